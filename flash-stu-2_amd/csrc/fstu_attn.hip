@@ -1,0 +1,289 @@
+// Sliding-window attention with ALiBi and tanh soft-capping: ring KV cache
+// maintenance, the single-query decode kernel and a simple prefill kernel.
+//
+// Work split: 8 lanes share one key (each lane owns hd/8 head dims), so a wave
+// visits 8 keys at a time and a lane reads 16..64 contiguous bytes per key.
+// Each 8-lane group keeps an online-softmax partial (max, sum, weighted V);
+// partials are merged through LDS at the end.
+#include "fstu_common.h"
+
+template <typename T, int N>
+__device__ __forceinline__ void load_vec(const T* p, float* o);
+
+template <> __device__ __forceinline__ void load_vec<bf16_t, 4>(const bf16_t* p, float* o) {
+  uint2 v = *(const uint2*)p;
+  o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+  o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void load_vec<bf16_t, 8>(const bf16_t* p, float* o) {
+  uint4 v = *(const uint4*)p;
+  unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(w[i] << 16); o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+}
+template <> __device__ __forceinline__ void load_vec<bf16_t, 16>(const bf16_t* p, float* o) {
+  load_vec<bf16_t, 8>(p, o);
+  load_vec<bf16_t, 8>(p + 8, o + 8);
+}
+template <> __device__ __forceinline__ void load_vec<bf16_t, 32>(const bf16_t* p, float* o) {
+  load_vec<bf16_t, 16>(p, o);
+  load_vec<bf16_t, 16>(p + 16, o + 16);
+}
+template <> __device__ __forceinline__ void load_vec<float, 4>(const float* p, float* o) {
+  float4 v = *(const float4*)p;
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+template <> __device__ __forceinline__ void load_vec<float, 8>(const float* p, float* o) {
+  load_vec<float, 4>(p, o); load_vec<float, 4>(p + 4, o + 4);
+}
+template <> __device__ __forceinline__ void load_vec<float, 16>(const float* p, float* o) {
+  load_vec<float, 8>(p, o); load_vec<float, 8>(p + 8, o + 8);
+}
+template <> __device__ __forceinline__ void load_vec<float, 32>(const float* p, float* o) {
+  load_vec<float, 16>(p, o); load_vec<float, 16>(p + 16, o + 16);
+}
+
+// Online-softmax partial of one 8-lane key group.
+template <int DPL>
+struct Partial {
+  float m, l;
+  float acc[DPL];
+};
+
+// Visits keys j = jb+u (u<U) for jb = j_first, j_first+j_step, ... < j_end.
+// kb/vb point at this lane's dims of slot 0; consecutive slots are `stride`
+// elements apart; cap > 0 maps position j to slot j % cap.
+template <typename T, int DPL, int U>
+__device__ __forceinline__ void attend_keys(Partial<DPL>& P, const T* kb, const T* vb, size_t stride, int cap,
+                                            const float* q, int j_first, int j_end, int j_step, int pos, float scale,
+                                            float softcap, float slope) {
+  for (int jb = j_first; jb < j_end; jb += j_step) {
+    float kk[U][DPL], vv[U][DPL];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int j = jb + u;
+      if (j < j_end) {
+        size_t slot = cap > 0 ? (size_t)(j % cap) : (size_t)j;
+        load_vec<T, DPL>(kb + slot * stride, kk[u]);
+        load_vec<T, DPL>(vb + slot * stride, vv[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int j = jb + u;
+      const bool valid = j < j_end;  // uniform within the 8-lane group
+      float s = 0.f;
+      if (valid) {
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) s = fmaf(q[i], kk[u][i], s);
+      }
+      s += __shfl_xor(s, 1, FSTU_WAVE);
+      s += __shfl_xor(s, 2, FSTU_WAVE);
+      s += __shfl_xor(s, 4, FSTU_WAVE);
+      if (valid) {
+        s *= scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        s -= slope * (float)(pos - j);
+        float mn = fmaxf(P.m, s);
+        float corr = __expf(P.m - mn);
+        float p = __expf(s - mn);
+        P.l = P.l * corr + p;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) P.acc[i] = fmaf(p, vv[u][i], P.acc[i] * corr);
+        P.m = mn;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- ring maintenance
+template <typename T>
+__global__ void kv_fill_kernel(const T* __restrict__ qkv, T* __restrict__ kring, T* __restrict__ vring, int B, int Tn,
+                               int H, int hd, int cap, int pos0, int tstart) {
+  // one thread per (b, tt, h, i) over tt in [tstart, Tn)
+  const int d = H * hd;
+  size_t n = (size_t)B * (Tn - tstart) * d;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+    int i = idx % hd;
+    size_t r = idx / hd;
+    int h = r % H;
+    r /= H;
+    int tt = tstart + (int)(r % (Tn - tstart));
+    int b = (int)(r / (Tn - tstart));
+    const T* src = qkv + ((size_t)b * Tn + tt) * 3 * d + h * hd + i;
+    int slot = (pos0 + tt) % cap;
+    size_t dst = (((size_t)b * H + h) * cap + slot) * hd + i;
+    kring[dst] = src[d];
+    vring[dst] = src[2 * d];
+  }
+}
+
+static int check_kv(const char* name, const void* a, const void* b, const void* c, int B, int H, int hd, int cap) {
+  FSTU_REQUIRE(a && b && c, FSTU_ENULL, "%s: null pointer", name);
+  FSTU_REQUIRE(B >= 1 && H >= 1 && hd >= 1 && cap >= 1, FSTU_ESHAPE, "%s: bad shape B=%d H=%d hd=%d cap=%d", name, B, H, hd, cap);
+  return FSTU_OK;
+}
+
+extern "C" int fstu_kv_fill(const void* qkv, void* kring, void* vring, int B, int T_, int H, int hd, int cap, int pos0,
+                            int dtype, void* stream) {
+  int rc = check_kv("fstu_kv_fill", qkv, kring, vring, B, H, hd, cap);
+  if (rc) return rc;
+  FSTU_REQUIRE(T_ >= 1 && pos0 >= 0, FSTU_EARG, "fstu_kv_fill: T=%d pos0=%d", T_, pos0);
+  int tstart = T_ > cap ? T_ - cap : 0;
+  size_t n = (size_t)B * (T_ - tstart) * H * hd;
+  unsigned blocks = (unsigned)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_kv_fill",
+                      hipLaunchKernelGGL(kv_fill_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                                         (const T*)qkv, (T*)kring, (T*)vring, B, T_, H, hd, cap, pos0, tstart));
+  FSTU_CHECK_LAUNCH("fstu_kv_fill");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, int H, int hd, int cap, int pos,
+                              int dtype, void* stream) {
+  FSTU_REQUIRE(pos >= 0, FSTU_EARG, "fstu_kv_append: pos<0");
+  return fstu_kv_fill(qkv, kring, vring, B, 1, H, hd, cap, pos, dtype, stream);
+}
+
+// ---------------------------------------------------------------- decode
+#define SWA_U 4
+template <typename T, int HD>
+__global__ void __launch_bounds__(256)
+swa_decode_kernel(const T* __restrict__ qkv, const T* __restrict__ kring, const T* __restrict__ vring,
+                  T* __restrict__ out, const float* __restrict__ slopes, int H, int cap, int pos, int window,
+                  float softcap) {
+  constexpr int DPL = HD / 8;
+  __shared__ float sm[32], sl[32];
+  __shared__ float sacc[32][HD];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int grp = lane >> 3, gl = lane & 7;
+  const int G = w * 8 + grp;  // group index 0..31
+  const int d = H * HD;
+  float q[DPL];
+  load_vec<T, DPL>(qkv + (size_t)b * 3 * d + h * HD + gl * DPL, q);
+  const size_t base = ((size_t)b * H + h) * cap * HD + gl * DPL;
+  Partial<DPL> P;
+  P.m = -INFINITY;
+  P.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
+  const int lo = max(0, pos - window);
+  attend_keys<T, DPL, SWA_U>(P, kring + base, vring + base, HD, cap, q, lo + G * SWA_U, pos + 1, 32 * SWA_U, pos,
+                             rsqrtf((float)HD), softcap, slopes[h]);
+  if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];
+  __syncthreads();
+  if (threadIdx.x < HD) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < 32; ++g) M = fmaxf(M, sm[g]);
+    float Lsum = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < 32; ++g) {
+      float e = __expf(sm[g] - M);
+      Lsum = fmaf(sl[g], e, Lsum);
+      o = fmaf(sacc[g][threadIdx.x], e, o);
+    }
+    DT<T>::st(out + (size_t)b * d + h * HD + threadIdx.x, o / Lsum);
+  }
+}
+
+static int check_swa(const char* name, int H, int hd, int window, const void* slopes) {
+  FSTU_REQUIRE(slopes, FSTU_ENULL, "%s: slopes is null", name);
+  FSTU_REQUIRE(hd == 32 || hd == 64 || hd == 128 || hd == 256, FSTU_ESHAPE, "%s: head dim %d not in {32,64,128,256}", name, hd);
+  FSTU_REQUIRE(window >= 0, FSTU_EARG, "%s: window<0", name);
+  return FSTU_OK;
+}
+
+#define SWA_DISPATCH_HD(KERNEL, hd, ...)                                   \
+  do {                                                                     \
+    if (hd == 32) hipLaunchKernelGGL((KERNEL<T, 32>), __VA_ARGS__);        \
+    else if (hd == 64) hipLaunchKernelGGL((KERNEL<T, 64>), __VA_ARGS__);   \
+    else if (hd == 128) hipLaunchKernelGGL((KERNEL<T, 128>), __VA_ARGS__); \
+    else hipLaunchKernelGGL((KERNEL<T, 256>), __VA_ARGS__);                \
+  } while (0)
+
+extern "C" int fstu_swa_decode(const void* qkv, const void* kring, const void* vring, void* out, const float* slopes,
+                               int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
+                               void* stream) {
+  int rc = check_kv("fstu_swa_decode", qkv, kring, vring, B, H, hd, cap);
+  if (rc) return rc;
+  rc = check_swa("fstu_swa_decode", H, hd, window, slopes);
+  if (rc) return rc;
+  FSTU_REQUIRE(out, FSTU_ENULL, "fstu_swa_decode: out is null");
+  FSTU_REQUIRE(pos >= 0 && cap >= window + 1, FSTU_EARG, "fstu_swa_decode: pos=%d, ring capacity %d < window+1=%d", pos, cap, window + 1);
+  FSTU_REQUIRE(fstu_aligned(qkv, 16) && fstu_aligned(kring, 16) && fstu_aligned(vring, 16), FSTU_EALIGN, "fstu_swa_decode: pointers must be 16-byte aligned");
+  FSTU_REQUIRE(B <= 65535, FSTU_ESHAPE, "fstu_swa_decode: B too large");
+  hipStream_t s = (hipStream_t)stream;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_decode",
+                      SWA_DISPATCH_HD(swa_decode_kernel, hd, dim3(H, B), dim3(256), 0, s, (const T*)qkv,
+                                      (const T*)kring, (const T*)vring, (T*)out, slopes, H, cap, pos, window, softcap));
+  FSTU_CHECK_LAUNCH("fstu_swa_decode");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- prefill
+// One wave per (batch, head, query); 4 queries per workgroup.
+template <typename T, int HD>
+__global__ void __launch_bounds__(256)
+swa_prefill_kernel(const T* __restrict__ qkv, T* __restrict__ out, const float* __restrict__ slopes, int Tn, int H,
+                   int window, float softcap) {
+  constexpr int DPL = HD / 8;
+  __shared__ float sm[4][8], sl[4][8];
+  __shared__ float sacc[4][8][HD];
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int grp = lane >> 3, gl = lane & 7;
+  const int t = blockIdx.x * 4 + w;
+  const int d = H * HD;
+  const bool live = t < Tn;
+  Partial<DPL> P;
+  P.m = -INFINITY;
+  P.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
+  if (live) {
+    float q[DPL];
+    const T* row0 = qkv + (size_t)b * Tn * 3 * d + h * HD + gl * DPL;
+    load_vec<T, DPL>(row0 + (size_t)t * 3 * d, q);
+    const int lo = max(0, t - window);
+    attend_keys<T, DPL, SWA_U>(P, row0 + d, row0 + 2 * d, (size_t)3 * d, 0, q, lo + grp * SWA_U, t + 1, 8 * SWA_U, t,
+                               rsqrtf((float)HD), softcap, slopes[h]);
+  }
+  if (gl == 0) { sm[w][grp] = P.m; sl[w][grp] = P.l; }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) sacc[w][grp][gl * DPL + i] = P.acc[i];
+  __syncthreads();
+  if (live) {
+    for (int i = lane; i < HD; i += 64) {
+      float M = -INFINITY;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) M = fmaxf(M, sm[w][g]);
+      float Lsum = 0.f, o = 0.f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        float e = __expf(sm[w][g] - M);
+        Lsum = fmaf(sl[w][g], e, Lsum);
+        o = fmaf(sacc[w][g][i], e, o);
+      }
+      DT<T>::st(out + ((size_t)b * Tn + t) * d + h * HD + i, o / Lsum);
+    }
+  }
+}
+
+extern "C" int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T_, int H, int hd,
+                                int window, float softcap, int dtype, void* stream) {
+  FSTU_REQUIRE(qkv && out, FSTU_ENULL, "fstu_swa_prefill: null pointer");
+  FSTU_REQUIRE(B >= 1 && T_ >= 1 && H >= 1 && B <= 65535 && H <= 65535, FSTU_ESHAPE, "fstu_swa_prefill: bad shape B=%d T=%d H=%d", B, T_, H);
+  int rc = check_swa("fstu_swa_prefill", H, hd, window, slopes);
+  if (rc) return rc;
+  FSTU_REQUIRE(fstu_aligned(qkv, 16), FSTU_EALIGN, "fstu_swa_prefill: qkv must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_prefill",
+                      SWA_DISPATCH_HD(swa_prefill_kernel, hd, dim3((T_ + 3) / 4, H, B), dim3(256), 0, s,
+                                      (const T*)qkv, (T*)out, slopes, T_, H, window, softcap));
+  FSTU_CHECK_LAUNCH("fstu_swa_prefill");
+  return FSTU_OK;
+}

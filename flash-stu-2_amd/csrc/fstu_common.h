@@ -1,0 +1,91 @@
+// Shared device/host helpers for the gfx950 kernels of libflashstu_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/flashstu_hip.h"
+
+#define FSTU_WAVE 64
+
+// ---------------------------------------------------------------- errors
+void fstu_set_error(const char* fmt, ...);
+
+#define FSTU_REQUIRE(cond, code, ...)                 \
+  do {                                                \
+    if (!(cond)) {                                    \
+      fstu_set_error(__VA_ARGS__);                    \
+      return (code);                                  \
+    }                                                 \
+  } while (0)
+
+#define FSTU_CHECK_LAUNCH(name)                                           \
+  do {                                                                    \
+    hipError_t e__ = hipGetLastError();                                   \
+    if (e__ != hipSuccess) {                                              \
+      fstu_set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+      return (int)e__;                                                    \
+    }                                                                     \
+  } while (0)
+
+static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// ---------------------------------------------------------------- dtypes
+typedef unsigned short bf16_t;  // raw bf16 bits
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((unsigned)v) << 16); }
+
+// round-to-nearest-even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct DT;
+template <> struct DT<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+};
+template <> struct DT<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+  static __device__ __forceinline__ float rnd(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+// ---------------------------------------------------------------- wave ops
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, FSTU_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, FSTU_WAVE));
+  return v;
+}
+
+// tanh-approximated GELU as torch evaluates it in fp32
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+  const float kBeta = 0.7978845608028654f;  // sqrt(2/pi)
+  const float kKappa = 0.044715f;
+  float inner = kBeta * (x + kKappa * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+#define FSTU_DISPATCH_DTYPE(dtype, NAME, ...)                      \
+  do {                                                             \
+    if ((dtype) == FSTU_F32) {                                     \
+      typedef float T;                                             \
+      __VA_ARGS__;                                                 \
+    } else if ((dtype) == FSTU_BF16) {                             \
+      typedef bf16_t T;                                            \
+      __VA_ARGS__;                                                 \
+    } else {                                                       \
+      fstu_set_error("%s: unknown dtype %d", NAME, (int)(dtype));  \
+      return FSTU_EDTYPE;                                          \
+    }                                                              \
+  } while (0)

@@ -1,0 +1,408 @@
+// Error reporting, embedding gather, fused residual + RMSNorm, GELU-gate and
+// the sampling kernel.  All bandwidth-bound, one workgroup per row.
+#include "fstu_common.h"
+#include <string.h>
+
+// ---------------------------------------------------------------- errors
+static thread_local char g_err[512] = "";
+
+void fstu_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* fstu_last_error(void) { return g_err; }
+extern "C" int fstu_version(void) { return FSTU_VERSION; }
+
+// ---------------------------------------------------------------- embed
+template <typename T>
+__global__ void embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
+                             int d, int vocab) {
+  int r = blockIdx.x;
+  int64_t id = ids[r];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* src = table + (size_t)id * d;
+  T* dst = out + (size_t)r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int fstu_embed(const int64_t* ids, const void* table, void* out, int rows, int d, int vocab, int dtype,
+                          void* stream) {
+  FSTU_REQUIRE(ids && table && out, FSTU_ENULL, "fstu_embed: null pointer");
+  FSTU_REQUIRE(rows >= 0 && d > 0 && vocab > 0, FSTU_ESHAPE, "fstu_embed: bad shape rows=%d d=%d vocab=%d", rows, d, vocab);
+  if (rows == 0) return FSTU_OK;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_embed",
+                      hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids,
+                                         (const T*)table, (T*)out, d, vocab));
+  FSTU_CHECK_LAUNCH("fstu_embed");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- add + rmsnorm
+// One workgroup (256 threads) per row; the row lives in registers between the
+// residual update and the normalisation.  d <= 256*FSTU_NORM_MAX_PER_THREAD.
+#define FSTU_NORM_THREADS 256
+#define FSTU_NORM_MAX_PER_THREAD 32
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float s = red[0] + red[1] + red[2] + red[3];
+  __syncthreads();
+  return s;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(FSTU_NORM_THREADS)
+add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_mode, int nslices, int single_branch,
+                   const T* __restrict__ w, T* __restrict__ y, int rows, int d, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  T* xr = x + (size_t)r * d;
+  float v[FSTU_NORM_MAX_PER_THREAD];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < FSTU_NORM_MAX_PER_THREAD; ++i) {
+    int c = threadIdx.x + i * FSTU_NORM_THREADS;
+    v[i] = 0.f;
+    if (c < d) {
+      float xv = DT<T>::ld(xr + c);
+      if (delta != nullptr) {
+        float dv;
+        if (delta_mode == 0) {
+          dv = DT<T>::ld((const T*)delta + (size_t)r * d + c);
+        } else if (delta_mode == 1) {
+          const float* p = (const float*)delta + (size_t)r * d + c;
+          float acc = 0.f;
+          for (int s = 0; s < nslices; ++s) acc += p[(size_t)s * rows * d];
+          dv = DT<T>::rnd(acc);
+        } else {
+          const float* p = (const float*)delta + (size_t)r * d + c;
+          float e = 0.f, o = 0.f;
+          for (int s = 0; s < nslices; ++s) {
+            e += p[(size_t)(2 * s) * rows * d];
+            o += p[(size_t)(2 * s + 1) * rows * d];
+          }
+          dv = single_branch ? DT<T>::rnd(e + o) : DT<T>::rnd(DT<T>::rnd(e + o) + DT<T>::rnd(e - o));
+        }
+        xv = DT<T>::rnd(xv + dv);
+        DT<T>::st(xr + c, xv);
+      }
+      v[i] = xv;
+      ss += xv * xv;
+    }
+  }
+  if (y == nullptr) return;
+  float tot = block_sum_256(ss, red);
+  float rstd = rsqrtf(tot / (float)d + eps);
+  T* yr = y + (size_t)r * d;
+#pragma unroll
+  for (int i = 0; i < FSTU_NORM_MAX_PER_THREAD; ++i) {
+    int c = threadIdx.x + i * FSTU_NORM_THREADS;
+    if (c < d) DT<T>::st(yr + c, (v[i] * rstd) * DT<T>::ld(w + c));
+  }
+}
+
+extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch,
+                                const void* w, void* y, int rows, int d, float eps, int dtype, void* stream) {
+  FSTU_REQUIRE(x, FSTU_ENULL, "fstu_add_rmsnorm: x is null");
+  FSTU_REQUIRE((y == nullptr) || (w != nullptr), FSTU_ENULL, "fstu_add_rmsnorm: y given without weight");
+  FSTU_REQUIRE(delta || y, FSTU_EARG, "fstu_add_rmsnorm: nothing to do (no delta and no y)");
+  FSTU_REQUIRE(rows >= 0 && d > 0 && d <= FSTU_NORM_THREADS * FSTU_NORM_MAX_PER_THREAD, FSTU_ESHAPE,
+               "fstu_add_rmsnorm: d=%d out of range (1..%d)", d, FSTU_NORM_THREADS * FSTU_NORM_MAX_PER_THREAD);
+  FSTU_REQUIRE(delta_mode >= 0 && delta_mode <= 2, FSTU_EARG, "fstu_add_rmsnorm: delta_mode=%d", delta_mode);
+  FSTU_REQUIRE(delta == nullptr || delta_mode == 0 || nslices >= 1, FSTU_EARG, "fstu_add_rmsnorm: nslices=%d", nslices);
+  if (rows == 0) return FSTU_OK;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_add_rmsnorm",
+                      hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(rows), dim3(FSTU_NORM_THREADS), 0,
+                                         (hipStream_t)stream, (T*)x, delta, delta_mode, nslices, single_branch,
+                                         (const T*)w, (T*)y, rows, d, eps));
+  FSTU_CHECK_LAUNCH("fstu_add_rmsnorm");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- gelu * up
+template <typename T>
+__global__ void gelu_mul_kernel(const T* __restrict__ g, const T* __restrict__ u, T* __restrict__ act, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    float ge = DT<T>::rnd(gelu_tanh_f32(DT<T>::ld(g + i)));
+    DT<T>::st(act + i, ge * DT<T>::ld(u + i));
+  }
+}
+
+extern "C" int fstu_gelu_mul(const void* g, const void* u, void* act, int64_t n, int dtype, void* stream) {
+  FSTU_REQUIRE(g && u && act, FSTU_ENULL, "fstu_gelu_mul: null pointer");
+  FSTU_REQUIRE(n >= 0, FSTU_ESHAPE, "fstu_gelu_mul: n<0");
+  if (n == 0) return FSTU_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_gelu_mul",
+                      hipLaunchKernelGGL(gelu_mul_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                                         (const T*)g, (const T*)u, (T*)act, n));
+  FSTU_CHECK_LAUNCH("fstu_gelu_mul");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- sampling
+// One workgroup of 1024 threads per row; the row (V logits) is re-read from
+// L2 in each pass instead of being staged.
+#define FSTU_SAMPLE_THREADS 1024
+
+struct SampleShared {
+  float redf[16];
+  int redi[16];
+  double redd[16];
+  unsigned hist[256];
+  unsigned long long mass[256];
+  unsigned sel_prefix;
+  unsigned sel_k;
+  unsigned long long sel_mass;
+  int bcast_i;
+  double bcast_d;
+};
+
+__device__ __forceinline__ unsigned f32_key(float f) {  // larger float -> larger key
+  unsigned u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_f32(unsigned k) {
+  unsigned u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+template <typename T>
+__device__ __forceinline__ float sample_transform(const T* row, int i, float inv_temp_is_one, float temperature) {
+  float x = DT<T>::ld(row + i);
+  if (!inv_temp_is_one) x = DT<T>::rnd(x / temperature);
+  x = fminf(fmaxf(x, -1e4f), 1e4f);
+  return DT<T>::rnd(x);
+}
+
+__device__ __forceinline__ double block_excl_scan_d(double v, double* red, double* total) {
+  // exclusive scan over 1024 threads (16 waves), fixed order
+  int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  double inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    double t = __shfl_up(inc, o, FSTU_WAVE);
+    if (lane >= o) inc += t;
+  }
+  if (lane == 63) red[w] = inc;
+  __syncthreads();
+  double base = 0.0, tot = 0.0;
+  for (int i = 0; i < 16; ++i) {
+    if (i < w) base += red[i];
+    tot += red[i];
+  }
+  __syncthreads();
+  *total = tot;
+  return base + inc - v;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
+sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
+              int top_k, float top_p, int do_sample, uint64_t seed, int step) {
+  __shared__ SampleShared sh;
+  const int b = blockIdx.x;
+  const T* row = logits + (size_t)b * V;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const bool t1 = (temperature == 1.0f);
+
+  // ---- pass A: maximum (lowest index on ties) over a strided walk
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
+    float l = sample_transform(row, i, t1, temperature);
+    if (besti == 0x7fffffff || l > best) { best = l; besti = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ob = __shfl_xor(best, o, FSTU_WAVE);
+    int oi = __shfl_xor(besti, o, FSTU_WAVE);
+    if (ob > best || (ob == best && oi < besti)) { best = ob; besti = oi; }
+  }
+  if (lane == 0) { sh.redf[w] = best; sh.redi[w] = besti; }
+  __syncthreads();
+  if (tid == 0) {
+    float bb = sh.redf[0];
+    int bi = sh.redi[0];
+    for (int i = 1; i < 16; ++i)
+      if (sh.redf[i] > bb || (sh.redf[i] == bb && sh.redi[i] < bi)) { bb = sh.redf[i]; bi = sh.redi[i]; }
+    sh.redf[0] = bb;
+    sh.bcast_i = bi;
+  }
+  __syncthreads();
+  const float m = sh.redf[0];
+  const int arg = sh.bcast_i;
+  __syncthreads();
+  if (!do_sample) {
+    if (tid == 0) out[(size_t)b * out_stride] = arg;
+    return;
+  }
+
+  // ---- top-k threshold by radix select on the monotone key
+  unsigned thr_key = 0;  // keep keys >= thr_key
+  if (top_k > 0 && top_k < V) {
+    unsigned prefix = 0, kk = (unsigned)top_k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.hist[i] = 0;
+      __syncthreads();
+      unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
+      for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
+        unsigned k = f32_key(sample_transform(row, i, t1, temperature));
+        if ((k & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        unsigned acc = 0;
+        int bin = 255;
+        for (; bin > 0; --bin) {
+          if (acc + sh.hist[bin] >= kk) break;
+          acc += sh.hist[bin];
+        }
+        sh.sel_prefix = prefix | ((unsigned)bin << shift);
+        sh.sel_k = kk - acc;
+      }
+      __syncthreads();
+      prefix = sh.sel_prefix;
+      kk = sh.sel_k;
+      __syncthreads();
+    }
+    thr_key = prefix;
+  }
+
+  // ---- top-p over the survivors
+  // kept set = {key > vb} U {key == vb with tie rank < tie_keep}
+  unsigned vb_key = thr_key;
+  long long tie_keep = -1;  // -1: keep every tied token
+  if (top_p > 0.f && top_p < 1.f) {
+    double e = 0.0;
+    for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
+      float l = sample_transform(row, i, t1, temperature);
+      if (f32_key(l) >= thr_key) e += (double)expf(l - m);
+    }
+    double Z1;
+    block_excl_scan_d(e, sh.redd, &Z1);
+    const double scale = 17592186044416.0 / Z1;  // 2^44 / Z1: fixed-point probabilities
+    const unsigned long long target = (unsigned long long)((double)top_p * 17592186044416.0);
+    unsigned prefix = 0;
+    unsigned long long above = 0;  // mass of keys strictly above the current prefix range
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.mass[i] = 0ull;
+      __syncthreads();
+      unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
+      for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
+        float l = sample_transform(row, i, t1, temperature);
+        unsigned k = f32_key(l);
+        if (k >= thr_key && (k & himask) == (prefix & himask))
+          atomicAdd(&sh.mass[(k >> shift) & 255u], (unsigned long long)((double)expf(l - m) * scale));
+      }
+      __syncthreads();
+      if (tid == 0) {
+        // lowest bin whose strictly-above mass is still <= target
+        unsigned long long acc = above;
+        int bin = 255;
+        for (; bin > 0; --bin) {
+          if (acc + sh.mass[bin] > target) break;  // bins below `bin` have mass-above > target
+          acc += sh.mass[bin];
+        }
+        sh.sel_prefix = prefix | ((unsigned)bin << shift);
+        sh.sel_mass = acc;
+      }
+      __syncthreads();
+      prefix = sh.sel_prefix;
+      above = sh.sel_mass;
+      __syncthreads();
+    }
+    // prefix = boundary key vb: mass strictly above it is `above` (<= target);
+    // tokens tied at vb are kept while above + rank*p_b <= target.
+    if (prefix >= thr_key) {
+      vb_key = prefix;
+      float lb = key_f32(vb_key);
+      unsigned long long pb = (unsigned long long)((double)expf(lb - m) * scale);
+      if (pb == 0ull) pb = 1ull;
+      tie_keep = (long long)((target - above) / pb) + 1;  // above <= target by construction
+    }  // else: top-p keeps every top-k survivor
+  }
+
+  // ---- draw: inverse CDF in index order over contiguous per-thread chunks
+  const int chunk = (V + FSTU_SAMPLE_THREADS - 1) / FSTU_SAMPLE_THREADS;
+  const int i0 = tid * chunk, i1 = min(V, i0 + chunk);
+  // tie ranks need an index-ordered count of tokens equal to vb
+  double tcount = 0.0;
+  if (tie_keep >= 0)
+    for (int i = i0; i < i1; ++i)
+      if (f32_key(sample_transform(row, i, t1, temperature)) == vb_key) tcount += 1.0;
+  double ttotal = 0.0;
+  double tbase = (tie_keep >= 0) ? block_excl_scan_d(tcount, sh.redd, &ttotal) : 0.0;
+  double mysum = 0.0;
+  {
+    long long rank = (long long)tbase;
+    for (int i = i0; i < i1; ++i) {
+      float l = sample_transform(row, i, t1, temperature);
+      unsigned k = f32_key(l);
+      bool keep = k > vb_key;
+      if (k == vb_key) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
+      if (keep) mysum += (double)expf(l - m);
+    }
+  }
+  double Z;
+  double mybase = block_excl_scan_d(mysum, sh.redd, &Z);
+  // counter-based uniform (splitmix64 finaliser), 24 bits
+  unsigned long long z = seed * 0x9E3779B97F4A7C15ull + (unsigned long long)step * 0xBF58476D1CE4E5B9ull +
+                         (unsigned long long)b * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z = z ^ (z >> 31);
+  const double u = (double)(z >> 40) / 16777216.0;
+  const double tgt = u * Z;
+  if (tid == 0) sh.bcast_i = -1;
+  __syncthreads();
+  if (mysum > 0.0 && tgt >= mybase && tgt < mybase + mysum) {
+    double acc = mybase;
+    long long rank = (long long)tbase;
+    int pick = -1, lastkept = -1;
+    for (int i = i0; i < i1; ++i) {
+      float l = sample_transform(row, i, t1, temperature);
+      unsigned k = f32_key(l);
+      bool keep = k > vb_key;
+      if (k == vb_key) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
+      if (keep) {
+        acc += (double)expf(l - m);
+        lastkept = i;
+        if (acc > tgt) { pick = i; break; }
+      }
+    }
+    if (pick < 0) pick = lastkept;
+    sh.bcast_i = pick;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pick = sh.bcast_i;
+    if (pick < 0) pick = arg;  // rounding left the target past the last chunk
+    out[(size_t)b * out_stride] = pick;
+  }
+}
+
+extern "C" int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature,
+                           int top_k, float top_p, int do_sample, uint64_t seed, int step, int dtype,
+                           void* stream) {
+  FSTU_REQUIRE(logits && out, FSTU_ENULL, "fstu_sample: null pointer");
+  FSTU_REQUIRE(B >= 0 && V > 0, FSTU_ESHAPE, "fstu_sample: bad shape B=%d V=%d", B, V);
+  FSTU_REQUIRE(temperature > 0.f, FSTU_EARG, "fstu_sample: temperature must be > 0");
+  FSTU_REQUIRE(out_stride >= 1, FSTU_EARG, "fstu_sample: out_stride < 1");
+  if (B == 0) return FSTU_OK;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_sample",
+                      hipLaunchKernelGGL(sample_kernel<T>, dim3(B), dim3(FSTU_SAMPLE_THREADS), 0, (hipStream_t)stream,
+                                         (const T*)logits, out, out_stride, V, temperature, top_k, top_p, do_sample,
+                                         seed, step));
+  FSTU_CHECK_LAUNCH("fstu_sample");
+  return FSTU_OK;
+}

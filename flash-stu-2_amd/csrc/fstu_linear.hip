@@ -1,0 +1,277 @@
+// Skinny linear layers for decode: up to 16 activation rows against an (N,K)
+// weight that is streamed from HBM exactly once.
+//
+// bf16 path: one wave owns a 16-feature row tile and a K range.  The weight
+// tile is the MFMA A operand (16 features x 32 k), the activations the B
+// operand (32 k x 16 batch rows, rows >= `rows` are zero), accumulated with
+// v_mfma_f32_16x16x32_bf16.  Within one 64-wide k step lane (r,g) reads the 32
+// contiguous bytes W[r, k+16g .. k+16g+15], so the four lanes of a row cover a
+// full 128-byte line; the two MFMAs of the step take the low and high 8
+// elements and the activation operand is permuted identically (a dot product
+// does not care about the order of k).
+// Waves of a workgroup that share a row tile but own different K ranges are
+// reduced through LDS in a fixed order, so results are deterministic.
+//
+// Other dtypes/shapes: a vector-ALU kernel, one wave per output feature.
+#include "fstu_common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+enum { LIN_PLAIN = 0, LIN_GLU = 1, LIN_PARTIAL = 2 };
+
+struct LinArgs {
+  const void* x;
+  int ldx;
+  const void* W;   // plain weight or gate weight
+  const void* W2;  // up weight (GLU)
+  void* y;         // T output (plain/GLU) or fp32 partial slices
+  int ldy;
+  int rows, N, K;
+  int kw;          // k range per wave
+};
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
+
+template <int KSW, int MODE>
+__global__ void __launch_bounds__(256)
+linear_mfma_bf16_kernel(LinArgs a) {
+  constexpr int RT = 4 / KSW;
+  constexpr int U = 4;  // k steps (of 64) whose loads are issued back to back
+  __shared__ float red[(KSW > 1) ? 4 * 64 * 4 * ((MODE == LIN_GLU) ? 2 : 1) : 1];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int rt = w / KSW, ks = w % KSW;
+  const int tile = blockIdx.x * RT + rt;
+  const int ntiles = (a.N + 15) >> 4;
+  const bool tile_ok = tile < ntiles;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = min(tile * 16 + r, a.N - 1);
+  const int k0 = (blockIdx.y * KSW + ks) * a.kw + g * 16;
+  const bf16_t* wp = (const bf16_t*)a.W + (size_t)max(n, 0) * a.K + k0;
+  const bf16_t* wp2 = (MODE == LIN_GLU) ? (const bf16_t*)a.W2 + (size_t)max(n, 0) * a.K + k0 : nullptr;
+  const bool xrow = r < a.rows;
+  const bf16_t* xp = (const bf16_t*)a.x + (size_t)(xrow ? r : 0) * a.ldx + k0;
+  floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  const int iters = a.kw >> 6;
+  if (tile_ok) {
+    for (int i0 = 0; i0 < iters; i0 += U) {
+      uint4 wa[U][2], wb[U][2], xa[U][2];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u < iters) {
+          const uint4* p = (const uint4*)(wp + (size_t)(i0 + u) * 64);
+          wa[u][0] = p[0];
+          wa[u][1] = p[1];
+          if (MODE == LIN_GLU) {
+            const uint4* p2 = (const uint4*)(wp2 + (size_t)(i0 + u) * 64);
+            wb[u][0] = p2[0];
+            wb[u][1] = p2[1];
+          }
+          if (xrow) {
+            const uint4* q = (const uint4*)(xp + (size_t)(i0 + u) * 64);
+            xa[u][0] = q[0];
+            xa[u][1] = q[1];
+          } else {
+            xa[u][0] = make_uint4(0, 0, 0, 0);
+            xa[u][1] = make_uint4(0, 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u < iters) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][0]), as_bf16x8(xa[u][0]), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][1]), as_bf16x8(xa[u][1]), acc, 0, 0, 0);
+          if (MODE == LIN_GLU) {
+            acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][0]), as_bf16x8(xa[u][0]), acc2, 0, 0, 0);
+            acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][1]), as_bf16x8(xa[u][1]), acc2, 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (KSW > 1) {
+    float* mine = red + (size_t)(w * 64 + lane) * 4;
+    constexpr int GLU_OFF = 4 * 64 * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      mine[i] = acc[i];
+      if (MODE == LIN_GLU) mine[GLU_OFF + i] = acc2[i];
+    }
+    __syncthreads();
+    if (ks != 0) return;
+#pragma unroll
+    for (int s = 1; s < KSW; ++s) {
+      const float* o = red + (size_t)((w + s) * 64 + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[i] += o[i];
+        if (MODE == LIN_GLU) acc2[i] += o[GLU_OFF + i];
+      }
+    }
+  }
+  if (!tile_ok) return;
+  // D layout: lane holds features 4*(lane/16)+i, batch row lane%16
+  const int b = r;
+  if (b >= a.rows) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int f = tile * 16 + g * 4 + i;
+    if (f >= a.N) continue;
+    if (MODE == LIN_PLAIN) {
+      ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(acc[i]);
+    } else if (MODE == LIN_GLU) {
+      float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[i])));
+      ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(ge * DT<bf16_t>::rnd(acc2[i]));
+    } else {
+      ((float*)a.y)[((size_t)blockIdx.y * a.rows + b) * a.N + f] = acc[i];
+    }
+  }
+}
+
+// Vector-ALU kernel: one wave per output feature (and K split), lanes stride
+// over k.  Any dtype, any K.
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+linear_valu_kernel(LinArgs a) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int n = blockIdx.x * 4 + w;
+  if (n >= a.N) return;
+  const int k0 = blockIdx.y * a.kw, k1 = min(a.K, k0 + a.kw);
+  const T* wr = (const T*)a.W + (size_t)n * a.K;
+  const T* wr2 = (MODE == LIN_GLU) ? (const T*)a.W2 + (size_t)n * a.K : nullptr;
+  const T* x = (const T*)a.x;
+  float acc[FSTU_MAX_DECODE_ROWS], acc2[FSTU_MAX_DECODE_ROWS];
+#pragma unroll
+  for (int b = 0; b < FSTU_MAX_DECODE_ROWS; ++b) { acc[b] = 0.f; acc2[b] = 0.f; }
+  for (int k = k0 + lane; k < k1; k += 64) {
+    float wv = DT<T>::ld(wr + k);
+    float wv2 = (MODE == LIN_GLU) ? DT<T>::ld(wr2 + k) : 0.f;
+#pragma unroll
+    for (int b = 0; b < FSTU_MAX_DECODE_ROWS; ++b) {
+      if (b < a.rows) {
+        float xv = DT<T>::ld(x + (size_t)b * a.ldx + k);
+        acc[b] = fmaf(wv, xv, acc[b]);
+        if (MODE == LIN_GLU) acc2[b] = fmaf(wv2, xv, acc2[b]);
+      }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < FSTU_MAX_DECODE_ROWS; ++b) {
+    if (b < a.rows) {
+      float s = wave_sum(acc[b]);
+      float s2 = (MODE == LIN_GLU) ? wave_sum(acc2[b]) : 0.f;
+      if (lane == 0) {
+        if (MODE == LIN_PLAIN) {
+          DT<T>::st((T*)a.y + (size_t)b * a.ldy + n, s);
+        } else if (MODE == LIN_GLU) {
+          float ge = DT<T>::rnd(gelu_tanh_f32(DT<T>::rnd(s)));
+          DT<T>::st((T*)a.y + (size_t)b * a.ldy + n, ge * DT<T>::rnd(s2));
+        } else {
+          ((float*)a.y)[((size_t)blockIdx.y * a.rows + b) * a.N + n] = s;
+        }
+      }
+    }
+  }
+}
+
+static int check_common(const char* name, const void* x, const void* W, const void* y, int ldx, int rows, int N, int K) {
+  FSTU_REQUIRE(x && W && y, FSTU_ENULL, "%s: null pointer", name);
+  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS, FSTU_ESHAPE, "%s: rows=%d outside 1..%d", name, rows,
+               FSTU_MAX_DECODE_ROWS);
+  FSTU_REQUIRE(N >= 1 && K >= 1, FSTU_ESHAPE, "%s: N=%d K=%d", name, N, K);
+  FSTU_REQUIRE(ldx >= K, FSTU_ESHAPE, "%s: ldx=%d < K=%d", name, ldx, K);
+  return FSTU_OK;
+}
+
+static bool mfma_ok(const void* x, int ldx, const void* W, const void* W2, int K, int ksplit) {
+  return K % (64 * ksplit) == 0 && ldx % 8 == 0 && fstu_aligned(x, 16) && fstu_aligned(W, 16) &&
+         (W2 == nullptr || fstu_aligned(W2, 16));
+}
+
+// in-workgroup K split: use the deepest split that keeps >= 128 k per wave
+static int pick_ksw(int N, int kper) {
+  int tiles = (N + 15) / 16;
+  if (kper % 256 == 0 && kper >= 512 && tiles < 4096) return 4;
+  if (kper % 128 == 0 && kper >= 256 && tiles < 8192) return 2;
+  return 1;
+}
+
+template <int MODE>
+static int launch_mfma(LinArgs a, int ksplit, hipStream_t s) {
+  int kper = a.K / ksplit;
+  int ksw = pick_ksw(a.N, kper);
+  a.kw = kper / ksw;
+  int tiles = (a.N + 15) / 16;
+  int rt = 4 / ksw;
+  dim3 grid((tiles + rt - 1) / rt, ksplit);
+  if (ksw == 4) hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, MODE>), grid, dim3(256), 0, s, a);
+  else if (ksw == 2) hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, MODE>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, MODE>), grid, dim3(256), 0, s, a);
+  return 0;
+}
+
+template <typename T, int MODE>
+static void launch_valu(LinArgs a, int ksplit, hipStream_t s) {
+  a.kw = (a.K + ksplit - 1) / ksplit;
+  dim3 grid((a.N + 3) / 4, ksplit);
+  hipLaunchKernelGGL((linear_valu_kernel<T, MODE>), grid, dim3(256), 0, s, a);
+}
+
+extern "C" int fstu_linear_decode(const void* x, int ldx, const void* W, void* y, int ldy, int rows, int N, int K,
+                                  int dtype, void* stream) {
+  int rc = check_common("fstu_linear_decode", x, W, y, ldx, rows, N, K);
+  if (rc) return rc;
+  FSTU_REQUIRE(ldy >= N, FSTU_ESHAPE, "fstu_linear_decode: ldy=%d < N=%d", ldy, N);
+  LinArgs a{x, ldx, W, nullptr, y, ldy, rows, N, K, K};
+  if (dtype == FSTU_BF16) {
+    if (mfma_ok(x, ldx, W, nullptr, K, 1)) launch_mfma<LIN_PLAIN>(a, 1, (hipStream_t)stream);
+    else launch_valu<bf16_t, LIN_PLAIN>(a, 1, (hipStream_t)stream);
+  } else if (dtype == FSTU_F32) {
+    launch_valu<float, LIN_PLAIN>(a, 1, (hipStream_t)stream);
+  } else {
+    fstu_set_error("fstu_linear_decode: unknown dtype %d", dtype);
+    return FSTU_EDTYPE;
+  }
+  FSTU_CHECK_LAUNCH("fstu_linear_decode");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_glu_decode(const void* x, int ldx, const void* Wg, const void* Wu, void* act, int ldact, int rows,
+                               int I, int K, int dtype, void* stream) {
+  int rc = check_common("fstu_glu_decode", x, Wg, act, ldx, rows, I, K);
+  if (rc) return rc;
+  FSTU_REQUIRE(Wu, FSTU_ENULL, "fstu_glu_decode: Wu is null");
+  FSTU_REQUIRE(ldact >= I, FSTU_ESHAPE, "fstu_glu_decode: ldact=%d < I=%d", ldact, I);
+  LinArgs a{x, ldx, Wg, Wu, act, ldact, rows, I, K, K};
+  if (dtype == FSTU_BF16) {
+    if (mfma_ok(x, ldx, Wg, Wu, K, 1)) launch_mfma<LIN_GLU>(a, 1, (hipStream_t)stream);
+    else launch_valu<bf16_t, LIN_GLU>(a, 1, (hipStream_t)stream);
+  } else if (dtype == FSTU_F32) {
+    launch_valu<float, LIN_GLU>(a, 1, (hipStream_t)stream);
+  } else {
+    fstu_set_error("fstu_glu_decode: unknown dtype %d", dtype);
+    return FSTU_EDTYPE;
+  }
+  FSTU_CHECK_LAUNCH("fstu_glu_decode");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, float* partial, int rows, int N, int K,
+                                         int ksplit, int dtype, void* stream) {
+  int rc = check_common("fstu_linear_decode_splitk", x, W, partial, ldx, rows, N, K);
+  if (rc) return rc;
+  FSTU_REQUIRE(ksplit >= 1 && ksplit <= 1024 && ksplit <= K, FSTU_EARG, "fstu_linear_decode_splitk: ksplit=%d", ksplit);
+  LinArgs a{x, ldx, W, nullptr, partial, N, rows, N, K, K};
+  if (dtype == FSTU_BF16) {
+    if (mfma_ok(x, ldx, W, nullptr, K, ksplit)) launch_mfma<LIN_PARTIAL>(a, ksplit, (hipStream_t)stream);
+    else launch_valu<bf16_t, LIN_PARTIAL>(a, ksplit, (hipStream_t)stream);
+  } else if (dtype == FSTU_F32) {
+    launch_valu<float, LIN_PARTIAL>(a, ksplit, (hipStream_t)stream);
+  } else {
+    fstu_set_error("fstu_linear_decode_splitk: unknown dtype %d", dtype);
+    return FSTU_EDTYPE;
+  }
+  FSTU_CHECK_LAUNCH("fstu_linear_decode_splitk");
+  return FSTU_OK;
+}

@@ -1,0 +1,336 @@
+// STU kernels: per-token decode step in the exact history form and in the
+// distilled diagonal-recurrence (LDS) form, the state builder that turns a
+// prefilled history into recurrence state, the time-domain prefill
+// convolution, and the dense LDS step of mini_stu.
+#include "fstu_common.h"
+
+// ---------------------------------------------------------------- history step
+// Lags are rows of the (lag, channel) plane; a workgroup walks a contiguous
+// lag range with all loads coalesced along channels.  Thread (row, chunk)
+// accumulates VEC channels for lags row, row+RW, ...; rows are then reduced
+// through LDS.  Even and odd lags are kept apart because the reference rounds
+// the two sign branches separately.
+template <typename T, int VEC>
+struct VecLd;
+template <> struct VecLd<bf16_t, 8> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* o) {
+    uint4 v = *(const uint4*)p;
+    unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __uint_as_float(w[i] << 16);
+      o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+template <> struct VecLd<float, 8> {
+  static __device__ __forceinline__ void ld(const float* p, float* o) {
+    float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+};
+template <typename T> struct VecLd<T, 1> {
+  static __device__ __forceinline__ void ld(const T* p, float* o) { o[0] = DT<T>::ld(p); }
+};
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+stu_step_hist_kernel(const T* __restrict__ hist, const T* __restrict__ filt, float* __restrict__ eo, int B, int d,
+                     int t, int cap, int nl, int per, int CW, int RW) {
+  __shared__ float sh[256 * 2 * VEC];
+  const int b = blockIdx.y, split = blockIdx.x;
+  const int nch = d / VEC;
+  const int chunk = blockIdx.z * CW + (threadIdx.x % CW);
+  const int row = threadIdx.x / CW;
+  const bool active = row < RW && chunk < nch;
+  float aE[VEC], aO[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) { aE[v] = 0.f; aO[v] = 0.f; }
+  const int lag0 = split * per, lag1 = min(nl, lag0 + per);
+  if (active) {
+    const T* hb = hist + ((size_t)b * cap + t) * d + (size_t)chunk * VEC;
+    const T* fb = filt + (size_t)chunk * VEC;
+#pragma unroll 4
+    for (int lag = lag0 + row; lag < lag1; lag += RW) {
+      float h[VEC], f[VEC];
+      VecLd<T, VEC>::ld(hb - (size_t)lag * d, h);
+      VecLd<T, VEC>::ld(fb + (size_t)lag * d, f);
+      if (lag & 1) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) aO[v] = fmaf(f[v], h[v], aO[v]);
+      } else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) aE[v] = fmaf(f[v], h[v], aE[v]);
+      }
+    }
+  }
+  float* mine = sh + (size_t)threadIdx.x * 2 * VEC;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) { mine[v] = aE[v]; mine[VEC + v] = aO[v]; }
+  __syncthreads();
+  if (active && row == 0) {
+    for (int r2 = 1; r2 < RW; ++r2) {
+      const float* o = sh + (size_t)(r2 * CW + (threadIdx.x % CW)) * 2 * VEC;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { aE[v] += o[v]; aO[v] += o[VEC + v]; }
+    }
+    float* pe = eo + ((size_t)(2 * split) * B + b) * d + (size_t)chunk * VEC;
+    float* po = eo + ((size_t)(2 * split + 1) * B + b) * d + (size_t)chunk * VEC;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { pe[v] = aE[v]; po[v] = aO[v]; }
+  }
+}
+
+extern "C" int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int d, int t, int cap, int L,
+                                  int nsplit, int dtype, void* stream) {
+  FSTU_REQUIRE(hist && filt && eo, FSTU_ENULL, "fstu_stu_step_hist: null pointer");
+  FSTU_REQUIRE(B >= 1 && d >= 1 && L >= 1 && cap >= 1, FSTU_ESHAPE, "fstu_stu_step_hist: bad shape B=%d d=%d L=%d cap=%d", B, d, L, cap);
+  FSTU_REQUIRE(t >= 0 && t < cap, FSTU_EARG, "fstu_stu_step_hist: t=%d outside history capacity %d", t, cap);
+  FSTU_REQUIRE(nsplit >= 1 && nsplit <= 4096, FSTU_EARG, "fstu_stu_step_hist: nsplit=%d", nsplit);
+  const int nl = (t + 1 < L) ? t + 1 : L;
+  const int per = (nl + nsplit - 1) / nsplit;
+  const bool vec8 = (d % 8 == 0) && fstu_aligned(hist, 16) && fstu_aligned(filt, 16);
+  const int nch = vec8 ? d / 8 : d;
+  const int CW = nch < 256 ? nch : 256;
+  const int RW = 256 / CW;
+  dim3 grid(nsplit, B, (nch + CW - 1) / CW);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == FSTU_BF16) {
+    if (vec8) hipLaunchKernelGGL((stu_step_hist_kernel<bf16_t, 8>), grid, dim3(256), 0, s, (const bf16_t*)hist, (const bf16_t*)filt, eo, B, d, t, cap, nl, per, CW, RW);
+    else hipLaunchKernelGGL((stu_step_hist_kernel<bf16_t, 1>), grid, dim3(256), 0, s, (const bf16_t*)hist, (const bf16_t*)filt, eo, B, d, t, cap, nl, per, CW, RW);
+  } else if (dtype == FSTU_F32) {
+    if (vec8) hipLaunchKernelGGL((stu_step_hist_kernel<float, 8>), grid, dim3(256), 0, s, (const float*)hist, (const float*)filt, eo, B, d, t, cap, nl, per, CW, RW);
+    else hipLaunchKernelGGL((stu_step_hist_kernel<float, 1>), grid, dim3(256), 0, s, (const float*)hist, (const float*)filt, eo, B, d, t, cap, nl, per, CW, RW);
+  } else {
+    fstu_set_error("fstu_stu_step_hist: unknown dtype %d", dtype);
+    return FSTU_EDTYPE;
+  }
+  FSTU_CHECK_LAUNCH("fstu_stu_step_hist");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- LDS-form step
+// Workgroup = 32 channel quads (128 channels) x 8 mode groups.  Each thread
+// advances S/8 modes of 4 channels (float4 state accesses, 512 contiguous
+// bytes per mode row and wave half), then the 8 mode groups are reduced in LDS.
+#define LDS_JG 8
+template <typename T>
+__global__ void __launch_bounds__(256)
+stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
+                    const float* __restrict__ ce, T* __restrict__ y, int ldy, int S, int d, int parity) {
+  __shared__ float sh[LDS_JG][32][4];
+  const int b = blockIdx.y;
+  const int q = threadIdx.x & 31, jg = threadIdx.x >> 5;
+  const int c = (blockIdx.x * 32 + q) * 4;
+  const bool ok = c < d;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (ok) {
+    float x[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) x[v] = DT<T>::ld(xp + (size_t)b * ldxp + c + v);
+    float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
+#pragma unroll 4
+    for (int j = jg; j < S; j += LDS_JG) {
+      float4 h = *(float4*)(st + (size_t)j * d);
+      const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
+      const float aj = a[j];
+      h.x = fmaf(aj, h.x, x[0]);
+      h.y = fmaf(aj, h.y, x[1]);
+      h.z = fmaf(aj, h.z, x[2]);
+      h.w = fmaf(aj, h.w, x[3]);
+      *(float4*)(st + (size_t)j * d) = h;
+      acc[0] = fmaf(cj.x, h.x, acc[0]);
+      acc[1] = fmaf(cj.y, h.y, acc[1]);
+      acc[2] = fmaf(cj.z, h.z, acc[2]);
+      acc[3] = fmaf(cj.w, h.w, acc[3]);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) sh[jg][q][v] = acc[v];
+  __syncthreads();
+  if (jg == 0 && ok) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < LDS_JG; ++g) s += sh[g][q][v];
+      DT<T>::st(y + (size_t)b * ldy + c + v, 2.0f * s);
+    }
+  }
+}
+
+extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y,
+                                 int ldy, int B, int S, int d, int t, int dtype, void* stream) {
+  FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
+  FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
+  FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
+  FSTU_REQUIRE(t >= 0, FSTU_EARG, "fstu_stu_step_lds: t<0");
+  FSTU_REQUIRE(fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_step_lds: state/ce must be 16-byte aligned");
+  dim3 grid((d / 4 + 31) / 32, B);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
+                      hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
+                                         (const T*)xp, ldxp, a, ce, (T*)y, ldy, S, d, t & 1));
+  FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- state from history
+#define LSH_JG 4
+#define LSH_MAXJ 32
+template <typename T>
+__global__ void __launch_bounds__(256)
+lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__ a, float* __restrict__ state, int S,
+                           int d, int t_last, int cap) {
+  const int b = blockIdx.y, p = blockIdx.z;
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int jg = threadIdx.x >> 6;
+  const int per = (S + LSH_JG - 1) / LSH_JG;
+  const int j0 = jg * per;
+  if (c >= d) return;
+  float h[LSH_MAXJ], aj[LSH_MAXJ];
+#pragma unroll
+  for (int i = 0; i < LSH_MAXJ; ++i) {
+    h[i] = 0.f;
+    aj[i] = (i < per && j0 + i < S) ? a[j0 + i] : 0.f;
+  }
+  const T* hb = hist + (size_t)b * cap * d + c;
+  for (int tt = p; tt <= t_last; tt += 2) {
+    float x = DT<T>::ld(hb + (size_t)tt * d);
+#pragma unroll
+    for (int i = 0; i < LSH_MAXJ; ++i) h[i] = fmaf(aj[i], h[i], x);
+  }
+  float* st = state + (((size_t)b * 2 + p) * S) * d + c;
+#pragma unroll
+  for (int i = 0; i < LSH_MAXJ; ++i)
+    if (i < per && j0 + i < S) st[(size_t)(j0 + i) * d] = h[i];
+}
+
+extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, float* state, int B, int S, int d,
+                                            int t_last, int cap, int dtype, void* stream) {
+  FSTU_REQUIRE(hist && a && state, FSTU_ENULL, "fstu_stu_lds_state_from_hist: null pointer");
+  FSTU_REQUIRE(B >= 1 && d >= 1 && S >= 1 && S <= LSH_JG * LSH_MAXJ, FSTU_ESHAPE,
+               "fstu_stu_lds_state_from_hist: S=%d outside 1..%d", S, LSH_JG * LSH_MAXJ);
+  FSTU_REQUIRE(t_last >= -1 && t_last < cap, FSTU_EARG, "fstu_stu_lds_state_from_hist: t_last=%d cap=%d", t_last, cap);
+  dim3 grid((d + 63) / 64, B, 2);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
+                      hipLaunchKernelGGL(lds_state_from_hist_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream,
+                                         (const T*)hist, a, state, S, d, t_last, cap));
+  FSTU_CHECK_LAUNCH("fstu_stu_lds_state_from_hist");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- direct prefill convolution
+// Thread = (channel, tile of 16 output positions).  The 16 filter taps that
+// meet the current input row form a sliding window in registers: advancing the
+// input row by one shifts the window by one tap.
+#define CONV_TT 16
+template <typename T>
+__global__ void __launch_bounds__(256)
+stu_conv_direct_kernel(const T* __restrict__ xp, const T* __restrict__ filt, T* __restrict__ y, int Tn, int d, int L,
+                       int single_branch) {
+  const int b = blockIdx.z;
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int t0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * CONV_TT;
+  if (c >= d || t0 >= Tn) return;
+  float aE[CONV_TT], aO[CONV_TT], fw[CONV_TT];
+#pragma unroll
+  for (int i = 0; i < CONV_TT; ++i) {
+    aE[i] = 0.f;
+    aO[i] = 0.f;
+    int lag = t0 + i;
+    fw[i] = (lag < L) ? DT<T>::ld(filt + (size_t)lag * d + c) : 0.f;
+  }
+  const T* xb = xp + (size_t)b * Tn * d + c;
+  const int ulast = min(Tn - 1, t0 + CONV_TT - 1);
+  for (int u = 0; u <= ulast; ++u) {
+    const float xv = DT<T>::ld(xb + (size_t)u * d);
+    const int sel = (t0 - u) & 1;  // parity of the lag seen by output i=0
+    if (sel == 0) {
+#pragma unroll
+      for (int i = 0; i < CONV_TT; ++i) {
+        if (i & 1) aO[i] = fmaf(fw[i], xv, aO[i]); else aE[i] = fmaf(fw[i], xv, aE[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CONV_TT; ++i) {
+        if (i & 1) aE[i] = fmaf(fw[i], xv, aE[i]); else aO[i] = fmaf(fw[i], xv, aO[i]);
+      }
+    }
+#pragma unroll
+    for (int i = CONV_TT - 1; i > 0; --i) fw[i] = fw[i - 1];
+    const int lag = t0 - u - 1;
+    fw[0] = (lag >= 0 && lag < L) ? DT<T>::ld(filt + (size_t)lag * d + c) : 0.f;
+  }
+  T* yb = y + (size_t)b * Tn * d + c;
+#pragma unroll
+  for (int i = 0; i < CONV_TT; ++i) {
+    int t = t0 + i;
+    if (t < Tn) {
+      float v = single_branch ? (aE[i] + aO[i]) : (DT<T>::rnd(aE[i] + aO[i]) + DT<T>::rnd(aE[i] - aO[i]));
+      DT<T>::st(yb + (size_t)t * d, v);
+    }
+  }
+}
+
+extern "C" int fstu_stu_conv_direct(const void* xp, const void* filt, void* y, int B, int T_, int d, int L,
+                                    int single_branch, int dtype, void* stream) {
+  FSTU_REQUIRE(xp && filt && y, FSTU_ENULL, "fstu_stu_conv_direct: null pointer");
+  FSTU_REQUIRE(B >= 1 && T_ >= 1 && d >= 1 && L >= 1 && B <= 65535, FSTU_ESHAPE, "fstu_stu_conv_direct: bad shape B=%d T=%d d=%d L=%d", B, T_, d, L);
+  dim3 grid((d + 63) / 64, (T_ + 4 * CONV_TT - 1) / (4 * CONV_TT), B);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_conv_direct",
+                      hipLaunchKernelGGL(stu_conv_direct_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream,
+                                         (const T*)xp, (const T*)filt, (T*)y, T_, d, L, single_branch));
+  FSTU_CHECK_LAUNCH("fstu_stu_conv_direct");
+  return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- dense LDS steps
+// One workgroup per batch row; the state element s lives in a register of
+// thread s for the whole launch.
+template <typename T>
+__global__ void __launch_bounds__(256)
+lds_steps_kernel(float* __restrict__ h, const T* __restrict__ x, const float* __restrict__ A, const T* __restrict__ Bm,
+                 const T* __restrict__ Cm, T* __restrict__ y, int Tn, int Bt, int d_in, int S, int d_out) {
+  extern __shared__ float smem[];
+  float* xs = smem;          // d_in
+  float* hs = smem + d_in;   // S
+  const int b = blockIdx.x, tid = threadIdx.x;
+  float hreg = (tid < S) ? h[(size_t)b * S + tid] : 0.f;
+  const float areg = (tid < S) ? A[tid] : 0.f;
+  for (int t = 0; t < Tn; ++t) {
+    const T* xt = x + ((size_t)t * Bt + b) * d_in;
+    for (int k = tid; k < d_in; k += 256) xs[k] = DT<T>::ld(xt + k);
+    __syncthreads();
+    if (tid < S) {
+      float u = 0.f;
+      for (int k = 0; k < d_in; ++k) u = fmaf(xs[k], DT<T>::ld(Bm + (size_t)k * S + tid), u);
+      hreg = hreg * areg + u;
+      hs[tid] = hreg;
+    }
+    __syncthreads();
+    T* yt = y + ((size_t)t * Bt + b) * d_out;
+    for (int o = tid; o < d_out; o += 256) {
+      float acc = 0.f;
+      for (int s = 0; s < S; ++s) acc = fmaf(hs[s], DT<T>::ld(Cm + (size_t)s * d_out + o), acc);
+      DT<T>::st(yt + o, acc);
+    }
+    __syncthreads();
+  }
+  if (tid < S) h[(size_t)b * S + tid] = hreg;
+}
+
+extern "C" int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, const void* Cm, void* y,
+                              int T_steps, int Bt, int d_in, int S, int d_out, int dtype, void* stream) {
+  FSTU_REQUIRE(h && x && A && Bm && Cm && y, FSTU_ENULL, "fstu_lds_steps: null pointer");
+  FSTU_REQUIRE(T_steps >= 0 && Bt >= 1 && d_in >= 1 && d_out >= 1, FSTU_ESHAPE, "fstu_lds_steps: bad shape");
+  FSTU_REQUIRE(S >= 1 && S <= 256, FSTU_ESHAPE, "fstu_lds_steps: S=%d outside 1..256", S);
+  FSTU_REQUIRE((size_t)(d_in + S) * 4 <= 64 * 1024, FSTU_ESHAPE, "fstu_lds_steps: d_in=%d too large for LDS staging", d_in);
+  if (T_steps == 0) return FSTU_OK;
+  size_t shm = (size_t)(d_in + S) * sizeof(float);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_lds_steps",
+                      hipLaunchKernelGGL(lds_steps_kernel<T>, dim3(Bt), dim3(256), shm, (hipStream_t)stream, h,
+                                         (const T*)x, A, (const T*)Bm, (const T*)Cm, (T*)y, T_steps, Bt, d_in, S, d_out));
+  FSTU_CHECK_LAUNCH("fstu_lds_steps");
+  return FSTU_OK;
+}

@@ -1,0 +1,328 @@
+"""ctypes binding of libflashstu_hip.so (the C ABI declared in include/flashstu_hip.h).
+
+Every wrapper takes torch tensors that already live on the GPU, checks what the
+kernels assume (device, dtype, contiguity, shapes) and launches on torch's
+current HIP stream.  There is no CPU or eager fallback: if the shared library
+is missing or a tensor is not on the GPU the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libflashstu_hip.so")
+
+FSTU_F32, FSTU_BF16 = 0, 1
+MAX_DECODE_ROWS = 16
+
+_lib = None
+
+_vp, _i, _i64, _f, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_uint64
+
+# name -> argtypes; the complete export list of the library
+SIGNATURES = {
+    "fstu_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_add_rmsnorm": [_vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _f, _i, _vp],
+    "fstu_linear_decode": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_glu_decode": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_linear_decode_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_gelu_mul": [_vp, _vp, _vp, _i64, _i, _vp],
+    "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_kv_append": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
+    "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+}
+
+
+class FlashSTUHipError(RuntimeError):
+    pass
+
+
+def load(path: Optional[str] = None):
+    """Loads the shared library (once) and declares every entry point."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise FlashSTUHipError(
+            f"{p} not found: build it with `python flash-stu-2_amd/csrc/build.py` "
+            "(hipcc --offload-arch=gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(p)
+    lib.fstu_version.restype = ctypes.c_int
+    lib.fstu_last_error.restype = ctypes.c_char_p
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = ctypes.c_int
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def is_available() -> bool:
+    return os.path.exists(LIB_PATH) and torch.cuda.is_available()
+
+
+def _check(rc: int, name: str):
+    if rc != 0:
+        msg = load().fstu_last_error().decode("utf-8", "replace")
+        raise FlashSTUHipError(f"{name} failed (code {rc}): {msg}")
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return FSTU_F32
+    if t.dtype == torch.bfloat16:
+        return FSTU_BF16
+    raise FlashSTUHipError(f"unsupported dtype {t.dtype}: the HIP kernels take float32 or bfloat16")
+
+
+def _dev(*ts: Optional[torch.Tensor]):
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+        if not t.is_contiguous():
+            raise FlashSTUHipError(f"tensor of shape {tuple(t.shape)} must be contiguous")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _rows_view(t: torch.Tensor):
+    """(rows, row stride in elements) of a 2-D tensor whose rows are dense."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise FlashSTUHipError(f"expected a 2-D tensor with dense rows, got shape {tuple(t.shape)} stride {t.stride()}")
+    if not t.is_cuda:
+        raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    return t.shape[0], t.stride(0)
+
+
+# ---------------------------------------------------------------- wrappers
+def embed(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    ids = ids.contiguous()
+    _dev(ids, table, out)
+    assert ids.dtype == torch.int64
+    rows = ids.numel()
+    V, d = table.shape
+    if out is None:
+        out = torch.empty(*ids.shape, d, dtype=table.dtype, device=table.device)
+    _check(load().fstu_embed(_p(ids), _p(table), _p(out), rows, d, V, _dt(table), _stream()), "fstu_embed")
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float,
+                y: Optional[torch.Tensor] = None, delta_mode: int = 0, nslices: int = 1,
+                single_branch: bool = False, want_norm: bool = True) -> Optional[torch.Tensor]:
+    """x (rows..., d) is updated in place by delta (if given); returns rmsnorm(x)*w if want_norm."""
+    _dev(x, delta, w, y)
+    d = x.shape[-1]
+    rows = x.numel() // d
+    if want_norm and y is None:
+        y = torch.empty_like(x)
+    if delta is not None:
+        if delta_mode == 0:
+            assert delta.dtype == x.dtype and delta.numel() == x.numel()
+        else:
+            assert delta.dtype == torch.float32
+            assert delta.numel() == nslices * (2 if delta_mode == 2 else 1) * rows * d, "partial-sum buffer has the wrong size"
+    _check(load().fstu_add_rmsnorm(_p(x), _p(delta), delta_mode, nslices, int(single_branch),
+                                   _p(w) if want_norm else None, _p(y) if want_norm else None,
+                                   rows, d, float(eps), _dt(x), _stream()), "fstu_add_rmsnorm")
+    return y if want_norm else None
+
+
+def linear_decode(x: torch.Tensor, W: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (rows<=16, K) @ W(N,K)^T -> (rows, N); x and out may be row-strided views."""
+    rows, ldx = _rows_view(x)
+    _dev(W)
+    N, K = W.shape
+    assert x.shape[1] == K and x.dtype == W.dtype
+    if out is None:
+        out = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    orow, ldy = _rows_view(out)
+    assert orow == rows and out.shape[1] == N
+    _check(load().fstu_linear_decode(_p(x), ldx, _p(W), _p(out), ldy, rows, N, K, _dt(x), _stream()), "fstu_linear_decode")
+    return out
+
+
+def glu_decode(x: torch.Tensor, Wg: torch.Tensor, Wu: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    rows, ldx = _rows_view(x)
+    _dev(Wg, Wu)
+    I, K = Wg.shape
+    assert Wu.shape == Wg.shape and x.shape[1] == K and x.dtype == Wg.dtype == Wu.dtype
+    if out is None:
+        out = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    orow, ldo = _rows_view(out)
+    assert orow == rows and out.shape[1] == I
+    _check(load().fstu_glu_decode(_p(x), ldx, _p(Wg), _p(Wu), _p(out), ldo, rows, I, K, _dt(x), _stream()), "fstu_glu_decode")
+    return out
+
+
+def linear_decode_splitk(x: torch.Tensor, W: torch.Tensor, ksplit: int, partial: Optional[torch.Tensor] = None) -> torch.Tensor:
+    rows, ldx = _rows_view(x)
+    _dev(W, partial)
+    N, K = W.shape
+    assert x.shape[1] == K and x.dtype == W.dtype
+    if partial is None:
+        partial = torch.empty(ksplit, rows, N, dtype=torch.float32, device=x.device)
+    assert partial.dtype == torch.float32 and partial.numel() >= ksplit * rows * N
+    _check(load().fstu_linear_decode_splitk(_p(x), ldx, _p(W), _p(partial), rows, N, K, ksplit, _dt(x), _stream()),
+           "fstu_linear_decode_splitk")
+    return partial
+
+
+def gelu_mul(g: torch.Tensor, u: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(g, u, out)
+    assert g.shape == u.shape and g.dtype == u.dtype
+    if out is None:
+        out = torch.empty_like(g)
+    _check(load().fstu_gelu_mul(_p(g), _p(u), _p(out), g.numel(), _dt(g), _stream()), "fstu_gelu_mul")
+    return out
+
+
+def stu_step_hist(hist: torch.Tensor, filt: torch.Tensor, t: int, nsplit: int, eo: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """hist (B,cap,d), filt (L,d) -> fp32 partial sums (nsplit,2,B,d)."""
+    _dev(hist, filt, eo)
+    B, cap, d = hist.shape
+    L = filt.shape[0]
+    assert filt.shape[1] == d and filt.dtype == hist.dtype
+    if eo is None:
+        eo = torch.empty(nsplit, 2, B, d, dtype=torch.float32, device=hist.device)
+    assert eo.dtype == torch.float32 and eo.numel() >= nsplit * 2 * B * d
+    _check(load().fstu_stu_step_hist(_p(hist), _p(filt), _p(eo), B, d, t, cap, L, nsplit, _dt(hist), _stream()),
+           "fstu_stu_step_hist")
+    return eo
+
+
+def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d)."""
+    _dev(state, a, ce)
+    B, two, S, d = state.shape
+    assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
+    assert a.numel() == S and ce.shape == (S, d)
+    rows, ldxp = _rows_view(xp)
+    assert rows == B and xp.shape[1] == d
+    if out is None:
+        out = torch.empty(B, d, dtype=xp.dtype, device=xp.device)
+    orow, ldy = _rows_view(out)
+    assert orow == B and out.dtype == xp.dtype
+    _check(load().fstu_stu_step_lds(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
+           "fstu_stu_step_lds")
+    return out
+
+
+def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, state: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(hist, a, state)
+    B, cap, d = hist.shape
+    S = a.numel()
+    assert a.dtype == torch.float32
+    if state is None:
+        state = torch.empty(B, 2, S, d, dtype=torch.float32, device=hist.device)
+    assert state.shape == (B, 2, S, d) and state.dtype == torch.float32
+    _check(load().fstu_stu_lds_state_from_hist(_p(hist), _p(a), _p(state), B, S, d, t_last, cap, _dt(hist), _stream()),
+           "fstu_stu_lds_state_from_hist")
+    return state
+
+
+def stu_conv_direct(xp: torch.Tensor, filt: torch.Tensor, single_branch: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(xp, filt, out)
+    B, T, d = xp.shape
+    L = filt.shape[0]
+    assert filt.shape[1] == d and filt.dtype == xp.dtype
+    if out is None:
+        out = torch.empty_like(xp)
+    _check(load().fstu_stu_conv_direct(_p(xp), _p(filt), _p(out), B, T, d, L, int(single_branch), _dt(xp), _stream()),
+           "fstu_stu_conv_direct")
+    return out
+
+
+def kv_fill(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, pos0: int):
+    """qkv (B,T,3d) -> ring (B,H,cap,hd) slots of positions pos0..pos0+T-1 (the last cap of them)."""
+    _dev(qkv, kring, vring)
+    B, T, d3 = qkv.shape
+    Bk, H, cap, hd = kring.shape
+    assert Bk == B and d3 == 3 * H * hd and vring.shape == kring.shape and qkv.dtype == kring.dtype == vring.dtype
+    _check(load().fstu_kv_fill(_p(qkv), _p(kring), _p(vring), B, T, H, hd, cap, pos0, _dt(qkv), _stream()), "fstu_kv_fill")
+
+
+def kv_append(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, pos: int):
+    _dev(qkv, kring, vring)
+    B, d3 = qkv.shape
+    Bk, H, cap, hd = kring.shape
+    assert Bk == B and d3 == 3 * H * hd and vring.shape == kring.shape and qkv.dtype == kring.dtype == vring.dtype
+    _check(load().fstu_kv_append(_p(qkv), _p(kring), _p(vring), B, H, hd, cap, pos, _dt(qkv), _stream()), "fstu_kv_append")
+
+
+def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slopes: torch.Tensor, pos: int,
+               window: int, softcap: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(qkv, kring, vring, slopes, out)
+    B, d3 = qkv.shape
+    Bk, H, cap, hd = kring.shape
+    assert Bk == B and d3 == 3 * H * hd and slopes.dtype == torch.float32 and slopes.numel() == H
+    assert qkv.dtype == kring.dtype == vring.dtype
+    if out is None:
+        out = torch.empty(B, H * hd, dtype=qkv.dtype, device=qkv.device)
+    _check(load().fstu_swa_decode(_p(qkv), _p(kring), _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window,
+                                  float(softcap or 0.0), _dt(qkv), _stream()), "fstu_swa_decode")
+    return out
+
+
+def swa_prefill(qkv: torch.Tensor, slopes: torch.Tensor, n_heads: int, window: int, softcap: float,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(qkv, slopes, out)
+    B, T, d3 = qkv.shape
+    d = d3 // 3
+    hd = d // n_heads
+    assert slopes.dtype == torch.float32 and slopes.numel() == n_heads
+    if out is None:
+        out = torch.empty(B, T, d, dtype=qkv.dtype, device=qkv.device)
+    _check(load().fstu_swa_prefill(_p(qkv), _p(out), _p(slopes), B, T, n_heads, hd, window, float(softcap or 0.0),
+                                   _dt(qkv), _stream()), "fstu_swa_prefill")
+    return out
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float = 1.0, top_k: Optional[int] = None,
+           top_p: Optional[float] = None, do_sample: bool = True, seed: int = 0, step: int = 0):
+    """logits (B,V); writes one int64 per row into `out`, a (B,) view that may be strided."""
+    _dev(logits)
+    B, V = logits.shape
+    assert out.dtype == torch.int64 and out.is_cuda and out.dim() == 1 and out.shape[0] == B
+    _check(load().fstu_sample(_p(logits), out.data_ptr(), out.stride(0), B, V, float(temperature),
+                              int(top_k) if top_k else 0, float(top_p) if top_p else 0.0, int(bool(do_sample)),
+                              int(seed) & ((1 << 64) - 1), int(step), _dt(logits), _stream()), "fstu_sample")
+    return out
+
+
+def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense LDS: h fp32 (Bt,S) carried in place over x (T,Bt,d_in) -> y (T,Bt,d_out)."""
+    _dev(h, x, A, Bm, Cm, out)
+    T, Bt, d_in = x.shape
+    S = A.numel()
+    d_out = Cm.shape[1]
+    assert h.shape == (Bt, S) and h.dtype == torch.float32 and A.dtype == torch.float32
+    assert Bm.shape == (d_in, S) and Cm.shape == (S, d_out) and Bm.dtype == Cm.dtype == x.dtype
+    if out is None:
+        out = torch.empty(T, Bt, d_out, dtype=x.dtype, device=x.device)
+    _check(load().fstu_lds_steps(_p(h), _p(x), _p(A), _p(Bm), _p(Cm), _p(out), T, Bt, d_in, S, d_out, _dt(x), _stream()),
+           "fstu_lds_steps")
+    return out

@@ -1,0 +1,191 @@
+/*
+ * flashstu_hip.h -- C ABI of libflashstu_hip.so: hand-written gfx950 (MI355X)
+ * kernels for Flash STU's autoregressive token loop.
+ *
+ * The reference (hazan-lab/flash-stu-2) has no native code of its own: every
+ * device computation on this path is delegated to torch ops or third-party
+ * CUDA/Triton wheels.  Each entry point below names the reference call site
+ * (file:line, relative to the reference checkout) whose arithmetic it replaces.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers owned by the caller unless stated.
+ *     The library allocates nothing.
+ *   - `dtype` selects the model dtype of activations and weights:
+ *     FSTU_F32 or FSTU_BF16.  Accumulation is always fp32; values are rounded
+ *     to the model dtype (round-to-nearest-even) at the points where the
+ *     reference's torch ops round.
+ *   - All tensors are dense row-major; row strides are given where a tensor
+ *     may be a view.
+ *   - `stream` is a hipStream_t passed as void*.  Launches are asynchronous on
+ *     that stream; no entry point synchronises.
+ *   - Return value: 0 on success; negative FSTU_E* for rejected arguments
+ *     (nothing is launched); positive values are hipError_t codes.
+ *     fstu_last_error() returns a thread-local description of the last failure.
+ */
+#ifndef FLASHSTU_HIP_H
+#define FLASHSTU_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSTU_VERSION 100
+
+enum { FSTU_F32 = 0, FSTU_BF16 = 1 };
+
+enum {
+  FSTU_OK = 0,
+  FSTU_ENULL = -1,   /* null pointer */
+  FSTU_EDTYPE = -2,  /* unknown dtype */
+  FSTU_ESHAPE = -3,  /* dimension out of the supported range */
+  FSTU_EALIGN = -4,  /* pointer or stride not aligned as required */
+  FSTU_EARG = -5     /* other invalid argument */
+};
+
+int fstu_version(void);
+const char* fstu_last_error(void);
+
+/* Maximum number of activation rows the skinny (decode) kernels accept. */
+#define FSTU_MAX_DECODE_ROWS 16
+
+/* ---- embedding ---------------------------------------------------------
+ * out[r,:] = table[ids[r],:].   Replaces nn.Embedding at flash_stu/model.py:152.
+ * ids are int64; an id outside [0,vocab) is rejected on the device by clamping
+ * (the row of id clamp(id,0,vocab-1) is returned). */
+int fstu_embed(const int64_t* ids, const void* table, void* out, int rows, int d, int vocab,
+               int dtype, void* stream);
+
+/* ---- RMSNorm with fused residual add -------------------------------------
+ * Optional residual update followed by optional RMSNorm:
+ *   if delta != NULL:  x[r,:] = T( x[r,:] + D[r,:] )   (in place)
+ *   if y != NULL:      y[r,:] = T( x[r,:] * rsqrt(mean(x[r,:]^2)+eps) * w )
+ * D depends on delta_mode:
+ *   0: delta is (rows,d) in the model dtype.
+ *   1: delta is `nslices` fp32 slices (nslices,rows,d); D = T(sum of slices in
+ *      slice order)  -- the split-K partial sums of fstu_linear_decode_splitk.
+ *   2: delta is fp32 (nslices,2,rows,d) holding even-lag / odd-lag partial sums
+ *      E,O of the STU convolution; D = T( T(E+O) + T(E-O) ) when both branches
+ *      are used (single_branch==0) or T(E+O) otherwise
+ *      (flash_stu/utils/stu_utils.py:226-228, modules/stu.py:120).
+ * Replaces torch.nn.RMSNorm + x.add_() at flash_stu/layers/stu_layer.py:81,93,96,
+ * layers/attention_layer.py:53-62, model.py:173. */
+int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch,
+                     const void* w, void* y, int rows, int d, float eps, int dtype, void* stream);
+
+/* ---- skinny linear layers for decode (rows <= 16) -------------------------
+ * y[m, n] = T( sum_k x[m,k] * W[n,k] ),  W is (N,K) row-major (nn.Linear layout).
+ * x rows have stride ldx elements, y rows stride ldy.  bf16 uses MFMA and needs
+ * K % 64 == 0; other shapes and fp32 take a vector-ALU kernel.
+ * Replaces nn.Linear / `@` at flash_stu/modules/attention.py:74,101,
+ * modules/stu.py:87 (with M_inputs pre-transposed), model.py:176. */
+int fstu_linear_decode(const void* x, int ldx, const void* W, void* y, int ldy, int rows, int N, int K,
+                       int dtype, void* stream);
+
+/* act[m,i] = T( T(gelu_tanh(T(x.Wg[i]))) * T(x.Wu[i]) ), Wg/Wu (I,K).
+ * Replaces gate_proj/up_proj/gelu/mul at flash_stu/modules/swiglu.py:23-26. */
+int fstu_glu_decode(const void* x, int ldx, const void* Wg, const void* Wu, void* act, int ldact, int rows,
+                    int I, int K, int dtype, void* stream);
+
+/* Split-K form: partial[s, m, n] = sum over the s-th K range of x[m,k] W[n,k]
+ * (fp32, no rounding), s < ksplit.  The consumer (fstu_add_rmsnorm mode 1) adds
+ * the slices in order, so results are deterministic.  K % (64*ksplit) == 0 for
+ * bf16.  Replaces down_proj at flash_stu/modules/swiglu.py:27. */
+int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, float* partial, int rows, int N, int K,
+                              int ksplit, int dtype, void* stream);
+
+/* Elementwise act = T( T(gelu_tanh(g)) * u ) over n elements (prefill form of
+ * flash_stu/modules/swiglu.py:24-26). */
+int fstu_gelu_mul(const void* g, const void* u, void* act, int64_t n, int dtype, void* stream);
+
+/* ---- STU decode step: exact history form ----------------------------------
+ * hist is the (B,cap,d) history of projected inputs x_proj (model dtype), the
+ * newest at time index t (0-based, t < cap); filt is the (L,d) per-channel
+ * filter phi_proj in the model dtype.  Writes fp32 partial sums
+ *   eo[s,0,b,c] = sum over even lags in lag range s of filt[lag,c]*hist[b,t-lag,c]
+ *   eo[s,1,b,c] = same over odd lags
+ * for nsplit lag ranges covering lags 0..min(t,L-1); consumed by
+ * fstu_add_rmsnorm mode 2.  Restates convolve() at
+ * flash_stu/utils/stu_utils.py:223-228 at the newest position. */
+int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int d, int t, int cap, int L,
+                       int nsplit, int dtype, void* stream);
+
+/* ---- STU decode step: distilled diagonal recurrence (LDS form) -------------
+ * state is fp32 (B,2,S,d): two parity banks of S modes per (batch,channel).
+ * The bank of parity t&1 is advanced h_j <- a[j]*h_j + xp[b,c] and
+ *   y[b,c] = T( 2 * sum_j ce[j,c]*h_j )
+ * where a (S) are the two-step poles and ce (S,d) the per-channel output
+ * weights fitted to phi_proj's even lags.  Per-token form of
+ * mini_stu/stu_lds.py:213-338 merged with the approx-mode contraction of
+ * flash_stu/modules/stu.py:87-98,120. */
+int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
+                      int B, int S, int d, int t, int dtype, void* stream);
+
+/* Builds that state from a prefilled history: for both parities p,
+ *   state[b,p,j,c] = sum_{m>=0} a[j]^m * hist[b, tp-2m, c],  tp = newest index
+ *   of parity p that is <= t_last.  hist is (B,cap,d). */
+int fstu_stu_lds_state_from_hist(const void* hist, const float* a, float* state, int B, int S, int d,
+                                 int t_last, int cap, int dtype, void* stream);
+
+/* ---- STU prefill convolution (approx mode), time-domain form ---------------
+ * y[b,t,c] = T(E+O) + T(E-O)  (or T(E+O) if single_branch) with E/O the even-/
+ * odd-lag parts of sum_{s<=t} filt[s,c]*xp[b,t-s,c].  xp,y (B,T,d); filt (L,d).
+ * Replaces convolve() at flash_stu/utils/stu_utils.py:195-228 + stu.py:120. */
+int fstu_stu_conv_direct(const void* xp, const void* filt, void* y, int B, int T, int d, int L,
+                         int single_branch, int dtype, void* stream);
+
+/* ---- sliding-window attention ----------------------------------------------
+ * KV ring layout: (B,H,cap,hd), absolute position j lives in slot j % cap,
+ * cap >= window+1.
+ * fstu_kv_append copies k,v of one new token per batch row out of a fused qkv
+ * row (B,3*H*hd; q,k,v order) into slot pos % cap.
+ * fstu_kv_fill copies the last min(T,cap) positions of a prefill qkv (B,T,3*H*hd)
+ * whose first row is absolute position pos0. */
+int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, int H, int hd, int cap, int pos,
+                   int dtype, void* stream);
+int fstu_kv_fill(const void* qkv, void* kring, void* vring, int B, int T, int H, int hd, int cap, int pos0,
+                 int dtype, void* stream);
+
+/* One query per (batch,head) at absolute position pos (its own k,v already in
+ * the ring) against keys max(0,pos-window)..pos:
+ *   s_j = softcap*tanh(q.k_j*hd^-0.5/softcap) - slope[h]*(pos-j)  (softcap<=0: no cap)
+ *   out = softmax_j(s) . v   in fp32, rounded to the model dtype.
+ * q is read from qkv (B,3*H*hd) columns [0,H*hd); out is (B,H*hd).
+ * Replaces flash_attn_func(causal, window_size=(W,0), alibi_slopes, softcap) at
+ * flash_stu/modules/attention.py:90-99 for the decode shape. */
+int fstu_swa_decode(const void* qkv, const void* kring, const void* vring, void* out, const float* slopes,
+                    int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
+                    void* stream);
+
+/* Prefill form: qkv (B,T,3*H*hd), positions 0..T-1, out (B,T,H*hd). */
+int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T, int H, int hd,
+                     int window, float softcap, int dtype, void* stream);
+
+/* ---- sampling --------------------------------------------------------------
+ * Per row of logits (B,V): l = clamp(T(logit/temperature), -1e4, 1e4); optional
+ * top-k (keep every l >= k-th largest), optional top-p over the survivors
+ * (descending order, ties by lower index first; a token is kept iff the
+ * probability mass ranked before it is <= top_p), then
+ *   do_sample == 0: argmax, lowest index on ties;
+ *   do_sample != 0: inverse-CDF draw in index order with the counter-based
+ *                   uniform u(seed, step, row).
+ * Writes out[b*out_stride] (int64).  top_k <= 0 (or >= V) and top_p outside
+ * (0,1) disable the respective filter.  Probabilities are fp32 exponentials
+ * relative to the row maximum, summed in float64.
+ * Replaces flash_stu/model.py:267-299. */
+int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature,
+                int top_k, float top_p, int do_sample, uint64_t seed, int step, int dtype, void* stream);
+
+/* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
+ * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:
+ *   h <- h*A + x_t @ Bm ;  y_t = T(h @ Cm)
+ * x (T_steps,Bt,d_in), y (T_steps,Bt,d_out) in the model dtype; A (S) fp32;
+ * Bm (d_in,S), Cm (S,d_out) in the model dtype.  S <= 256. */
+int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, const void* Cm, void* y,
+                   int T_steps, int Bt, int d_in, int S, int d_out, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHSTU_HIP_H */

@@ -1,0 +1,316 @@
+"""GPU parity of every C-ABI entry point against the CPU oracle on the same
+seeded inputs.  All calls go through libflashstu_hip.so (ctypes).
+
+Tolerances: fp32 results differ from the oracle only by summation order
+(1e-5 relative to the result scale); bf16 results must equal the oracle's
+rounded values except where a different fp32 summation order flips a rounding:
+at most one bf16 ulp (2^-7 relative) on a small fraction of elements."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import flashstu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from flash_stu import _hip
+    _hip.load()
+    return _hip
+
+
+def dev(t):
+    return t.cuda()
+
+
+def check(got, ref, dtype, frac=0.02, scale=None, atol=0.0):
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    s = float(ref.abs().max()) if scale is None else scale
+    diff = (got - ref).abs()
+    if dtype == torch.float32:
+        assert float(diff.max()) <= 2e-5 * max(s, 1e-30), f"fp32 max diff {float(diff.max())} scale {s}"
+    else:
+        tol = ref.abs() * 2.0 ** -7 + 1e-3 * 2.0 ** -7 * max(s, 1e-30) + atol
+        assert bool((diff <= tol).all()), f"bf16 diff beyond one ulp: {float((diff - tol).max())}"
+        assert float((diff > 0).float().mean()) <= frac, f"too many rounding flips: {float((diff > 0).float().mean())}"
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(hip, dtype):
+    g = gen(0)
+    table = torch.randn(101, 48, generator=g).to(dtype)
+    ids = torch.randint(0, 101, (3, 7), generator=g)
+    out = hip.embed(dev(ids), dev(table))
+    assert torch.equal(out.cpu(), table[ids])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,d", [(8, 768), (3, 100), (64, 2048), (1, 256)])
+def test_rmsnorm_plain_and_residual(hip, dtype, rows, d):
+    g = gen(1)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    delta = torch.randn(rows, d, generator=g).to(dtype)
+    w = (1 + 0.2 * torch.randn(d, generator=g)).to(dtype)
+    y = hip.add_rmsnorm(dev(x), None, dev(w), O.RMS_EPS_DEFAULT)
+    check(y, O.rms_norm(x, w), dtype)
+    xd = dev(x.clone())
+    y2 = hip.add_rmsnorm(xd, dev(delta), dev(w), O.RMS_EPS_DEFAULT)
+    xr = x + delta
+    assert torch.equal(xd.cpu(), xr)
+    check(y2, O.rms_norm(xr, w), dtype)
+    xd = dev(x.clone())
+    assert hip.add_rmsnorm(xd, dev(delta), None, O.RMS_EPS_DEFAULT, want_norm=False) is None
+    assert torch.equal(xd.cpu(), xr)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,N,K", [(8, 768, 768), (8, 2304, 768), (1, 50257, 256), (16, 1000, 320),
+                                       (5, 37, 100), (8, 50257, 768)])
+def test_linear_decode(hip, dtype, rows, N, K):
+    g = gen(2)
+    x = torch.randn(rows, K, generator=g).to(dtype)
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    y = hip.linear_decode(dev(x), dev(W))
+    check(y, F.linear(x.float(), W.float()).to(dtype), dtype)
+
+
+def test_linear_decode_strided_rows(hip):
+    g = gen(3)
+    big = torch.randn(4, 5, 256, generator=g).bfloat16()
+    W = (torch.randn(128, 256, generator=g) / 16).bfloat16()
+    bd = dev(big)
+    out = torch.zeros(4, 3, 128, dtype=torch.bfloat16, device="cuda")
+    hip.linear_decode(bd[:, 2, :], dev(W), out[:, 1, :])
+    check(out[:, 1].cpu(), F.linear(big[:, 2].float(), W.float()).bfloat16(), torch.bfloat16)
+    assert float(out[:, 0].abs().max()) == 0 and float(out[:, 2].abs().max()) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 3072), (2, 256, 1024), (3, 96, 200)])
+def test_mlp_decode_chain(hip, dtype, rows, d, I):
+    """glu -> split-K down projection -> residual add equals x + MLP(x)."""
+    g = gen(4)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    res = torch.randn(rows, d, generator=g).to(dtype)
+    p = {"gate_proj.weight": (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype),
+         "up_proj.weight": (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype),
+         "down_proj.weight": (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)}
+    act = hip.glu_decode(dev(x), dev(p["gate_proj.weight"]), dev(p["up_proj.weight"]))
+    ref_act = F.gelu(F.linear(x, p["gate_proj.weight"]), approximate="tanh") * F.linear(x, p["up_proj.weight"])
+    check(act, ref_act, dtype)
+    for ks in ([1, 4] if I % 256 == 0 else [1, 2]):
+        part = hip.linear_decode_splitk(act, dev(p["down_proj.weight"]), ks)
+        rd = dev(res.clone())
+        hip.add_rmsnorm(rd, part, None, O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ks, want_norm=False)
+        down = F.linear(act.cpu(), p["down_proj.weight"])
+        ref = res + down
+        # a one-ulp flip of the projection survives the residual add at the projection's scale
+        check(rd, ref, dtype, frac=0.05, atol=(2.0 ** -7 * float(down.float().abs().max())) if dtype == torch.bfloat16 else 0.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gelu_mul(hip, dtype):
+    g = gen(5)
+    a = (3 * torch.randn(4, 1000, generator=g)).to(dtype)
+    b = torch.randn(4, 1000, generator=g).to(dtype)
+    check(hip.gelu_mul(dev(a), dev(b)), F.gelu(a, approximate="tanh") * b, dtype)
+
+
+def _stu_setup(dtype, B, T, d, L, K, seed):
+    g = gen(seed)
+    phi = torch.tensor(O.get_spectral_filters_f64(L, K)).to(dtype)
+    Mf = (torch.randn(K, d, generator=g) / math.sqrt(K)).to(dtype)
+    xp = torch.randn(B, T, d, generator=g).to(dtype)
+    filt = phi @ Mf
+    n = O.nearest_power_of_two(2 * L - 1, True)
+    plus, minus = O.convolve(xp, filt, n, use_approx=True)
+    return xp, filt, plus + minus, plus
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d,L", [(2, 100, 96, 128), (1, 64, 256, 1024), (3, 120, 100, 128)])
+def test_stu_conv_direct(hip, dtype, B, T, d, L):
+    xp, filt, ref, plus = _stu_setup(dtype, B, T, d, L, 8, 6)
+    # the two branches are rounded before they are added: a flip costs one ulp of a branch
+    atol = 2.0 ** -7 * float(plus.float().abs().max()) if dtype == torch.bfloat16 else 0.0
+    check(hip.stu_conv_direct(dev(xp), dev(filt)), ref, dtype, frac=0.05, atol=atol)
+    check(hip.stu_conv_direct(dev(xp), dev(filt), single_branch=True), plus, dtype, frac=0.05)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d,L,nsplit", [(2, 100, 96, 128, 3), (8, 257, 768, 512, 4), (1, 50, 100, 64, 1),
+                                             (2, 128, 2048, 128, 2)])  # T <= L: the reference's FFT length assumes it
+def test_stu_step_hist(hip, dtype, B, T, d, L, nsplit):
+    """Newest-position output of the history step == last row of the oracle's
+    FFT convolution, at several t including t >= L-1."""
+    xp, filt, ref, plus = _stu_setup(dtype, B, T, d, L, 8, 7)
+    atol = 2.0 ** -7 * float(plus.float().abs().max()) if dtype == torch.bfloat16 else 0.0
+    cap = T + 3
+    hist = torch.zeros(B, cap, d, dtype=dtype)
+    hist[:, :T] = xp
+    hd_, fd = dev(hist), dev(filt)
+    for t in (0, 1, T // 2, T - 1):
+        eo = hip.stu_step_hist(hd_, fd, t, nsplit)
+        x = torch.zeros(B, d, dtype=dtype, device="cuda")
+        hip.add_rmsnorm(x, eo, None, O.RMS_EPS_DEFAULT, delta_mode=2, nslices=nsplit, want_norm=False)
+        check(x, ref[:, t], dtype, frac=0.05, scale=float(ref.abs().max()), atol=atol)
+
+
+def _fit_lds(filt_even, S):
+    """ridge fit of the even-lag filter by S real poles (host-side helper of the product)."""
+    from flash_stu.utils.lds_fit import fit_even_lag_lds
+    return fit_even_lag_lds(filt_even, S)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stu_step_lds_recurrence(hip, dtype):
+    """The kernel's recurrence equals a float64 evaluation of the same
+    recurrence, and the state builder equals stepping from zero."""
+    g = gen(8)
+    B, S, d, T = 3, 64, 256, 41
+    a = (0.5 + 0.49 * torch.rand(S, generator=g)).float()
+    ce = (torch.randn(S, d, generator=g) / S).float()
+    xs = torch.randn(T, B, d, generator=g).to(dtype)
+    state = torch.zeros(B, 2, S, d, device="cuda")
+    h64 = torch.zeros(B, 2, S, d, dtype=torch.float64)
+    ad, ced = dev(a), dev(ce)
+    for t in range(T):
+        y = hip.stu_step_lds(state, dev(xs[t]), ad, ced, t)
+        p = t & 1
+        h64[:, p] = a.double()[None, :, None] * h64[:, p] + xs[t].double()[:, None, :]
+        ref = 2 * (ce.double()[None] * h64[:, p]).sum(1)
+        check(y, ref.to(dtype), dtype, frac=0.05, scale=float(ref.abs().max()))
+    assert float((state.cpu().double() - h64).abs().max()) < 1e-4 * float(h64.abs().max())
+    hist = torch.zeros(B, T + 5, d, dtype=dtype)
+    hist[:, :T] = xs.transpose(0, 1)
+    st2 = hip.stu_lds_state_from_hist(dev(hist), ad, T - 1)
+    assert float((st2.cpu().double() - h64).abs().max()) < 1e-4 * float(h64.abs().max())
+
+
+@pytest.mark.parametrize("L", [128, 1024])
+def test_stu_step_lds_tracks_the_convolution(hip, L):
+    """With poles/weights fitted to the effective filter, the recurrence
+    reproduces the oracle's convolution output to well below one bf16 ulp."""
+    dtype = torch.float32
+    B, d, K, S = 2, 128, 24 if L >= 256 else 8, 64
+    T = L
+    xp, filt, ref, _ = _stu_setup(dtype, B, T, d, L, K, 9)
+    a, ce, err = _fit_lds(filt.double()[0::2], S)
+    state = torch.zeros(B, 2, S, d, device="cuda")
+    ad, ced = dev(a), dev(ce)
+    worst = 0.0
+    for t in range(T):
+        y = hip.stu_step_lds(state, dev(xp[:, t].contiguous()), ad, ced, t)
+        worst = max(worst, float((y.cpu() - ref[:, t]).abs().max()))
+    assert worst < 1e-3 * float(ref.abs().max()), (worst, float(ref.abs().max()), err)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,hd,W,T", [(2, 4, 64, 16, 50), (8, 12, 64, 512, 600), (1, 16, 128, 32, 40),
+                                         (2, 2, 32, 7, 20)])
+def test_swa_ring_decode_and_prefill(hip, dtype, B, H, hd, W, T):
+    g = gen(10)
+    d = H * hd
+    qkv = torch.randn(B, T, 3 * d, generator=g).to(dtype)
+    slopes = O.alibi_slopes(H)
+    q, k, v = (t.reshape(B, T, H, hd) for t in torch.chunk(qkv, 3, dim=2))
+    full = O.attention_core(q, k, v, W, slopes, 50.0).reshape(B, T, d)
+    out = hip.swa_prefill(dev(qkv), dev(slopes), H, W, 50.0)
+    check(out, full, dtype, frac=0.05)
+    # ring: prefill P positions, then append/decode the rest one by one
+    cap = W + 1
+    P = T // 2
+    kr = torch.zeros(B, H, cap, hd, dtype=dtype, device="cuda")
+    vr = torch.zeros_like(kr)
+    qd = dev(qkv)
+    hip.kv_fill(qd[:, :P].contiguous(), kr, vr, 0)
+    sd = dev(slopes)
+    for pos in range(P, T):
+        row = qd[:, pos].contiguous()
+        hip.kv_append(row, kr, vr, pos)
+        o = hip.swa_decode(row, kr, vr, sd, pos, W, 50.0)
+        check(o, full[:, pos], dtype, frac=0.05, scale=float(full.abs().max()))
+    # softcap disabled
+    o2 = hip.swa_decode(qd[:, T - 1].contiguous(), kr, vr, sd, T - 1, W, 0.0)
+    ref2 = O.attention_core(q[:, -1:], k, v, W, slopes, 0.0).reshape(B, d)
+    check(o2, ref2, dtype, frac=0.05)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sample_greedy_matches_oracle_ties_included(hip, dtype):
+    g = gen(11)
+    B, V = 8, 50257
+    logits = torch.randn(B, V, generator=g).to(dtype)
+    logits[0, 100] = logits[0, 40000] = 9.0        # tie -> lowest index
+    logits[1, :] = 0.0                               # all equal -> 0
+    out = torch.full((B, 4), -1, dtype=torch.int64, device="cuda")
+    hip.sample(dev(logits), out[:, 2], do_sample=False)
+    ref = O.next_token(logits, do_sample=False)
+    assert torch.equal(out[:, 2].cpu(), ref[:, 0])
+    assert int(out[0, 2]) == 100 and int(out[1, 2]) == 0
+    assert bool((out[:, [0, 1, 3]] == -1).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 40, None), (1.0, None, None), (1.0, 5, 0.7),
+                                                      (1.3, None, 0.9), (0.7, 1, None)])
+def test_sample_draws_match_oracle(hip, dtype, temperature, top_k, top_p):
+    """Same counter-based stream, same filters: ids equal the oracle's draw.
+    (fp32 only for top-p: the oracle restates the reference's model-dtype
+    softmax/cumsum, which the kernel evaluates in fp32.)"""
+    if top_p is not None and dtype == torch.bfloat16:
+        pytest.skip("top-p cumulative sums in bf16 are not reproduced bit-wise; covered in fp32")
+    g = gen(12)
+    B, V = 4, 3001
+    logits = (2.5 * torch.randn(B, V, generator=g)).to(dtype)
+    ld = dev(logits)
+    agree = total = 0
+    for step in range(40):
+        out = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample(ld, out, temperature, top_k, top_p, True, seed=77, step=step)
+        ref = O.next_token(logits, temperature, top_k, top_p, True, seed=77, step=step)[:, 0]
+        agree += int((out.cpu() == ref).sum())
+        total += B
+        filt = O.filter_logits(logits.float() if dtype == torch.float32 else logits, temperature, top_k, top_p)
+        assert bool(torch.isfinite(filt.float().gather(1, out.cpu()[:, None])).all()), "drew a filtered token"
+    assert agree >= total - 1, (agree, total)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_lds_steps_dense(hip, dtype):
+    g = gen(13)
+    T, Bt, din, S, dout = 12, 5, 96, 40, 72
+    A = (0.9 + 0.099 * torch.rand(S, generator=g)).float()
+    Bm = (torch.randn(din, S, generator=g) / din).to(dtype)
+    Cm = (torch.randn(S, dout, generator=g) / S).to(dtype)
+    x = torch.randn(T, Bt, din, generator=g).to(dtype)
+    yref, href = O.lds_sequence(x, A, Bm, Cm)
+    h = torch.zeros(Bt, S, device="cuda")
+    y = hip.lds_steps(h, dev(x[:7]), dev(A), dev(Bm), dev(Cm))
+    y2 = hip.lds_steps(h, dev(x[7:]), dev(A), dev(Bm), dev(Cm))     # state carried across launches
+    check(torch.cat([y, y2]), yref, dtype, frac=0.05)
+    assert float((h.cpu() - href).abs().max()) < 1e-5 * max(1.0, float(href.abs().max()))
+
+
+def test_argument_errors_do_not_launch(hip):
+    x = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
+    W = torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(hip.FlashSTUHipError, match="rows=17"):
+        hip.linear_decode(x, W)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.linear_decode(torch.zeros(2, 64), W.cpu())
+    kr = torch.zeros(1, 2, 4, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(hip.FlashSTUHipError, match="ring capacity"):
+        hip.swa_decode(torch.zeros(1, 384, dtype=torch.bfloat16, device="cuda"), kr, kr.clone(),
+                       torch.zeros(2, device="cuda"), 3, 8, 50.0)
