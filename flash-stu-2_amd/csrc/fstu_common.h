@@ -29,6 +29,10 @@ void fstu_set_error(const char* fmt, ...);
     }                                                                     \
   } while (0)
 
+// library-internal: embedding gather of ids[r*id_stride]
+int fstu_embed_strided(const int64_t* ids, int64_t id_stride, const void* table, void* out, int rows, int d, int vocab,
+                       int dtype, void* stream);
+
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // ---------------------------------------------------------------- dtypes

@@ -18,10 +18,10 @@ extern "C" int fstu_version(void) { return FSTU_VERSION; }
 
 // ---------------------------------------------------------------- embed
 template <typename T>
-__global__ void embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, T* __restrict__ out,
-                             int d, int vocab) {
+__global__ void embed_kernel(const int64_t* __restrict__ ids, int64_t id_stride, const T* __restrict__ table,
+                             T* __restrict__ out, int d, int vocab) {
   int r = blockIdx.x;
-  int64_t id = ids[r];
+  int64_t id = ids[(size_t)r * id_stride];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + (size_t)id * d;
   T* dst = out + (size_t)r * d;
@@ -35,7 +35,18 @@ extern "C" int fstu_embed(const int64_t* ids, const void* table, void* out, int 
   if (rows == 0) return FSTU_OK;
   FSTU_DISPATCH_DTYPE(dtype, "fstu_embed",
                       hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids,
-                                         (const T*)table, (T*)out, d, vocab));
+                                         (int64_t)1, (const T*)table, (T*)out, d, vocab));
+  FSTU_CHECK_LAUNCH("fstu_embed");
+  return FSTU_OK;
+}
+
+// ids[r*id_stride]: one column of a (rows, id_stride) token buffer (library-internal)
+int fstu_embed_strided(const int64_t* ids, int64_t id_stride, const void* table, void* out, int rows, int d, int vocab,
+                       int dtype, void* stream) {
+  FSTU_REQUIRE(ids && table && out, FSTU_ENULL, "fstu_embed: null pointer");
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_embed",
+                      hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids,
+                                         id_stride, (const T*)table, (T*)out, d, vocab));
   FSTU_CHECK_LAUNCH("fstu_embed");
   return FSTU_OK;
 }

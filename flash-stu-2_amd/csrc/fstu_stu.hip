@@ -224,22 +224,27 @@ extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, fl
 // Thread = (channel, tile of 16 output positions).  The 16 filter taps that
 // meet the current input row form a sliding window in registers: advancing the
 // input row by one shifts the window by one tap.
+// The filter element of (lag, channel c) is filt[lag*f_ls + c*f_cs], so the same
+// kernel serves a per-channel filter (f_ls=d, f_cs=1) and one column of a
+// shared filter bank (f_ls=K, f_cs=0).  Output rows are ldy elements apart.
+// mode 0: y = T(E+O) + T(E-O);  mode 1: y = T(E+O);  mode 2: y = T(E+O), y2 = T(E-O).
 #define CONV_TT 16
 template <typename T>
 __global__ void __launch_bounds__(256)
-stu_conv_direct_kernel(const T* __restrict__ xp, const T* __restrict__ filt, T* __restrict__ y, int Tn, int d, int L,
-                       int single_branch) {
+stu_conv_direct_kernel(const T* __restrict__ xp, const T* __restrict__ filt, size_t f_ls, size_t f_cs,
+                       T* __restrict__ y, T* __restrict__ y2, size_t ldy, int Tn, int d, int L, int mode) {
   const int b = blockIdx.z;
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int t0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * CONV_TT;
   if (c >= d || t0 >= Tn) return;
+  const T* fc = filt + (size_t)c * f_cs;
   float aE[CONV_TT], aO[CONV_TT], fw[CONV_TT];
 #pragma unroll
   for (int i = 0; i < CONV_TT; ++i) {
     aE[i] = 0.f;
     aO[i] = 0.f;
     int lag = t0 + i;
-    fw[i] = (lag < L) ? DT<T>::ld(filt + (size_t)lag * d + c) : 0.f;
+    fw[i] = (lag < L) ? DT<T>::ld(fc + (size_t)lag * f_ls) : 0.f;
   }
   const T* xb = xp + (size_t)b * Tn * d + c;
   const int ulast = min(Tn - 1, t0 + CONV_TT - 1);
@@ -260,15 +265,20 @@ stu_conv_direct_kernel(const T* __restrict__ xp, const T* __restrict__ filt, T* 
 #pragma unroll
     for (int i = CONV_TT - 1; i > 0; --i) fw[i] = fw[i - 1];
     const int lag = t0 - u - 1;
-    fw[0] = (lag >= 0 && lag < L) ? DT<T>::ld(filt + (size_t)lag * d + c) : 0.f;
+    fw[0] = (lag >= 0 && lag < L) ? DT<T>::ld(fc + (size_t)lag * f_ls) : 0.f;
   }
-  T* yb = y + (size_t)b * Tn * d + c;
+  T* yb = y + (size_t)b * Tn * ldy + c;
+  T* yb2 = (mode == 2) ? y2 + (size_t)b * Tn * ldy + c : nullptr;
 #pragma unroll
   for (int i = 0; i < CONV_TT; ++i) {
     int t = t0 + i;
     if (t < Tn) {
-      float v = single_branch ? (aE[i] + aO[i]) : (DT<T>::rnd(aE[i] + aO[i]) + DT<T>::rnd(aE[i] - aO[i]));
-      DT<T>::st(yb + (size_t)t * d, v);
+      if (mode == 0) {
+        DT<T>::st(yb + (size_t)t * ldy, DT<T>::rnd(aE[i] + aO[i]) + DT<T>::rnd(aE[i] - aO[i]));
+      } else {
+        DT<T>::st(yb + (size_t)t * ldy, aE[i] + aO[i]);
+        if (mode == 2) DT<T>::st(yb2 + (size_t)t * ldy, aE[i] - aO[i]);
+      }
     }
   }
 }
@@ -280,8 +290,25 @@ extern "C" int fstu_stu_conv_direct(const void* xp, const void* filt, void* y, i
   dim3 grid((d + 63) / 64, (T_ + 4 * CONV_TT - 1) / (4 * CONV_TT), B);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_conv_direct",
                       hipLaunchKernelGGL(stu_conv_direct_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream,
-                                         (const T*)xp, (const T*)filt, (T*)y, T_, d, L, single_branch));
+                                         (const T*)xp, (const T*)filt, (size_t)d, (size_t)1, (T*)y, (T*)nullptr,
+                                         (size_t)d, T_, d, L, single_branch ? 1 : 0));
   FSTU_CHECK_LAUNCH("fstu_stu_conv_direct");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_stu_conv_bank(const void* x, const void* phi, void* u_plus, void* u_minus, int B, int T_, int d,
+                                  int L, int K, int dtype, void* stream) {
+  FSTU_REQUIRE(x && phi && u_plus, FSTU_ENULL, "fstu_stu_conv_bank: null pointer");
+  FSTU_REQUIRE(B >= 1 && T_ >= 1 && d >= 1 && L >= 1 && K >= 1 && B <= 65535, FSTU_ESHAPE, "fstu_stu_conv_bank: bad shape B=%d T=%d d=%d L=%d K=%d", B, T_, d, L, K);
+  dim3 grid((d + 63) / 64, (T_ + 4 * CONV_TT - 1) / (4 * CONV_TT), B);
+  for (int k = 0; k < K; ++k) {
+    FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_conv_bank",
+                        hipLaunchKernelGGL(stu_conv_direct_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream,
+                                           (const T*)x, (const T*)phi + k, (size_t)K, (size_t)0,
+                                           (T*)u_plus + (size_t)k * d, u_minus ? (T*)u_minus + (size_t)k * d : (T*)nullptr,
+                                           (size_t)K * d, T_, d, L, u_minus ? 2 : 1));
+  }
+  FSTU_CHECK_LAUNCH("fstu_stu_conv_bank");
   return FSTU_OK;
 }
 

@@ -35,6 +35,7 @@ SIGNATURES = {
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_append": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -253,6 +254,17 @@ def stu_conv_direct(xp: torch.Tensor, filt: torch.Tensor, single_branch: bool = 
     _check(load().fstu_stu_conv_direct(_p(xp), _p(filt), _p(out), B, T, d, L, int(single_branch), _dt(xp), _stream()),
            "fstu_stu_conv_direct")
     return out
+
+
+def stu_conv_bank(x: torch.Tensor, phi: torch.Tensor, u_plus: torch.Tensor, u_minus: Optional[torch.Tensor]):
+    """x (B,T,d), phi (L,K) -> u_plus/u_minus (B,T,K,d) written in place."""
+    _dev(x, phi, u_plus, u_minus)
+    B, T, d = x.shape
+    L, K = phi.shape
+    assert u_plus.shape == (B, T, K, d) and phi.dtype == x.dtype == u_plus.dtype
+    assert u_minus is None or (u_minus.shape == u_plus.shape and u_minus.dtype == x.dtype)
+    _check(load().fstu_stu_conv_bank(_p(x), _p(phi), _p(u_plus), _p(u_minus), B, T, d, L, K, _dt(x), _stream()),
+           "fstu_stu_conv_bank")
 
 
 def kv_fill(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, pos0: int):

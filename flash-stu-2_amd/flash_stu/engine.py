@@ -1,0 +1,195 @@
+"""Decode engine behind FlashSTU.generate(): prefill through the module path,
+then one C-ABI call per token (fstu_decode_step) that launches the fused kernel
+sequence for the whole layer stack against preallocated state and workspaces.
+
+The token buffer (B, max_length) lives on the GPU for the whole loop; each step
+reads column pos and writes column pos+1, so the host never sees a token until
+generate() returns (reference loop: flash_stu/model.py:245-302, which re-allocates
+the sequence with torch.cat every step).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from . import _hip
+from .layers.attention_layer import AttentionLayer
+from .layers.stu_layer import STULayer
+
+_vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+
+
+class LayerDesc(ctypes.Structure):
+    _fields_ = [("kind", _i), ("norm1_w", _vp), ("mlp_norm_w", _vp), ("w_gate", _vp), ("w_up", _vp), ("w_down", _vp),
+                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_state", _vp),
+                ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp)]
+
+
+class ModelDesc(ctypes.Structure):
+    _fields_ = [("dtype", _i), ("B", _i), ("d", _i), ("I", _i), ("V", _i), ("n_layers", _i), ("n_heads", _i),
+                ("head_dim", _i), ("window", _i), ("kv_cap", _i), ("L", _i), ("hist_cap", _i), ("stu_mode", _i),
+                ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i),
+                ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
+                ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
+                ("partial", _vp), ("eo", _vp), ("logits", _vp)]
+
+
+def pick_ksplit_down(I: int) -> int:
+    """K split of the down projection: enough waves to fill 256 CUs while every
+    slice still divides into the 64-wide k steps of the MFMA kernel."""
+    for ks in (12, 16, 8, 6, 4, 3, 2):
+        if I % (ks * 256) == 0:
+            return ks
+    for ks in (8, 4, 2):
+        if I % (ks * 64) == 0:
+            return ks
+    return 1
+
+
+class DecodeEngine:
+    HIST_NSPLIT_MAX = 16
+
+    def __init__(self, model):
+        cfg = model.config
+        if not cfg.use_approx:
+            raise NotImplementedError("the fused decode engine covers use_approx=True; use generate(use_cache=False)")
+        self.model = model
+        self.cfg = cfg
+        self.lib = _hip.load()
+        self.lib.fstu_decode_step.argtypes = [ctypes.POINTER(ModelDesc), _vp, _vp, ctypes.c_int64, _i, _f, _i, _f, _i,
+                                              ctypes.c_uint64, _i, _vp]
+        self.lib.fstu_decode_step.restype = _i
+        self._keep: List[torch.Tensor] = []
+
+    # ------------------------------------------------------------------
+    def _build(self, caches, B: int, total_len: int):
+        model, cfg = self.model, self.cfg
+        dev = model.lm_head.weight.device
+        dt = cfg.torch_dtype
+        d, I, V = cfg.n_embd, cfg.n_embd * cfg.mlp_scale, cfg.vocab_size
+        mode = cfg.resolved_stu_decode_mode()
+        self._keep = []
+        keep = self._keep.append
+        n = len(model.layers)
+        arr = (LayerDesc * n)()
+        hist_cap = 0
+        new_caches = list(caches)
+        for i, layer in enumerate(model.layers):
+            ld = arr[i]
+            ld.w_gate = layer.mlp.gate_proj.weight.data_ptr()
+            ld.w_up = layer.mlp.up_proj.weight.data_ptr()
+            ld.w_down = layer.mlp.down_proj.weight.data_ptr()
+            ld.mlp_norm_w = layer.mlp_norm.weight.data_ptr()
+            if isinstance(layer, STULayer):
+                stu = layer.stu
+                ld.kind = 0
+                ld.norm1_w = layer.stu_norm.weight.data_ptr()
+                mit = stu.m_inputs_t()
+                keep(mit)
+                ld.m_inputs_t = mit.data_ptr()
+                hist, state, pos = caches[i]
+                if mode == "lds":
+                    a, ce = stu.lds_params()
+                    keep(a), keep(ce), keep(state)
+                    ld.lds_a, ld.lds_ce, ld.lds_state = a.data_ptr(), ce.data_ptr(), state.data_ptr()
+                else:
+                    if hist.shape[1] < total_len:
+                        bigger = hist.new_zeros(B, total_len, d)
+                        bigger[:, : hist.shape[1]] = hist
+                        hist = bigger
+                        new_caches[i] = (hist, state, pos)
+                    if hist_cap and hist.shape[1] != hist_cap:
+                        raise RuntimeError("STU histories must share one capacity")
+                    hist_cap = hist.shape[1]
+                    filt = stu.effective_filter()
+                    keep(filt), keep(hist)
+                    ld.filt, ld.hist = filt.data_ptr(), hist.data_ptr()
+            elif isinstance(layer, AttentionLayer):
+                att = layer.attn
+                ld.kind = 1
+                ld.norm1_w = layer.attn_norm.weight.data_ptr()
+                ld.w_qkv = att.c_attn.weight.data_ptr()
+                ld.w_proj = att.c_proj.weight.data_ptr()
+                kr, vr, pos = caches[i]
+                keep(kr), keep(vr)
+                ld.kring, ld.vring = kr.data_ptr(), vr.data_ptr()
+                ld.slopes = att.alibi_slopes.data_ptr()
+            else:
+                raise TypeError(type(layer))
+        m = ModelDesc()
+        m.dtype = _hip.FSTU_BF16 if dt == torch.bfloat16 else _hip.FSTU_F32
+        m.B, m.d, m.I, m.V, m.n_layers = B, d, I, V, n
+        m.n_heads, m.head_dim = cfg.n_heads, d // cfg.n_heads
+        m.window, m.kv_cap = cfg.window_left, cfg.window_left + 1
+        m.L, m.hist_cap = cfg.seq_len, hist_cap
+        m.stu_mode = 1 if mode == "lds" else 0
+        m.lds_S = cfg.stu_lds_state_dim
+        m.single_branch = int(cfg.use_hankel_L)
+        m.ksplit_down = pick_ksplit_down(I) if dt == torch.bfloat16 else min(8, max(1, I // 512))
+        m.hist_nsplit_max = self.HIST_NSPLIT_MAX
+        m.eps, m.softcap = float(cfg.rms_norm_eps), float(cfg.softcap or 0.0)
+        m.emb = model.lm_head.weight.data_ptr()
+        m.final_norm_w = model.norm.weight.data_ptr()
+        m.layers = ctypes.cast(arr, ctypes.POINTER(LayerDesc))
+
+        def buf(*shape, dtype=dt):
+            t = torch.zeros(*shape, dtype=dtype, device=dev)
+            keep(t)
+            return t
+        self.x, self.h = buf(B, d), buf(B, d)
+        self.logits = buf(B, V)
+        m.x, m.h = self.x.data_ptr(), self.h.data_ptr()
+        m.qkv, m.attn = buf(B, 3 * d).data_ptr(), buf(B, d).data_ptr()
+        m.act, m.xp, m.y = buf(B, I).data_ptr(), buf(B, d).data_ptr(), buf(B, d).data_ptr()
+        m.partial = buf(m.ksplit_down, B, d, dtype=torch.float32).data_ptr()
+        m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
+        m.logits = self.logits.data_ptr()
+        self._arr, self.desc = arr, m
+        return tuple(new_caches)
+
+    def step(self, tokens: torch.Tensor, pos: int, temperature, top_k, top_p, do_sample, seed, step_idx):
+        """Feeds tokens[:, pos], writes the sampled id to tokens[:, pos+1]."""
+        rc = self.lib.fstu_decode_step(ctypes.byref(self.desc), tokens.data_ptr() + 8 * pos,
+                                       tokens.data_ptr() + 8 * (pos + 1), tokens.stride(0), pos, float(temperature),
+                                       int(top_k) if top_k else 0, float(top_p) if top_p else 0.0, int(bool(do_sample)),
+                                       int(seed) & ((1 << 64) - 1), int(step_idx),
+                                       torch.cuda.current_stream().cuda_stream)
+        _hip._check(rc, "fstu_decode_step")
+
+    # ------------------------------------------------------------------
+    @torch.no_grad()
+    def prefill(self, input_ids: torch.Tensor, total_len: int):
+        """Runs the prompt through the module path with caches, returns the
+        logits of the last position (B,V) and prepares the step descriptor."""
+        model = self.model
+        B, P = input_ids.shape
+        x = model._embed(input_ids.contiguous())
+        x, caches = model._run_layers(x, None, True, None)
+        xn = model.norm(x[:, -1:, :].contiguous())
+        logits = model._head(xn)[:, 0, :].contiguous()
+        self.caches = self._build(caches, B, total_len)
+        return logits
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, n_new: int, temperature=1.0, top_k=None, top_p=None, do_sample=True,
+                 seed: int = 0, return_logits: bool = False):
+        if not input_ids.is_cuda:
+            raise _hip.FlashSTUHipError("input_ids must be on the GPU: this model has no CPU path")
+        B, P = input_ids.shape
+        if B > _hip.MAX_DECODE_ROWS:
+            raise _hip.FlashSTUHipError(f"batch {B} exceeds the decode kernels' limit of {_hip.MAX_DECODE_ROWS} rows")
+        total = P + n_new
+        if self.cfg.resolved_stu_decode_mode() == "history" and total > self.cfg.seq_len:
+            raise ValueError(f"history-mode decode needs prompt+new tokens ({total}) <= seq_len ({self.cfg.seq_len})")
+        tokens = torch.zeros(B, total, dtype=torch.int64, device=input_ids.device)
+        tokens[:, :P] = input_ids
+        logits = self.prefill(input_ids, total)
+        _hip.sample(logits, tokens[:, P], temperature, top_k, top_p, do_sample, seed, 0)
+        all_logits = [logits.clone()] if return_logits else None
+        for s in range(1, n_new):
+            self.step(tokens, P + s - 1, temperature, top_k, top_p, do_sample, seed, s)
+            if return_logits:
+                all_logits.append(self.logits.clone())
+        return (tokens, torch.stack(all_logits, 1)) if return_logits else tokens

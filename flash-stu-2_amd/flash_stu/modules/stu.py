@@ -1,0 +1,178 @@
+"""Spectral Transform Unit (reference: flash_stu/modules/stu.py:12-120).
+
+Same parameters and forward semantics as the reference module; in addition the
+module can carry decode state so that one token per call reproduces what the
+reference obtains by re-running the whole sequence:
+
+  history mode  the projected inputs x_proj of every past position are kept and
+                the causal convolution is evaluated at the newest position by
+                the HIP history kernel (exact; fp32 parity mode);
+  lds mode      the even-lag effective filter is distilled into S real modes
+                per channel and two parity banks of recurrence state replace
+                the history (bounded state; bf16 performance mode).
+
+State tuples are batch-first tensors: (hist (B,cap,d), state (B,2,S,d) fp32, pos (B,) int64 on the host).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from .. import _hip
+from ..utils.lds_fit import fit_even_lag_lds
+
+
+class STU(nn.Module):
+    def __init__(self, config, phi: torch.Tensor, n: int, feature_dim: Optional[int] = None) -> None:
+        super().__init__()
+        self.config = config
+        self.register_buffer("phi", phi, persistent=False)
+        self.n = n
+        self.K = config.num_eigh
+        self.d_in = feature_dim if feature_dim is not None else config.n_embd
+        self.d_out = self.d_in
+        self.use_hankel_L = config.use_hankel_L
+        self.use_approx = config.use_approx
+        dt = config.torch_dtype
+        if self.use_approx:
+            self.M_inputs = nn.Parameter(torch.empty(self.d_in, self.d_out, dtype=dt))
+            self.M_filters = nn.Parameter(torch.empty(self.K, self.d_in, dtype=dt))
+        else:
+            self.M_phi_plus = nn.Parameter(torch.empty(self.K, self.d_in, self.d_out, dtype=dt))
+            if not self.use_hankel_L:
+                self.M_phi_minus = nn.Parameter(torch.empty(self.K, self.d_in, self.d_out, dtype=dt))
+        tile = min(config.d_in_tile or self.d_in, config.d_out_tile or self.d_in)
+        if tile < self.d_in:
+            raise NotImplementedError("channel tiling (d_in_tile/d_out_tile) is not implemented on the HIP path")
+        self._derived = {}
+
+    # ---- tensors derived from the parameters, rebuilt when a parameter changes
+    def _cached(self, key, params, build):
+        ver = tuple((p._version, p.data_ptr()) for p in params)
+        hit = self._derived.get(key)
+        if hit is None or hit[0] != ver:
+            hit = (ver, build())
+            self._derived[key] = hit
+        return hit[1]
+
+    def decode_mode(self) -> str:
+        return self.config.resolved_stu_decode_mode()
+
+    def effective_filter(self) -> torch.Tensor:
+        """phi_proj = phi @ M_filters, (L,d) in the model dtype (stu.py:88)."""
+        return self._cached("filt", (self.phi, self.M_filters),
+                            lambda: torch.matmul(self.phi, self.M_filters).contiguous())
+
+    def m_inputs_t(self) -> torch.Tensor:
+        return self._cached("mit", (self.M_inputs,), lambda: self.M_inputs.t().contiguous())
+
+    def lds_params(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        def build():
+            a, ce, err = fit_even_lag_lds(self.effective_filter()[0::2], self.config.stu_lds_state_dim)
+            self.lds_fit_error = err
+            dev = self.M_filters.device
+            return a.to(dev), ce.to(dev).contiguous()
+        return self._cached("lds", (self.phi, self.M_filters), build)
+
+    def exact_flat_weights(self):
+        def build():
+            Kd = self.K * self.d_in
+            wp = self.M_phi_plus.reshape(Kd, self.d_out)
+            wm = self.M_phi_minus.reshape(Kd, self.d_out) if not self.use_hankel_L else None
+            return wp, wm
+        params = (self.M_phi_plus,) + (() if self.use_hankel_L else (self.M_phi_minus,))
+        return self._cached("flat", params, build)
+
+    # ---- full-sequence evaluation
+    def _project(self, x: torch.Tensor) -> torch.Tensor:
+        B, T, d = x.shape
+        if B * T <= _hip.MAX_DECODE_ROWS:
+            return _hip.linear_decode(x.reshape(B * T, d), self.m_inputs_t()).reshape(B, T, self.d_out)
+        return torch.matmul(x, self.M_inputs)
+
+    def _exact_sequence(self, x: torch.Tensor) -> torch.Tensor:
+        """use_approx=False: U+-[b,t,k,i] by the time-domain kernel, one filter at a
+        time, then the (K*d_in, d_out) contractions as library GEMMs with the
+        reference's rounding points (stu.py:107-120)."""
+        B, T, d = x.shape
+        Up = torch.empty(B, T, self.K, d, dtype=x.dtype, device=x.device)
+        Um = None if self.use_hankel_L else torch.empty_like(Up)
+        _hip.stu_conv_bank(x, self.phi, Up, Um)
+        wp, wm = self.exact_flat_weights()
+        y = torch.matmul(Up.reshape(B * T, self.K * d), wp)
+        if Um is not None:
+            y = y + torch.matmul(Um.reshape(B * T, self.K * d), wm)
+        return y.reshape(B, T, self.d_out)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, past_state=None, use_cache: bool = False):
+        """x (B,T,d).  Without past_state the whole sequence is convolved from
+        position 0 (the reference's forward).  With past_state, T must be 1 and
+        the call is one decode step.  Returns y, or (y, state) if use_cache."""
+        x = x.contiguous()
+        B, T, d = x.shape
+        if past_state is None:
+            if T > self.phi.shape[0]:
+                raise ValueError(f"sequence length {T} exceeds the filter length {self.phi.shape[0]}")
+            if self.use_approx:
+                xp = self._project(x)
+                y = _hip.stu_conv_direct(xp, self.effective_filter(), single_branch=self.use_hankel_L)
+                hist_src = xp
+            else:
+                y = self._exact_sequence(x)
+                hist_src = x
+            if not use_cache:
+                return y
+            return y, self._state_from_sequence(hist_src)
+        if T != 1:
+            raise ValueError("a decode call with past_state takes exactly one new position")
+        y, state = self._step(x.reshape(B, d), past_state)
+        y = y.reshape(B, 1, self.d_out)
+        return (y, state) if use_cache else y
+
+    # ---- decode state
+    def _state_from_sequence(self, src: torch.Tensor):
+        B, T, d = src.shape
+        pos = torch.full((B,), T, dtype=torch.int64)
+        if self.use_approx and self.decode_mode() == "lds":
+            a, _ = self.lds_params()
+            state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1)
+            return (src.new_empty(B, 0, d), state, pos)
+        cap = max(self.config.seq_len, T)
+        hist = src.new_zeros(B, cap, d)
+        hist[:, :T] = src
+        return (hist, torch.empty(B, 0, dtype=torch.float32, device=src.device), pos)
+
+    def _step(self, x: torch.Tensor, past_state):
+        hist, state, pos_t = past_state
+        pos = int(pos_t[0])
+        B, d = x.shape
+        if self.use_approx and state.numel() > 0:
+            a, ce = self.lds_params()
+            xp = _hip.linear_decode(x, self.m_inputs_t())
+            y = _hip.stu_step_lds(state, xp, a, ce, pos)
+            return y, (hist, state, pos_t + 1)
+        if pos >= hist.shape[1]:
+            hist = torch.cat([hist, torch.zeros_like(hist)], dim=1)
+        if pos >= self.phi.shape[0]:
+            raise ValueError(f"position {pos} is past the filter length {self.phi.shape[0]}")
+        if self.use_approx:
+            _hip.linear_decode(x, self.m_inputs_t(), hist[:, pos, :])
+            nsplit = _hist_nsplit(pos + 1)
+            eo = _hip.stu_step_hist(hist, self.effective_filter(), pos, nsplit)
+            y = torch.zeros(B, d, dtype=x.dtype, device=x.device)
+            _hip.add_rmsnorm(y, eo, None, 0.0, delta_mode=2, nslices=nsplit, single_branch=self.use_hankel_L,
+                             want_norm=False)
+            return y, (hist, state, pos_t + 1)
+        # exact mode: re-evaluate the bank over the stored inputs and keep the newest row
+        hist[:, pos, :] = x
+        y = self._exact_sequence(hist[:, : pos + 1].contiguous())[:, -1]
+        return y, (hist, state, pos_t + 1)
+
+
+def _hist_nsplit(nlags: int) -> int:
+    """Lag ranges per (batch) for the history kernel: enough workgroups to pull
+    bandwidth without making the partial-sum traffic comparable to the history."""
+    return max(1, min(16, nlags // 64))

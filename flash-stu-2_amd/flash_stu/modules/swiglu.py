@@ -1,0 +1,37 @@
+"""Gated MLP of Flash STU: down(gelu_tanh(gate(x)) * up(x))
+(reference: flash_stu/modules/swiglu.py:4-29; the gate is tanh-GELU despite the
+file name)."""
+import torch
+import torch.nn as nn
+
+from .. import _hip
+
+
+class MLP(nn.Module):
+    def __init__(self, config, dtype=None):
+        super().__init__()
+        dtype = dtype if dtype is not None else config.torch_dtype
+        self.hidden_size = config.n_embd
+        self.intermediate_size = config.n_embd * config.mlp_scale
+        self.gate_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=config.bias, dtype=dtype)
+        self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=config.bias, dtype=dtype)
+        self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=config.bias, dtype=dtype)
+        if config.bias:
+            raise NotImplementedError("bias=True is not supported by the HIP path")
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x (..., d).  Up to 16 rows take the skinny MFMA kernels with the gate
+        fused; more rows use library GEMMs plus the fused gelu*up kernel."""
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        rows = x2.shape[0]
+        if rows <= _hip.MAX_DECODE_ROWS:
+            act = _hip.glu_decode(x2, self.gate_proj.weight, self.up_proj.weight)
+            out = _hip.linear_decode(act, self.down_proj.weight)
+        else:
+            g = torch.matmul(x2, self.gate_proj.weight.t())
+            u = torch.matmul(x2, self.up_proj.weight.t())
+            act = _hip.gelu_mul(g, u, out=g)
+            out = torch.matmul(act, self.down_proj.weight.t())
+        return out.reshape(shape)

@@ -135,6 +135,14 @@ int fstu_stu_lds_state_from_hist(const void* hist, const float* a, float* state,
 int fstu_stu_conv_direct(const void* xp, const void* filt, void* y, int B, int T, int d, int L,
                          int single_branch, int dtype, void* stream);
 
+/* Exact mode (use_approx=False): the whole filter bank at once.
+ *   u_plus[b,t,k,c]  = T( sum_{s<=t} phi[s,k] x[b,t-s,c] )
+ *   u_minus[b,t,k,c] = T( sum_{s<=t} (-1)^s phi[s,k] x[b,t-s,c] )   (skipped if NULL)
+ * x (B,T,d), phi (L,K), outputs (B,T,K,d).  Replaces convolve(..., use_approx=False)
+ * at flash_stu/utils/stu_utils.py:214-228 without expanding x K-fold. */
+int fstu_stu_conv_bank(const void* x, const void* phi, void* u_plus, void* u_minus, int B, int T, int d,
+                       int L, int K, int dtype, void* stream);
+
 /* ---- sliding-window attention ----------------------------------------------
  * KV ring layout: (B,H,cap,hd), absolute position j lives in slot j % cap,
  * cap >= window+1.
@@ -184,6 +192,69 @@ int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int
  * Bm (d_in,S), Cm (S,d_out) in the model dtype.  S <= 256. */
 int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, const void* Cm, void* y,
                    int T_steps, int Bt, int d_in, int S, int d_out, int dtype, void* stream);
+
+/* ---- whole decode step -----------------------------------------------------
+ * One call launches every kernel of one token step for all layers: embedding of
+ * the input token, the layer stack against its decode state, final norm, tied
+ * head, and sampling of the next token.  It is the body of the loop at
+ * flash_stu/model.py:245-302 for steps after the first, with the per-layer state
+ * the reference lacks for STU layers (flash_stu/layers/stu_layer.py:99-120).
+ * The descriptors only carry device pointers owned by the caller. */
+typedef struct {
+  int kind;                 /* 0: STU layer (approx mode), 1: attention layer */
+  const void* norm1_w;      /* stu_norm / attn_norm weight (d) */
+  const void* mlp_norm_w;   /* (d) */
+  const void* w_gate;       /* (I,d) */
+  const void* w_up;         /* (I,d) */
+  const void* w_down;       /* (d,I) */
+  /* STU */
+  const void* m_inputs_t;   /* (d,d): M_inputs transposed, [out][in] */
+  const void* filt;         /* (L,d) phi_proj, model dtype       (history mode) */
+  void* hist;               /* (B,hist_cap,d) x_proj history      (history mode) */
+  const float* lds_a;       /* (S)                                (lds mode) */
+  const float* lds_ce;      /* (S,d)                              (lds mode) */
+  float* lds_state;         /* (B,2,S,d)                          (lds mode) */
+  /* attention */
+  const void* w_qkv;        /* (3d,d) */
+  const void* w_proj;       /* (d,d) */
+  void* kring;              /* (B,H,kv_cap,hd) */
+  void* vring;
+  const float* slopes;      /* (H) */
+} fstu_layer_desc;
+
+typedef struct {
+  int dtype;
+  int B, d, I, V, n_layers, n_heads, head_dim;
+  int window, kv_cap;
+  int L, hist_cap;
+  int stu_mode;             /* 0: history, 1: lds */
+  int lds_S;
+  int single_branch;        /* use_hankel_L */
+  int ksplit_down;          /* K split of the down projection (partial holds ksplit_down*B*d floats) */
+  int hist_nsplit_max;      /* eo holds hist_nsplit_max*2*B*d floats */
+  float eps, softcap;
+  const void* emb;          /* (V,d) tied embedding / head */
+  const void* final_norm_w; /* (d) */
+  const fstu_layer_desc* layers;   /* host array of n_layers entries */
+  /* workspaces, model dtype unless noted */
+  void* x;                  /* (B,d) residual stream */
+  void* h;                  /* (B,d) normalised activations */
+  void* qkv;                /* (B,3d) */
+  void* attn;               /* (B,d) */
+  void* act;                /* (B,I) */
+  void* xp;                 /* (B,d) */
+  void* y;                  /* (B,d) */
+  float* partial;           /* fp32 */
+  float* eo;                /* fp32 */
+  void* logits;             /* (B,V) */
+} fstu_model_desc;
+
+/* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next
+ * token is written to tok_out[b*tok_stride].  `step` indexes the sampling
+ * stream.  Sampling arguments as in fstu_sample. */
+int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
+                     int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                     int step, void* stream);
 
 #ifdef __cplusplus
 }
