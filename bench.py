@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Decode-throughput benchmark of the Flash STU token loop on one MI355X.
+
+Workload (BASELINE config 2): FlashSTU 768-d / 12 layers (STU, SWA alternating)
+/ 12 heads / window 512 / 24 filters / seq_len 2048 / vocab 50257, random-init
+bf16 (seed 1), batch 8, 512-token prompts of uniform random ids, greedy decode.
+One "step" is one decode step of the whole batch (8 tokens).  The prompt is
+prefilled (untimed, reported separately), W warm-up steps run, then exactly K
+steps are timed with the inputs, weights and decode state resident in HBM.
+
+Prints one JSON line; see the keys below.  `roofline` is the dominant kernel
+(the gate/up GLU projection, the largest weight stream of a step), timed live
+with HIP events on the launch stream in a second pass over the same K steps;
+`step_roofline` is the whole step against the HBM roofline; `cpu_baseline` is
+the CPU oracle on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "flash-stu-2_amd"))
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def build_model(args, torch):
+    from flash_stu import FlashSTU, FlashSTUConfig
+    cfg = FlashSTUConfig(n_embd=768, n_layers=12, n_heads=12, window_size=512, num_eigh=24, seq_len=2048,
+                         vocab_size=50257, mlp_scale=args.mlp_scale, torch_dtype=torch.bfloat16,
+                         stu_decode_mode=args.stu_mode)
+    torch.manual_seed(1)
+    model = FlashSTU(cfg).cuda().eval()
+    return cfg, model
+
+
+def decode_step_bytes(cfg, B, t, mode, S):
+    """Algorithmic HBM bytes of one decode step at position t (every weight
+    once, visible KV window + one row written, STU state or history, logits)."""
+    d, I, V, w = cfg.n_embd, cfg.n_embd * cfg.mlp_scale, cfg.vocab_size, 2
+    n_att = sum(1 for i in range(cfg.n_layers) if i % 2 == 1 and cfg.use_attn)
+    n_stu = cfg.n_layers - n_att
+    weights = (cfg.n_layers * (3 * d * I + 2 * d) + n_att * 4 * d * d + n_stu * d * d + d + V * d) * w
+    kv = n_att * B * 2 * d * w * (min(t, cfg.window_left + 1) + 1)
+    if mode == "lds":
+        stu = n_stu * (B * S * d * 4 * 2 + S * d * 4)
+    else:
+        stu = n_stu * (B * (t + 1) * d * w + (t + 1) * d * w)
+    return weights + kv + stu + B * V * w
+
+
+def cpu_baseline(args, torch):
+    """CPU oracle (stateful decode) on a bounded sample: batch 8, 32-token
+    prompt, 6 decode steps, same architecture and dtype."""
+    from oracle import flashstu_oracle as O
+    ocfg = O.OracleConfig(n_embd=768, n_heads=12, n_layers=12, seq_len=2048, window_size=512, vocab_size=50257,
+                          mlp_scale=args.mlp_scale, num_eigh=24, dtype=torch.bfloat16)
+    phi = torch.zeros(2048, 24, dtype=torch.bfloat16)       # filter values do not change the cost
+    phi[:, :] = torch.linspace(0.1, 1.0, 24, dtype=torch.float32).bfloat16()
+    w = O.init_weights(ocfg, seed=1, mode="reference", phi=phi)
+    B, P, N = 8, 32, 6
+    ids = torch.randint(0, 50257, (B, P), generator=torch.Generator().manual_seed(0))
+    with torch.no_grad():
+        st = O.DecodeState(w, ocfg, B)
+        t0 = time.perf_counter()
+        logits = st.prefill(ids)
+        t_pre = time.perf_counter() - t0
+        tok = logits[:, -1].argmax(-1)
+        st.step(tok)                                   # warm-up step
+        t0 = time.perf_counter()
+        for _ in range(N):
+            tok = st.step(tok)[:, -1].argmax(-1)
+        t_dec = time.perf_counter() - t0
+    return {"value": B * N / t_dec, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"CPU oracle, bf16, batch {B}, {P}-token prompt, {N} stateful decode steps "
+                      f"(prefill {B * P / t_pre:.0f} tokens/s)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--mlp-scale", type=int, default=12, dest="mlp_scale")
+    ap.add_argument("--stu-mode", default="lds", choices=["lds", "history"], dest="stu_mode")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--breakdown", action="store_true", help="time every kernel class with HIP events")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (batch-sharded decode needs no exchange; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import ctypes
+    import torch
+    from flash_stu import _hip
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    cfg, model = build_model(args, torch)
+    B, P, K, W = args.batch, args.prompt, args.steps, args.warmup
+    total = P + W + 2 * K + 8
+    assert total <= cfg.seq_len or args.stu_mode == "lds"
+    ids = torch.randint(0, cfg.vocab_size, (B, P), generator=torch.Generator().manual_seed(1)).cuda()
+    eng = model.decode_engine()
+    tokens = torch.zeros(B, total, dtype=torch.int64, device="cuda")
+    tokens[:, :P] = ids
+    # ---- prefill (untimed for `value`, reported on its own)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = eng.prefill(ids, total)
+    _hip.sample(logits, tokens[:, P], do_sample=False)
+    torch.cuda.synchronize()
+    t_prefill_cold = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    logits = eng.prefill(ids, total)
+    _hip.sample(logits, tokens[:, P], do_sample=False)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    pos = P
+
+    def run(n):
+        nonlocal pos
+        for _ in range(n):
+            eng.step(tokens, pos, 1.0, None, None, False, 0, pos - P + 1)
+            pos += 1
+
+    run(W)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(K)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / K * 1e3
+    value = B * K / dt
+    t_mid = P + W + K // 2
+    S = cfg.stu_lds_state_dim
+    step_bytes = decode_step_bytes(cfg, B, t_mid, args.stu_mode, S)
+    # ---- second pass over K steps with events around the dominant kernel
+    lib = _hip.load()
+    lib.fstu_prof_begin.argtypes = [ctypes.c_int, ctypes.c_int]
+    lib.fstu_prof_end.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
+
+    def timed_class(cls, n):
+        nonlocal pos
+        save = pos
+        _hip._check(lib.fstu_prof_begin(cls, n * cfg.n_layers * 2 + 8), "fstu_prof_begin")
+        run(n)
+        ms, cnt = ctypes.c_double(), ctypes.c_int()
+        _hip._check(lib.fstu_prof_end(ctypes.byref(ms), ctypes.byref(cnt)), "fstu_prof_end")
+        pos = save
+        return ms.value, cnt.value
+
+    glu_ms, glu_n = timed_class(1, K)
+    d, I = cfg.n_embd, cfg.n_embd * cfg.mlp_scale
+    glu_bytes = 2 * I * d * 2 + B * d * 2 + B * I * 2          # gate+up weights, x in, act out
+    glu_avg_us = glu_ms / glu_n * 1e3
+    glu_gbps = glu_bytes / (glu_avg_us * 1e-6) / 1e9
+    out = {
+        "metric": "decode tokens/sec at 1 GPU (768-d FlashSTU, bs=8) + achieved HBM GB/s",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: FlashSTU 768-d/12-layer/12-head, window 512, K=24, seq_len 2048, "
+                               "vocab 50257, random-init bf16 seed 1, batch 8, 512-token prompt, greedy decode",
+                   "mlp_scale": cfg.mlp_scale, "params": model.get_num_params(), "batch": B, "prompt": P,
+                   "stu_decode_mode": args.stu_mode, "stu_state_dim": S if args.stu_mode == "lds" else None},
+        "roofline": {"bound": "hbm", "kernel": "linear_mfma_bf16_kernel<GLU> (gate/up projection + gelu*up)",
+                     "achieved": glu_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": glu_gbps / HBM_PEAK_GBPS,
+                     "traffic": None, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,
+                     "launches_timed": glu_n},
+        "step_roofline": {"bound": "hbm", "bytes_per_step": step_bytes, "achieved": step_bytes / (ms_per_step * 1e-3) / 1e9,
+                          "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                          "frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "prefill_tokens_per_s": B * P / t_prefill, "prefill_ms": t_prefill * 1e3, "prefill_first_call_ms": t_prefill_cold * 1e3,
+    }
+    if args.breakdown:
+        names = {1: "glu", 2: "down", 3: "head", 4: "attention", 5: "stu_step", 6: "proj_qkv", 7: "embed_add_norm", 8: "sample"}
+        n = min(K, 32)
+        out["kernel_us_per_step"] = {names[c]: timed_class(c, n)[0] / n * 1e3 for c in names}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args, torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

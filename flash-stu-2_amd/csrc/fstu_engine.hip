@@ -8,6 +8,56 @@
     if (rc__ != 0) return rc__; \
   } while (0)
 
+// ---------------------------------------------------------------- live kernel timing
+// Optional: HIP events recorded around every launch of one kernel class inside
+// fstu_decode_step, on the stream the kernels run on.
+enum { PC_NONE = 0, PC_GLU = 1, PC_DOWN = 2, PC_HEAD = 3, PC_SWA = 4, PC_STU = 5, PC_PROJ = 6, PC_NORM = 7, PC_SAMPLE = 8, PC_NCLASS = 9 };
+static int g_prof_class = PC_NONE;
+static hipEvent_t* g_prof_ev = nullptr;
+static int g_prof_cap = 0, g_prof_n = 0;
+
+extern "C" int fstu_prof_begin(int kernel_class, int max_launches) {
+  FSTU_REQUIRE(kernel_class > PC_NONE && kernel_class < PC_NCLASS && max_launches > 0, FSTU_EARG, "fstu_prof_begin: bad class %d / capacity %d", kernel_class, max_launches);
+  FSTU_REQUIRE(g_prof_ev == nullptr, FSTU_EARG, "fstu_prof_begin: already profiling");
+  g_prof_ev = new hipEvent_t[2 * (size_t)max_launches];
+  for (int i = 0; i < 2 * max_launches; ++i) {
+    hipError_t e = hipEventCreate(&g_prof_ev[i]);
+    if (e != hipSuccess) { fstu_set_error("fstu_prof_begin: hipEventCreate: %s", hipGetErrorString(e)); return (int)e; }
+  }
+  g_prof_class = kernel_class;
+  g_prof_cap = max_launches;
+  g_prof_n = 0;
+  return FSTU_OK;
+}
+
+extern "C" int fstu_prof_end(double* total_ms, int* launches) {
+  FSTU_REQUIRE(g_prof_ev != nullptr && total_ms && launches, FSTU_EARG, "fstu_prof_end: not profiling");
+  double tot = 0.0;
+  for (int i = 0; i < g_prof_n; ++i) {
+    (void)hipEventSynchronize(g_prof_ev[2 * i + 1]);
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, g_prof_ev[2 * i], g_prof_ev[2 * i + 1]);
+    tot += ms;
+  }
+  for (int i = 0; i < 2 * g_prof_cap; ++i) (void)hipEventDestroy(g_prof_ev[i]);
+  delete[] g_prof_ev;
+  g_prof_ev = nullptr;
+  *total_ms = tot;
+  *launches = g_prof_n;
+  g_prof_class = PC_NONE;
+  g_prof_cap = g_prof_n = 0;
+  return FSTU_OK;
+}
+
+#define TIMED(cls, call)                                                                        \
+  do {                                                                                          \
+    const bool t__ = (g_prof_class == (cls)) && g_prof_n < g_prof_cap;                          \
+    if (t__) (void)hipEventRecord(g_prof_ev[2 * g_prof_n], (hipStream_t)stream);                    \
+    int rc__ = (call);                                                                          \
+    if (t__) { (void)hipEventRecord(g_prof_ev[2 * g_prof_n + 1], (hipStream_t)stream); ++g_prof_n; }  \
+    if (rc__ != 0) return rc__;                                                                 \
+  } while (0)
+
 static int hist_nsplit(int nlags, int maxsplit) {
   int n = nlags / 64;
   if (n < 1) n = 1;
@@ -43,37 +93,37 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
                    "fstu_decode_step: layer %d has no attention state", l);
     }
   }
-  STEP(fstu_embed_strided(tok_in, tok_stride, m->emb, m->x, B, d, m->V, dt, stream));
+  TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, m->x, B, d, m->V, dt, stream));
   // h = norm(x) with the first layer's norm weight
-  STEP(fstu_add_rmsnorm(m->x, nullptr, 0, 1, 0, m->layers[0].norm1_w, m->h, B, d, m->eps, dt, stream));
+  TIMED(PC_NORM, fstu_add_rmsnorm(m->x, nullptr, 0, 1, 0, m->layers[0].norm1_w, m->h, B, d, m->eps, dt, stream));
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     if (L.kind == 0) {
       if (m->stu_mode == 0) {
         char* row = (char*)L.hist + (size_t)pos * d * esz;  // hist[:, pos, :] with row stride hist_cap*d
-        STEP(fstu_linear_decode(m->h, d, L.m_inputs_t, row, m->hist_cap * d, B, d, d, dt, stream));
+        TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, row, m->hist_cap * d, B, d, d, dt, stream));
         int ns = hist_nsplit(pos + 1, m->hist_nsplit_max);
-        STEP(fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
-        STEP(fstu_add_rmsnorm(m->x, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+        TIMED(PC_STU, fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
+        TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
-        STEP(fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-        STEP(fstu_stu_step_lds(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dt, stream));
-        STEP(fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+        TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
+        TIMED(PC_STU, fstu_stu_step_lds(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dt, stream));
+        TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       }
     } else {
-      STEP(fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
-      STEP(fstu_kv_append(m->qkv, L.kring, L.vring, B, m->n_heads, m->head_dim, m->kv_cap, pos, dt, stream));
-      STEP(fstu_swa_decode(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
+      TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
+      TIMED(PC_SWA, fstu_kv_append(m->qkv, L.kring, L.vring, B, m->n_heads, m->head_dim, m->kv_cap, pos, dt, stream));
+      TIMED(PC_SWA, fstu_swa_decode(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
                            m->window, m->softcap, dt, stream));
-      STEP(fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
-      STEP(fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+      TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
+      TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
     }
-    STEP(fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
-    STEP(fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
+    TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
+    TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
-    STEP(fstu_add_rmsnorm(m->x, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
+    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
-  STEP(fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
-  STEP(fstu_sample(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dt, stream));
+  TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
+  TIMED(PC_SAMPLE, fstu_sample(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dt, stream));
   return FSTU_OK;
 }

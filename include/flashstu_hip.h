@@ -256,6 +256,17 @@ int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* t
                      int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                      int step, void* stream);
 
+/* ---- live kernel timing (measurement aid; no counterpart in the reference) ----
+ * Between fstu_prof_begin and fstu_prof_end every launch of one kernel class
+ * inside fstu_decode_step is bracketed by HIP events on the launch stream
+ * (at most max_launches of them; events are created and destroyed by these two
+ * calls).  fstu_prof_end waits for the events and returns the summed kernel
+ * time and the number of launches.  Classes: 1 gate/up GLU, 2 down projection,
+ * 3 head, 4 attention (append+decode), 5 STU step, 6 d-by-d projections and
+ * QKV, 7 embed/add/RMSNorm, 8 sampling.  Not thread-safe. */
+int fstu_prof_begin(int kernel_class, int max_launches);
+int fstu_prof_end(double* total_ms, int* launches);
+
 #ifdef __cplusplus
 }
 #endif

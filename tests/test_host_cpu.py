@@ -23,7 +23,8 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_hip.LIB_PATH)
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
-    bound = set(_hip.SIGNATURES) | {"fstu_version", "fstu_last_error", "fstu_decode_step"}
+    bound = set(_hip.SIGNATURES) | {"fstu_version", "fstu_last_error", "fstu_decode_step", "fstu_prof_begin",
+                                       "fstu_prof_end"}
     assert declared == bound, declared ^ bound
     assert _hip.load().fstu_version() == 100
 
