@@ -89,6 +89,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch every step kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--breakdown", action="store_true", help="time every kernel class with HIP events")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -129,12 +130,29 @@ def main():
             eng.step(tokens, pos, 1.0, None, None, False, 0, pos - P + 1)
             pos += 1
 
-    run(W)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run(K)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    use_graph = eng.graph_supported() and not args.no_graph
+    if use_graph:
+        # one decode step captured once; every replay reads its position from device memory
+        eng.graph_begin(tokens, pos, pos - P + 1, 1.0, None, None, False, 0)
+        for _ in range(W):
+            eng.graph_step()
+        eng._gstream.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            eng.graph_step()
+        eng._gstream.synchronize()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        eng.graph_end()
+        pos += W + K
+    else:
+        run(W)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(K)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
     ms_per_step = dt / K * 1e3
     value = B * K / dt
     t_mid = P + W + K // 2
@@ -167,7 +185,7 @@ def main():
         "config": {"workload": "BASELINE config 2: FlashSTU 768-d/12-layer/12-head, window 512, K=24, seq_len 2048, "
                                "vocab 50257, random-init bf16 seed 1, batch 8, 512-token prompt, greedy decode",
                    "mlp_scale": cfg.mlp_scale, "params": model.get_num_params(), "batch": B, "prompt": P,
-                   "stu_decode_mode": args.stu_mode, "stu_state_dim": S if args.stu_mode == "lds" else None},
+                   "stu_decode_mode": args.stu_mode, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
         "roofline": {"bound": "hbm", "kernel": "linear_mfma_bf16_kernel<GLU> (gate/up projection + gelu*up)",
                      "achieved": glu_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": glu_gbps / HBM_PEAK_GBPS,
                      "traffic": None, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,

@@ -146,42 +146,54 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 }
 
 // ---------------------------------------------------------------- decode
+// One workgroup per (batch, head); NWAVES*8 key groups visit 4 keys each per
+// sweep, so a 513-key window is covered in two sweeps with every load of a
+// sweep in flight at once.  With append != 0 the workgroup first stores the new
+// token's k,v (read from the qkv row) into ring slot pos % cap.
 #define SWA_U 4
-template <typename T, int HD>
-__global__ void __launch_bounds__(256)
-swa_decode_kernel(const T* __restrict__ qkv, const T* __restrict__ kring, const T* __restrict__ vring,
-                  T* __restrict__ out, const float* __restrict__ slopes, int H, int cap, int pos, int window,
-                  float softcap) {
+template <typename T, int HD, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64)
+swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__ out, const float* __restrict__ slopes,
+                  int H, int cap, int pos, int window, float softcap, int append, const int* __restrict__ dyn) {
   constexpr int DPL = HD / 8;
-  __shared__ float sm[32], sl[32];
-  __shared__ float sacc[32][HD];
+  constexpr int NGRP = NWAVES * 8;
+  if (dyn) pos = dyn[0];
+  __shared__ float sm[NGRP], sl[NGRP];
+  __shared__ float sacc[NGRP][HD];
   const int h = blockIdx.x, b = blockIdx.y;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int grp = lane >> 3, gl = lane & 7;
-  const int G = w * 8 + grp;  // group index 0..31
+  const int G = w * 8 + grp;
   const int d = H * HD;
+  const T* row = qkv + (size_t)b * 3 * d + h * HD;
+  const size_t hbase = ((size_t)b * H + h) * cap * HD;
+  if (append) {
+    if (threadIdx.x < HD) {
+      size_t dst = hbase + (size_t)(pos % cap) * HD + threadIdx.x;
+      kring[dst] = row[d + threadIdx.x];
+      vring[dst] = row[2 * d + threadIdx.x];
+    }
+    __syncthreads();
+  }
   float q[DPL];
-  load_vec<T, DPL>(qkv + (size_t)b * 3 * d + h * HD + gl * DPL, q);
-  const size_t base = ((size_t)b * H + h) * cap * HD + gl * DPL;
+  load_vec<T, DPL>(row + gl * DPL, q);
   Partial<DPL> P;
   P.m = -INFINITY;
   P.l = 0.f;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
   const int lo = max(0, pos - window);
-  attend_keys<T, DPL, SWA_U>(P, kring + base, vring + base, HD, cap, q, lo + G * SWA_U, pos + 1, 32 * SWA_U, pos,
-                             rsqrtf((float)HD), softcap, slopes[h]);
+  attend_keys<T, DPL, SWA_U>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, q, lo + G * SWA_U, pos + 1,
+                             NGRP * SWA_U, pos, rsqrtf((float)HD), softcap, slopes[h]);
   if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
 #pragma unroll
   for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];
   __syncthreads();
   if (threadIdx.x < HD) {
     float M = -INFINITY;
-#pragma unroll
-    for (int g = 0; g < 32; ++g) M = fmaxf(M, sm[g]);
+    for (int g = 0; g < NGRP; ++g) M = fmaxf(M, sm[g]);
     float Lsum = 0.f, o = 0.f;
-#pragma unroll
-    for (int g = 0; g < 32; ++g) {
+    for (int g = 0; g < NGRP; ++g) {
       float e = __expf(sm[g] - M);
       Lsum = fmaf(sl[g], e, Lsum);
       o = fmaf(sacc[g][threadIdx.x], e, o);
@@ -205,9 +217,8 @@ static int check_swa(const char* name, int H, int hd, int window, const void* sl
     else hipLaunchKernelGGL((KERNEL<T, 256>), __VA_ARGS__);                \
   } while (0)
 
-extern "C" int fstu_swa_decode(const void* qkv, const void* kring, const void* vring, void* out, const float* slopes,
-                               int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
-                               void* stream) {
+int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B, int H, int hd,
+                         int cap, int pos, int window, float softcap, int append, const int* dyn, int dtype, void* stream) {
   int rc = check_kv("fstu_swa_decode", qkv, kring, vring, B, H, hd, cap);
   if (rc) return rc;
   rc = check_swa("fstu_swa_decode", H, hd, window, slopes);
@@ -217,11 +228,31 @@ extern "C" int fstu_swa_decode(const void* qkv, const void* kring, const void* v
   FSTU_REQUIRE(fstu_aligned(qkv, 16) && fstu_aligned(kring, 16) && fstu_aligned(vring, 16), FSTU_EALIGN, "fstu_swa_decode: pointers must be 16-byte aligned");
   FSTU_REQUIRE(B <= 65535, FSTU_ESHAPE, "fstu_swa_decode: B too large");
   hipStream_t s = (hipStream_t)stream;
-  FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_decode",
-                      SWA_DISPATCH_HD(swa_decode_kernel, hd, dim3(H, B), dim3(256), 0, s, (const T*)qkv,
-                                      (const T*)kring, (const T*)vring, (T*)out, slopes, H, cap, pos, window, softcap));
+  const int nkeys = dyn ? window + 1 : (pos < window ? pos : window) + 1;
+#define SWA_LAUNCH(HD, NW)                                                                                      \
+  hipLaunchKernelGGL((swa_decode_kernel<T, HD, NW>), dim3(H, B), dim3(NW * 64), 0, s, (const T*)qkv, (T*)kring, \
+                     (T*)vring, (T*)out, slopes, H, cap, pos, window, softcap, append, dyn)
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_decode", {
+    if (hd == 32) { if (nkeys > 128) SWA_LAUNCH(32, 16); else SWA_LAUNCH(32, 4); }
+    else if (hd == 64) { if (nkeys > 128) SWA_LAUNCH(64, 16); else SWA_LAUNCH(64, 4); }
+    else if (hd == 128) { if (nkeys > 128) SWA_LAUNCH(128, 8); else SWA_LAUNCH(128, 4); }
+    else SWA_LAUNCH(256, 4);
+  });
+#undef SWA_LAUNCH
   FSTU_CHECK_LAUNCH("fstu_swa_decode");
   return FSTU_OK;
+}
+
+extern "C" int fstu_swa_decode(const void* qkv, const void* kring, const void* vring, void* out, const float* slopes,
+                               int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
+                               void* stream) {
+  return fstu_swa_decode_impl(qkv, (void*)kring, (void*)vring, out, slopes, B, H, hd, cap, pos, window, softcap, 0, nullptr, dtype, stream);
+}
+
+extern "C" int fstu_swa_append_decode(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B,
+                                      int H, int hd, int cap, int pos, int window, float softcap, int dtype,
+                                      void* stream) {
+  return fstu_swa_decode_impl(qkv, kring, vring, out, slopes, B, H, hd, cap, pos, window, softcap, 1, nullptr, dtype, stream);
 }
 
 // ---------------------------------------------------------------- prefill

@@ -29,9 +29,21 @@ void fstu_set_error(const char* fmt, ...);
     }                                                                     \
   } while (0)
 
-// library-internal: embedding gather of ids[r*id_stride]
+// ---- library-internal launchers used by the decode-step driver.  `dyn`, when not null, is a device int[2]
+// {position, sampling step} read by the kernels instead of the host-side values, so that a captured graph of one
+// step can be replayed for every position.
 int fstu_embed_strided(const int64_t* ids, int64_t id_stride, const void* table, void* out, int rows, int d, int vocab,
-                       int dtype, void* stream);
+                       int dtype, void* stream, const int* dyn);
+int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
+                          int B, int S, int d, int t, const int* dyn, int dtype, void* stream);
+int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B, int H, int hd,
+                         int cap, int pos, int window, float softcap, int append, const int* dyn, int dtype, void* stream);
+int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, const int* dyn,
+                         int dtype, void* stream);
+int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
+                    float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream);
+int fstu_advance_dyn(int* dyn, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

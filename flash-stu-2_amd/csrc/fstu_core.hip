@@ -19,9 +19,9 @@ extern "C" int fstu_version(void) { return FSTU_VERSION; }
 // ---------------------------------------------------------------- embed
 template <typename T>
 __global__ void embed_kernel(const int64_t* __restrict__ ids, int64_t id_stride, const T* __restrict__ table,
-                             T* __restrict__ out, int d, int vocab) {
+                             T* __restrict__ out, int d, int vocab, const int* __restrict__ dyn) {
   int r = blockIdx.x;
-  int64_t id = ids[(size_t)r * id_stride];
+  int64_t id = ids[(size_t)r * id_stride + (dyn ? dyn[0] : 0)];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + (size_t)id * d;
   T* dst = out + (size_t)r * d;
@@ -35,27 +35,29 @@ extern "C" int fstu_embed(const int64_t* ids, const void* table, void* out, int 
   if (rows == 0) return FSTU_OK;
   FSTU_DISPATCH_DTYPE(dtype, "fstu_embed",
                       hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids,
-                                         (int64_t)1, (const T*)table, (T*)out, d, vocab));
+                                         (int64_t)1, (const T*)table, (T*)out, d, vocab, (const int*)nullptr));
   FSTU_CHECK_LAUNCH("fstu_embed");
   return FSTU_OK;
 }
 
-// ids[r*id_stride]: one column of a (rows, id_stride) token buffer (library-internal)
+// ids[r*id_stride (+ dyn[0])]: one column of a (rows, id_stride) token buffer (library-internal)
 int fstu_embed_strided(const int64_t* ids, int64_t id_stride, const void* table, void* out, int rows, int d, int vocab,
-                       int dtype, void* stream) {
+                       int dtype, void* stream, const int* dyn) {
   FSTU_REQUIRE(ids && table && out, FSTU_ENULL, "fstu_embed: null pointer");
   FSTU_DISPATCH_DTYPE(dtype, "fstu_embed",
                       hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids,
-                                         id_stride, (const T*)table, (T*)out, d, vocab));
+                                         id_stride, (const T*)table, (T*)out, d, vocab, dyn));
   FSTU_CHECK_LAUNCH("fstu_embed");
   return FSTU_OK;
 }
 
 // ---------------------------------------------------------------- add + rmsnorm
-// One workgroup (256 threads) per row; the row lives in registers between the
-// residual update and the normalisation.  d <= 256*FSTU_NORM_MAX_PER_THREAD.
+// One workgroup (256 threads) per row; a thread owns groups of 4 consecutive
+// channels (16-byte fp32 loads, 8-byte bf16 loads) and keeps them in registers
+// between the residual update and the normalisation.  Partial-sum slices are
+// read four at a time into independent accumulators so their load latencies
+// overlap; the summation order is fixed (deterministic).
 #define FSTU_NORM_THREADS 256
-#define FSTU_NORM_MAX_PER_THREAD 32
 
 __device__ __forceinline__ float block_sum_256(float v, float* red) {
   v = wave_sum(v);
@@ -67,44 +69,97 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return s;
 }
 
-template <typename T>
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void ld(const float* p, float* o) {
+    float4 v = *(const float4*)p;
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float* v) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float* o) {
+    uint2 v = *(const uint2*)p;
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
+    uint2 o;
+    o.x = (unsigned)f32_to_bf16(v[0]) | ((unsigned)f32_to_bf16(v[1]) << 16);
+    o.y = (unsigned)f32_to_bf16(v[2]) | ((unsigned)f32_to_bf16(v[3]) << 16);
+    *(uint2*)p = o;
+  }
+};
+
+// sum of `n` fp32 slices (stride `stride` floats) of 4 consecutive values in a fixed order; up to 16 slices are
+// loaded before any is added so their latencies overlap
+__device__ __forceinline__ void sum_slices4(const float* p, size_t stride, int n, float* out) {
+  float4 tot = make_float4(0, 0, 0, 0);
+  for (int s0 = 0; s0 < n; s0 += 16) {
+    float4 v[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) v[k] = (s0 + k < n) ? *(const float4*)(p + (size_t)(s0 + k) * stride) : make_float4(0, 0, 0, 0);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { tot.x += v[k].x; tot.y += v[k].y; tot.z += v[k].z; tot.w += v[k].w; }
+  }
+  out[0] = tot.x; out[1] = tot.y; out[2] = tot.z; out[3] = tot.w;
+}
+
+template <typename T, int NG, bool VEC>
 __global__ void __launch_bounds__(FSTU_NORM_THREADS)
 add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_mode, int nslices, int single_branch,
                    const T* __restrict__ w, T* __restrict__ y, int rows, int d, float eps) {
+  // VEC: d % 4 == 0 and all pointers 16-byte aligned; a group is 4 channels.  Otherwise a group is 1 channel.
+  constexpr int GW = VEC ? 4 : 1;
   __shared__ float red[4];
   const int r = blockIdx.x;
   T* xr = x + (size_t)r * d;
-  float v[FSTU_NORM_MAX_PER_THREAD];
+  const size_t slice = (size_t)rows * d;
+  float v[NG][GW];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < FSTU_NORM_MAX_PER_THREAD; ++i) {
-    int c = threadIdx.x + i * FSTU_NORM_THREADS;
-    v[i] = 0.f;
+  for (int i = 0; i < NG; ++i) {
+    const int c = (threadIdx.x + i * FSTU_NORM_THREADS) * GW;
+#pragma unroll
+    for (int k = 0; k < GW; ++k) v[i][k] = 0.f;
     if (c < d) {
-      float xv = DT<T>::ld(xr + c);
+      float xv[GW], dv[GW];
+      if (VEC) Vec4<T>::ld(xr + c, xv); else xv[0] = DT<T>::ld(xr + c);
       if (delta != nullptr) {
-        float dv;
         if (delta_mode == 0) {
-          dv = DT<T>::ld((const T*)delta + (size_t)r * d + c);
+          const T* dp = (const T*)delta + (size_t)r * d + c;
+          if (VEC) Vec4<T>::ld(dp, dv); else dv[0] = DT<T>::ld(dp);
         } else if (delta_mode == 1) {
           const float* p = (const float*)delta + (size_t)r * d + c;
-          float acc = 0.f;
-          for (int s = 0; s < nslices; ++s) acc += p[(size_t)s * rows * d];
-          dv = DT<T>::rnd(acc);
+          if (VEC) {
+            sum_slices4(p, slice, nslices, dv);
+          } else {
+            float acc = 0.f;
+            for (int s = 0; s < nslices; ++s) acc += p[(size_t)s * slice];
+            dv[0] = acc;
+          }
+#pragma unroll
+          for (int k = 0; k < GW; ++k) dv[k] = DT<T>::rnd(dv[k]);
         } else {
           const float* p = (const float*)delta + (size_t)r * d + c;
-          float e = 0.f, o = 0.f;
-          for (int s = 0; s < nslices; ++s) {
-            e += p[(size_t)(2 * s) * rows * d];
-            o += p[(size_t)(2 * s + 1) * rows * d];
+          float e[GW], o[GW];
+          if (VEC) {
+            sum_slices4(p, 2 * slice, nslices, e);
+            sum_slices4(p + slice, 2 * slice, nslices, o);
+          } else {
+            e[0] = o[0] = 0.f;
+            for (int s = 0; s < nslices; ++s) { e[0] += p[(size_t)(2 * s) * slice]; o[0] += p[(size_t)(2 * s + 1) * slice]; }
           }
-          dv = single_branch ? DT<T>::rnd(e + o) : DT<T>::rnd(DT<T>::rnd(e + o) + DT<T>::rnd(e - o));
+#pragma unroll
+          for (int k = 0; k < GW; ++k)
+            dv[k] = single_branch ? DT<T>::rnd(e[k] + o[k]) : DT<T>::rnd(DT<T>::rnd(e[k] + o[k]) + DT<T>::rnd(e[k] - o[k]));
         }
-        xv = DT<T>::rnd(xv + dv);
-        DT<T>::st(xr + c, xv);
+#pragma unroll
+        for (int k = 0; k < GW; ++k) xv[k] = DT<T>::rnd(xv[k] + dv[k]);
+        if (VEC) Vec4<T>::st(xr + c, xv); else DT<T>::st(xr + c, xv[0]);
       }
-      v[i] = xv;
-      ss += xv * xv;
+#pragma unroll
+      for (int k = 0; k < GW; ++k) { v[i][k] = xv[k]; ss += xv[k] * xv[k]; }
     }
   }
   if (y == nullptr) return;
@@ -112,10 +167,36 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
   float rstd = rsqrtf(tot / (float)d + eps);
   T* yr = y + (size_t)r * d;
 #pragma unroll
-  for (int i = 0; i < FSTU_NORM_MAX_PER_THREAD; ++i) {
-    int c = threadIdx.x + i * FSTU_NORM_THREADS;
-    if (c < d) DT<T>::st(yr + c, (v[i] * rstd) * DT<T>::ld(w + c));
+  for (int i = 0; i < NG; ++i) {
+    const int c = (threadIdx.x + i * FSTU_NORM_THREADS) * GW;
+    if (c < d) {
+      float wv[GW], o[GW];
+      if (VEC) Vec4<T>::ld(w + c, wv); else wv[0] = DT<T>::ld(w + c);
+#pragma unroll
+      for (int k = 0; k < GW; ++k) o[k] = (v[i][k] * rstd) * wv[k];
+      if (VEC) Vec4<T>::st(yr + c, o); else DT<T>::st(yr + c, o[0]);
+    }
   }
+}
+
+template <typename T>
+static int launch_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch, const void* w,
+                              void* y, int rows, int d, float eps, hipStream_t s) {
+  const bool vec = (d % 4 == 0) && fstu_aligned(x, 16) && fstu_aligned(delta, 16) && fstu_aligned(w, 16) && fstu_aligned(y, 16);
+  const int groups = vec ? d / 4 : d;
+  const int ng = (groups + FSTU_NORM_THREADS - 1) / FSTU_NORM_THREADS;
+#define LAUNCH_NORM(NG, VEC)                                                                                          \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<T, NG, VEC>), dim3(rows), dim3(FSTU_NORM_THREADS), 0, s, (T*)x, delta,      \
+                     delta_mode, nslices, single_branch, (const T*)w, (T*)y, rows, d, eps)
+  if (vec) {
+    if (ng <= 1) LAUNCH_NORM(1, true); else if (ng <= 2) LAUNCH_NORM(2, true); else if (ng <= 4) LAUNCH_NORM(4, true);
+    else if (ng <= 8) LAUNCH_NORM(8, true); else return -1;
+  } else {
+    if (ng <= 4) LAUNCH_NORM(4, false); else if (ng <= 8) LAUNCH_NORM(8, false); else if (ng <= 32) LAUNCH_NORM(32, false);
+    else return -1;
+  }
+#undef LAUNCH_NORM
+  return 0;
 }
 
 extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch,
@@ -123,15 +204,15 @@ extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int 
   FSTU_REQUIRE(x, FSTU_ENULL, "fstu_add_rmsnorm: x is null");
   FSTU_REQUIRE((y == nullptr) || (w != nullptr), FSTU_ENULL, "fstu_add_rmsnorm: y given without weight");
   FSTU_REQUIRE(delta || y, FSTU_EARG, "fstu_add_rmsnorm: nothing to do (no delta and no y)");
-  FSTU_REQUIRE(rows >= 0 && d > 0 && d <= FSTU_NORM_THREADS * FSTU_NORM_MAX_PER_THREAD, FSTU_ESHAPE,
-               "fstu_add_rmsnorm: d=%d out of range (1..%d)", d, FSTU_NORM_THREADS * FSTU_NORM_MAX_PER_THREAD);
+  FSTU_REQUIRE(rows >= 0 && d > 0 && d <= 8192, FSTU_ESHAPE, "fstu_add_rmsnorm: d=%d out of range (1..8192)", d);
   FSTU_REQUIRE(delta_mode >= 0 && delta_mode <= 2, FSTU_EARG, "fstu_add_rmsnorm: delta_mode=%d", delta_mode);
   FSTU_REQUIRE(delta == nullptr || delta_mode == 0 || nslices >= 1, FSTU_EARG, "fstu_add_rmsnorm: nslices=%d", nslices);
   if (rows == 0) return FSTU_OK;
+  int rc;
   FSTU_DISPATCH_DTYPE(dtype, "fstu_add_rmsnorm",
-                      hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(rows), dim3(FSTU_NORM_THREADS), 0,
-                                         (hipStream_t)stream, (T*)x, delta, delta_mode, nslices, single_branch,
-                                         (const T*)w, (T*)y, rows, d, eps));
+                      rc = launch_add_rmsnorm<T>(x, delta, delta_mode, nslices, single_branch, w, y, rows, d, eps,
+                                                 (hipStream_t)stream));
+  FSTU_REQUIRE(rc == 0, FSTU_ESHAPE, "fstu_add_rmsnorm: d=%d not supported", d);
   FSTU_CHECK_LAUNCH("fstu_add_rmsnorm");
   return FSTU_OK;
 }
@@ -219,9 +300,10 @@ __device__ __forceinline__ double block_excl_scan_d(double v, double* red, doubl
 template <typename T>
 __global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
 sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
-              int top_k, float top_p, int do_sample, uint64_t seed, int step) {
+              int top_k, float top_p, int do_sample, uint64_t seed, int step, const int* __restrict__ dyn) {
   __shared__ SampleShared sh;
   const int b = blockIdx.x;
+  if (dyn) { out += dyn[0]; step = dyn[1]; }
   const T* row = logits + (size_t)b * V;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const bool t1 = (temperature == 1.0f);
@@ -229,9 +311,21 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   // ---- pass A: maximum (lowest index on ties) over a strided walk
   float best = -INFINITY;
   int besti = 0x7fffffff;
-  for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
-    float l = sample_transform(row, i, t1, temperature);
-    if (besti == 0x7fffffff || l > best) { best = l; besti = i; }
+  {
+    // 8 strided loads in flight per thread; indices grow with k, so '>' keeps the lowest index on ties
+    int i = tid;
+    for (; i + 7 * FSTU_SAMPLE_THREADS < V; i += 8 * FSTU_SAMPLE_THREADS) {
+      float l[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) l[k] = sample_transform(row, i + k * FSTU_SAMPLE_THREADS, t1, temperature);
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (besti == 0x7fffffff || l[k] > best) { best = l[k]; besti = i + k * FSTU_SAMPLE_THREADS; }
+    }
+    for (; i < V; i += FSTU_SAMPLE_THREADS) {
+      float l = sample_transform(row, i, t1, temperature);
+      if (besti == 0x7fffffff || l > best) { best = l; besti = i; }
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -402,9 +496,25 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   }
 }
 
+__global__ void advance_dyn_kernel(int* dyn) {
+  if (threadIdx.x == 0) { dyn[0] += 1; dyn[1] += 1; }
+}
+
+int fstu_advance_dyn(int* dyn, void* stream) {
+  hipLaunchKernelGGL(advance_dyn_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, dyn);
+  FSTU_CHECK_LAUNCH("fstu_advance_dyn");
+  return FSTU_OK;
+}
+
 extern "C" int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature,
                            int top_k, float top_p, int do_sample, uint64_t seed, int step, int dtype,
                            void* stream) {
+  return fstu_sample_dyn(logits, out, out_stride, B, V, temperature, top_k, top_p, do_sample, seed, step, nullptr, dtype,
+                         stream);
+}
+
+int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
+                    float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream) {
   FSTU_REQUIRE(logits && out, FSTU_ENULL, "fstu_sample: null pointer");
   FSTU_REQUIRE(B >= 0 && V > 0, FSTU_ESHAPE, "fstu_sample: bad shape B=%d V=%d", B, V);
   FSTU_REQUIRE(temperature > 0.f, FSTU_EARG, "fstu_sample: temperature must be > 0");
@@ -413,7 +523,7 @@ extern "C" int fstu_sample(const void* logits, int64_t* out, int64_t out_stride,
   FSTU_DISPATCH_DTYPE(dtype, "fstu_sample",
                       hipLaunchKernelGGL(sample_kernel<T>, dim3(B), dim3(FSTU_SAMPLE_THREADS), 0, (hipStream_t)stream,
                                          (const T*)logits, out, out_stride, V, temperature, top_k, top_p, do_sample,
-                                         seed, step));
+                                         seed, step, dyn));
   FSTU_CHECK_LAUNCH("fstu_sample");
   return FSTU_OK;
 }

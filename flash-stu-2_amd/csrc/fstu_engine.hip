@@ -66,10 +66,13 @@ static int hist_nsplit(int nlags, int maxsplit) {
   return n;
 }
 
-extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
-                                int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
-                                int step, void* stream) {
+// dyn == nullptr: pos/step come from the host arguments.  dyn != nullptr (graph capture): every position-dependent
+// kernel reads {pos, step} from that device int[2]; tok_in/tok_out are then the bases of token columns 0 and 1.
+static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
+                            int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                            int step, const int* dyn, void* stream) {
   FSTU_REQUIRE(m && tok_in && tok_out, FSTU_ENULL, "fstu_decode_step: null pointer");
+  FSTU_REQUIRE(dyn == nullptr || m->stu_mode == 1, FSTU_EARG, "fstu_decode_step: graph replay needs the recurrence (lds) STU state");
   FSTU_REQUIRE(m->layers && m->emb && m->final_norm_w && m->x && m->h && m->act && m->partial && m->logits,
                FSTU_ENULL, "fstu_decode_step: incomplete model descriptor");
   FSTU_REQUIRE(m->B >= 1 && m->B <= FSTU_MAX_DECODE_ROWS, FSTU_ESHAPE, "fstu_decode_step: batch %d outside 1..%d", m->B,
@@ -93,7 +96,7 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
                    "fstu_decode_step: layer %d has no attention state", l);
     }
   }
-  TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, m->x, B, d, m->V, dt, stream));
+  TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, m->x, B, d, m->V, dt, stream, dyn));
   // h = norm(x) with the first layer's norm weight
   TIMED(PC_NORM, fstu_add_rmsnorm(m->x, nullptr, 0, 1, 0, m->layers[0].norm1_w, m->h, B, d, m->eps, dt, stream));
   for (int l = 0; l < m->n_layers; ++l) {
@@ -107,14 +110,13 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
         TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
         TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-        TIMED(PC_STU, fstu_stu_step_lds(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dt, stream));
+        TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
         TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       }
     } else {
       TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
-      TIMED(PC_SWA, fstu_kv_append(m->qkv, L.kring, L.vring, B, m->n_heads, m->head_dim, m->kv_cap, pos, dt, stream));
-      TIMED(PC_SWA, fstu_swa_decode(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
-                           m->window, m->softcap, dt, stream));
+      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
+                                         m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
       TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
       TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
     }
@@ -123,7 +125,62 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
     TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
-  TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
-  TIMED(PC_SAMPLE, fstu_sample(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dt, stream));
+  if (!do_sample && m->best) {
+    TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
+                                        tok_stride, dyn, dt, stream));
+  } else {
+    TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dyn, dt, stream));
+  }
+  return FSTU_OK;
+}
+
+extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
+                                int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                                int step, void* stream) {
+  return decode_step_impl(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, nullptr,
+                          stream);
+}
+
+// ---------------------------------------------------------------- one step as a replayable HIP graph
+struct fstu_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+
+extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn,
+                                        float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                                        void* stream, void** graph_out) {
+  FSTU_REQUIRE(m && tokens && dyn && graph_out && stream, FSTU_ENULL, "fstu_decode_graph_create: null pointer (a non-default stream is required)");
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+  if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_create: begin capture: %s", hipGetErrorString(e)); return (int)e; }
+  int rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
+  if (rc == 0) rc = fstu_advance_dyn(dyn, stream);
+  hipGraph_t g = nullptr;
+  e = hipStreamEndCapture(s, &g);
+  if (rc != 0) { if (g) (void)hipGraphDestroy(g); return rc; }
+  if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_create: end capture: %s", hipGetErrorString(e)); return (int)e; }
+  hipGraphExec_t ge = nullptr;
+  e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) { (void)hipGraphDestroy(g); fstu_set_error("fstu_decode_graph_create: instantiate: %s", hipGetErrorString(e)); return (int)e; }
+  fstu_graph* h = new fstu_graph{g, ge};
+  *graph_out = h;
+  return FSTU_OK;
+}
+
+extern "C" int fstu_decode_graph_launch(void* graph, void* stream) {
+  FSTU_REQUIRE(graph, FSTU_ENULL, "fstu_decode_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch(((fstu_graph*)graph)->exec, (hipStream_t)stream);
+  if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_launch: %s", hipGetErrorString(e)); return (int)e; }
+  return FSTU_OK;
+}
+
+extern "C" int fstu_decode_graph_destroy(void* graph) {
+  if (!graph) return FSTU_OK;
+  fstu_graph* h = (fstu_graph*)graph;
+  (void)hipGraphExecDestroy(h->exec);
+  (void)hipGraphDestroy(h->graph);
+  delete h;
   return FSTU_OK;
 }

@@ -18,7 +18,7 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-enum { LIN_PLAIN = 0, LIN_GLU = 1, LIN_PARTIAL = 2 };
+enum { LIN_PLAIN = 0, LIN_GLU = 1, LIN_PARTIAL = 2, LIN_ARGMAX = 3 };
 
 struct LinArgs {
   const void* x;
@@ -29,6 +29,8 @@ struct LinArgs {
   int ldy;
   int rows, N, K;
   int kw;          // k range per wave
+  unsigned long long* best;  // LIN_ARGMAX: per-row packed (value key, ~index) maxima, zero on entry
+  float temperature;         // LIN_ARGMAX: logits are divided by it before comparison
 };
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
@@ -110,6 +112,30 @@ linear_mfma_bf16_kernel(LinArgs a) {
       }
     }
   }
+  if (MODE == LIN_ARGMAX) {
+    // per batch row: best (value, lowest index) over this wave's 16 features, then one 64-bit atomic max
+    unsigned long long key = 0ull;
+    if (tile_ok && r < a.rows) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int f = tile * 16 + g * 4 + i;
+        if (f < a.N) {
+          float l = DT<bf16_t>::rnd(acc[i]);
+          if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
+          l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
+          unsigned u = __float_as_uint(l);
+          u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+          unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
+          key = k > key ? k : key;
+        }
+      }
+    }
+    unsigned long long o = __shfl_xor(key, 16, FSTU_WAVE);
+    key = o > key ? o : key;
+    o = __shfl_xor(key, 32, FSTU_WAVE);
+    key = o > key ? o : key;
+    if (tile_ok && g == 0 && r < a.rows && key != 0ull) atomicMax(a.best + r, key);
+  }
   if (!tile_ok) return;
   // D layout: lane holds features 4*(lane/16)+i, batch row lane%16
   const int b = r;
@@ -118,7 +144,7 @@ linear_mfma_bf16_kernel(LinArgs a) {
   for (int i = 0; i < 4; ++i) {
     int f = tile * 16 + g * 4 + i;
     if (f >= a.N) continue;
-    if (MODE == LIN_PLAIN) {
+    if (MODE == LIN_PLAIN || MODE == LIN_ARGMAX) {
       ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(acc[i]);
     } else if (MODE == LIN_GLU) {
       float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[i])));
@@ -223,7 +249,7 @@ extern "C" int fstu_linear_decode(const void* x, int ldx, const void* W, void* y
   int rc = check_common("fstu_linear_decode", x, W, y, ldx, rows, N, K);
   if (rc) return rc;
   FSTU_REQUIRE(ldy >= N, FSTU_ESHAPE, "fstu_linear_decode: ldy=%d < N=%d", ldy, N);
-  LinArgs a{x, ldx, W, nullptr, y, ldy, rows, N, K, K};
+  LinArgs a{x, ldx, W, nullptr, y, ldy, rows, N, K, K, nullptr, 1.0f};
   if (dtype == FSTU_BF16) {
     if (mfma_ok(x, ldx, W, nullptr, K, 1)) launch_mfma<LIN_PLAIN>(a, 1, (hipStream_t)stream);
     else launch_valu<bf16_t, LIN_PLAIN>(a, 1, (hipStream_t)stream);
@@ -243,7 +269,7 @@ extern "C" int fstu_glu_decode(const void* x, int ldx, const void* Wg, const voi
   if (rc) return rc;
   FSTU_REQUIRE(Wu, FSTU_ENULL, "fstu_glu_decode: Wu is null");
   FSTU_REQUIRE(ldact >= I, FSTU_ESHAPE, "fstu_glu_decode: ldact=%d < I=%d", ldact, I);
-  LinArgs a{x, ldx, Wg, Wu, act, ldact, rows, I, K, K};
+  LinArgs a{x, ldx, Wg, Wu, act, ldact, rows, I, K, K, nullptr, 1.0f};
   if (dtype == FSTU_BF16) {
     if (mfma_ok(x, ldx, Wg, Wu, K, 1)) launch_mfma<LIN_GLU>(a, 1, (hipStream_t)stream);
     else launch_valu<bf16_t, LIN_GLU>(a, 1, (hipStream_t)stream);
@@ -262,7 +288,7 @@ extern "C" int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, 
   int rc = check_common("fstu_linear_decode_splitk", x, W, partial, ldx, rows, N, K);
   if (rc) return rc;
   FSTU_REQUIRE(ksplit >= 1 && ksplit <= 1024 && ksplit <= K, FSTU_EARG, "fstu_linear_decode_splitk: ksplit=%d", ksplit);
-  LinArgs a{x, ldx, W, nullptr, partial, N, rows, N, K, K};
+  LinArgs a{x, ldx, W, nullptr, partial, N, rows, N, K, K, nullptr, 1.0f};
   if (dtype == FSTU_BF16) {
     if (mfma_ok(x, ldx, W, nullptr, K, ksplit)) launch_mfma<LIN_PARTIAL>(a, ksplit, (hipStream_t)stream);
     else launch_valu<bf16_t, LIN_PARTIAL>(a, ksplit, (hipStream_t)stream);
@@ -274,4 +300,44 @@ extern "C" int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, 
   }
   FSTU_CHECK_LAUNCH("fstu_linear_decode_splitk");
   return FSTU_OK;
+}
+
+// ---------------------------------------------------------------- head with fused greedy pick
+__global__ void argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows,
+                                     const int* __restrict__ dyn) {
+  int b = threadIdx.x;
+  if (b < rows) {
+    unsigned long long k = best[b];
+    tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
+    best[b] = 0ull;
+  }
+}
+
+extern "C" int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                                float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
+                                void* stream) {
+  return fstu_head_argmax_dyn(x, ldx, W, logits, ldy, rows, N, K, temperature, best_ws, tok_out, tok_stride, nullptr, dtype,
+                              stream);
+}
+
+int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, const int* dyn,
+                         int dtype, void* stream) {
+  int rc = check_common("fstu_head_argmax", x, W, logits, ldx, rows, N, K);
+  if (rc) return rc;
+  FSTU_REQUIRE(best_ws && tok_out, FSTU_ENULL, "fstu_head_argmax: null workspace or output");
+  FSTU_REQUIRE(ldy >= N && tok_stride >= 1 && temperature > 0.f, FSTU_EARG, "fstu_head_argmax: bad ldy / stride / temperature");
+  FSTU_REQUIRE(fstu_aligned(best_ws, 8), FSTU_EALIGN, "fstu_head_argmax: workspace must be 8-byte aligned");
+  if (dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1)) {
+    LinArgs a{x, ldx, W, nullptr, logits, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
+    launch_mfma<LIN_ARGMAX>(a, 1, (hipStream_t)stream);
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
+                       tok_out, tok_stride, rows, dyn);
+    FSTU_CHECK_LAUNCH("fstu_head_argmax");
+    return FSTU_OK;
+  }
+  rc = fstu_linear_decode(x, ldx, W, logits, ldy, rows, N, K, dtype, stream);
+  if (rc) return rc;
+  FSTU_REQUIRE(ldy == N, FSTU_ESHAPE, "fstu_head_argmax: this dtype/shape needs dense logits (ldy == N)");
+  return fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, dyn, dtype, stream);
 }

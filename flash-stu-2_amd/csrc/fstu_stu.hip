@@ -118,8 +118,10 @@ extern "C" int fstu_stu_step_hist(const void* hist, const void* filt, float* eo,
 template <typename T>
 __global__ void __launch_bounds__(256)
 stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
-                    const float* __restrict__ ce, T* __restrict__ y, int ldy, int S, int d, int parity) {
+                    const float* __restrict__ ce, T* __restrict__ y, int ldy, int S, int d, int parity,
+                    const int* __restrict__ dyn) {
   __shared__ float sh[LDS_JG][32][4];
+  if (dyn) parity = dyn[0] & 1;
   const int b = blockIdx.y;
   const int q = threadIdx.x & 31, jg = threadIdx.x >> 5;
   const int c = (blockIdx.x * 32 + q) * 4;
@@ -162,6 +164,11 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
 
 extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y,
                                  int ldy, int B, int S, int d, int t, int dtype, void* stream) {
+  return fstu_stu_step_lds_dyn(state, xp, ldxp, a, ce, y, ldy, B, S, d, t, nullptr, dtype, stream);
+}
+
+int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
+                          int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
   FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
@@ -170,7 +177,7 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
   dim3 grid((d / 4 + 31) / 32, B);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
                       hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
-                                         (const T*)xp, ldxp, a, ce, (T*)y, ldy, S, d, t & 1));
+                                         (const T*)xp, ldxp, a, ce, (T*)y, ldy, S, d, t & 1, dyn));
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }

@@ -39,8 +39,10 @@ SIGNATURES = {
     "fstu_kv_append": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "fstu_swa_append_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
+    "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -285,7 +287,8 @@ def kv_append(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, pos: 
 
 
 def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slopes: torch.Tensor, pos: int,
-               window: int, softcap: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               window: int, softcap: float, out: Optional[torch.Tensor] = None, append: bool = False) -> torch.Tensor:
+    """One query per (batch, head) at position pos; with append the new k,v are written to the ring first."""
     _dev(qkv, kring, vring, slopes, out)
     B, d3 = qkv.shape
     Bk, H, cap, hd = kring.shape
@@ -293,8 +296,9 @@ def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slop
     assert qkv.dtype == kring.dtype == vring.dtype
     if out is None:
         out = torch.empty(B, H * hd, dtype=qkv.dtype, device=qkv.device)
-    _check(load().fstu_swa_decode(_p(qkv), _p(kring), _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window,
-                                  float(softcap or 0.0), _dt(qkv), _stream()), "fstu_swa_decode")
+    fn = load().fstu_swa_append_decode if append else load().fstu_swa_decode
+    _check(fn(_p(qkv), _p(kring), _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window,
+              float(softcap or 0.0), _dt(qkv), _stream()), "fstu_swa_decode")
     return out
 
 
@@ -322,6 +326,24 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float = 1.0, to
                               int(top_k) if top_k else 0, float(top_p) if top_p else 0.0, int(bool(do_sample)),
                               int(seed) & ((1 << 64) - 1), int(step), _dt(logits), _stream()), "fstu_sample")
     return out
+
+
+def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best_ws: torch.Tensor,
+                temperature: float = 1.0, logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """logits = x @ W^T (rows<=16) and the greedy pick per row written to out_tokens (a strided (rows,) int64 view).
+    best_ws: int64 zeros of at least `rows` elements; it is zero again when the call completes."""
+    rows, ldx = _rows_view(x)
+    _dev(W, best_ws)
+    N, K = W.shape
+    assert x.shape[1] == K and x.dtype == W.dtype
+    if logits is None:
+        logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    assert out_tokens.dtype == torch.int64 and out_tokens.dim() == 1 and out_tokens.shape[0] == rows
+    assert best_ws.dtype == torch.int64 and best_ws.numel() >= rows
+    _check(load().fstu_head_argmax(_p(x), ldx, _p(W), _p(logits), logits.stride(0), rows, N, K, float(temperature),
+                                   _p(best_ws), out_tokens.data_ptr(), out_tokens.stride(0), _dt(x), _stream()),
+           "fstu_head_argmax")
+    return logits
 
 
 def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,

@@ -33,7 +33,7 @@ class ModelDesc(ctypes.Structure):
                 ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i),
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
-                ("partial", _vp), ("eo", _vp), ("logits", _vp)]
+                ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -61,7 +61,15 @@ class DecodeEngine:
         self.lib.fstu_decode_step.argtypes = [ctypes.POINTER(ModelDesc), _vp, _vp, ctypes.c_int64, _i, _f, _i, _f, _i,
                                               ctypes.c_uint64, _i, _vp]
         self.lib.fstu_decode_step.restype = _i
+        self.lib.fstu_decode_graph_create.argtypes = [ctypes.POINTER(ModelDesc), _vp, ctypes.c_int64, _vp, _f, _i, _f, _i,
+                                                      ctypes.c_uint64, _vp, ctypes.POINTER(_vp)]
+        self.lib.fstu_decode_graph_create.restype = _i
+        self.lib.fstu_decode_graph_launch.argtypes = [_vp, _vp]
+        self.lib.fstu_decode_graph_launch.restype = _i
+        self.lib.fstu_decode_graph_destroy.argtypes = [_vp]
+        self.lib.fstu_decode_graph_destroy.restype = _i
         self._keep: List[torch.Tensor] = []
+        self._graph = None
 
     # ------------------------------------------------------------------
     def _build(self, caches, B: int, total_len: int):
@@ -146,6 +154,7 @@ class DecodeEngine:
         m.partial = buf(m.ksplit_down, B, d, dtype=torch.float32).data_ptr()
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = self.logits.data_ptr()
+        m.best = buf(max(B, 16), dtype=torch.int64).data_ptr()
         self._arr, self.desc = arr, m
         return tuple(new_caches)
 
@@ -157,6 +166,37 @@ class DecodeEngine:
                                        int(seed) & ((1 << 64) - 1), int(step_idx),
                                        torch.cuda.current_stream().cuda_stream)
         _hip._check(rc, "fstu_decode_step")
+
+    # ------------------------------------------------------------------ graph replay
+    def graph_supported(self) -> bool:
+        return self.cfg.resolved_stu_decode_mode() == "lds"
+
+    def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed):
+        """Captures one decode step as a HIP graph on a side stream.  Each graph_step() then feeds
+        tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
+        self.graph_end()
+        self._dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
+        self._gstream = torch.cuda.Stream(device=tokens.device)
+        self._gstream.wait_stream(torch.cuda.current_stream())
+        handle = _vp()
+        rc = self.lib.fstu_decode_graph_create(ctypes.byref(self.desc), tokens.data_ptr(), tokens.stride(0),
+                                               self._dyn.data_ptr(), float(temperature), int(top_k) if top_k else 0,
+                                               float(top_p) if top_p else 0.0, int(bool(do_sample)),
+                                               int(seed) & ((1 << 64) - 1), self._gstream.cuda_stream,
+                                               ctypes.byref(handle))
+        _hip._check(rc, "fstu_decode_graph_create")
+        self._graph = handle
+        self._graph_tokens = tokens
+
+    def graph_step(self):
+        _hip._check(self.lib.fstu_decode_graph_launch(self._graph, self._gstream.cuda_stream), "fstu_decode_graph_launch")
+
+    def graph_end(self):
+        if self._graph is not None:
+            torch.cuda.current_stream().wait_stream(self._gstream)
+            self._gstream.synchronize()
+            self.lib.fstu_decode_graph_destroy(self._graph)
+            self._graph = None
 
     # ------------------------------------------------------------------
     @torch.no_grad()
@@ -174,7 +214,7 @@ class DecodeEngine:
 
     @torch.no_grad()
     def generate(self, input_ids: torch.Tensor, n_new: int, temperature=1.0, top_k=None, top_p=None, do_sample=True,
-                 seed: int = 0, return_logits: bool = False):
+                 seed: int = 0, return_logits: bool = False, use_graph: bool = True):
         if not input_ids.is_cuda:
             raise _hip.FlashSTUHipError("input_ids must be on the GPU: this model has no CPU path")
         B, P = input_ids.shape
@@ -188,6 +228,14 @@ class DecodeEngine:
         logits = self.prefill(input_ids, total)
         _hip.sample(logits, tokens[:, P], temperature, top_k, top_p, do_sample, seed, 0)
         all_logits = [logits.clone()] if return_logits else None
+        if use_graph and not return_logits and self.graph_supported() and n_new > 2:
+            self.graph_begin(tokens, P, 1, temperature, top_k, top_p, do_sample, seed)
+            try:
+                for s in range(1, n_new):
+                    self.graph_step()
+            finally:
+                self.graph_end()
+            return tokens
         for s in range(1, n_new):
             self.step(tokens, P + s - 1, temperature, top_k, top_p, do_sample, seed, s)
             if return_logits:

@@ -206,7 +206,7 @@ class FlashSTU(nn.Module):
             return input_ids
         if use_cache and P <= self.config.seq_len:
             return self.decode_engine().generate(input_ids, n_new, temperature, top_k, top_p, do_sample, seed,
-                                                 return_logits=return_logits)
+                                                 return_logits=return_logits, use_graph=kwargs.get("use_graph", True))
         tokens = torch.empty(B, max_length, dtype=torch.int64, device=input_ids.device)
         tokens[:, :P] = input_ids
         all_logits = []

@@ -88,7 +88,6 @@ class Attention(nn.Module):
         kr, vr, pos_t = past_key_value
         pos = int(pos_t[0])
         qkv = _hip.linear_decode(x.reshape(B, d), self.c_attn.weight)
-        _hip.kv_append(qkv, kr, vr, pos)
-        o = _hip.swa_decode(qkv, kr, vr, slopes, pos, W, self.softcap)
+        o = _hip.swa_decode(qkv, kr, vr, slopes, pos, W, self.softcap, append=True)
         y = _hip.linear_decode(o, self.c_proj.weight).reshape(B, 1, d)
         return (y, (kr, vr, pos_t + 1)) if use_cache else y

@@ -166,6 +166,12 @@ int fstu_swa_decode(const void* qkv, const void* kring, const void* vring, void*
                     int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
                     void* stream);
 
+/* Same, but first stores the new token's k,v (columns [H*hd,3*H*hd) of the qkv
+ * row) into ring slot pos % cap: fstu_kv_append + fstu_swa_decode in one launch. */
+int fstu_swa_append_decode(const void* qkv, void* kring, void* vring, void* out, const float* slopes,
+                           int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
+                           void* stream);
+
 /* Prefill form: qkv (B,T,3*H*hd), positions 0..T-1, out (B,T,H*hd). */
 int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T, int H, int hd,
                      int window, float softcap, int dtype, void* stream);
@@ -184,6 +190,15 @@ int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int
  * Replaces flash_stu/model.py:267-299. */
 int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature,
                 int top_k, float top_p, int do_sample, uint64_t seed, int step, int dtype, void* stream);
+
+/* Tied head + greedy pick in one pass: logits[m,:] = T(x[m,:] . W^T) as
+ * fstu_linear_decode, and tok_out[m*tok_stride] = argmax_n clamp(T(logit/temperature))
+ * with the lowest index on ties (same rule as fstu_sample with do_sample=0).
+ * best_ws: `rows` 64-bit words, zero on entry and zero again on return.
+ * Replaces lm_head + argmax at flash_stu/model.py:176,268-269,299. */
+int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                     float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
+                     void* stream);
 
 /* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
  * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:
@@ -247,6 +262,7 @@ typedef struct {
   float* partial;           /* fp32 */
   float* eo;                /* fp32 */
   void* logits;             /* (B,V) */
+  void* best;               /* B 64-bit words, zero-initialised once by the caller */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next
@@ -255,6 +271,19 @@ typedef struct {
 int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
                      int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                      int step, void* stream);
+
+/* One decode step captured as a HIP graph that can be replayed for every position:
+ * the position-dependent kernels read {position, sampling step} from `dyn`, a
+ * device int[2] the caller sets before the first launch; every launch feeds
+ * tokens[:, dyn[0]], writes tokens[:, dyn[0]+1] and then advances both counters.
+ * Requires the recurrence (lds) STU state.  `stream` must be a non-default stream;
+ * capture happens on it inside fstu_decode_graph_create (no memset nodes are
+ * recorded).  No counterpart in the reference. */
+int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn,
+                             float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                             void* stream, void** graph_out);
+int fstu_decode_graph_launch(void* graph, void* stream);
+int fstu_decode_graph_destroy(void* graph);
 
 /* ---- live kernel timing (measurement aid; no counterpart in the reference) ----
  * Between fstu_prof_begin and fstu_prof_end every launch of one kernel class

@@ -1,0 +1,150 @@
+"""BASELINE configs 3, 4 and 5 on the GPU: parity against the CPU oracle at sizes
+the oracle finishes in seconds, plus size-independent properties at the full
+BASELINE sizes (linearity, causality, delta response, state carry)."""
+import math
+
+import pytest
+import torch
+
+from oracle import flashstu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from flash_stu import _hip
+    _hip.load()
+    return _hip
+
+
+# ----------------------------------------------------------------- config 3
+def _exact_stu(dtype, d, L, K, seed):
+    from flash_stu import STU, FlashSTUConfig
+    cfg = FlashSTUConfig(n_embd=d, n_heads=1, n_layers=1, seq_len=L, num_eigh=K, use_approx=False, torch_dtype=dtype,
+                         vocab_size=3)
+    phi = O.get_spectral_filters(L, K, dtype=dtype)
+    g = torch.Generator().manual_seed(seed)
+    stu = STU(cfg, phi, O.nearest_power_of_two(2 * L - 1, True))
+    with torch.no_grad():
+        stu.M_phi_plus.copy_((torch.randn(K, d, d, generator=g) / math.sqrt(d)).to(dtype))
+        stu.M_phi_minus.copy_((torch.randn(K, d, d, generator=g) / math.sqrt(d)).to(dtype))
+    p = {"M_phi_plus": stu.M_phi_plus.detach().clone(), "M_phi_minus": stu.M_phi_minus.detach().clone()}
+    return stu.cuda(), phi, p
+
+
+def test_c3_exact_mode_prefill_parity_reduced():
+    """Config 3's operator (use_approx=False, K=24, M_phi ~ N(0,1/sqrt(d))) at B=2, L=1024, d=128, bf16."""
+    dtype = torch.bfloat16
+    stu, phi, p = _exact_stu(dtype, 128, 1024, 24, 0)
+    x = torch.randn(2, 1024, 128, generator=torch.Generator().manual_seed(1)).to(dtype)
+    ref = O.stu_forward(x, phi, p, 2048, use_approx=False).float()
+    y = stu(x.cuda()).float().cpu()
+    scale = float(ref.abs().max())
+    assert float((y - ref).abs().max()) <= 3e-2 * scale
+    assert float((y - ref).abs().mean()) <= 3e-3 * scale
+
+
+def test_c3_full_size_properties(hip):
+    """B=4, L=8192, d=1024, K=24, bf16: the filter-bank kernel at the BASELINE shape.
+    delta input returns the filters; the response is causal and shift-invariant; fp32 results
+    are linear in the input."""
+    B, L, d, K = 4, 8192, 1024, 24
+    dtype = torch.bfloat16
+    phi = O.get_spectral_filters(L, K, dtype=dtype).cuda()
+    x = torch.zeros(B, L, d, dtype=dtype, device="cuda")
+    x[0, 0, :] = 1.0                      # delta at t=0
+    x[1, 100, 5] = 2.0                    # delayed, scaled delta in one channel
+    x[2] = torch.randn(L, d, generator=torch.Generator().manual_seed(2)).to(dtype).cuda()
+    x[3, 4000:] = x[2, : L - 4000]        # batch 3 = batch 2 shifted by 4000
+    Up = torch.empty(B, L, K, d, dtype=dtype, device="cuda")
+    Um = torch.empty_like(Up)
+    hip.stu_conv_bank(x, phi, Up, Um)
+    torch.cuda.synchronize()
+    sg = torch.ones(L, 1, device="cuda")
+    sg[1::2] = -1
+    assert torch.equal(Up[0, :, :, 7], phi)                                   # delta -> filter (exact in bf16)
+    assert torch.equal(Um[0, :, :, 3].float(), (phi.float() * sg))
+    assert float(Up[1, :100].abs().max()) == 0.0                               # causal
+    assert torch.equal(Up[1, 100:, :, 5].float(), (2 * phi[: L - 100].float()).to(dtype).float())
+    assert float(Up[1, :, :, 6].abs().max()) == 0.0                            # channels do not mix
+    assert torch.equal(Up[3, 4000:], Up[2, : L - 4000])                        # shift invariance (same rounding)
+    assert float(Up[3, :4000].abs().max()) == 0.0
+    # spot-check one (b, t, k, channel) column against a float64 dot product
+    t, k, c = 6000, 11, 321
+    ref = (phi[: t + 1, k].double().flip(0) * x[2, : t + 1, c].double()).sum()
+    assert abs(float(Up[2, t, k, c]) - float(ref)) <= 2.0 ** -7 * abs(float(ref)) + 1e-6
+
+
+# ----------------------------------------------------------------- config 4
+def _c4_tensors(T, Bt=64, d=1024, S=160, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    A = (0.9 + 0.099 * torch.rand(S, generator=g)).float()
+    Bm = (torch.randn(d, S, generator=g) / d).bfloat16()
+    Cm = (torch.randn(S, d, generator=g) / S).bfloat16()
+    x = torch.randn(T, Bt, d, generator=g).bfloat16()
+    return A, Bm, Cm, x
+
+
+def test_c4_lds_step_parity_at_full_width(hip):
+    """Batch 64, d=1024, state 160, A~U(0.9,0.999) fp32, B~N(0,1/d), C~N(0,1/160) bf16, x~N(0,1):
+    256 consecutive steps against the oracle's literal loop, state carried across two launches."""
+    T = 256
+    A, Bm, Cm, x = _c4_tensors(T)
+    yref, href = O.lds_sequence(x, A, Bm, Cm)
+    h = torch.zeros(64, 160, device="cuda")
+    y1 = hip.lds_steps(h, x[:100].cuda(), A.cuda(), Bm.cuda(), Cm.cuda())
+    y2 = hip.lds_steps(h, x[100:].cuda(), A.cuda(), Bm.cuda(), Cm.cuda())
+    y = torch.cat([y1, y2]).float().cpu()
+    diff = (y - yref.float()).abs()
+    assert float(diff.max()) <= 2.0 ** -7 * float(yref.float().abs().max())
+    assert float((diff > 0).float().mean()) < 0.05
+    assert float((h.cpu() - href).abs().max()) <= 1e-4 * float(href.abs().max())
+
+
+def test_c4_4096_steps_state_is_the_closed_form(hip):
+    """The full 4096-step run: with a constant input the carried state converges to u/(1-A)
+    and two launches of 2048 steps equal one launch of 4096."""
+    T = 4096
+    A, Bm, Cm, x = _c4_tensors(1)
+    xs = x.expand(T, 64, 1024).contiguous().cuda()
+    Ad, Bd, Cd = A.cuda(), Bm.cuda(), Cm.cuda()
+    h1 = torch.zeros(64, 160, device="cuda")
+    y_full = hip.lds_steps(h1, xs, Ad, Bd, Cd)
+    h2 = torch.zeros(64, 160, device="cuda")
+    ya = hip.lds_steps(h2, xs[:2048], Ad, Bd, Cd)
+    yb = hip.lds_steps(h2, xs[2048:], Ad, Bd, Cd)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([ya, yb]), y_full) and torch.equal(h1, h2)
+    u = x[0].float() @ Bm.float()                                   # (64,160)
+    closed = u * (1 - A ** T) / (1 - A)
+    assert float((h1.cpu() - closed).abs().max()) <= 2e-4 * float(closed.abs().max())
+    ylast = (closed @ Cm.float())
+    assert float((y_full[-1].float().cpu() - ylast).abs().max()) <= 2.0 ** -6 * float(ylast.abs().max())
+
+
+# ----------------------------------------------------------------- config 5
+def test_c5_shape_sampling_parity_reduced():
+    """Config 5's structure (head dim 128, 24 filters, top-k 40 / temperature 0.8, seeded counter stream)
+    on a model small enough for the CPU oracle; fp32 so that ids must be identical."""
+    from test_gpu_model import make_pair, prompt
+    ocfg, w, model = make_pair(seed=2, init="healthy", mlp_scale=2, n_embd=256, n_layers=4, n_heads=2, window_size=24,
+                               num_eigh=24, seq_len=256, vocab_size=2003)
+    ids = prompt(16, 20, ocfg.vocab_size, 4)
+    ref = O.generate(w, ocfg, ids, max_length=52, temperature=0.8, top_k=40, do_sample=True, mode="stateful", seed=2)
+    got = model.generate(ids.cuda(), max_length=52, temperature=0.8, top_k=40, do_sample=True, seed=2)
+    assert torch.equal(got.cpu(), ref)
+
+
+def test_c5_shape_bf16_lds_teacher_forced():
+    """Same structure in bf16 with the recurrence state, logits within the bf16 tolerance."""
+    from test_gpu_model import make_pair, prompt, _teacher_forced
+    ocfg, w, model = make_pair(seed=2, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=256, n_layers=4,
+                               n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
+                               stu_decode_mode="lds")
+    P, N = 20, 60
+    ids = prompt(16, P, ocfg.vocab_size, 4)
+    got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
+    ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
+    err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
+    assert float(err.max()) <= 2e-2

@@ -75,6 +75,23 @@ def test_generate_without_cache_equals_with_cache():
     assert model.generate(ids, max_length=7).shape == (2, 7)
 
 
+@pytest.mark.parametrize("do_sample", [False, True])
+def test_graph_replay_equals_eager_steps(do_sample):
+    """The captured-step graph is replayed for many positions, with eager work and synchronisation in between,
+    and must reproduce the eager token sequence exactly (same kernels, position read from device memory)."""
+    ocfg, w, model = make_pair(seed=7, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=128, n_layers=4,
+                               n_heads=2, window_size=8, num_eigh=8, seq_len=128, vocab_size=1001, stu_decode_mode="lds")
+    ids = prompt(3, 6, ocfg.vocab_size, 9).cuda()
+    kw = dict(max_length=70, do_sample=do_sample, temperature=0.9, top_k=20, seed=5)
+    eager = model.generate(ids, use_graph=False, **kw)
+    for _ in range(3):
+        junk = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")   # unrelated eager work
+        torch.cuda.synchronize()
+        got = model.generate(ids, use_graph=True, **kw)
+        assert torch.equal(got, eager)
+    del junk
+
+
 def _teacher_forced(w, ocfg, tokens, P):
     logits, _ = O.model_forward(w, ocfg, tokens[:, :-1])
     return logits[:, P - 1:, :]          # predictions for positions P..end

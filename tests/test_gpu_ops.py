@@ -241,6 +241,11 @@ def test_swa_ring_decode_and_prefill(hip, dtype, B, H, hd, W, T):
         hip.kv_append(row, kr, vr, pos)
         o = hip.swa_decode(row, kr, vr, sd, pos, W, 50.0)
         check(o, full[:, pos], dtype, frac=0.05, scale=float(full.abs().max()))
+    # fused append + decode gives the same result as the two separate calls
+    kr2, vr2 = torch.zeros_like(kr), torch.zeros_like(vr)
+    hip.kv_fill(qd[:, :T - 1].contiguous(), kr2, vr2, 0)
+    o3 = hip.swa_decode(qd[:, T - 1].contiguous(), kr2, vr2, sd, T - 1, W, 50.0, append=True)
+    assert torch.equal(o3, o) and torch.equal(kr2, kr) and torch.equal(vr2, vr)
     # softcap disabled
     o2 = hip.swa_decode(qd[:, T - 1].contiguous(), kr, vr, sd, T - 1, W, 0.0)
     ref2 = O.attention_core(q[:, -1:], k, v, W, slopes, 0.0).reshape(B, d)
@@ -260,6 +265,27 @@ def test_sample_greedy_matches_oracle_ties_included(hip, dtype):
     assert torch.equal(out[:, 2].cpu(), ref[:, 0])
     assert int(out[0, 2]) == 100 and int(out[1, 2]) == 0
     assert bool((out[:, [0, 1, 3]] == -1).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_head_with_fused_greedy_pick(hip, dtype, temperature):
+    """logits as linear_decode; the pick equals the oracle's argmax of the filtered logits, ties to the lowest id."""
+    g = gen(14)
+    B, V, K = 8, 50257, 256
+    x = torch.randn(B, K, generator=g).to(dtype)
+    W = (torch.randn(V, K, generator=g) / 16).to(dtype)
+    W[40000] = W[123]                      # exact tie between ids 123 and 40000 in every row
+    x[0] = W[123].float().sign().to(dtype) * 3    # make that tied pair the maximum of row 0
+    ws = torch.zeros(16, dtype=torch.int64, device="cuda")
+    toks = torch.full((B, 3), -7, dtype=torch.int64, device="cuda")
+    logits = hip.head_argmax(dev(x), dev(W), toks[:, 1], ws, temperature)
+    ref_logits = F.linear(x.float(), W.float()).to(dtype)
+    check(logits, ref_logits, dtype)
+    ref = O.next_token(logits.cpu(), temperature=temperature, do_sample=False)[:, 0]
+    assert torch.equal(toks[:, 1].cpu(), ref)
+    assert int(toks[0, 1]) == 123
+    assert bool((ws == 0).all()) and bool((toks[:, [0, 2]] == -7).all())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
