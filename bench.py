@@ -160,8 +160,6 @@ def main():
     step_bytes = decode_step_bytes(cfg, B, t_mid, args.stu_mode, S)
     # ---- second pass over K steps with events around the dominant kernel
     lib = _hip.load()
-    lib.fstu_prof_begin.argtypes = [ctypes.c_int, ctypes.c_int]
-    lib.fstu_prof_end.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]
 
     def timed_class(cls, n):
         nonlocal pos

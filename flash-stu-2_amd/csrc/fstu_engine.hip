@@ -66,6 +66,84 @@ static int hist_nsplit(int nlags, int maxsplit) {
   return n;
 }
 
+// ---------------------------------------------------------------- fused bf16 step over packed weights
+// 58 launches: every residual add + RMSNorm runs as the prologue of the GEMV that consumes it, the down
+// projection reduces its K split in-kernel, the head picks the greedy token itself.
+static bool fused_available(const fstu_model_desc* m) {
+  if (m->dtype != FSTU_BF16 || m->stu_mode != 1 || !m->wp_emb || !m->x2 || !m->yd || !m->partial_fix || !m->counters || !m->best)
+    return false;
+  if (m->d % 128 != 0 || m->I % (128 * m->ksplit_down) != 0) return false;
+  if ((size_t)m->B * (m->d + 8) * 2 + 8192 > 64 * 1024) return false;
+  for (int l = 0; l < m->n_layers; ++l) {
+    const fstu_layer_desc& L = m->layers[l];
+    if (!L.wp_gate || !L.wp_up || !L.wp_down) return false;
+    if (L.kind == 0 ? !L.wp_m_inputs : (!L.wp_qkv || !L.wp_proj)) return false;
+  }
+  return true;
+}
+
+static int decode_step_fused(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
+                             int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                             int step, const int* dyn, void* stream) {
+  const int B = m->B, d = m->d, I = m->I, dt = m->dtype;
+  void* xb[2] = {m->x, m->x2};
+  int cur = 0;
+  TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, xb[0], B, d, m->V, dt, stream, dyn));
+  const void* pending = nullptr;   // output of the previous sub-layer, not yet added to the residual stream
+  auto pro = [&](fstu_gemv_args& g, const void* norm_w) {
+    g.res_in = xb[cur];
+    g.delta = pending;
+    g.res_out = pending ? xb[cur ^ 1] : nullptr;
+    g.norm_w = norm_w;
+    g.eps = m->eps;
+    if (pending) cur ^= 1;
+    pending = nullptr;
+  };
+  for (int l = 0; l < m->n_layers; ++l) {
+    const fstu_layer_desc& L = m->layers[l];
+    if (L.kind == 0) {
+      fstu_gemv_args g = {};
+      g.mode = 0; g.rows = B; g.N = d; g.K = d; g.Wp = L.wp_m_inputs; g.y = m->xp; g.ldy = d;
+      pro(g, L.norm1_w);
+      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&g, dyn, stream));
+      TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
+    } else {
+      fstu_gemv_args g = {};
+      g.mode = 0; g.rows = B; g.N = 3 * d; g.K = d; g.Wp = L.wp_qkv; g.y = m->qkv; g.ldy = 3 * d;
+      pro(g, L.norm1_w);
+      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&g, dyn, stream));
+      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
+                                         m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
+      fstu_gemv_args p = {};
+      p.mode = 0; p.rows = B; p.N = d; p.K = d; p.Wp = L.wp_proj; p.x = m->attn; p.ldx = d; p.y = m->y; p.ldy = d;
+      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&p, dyn, stream));
+    }
+    pending = m->y;
+    fstu_gemv_args u = {};
+    u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
+    pro(u, L.mlp_norm_w);
+    TIMED(PC_GLU, fstu_gemv_packed_dyn(&u, dyn, stream));
+    fstu_gemv_args dn = {};
+    dn.mode = 2; dn.rows = B; dn.N = d; dn.K = I; dn.Wp = L.wp_down; dn.x = m->act; dn.ldx = I; dn.y = m->yd; dn.ldy = d;
+    dn.ksplit = m->ksplit_down; dn.partial_ws = m->partial_fix; dn.counters = m->counters;
+    TIMED(PC_DOWN, fstu_gemv_packed_dyn(&dn, dyn, stream));
+    pending = m->yd;
+  }
+  fstu_gemv_args hd = {};
+  hd.rows = B; hd.N = m->V; hd.K = d; hd.Wp = m->wp_emb; hd.y = m->logits; hd.ldy = m->V;
+  if (!do_sample) {
+    hd.mode = 3; hd.temperature = temperature; hd.best_ws = m->best; hd.tok_out = tok_out; hd.tok_stride = tok_stride;
+    pro(hd, m->final_norm_w);
+    TIMED(PC_HEAD, fstu_gemv_packed_dyn(&hd, dyn, stream));
+  } else {
+    hd.mode = 0;
+    pro(hd, m->final_norm_w);
+    TIMED(PC_HEAD, fstu_gemv_packed_dyn(&hd, dyn, stream));
+    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dyn, dt, stream));
+  }
+  return FSTU_OK;
+}
+
 // dyn == nullptr: pos/step come from the host arguments.  dyn != nullptr (graph capture): every position-dependent
 // kernel reads {pos, step} from that device int[2]; tok_in/tok_out are then the bases of token columns 0 and 1.
 static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
@@ -96,6 +174,8 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                    "fstu_decode_step: layer %d has no attention state", l);
     }
   }
+  if (fused_available(m))
+    return decode_step_fused(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
   TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, m->x, B, d, m->V, dt, stream, dyn));
   // h = norm(x) with the first layer's norm weight
   TIMED(PC_NORM, fstu_add_rmsnorm(m->x, nullptr, 0, 1, 0, m->layers[0].norm1_w, m->h, B, d, m->eps, dt, stream));

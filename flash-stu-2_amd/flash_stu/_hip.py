@@ -43,6 +43,15 @@ SIGNATURES = {
     "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
+    "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
+    "fstu_packed_elems": [_i, _i],
+    "fstu_gemv_packed": [_vp, _vp],
+    "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
+    "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _f, _i, _f, _i, _u64, _vp, _vp],
+    "fstu_decode_graph_launch": [_vp, _vp],
+    "fstu_decode_graph_destroy": [_vp],
+    "fstu_prof_begin": [_i, _i],
+    "fstu_prof_end": [_vp, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -68,6 +77,7 @@ def load(path: Optional[str] = None):
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = ctypes.c_int
+    lib.fstu_packed_elems.restype = ctypes.c_int64
     if path is None:
         _lib = lib
     return lib
@@ -344,6 +354,54 @@ def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best
                                    _p(best_ws), out_tokens.data_ptr(), out_tokens.stride(0), _dt(x), _stream()),
            "fstu_head_argmax")
     return logits
+
+
+class GemvArgs(ctypes.Structure):
+    _fields_ = [("mode", _i), ("rows", _i), ("N", _i), ("K", _i), ("Wp", _vp), ("Wp2", _vp), ("x", _vp), ("ldx", _i),
+                ("res_in", _vp), ("delta", _vp), ("res_out", _vp), ("norm_w", _vp), ("eps", _f), ("y", _vp), ("ldy", _i),
+                ("ksplit", _i), ("partial_ws", _vp), ("counters", _vp), ("temperature", _f), ("best_ws", _vp),
+                ("tok_out", _vp), ("tok_stride", _i64)]
+
+
+def pack_rows(W: torch.Tensor) -> torch.Tensor:
+    """(N,K) bf16 row-major -> packed MFMA-fragment order (ceil(N/16)*16*K elements); K % 32 == 0."""
+    _dev(W)
+    if W.dtype != torch.bfloat16:
+        raise FlashSTUHipError("packed weights are bf16 only")
+    N, K = W.shape
+    lib = load()
+    out = torch.empty(lib.fstu_packed_elems(N, K), dtype=W.dtype, device=W.device)
+    _check(lib.fstu_pack_rows(_p(W), _p(out), N, K, _stream()), "fstu_pack_rows")
+    return out
+
+
+def gemv_packed(mode: int, Wp: torch.Tensor, N: int, K: int, out: torch.Tensor, x: Optional[torch.Tensor] = None,
+                Wp2: Optional[torch.Tensor] = None, res_in: Optional[torch.Tensor] = None,
+                delta: Optional[torch.Tensor] = None, res_out: Optional[torch.Tensor] = None,
+                norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ksplit: int = 1,
+                partial_ws: Optional[torch.Tensor] = None, counters: Optional[torch.Tensor] = None,
+                temperature: float = 1.0, best_ws: Optional[torch.Tensor] = None,
+                tok_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Thin wrapper over fstu_gemv_packed (see include/flashstu_hip.h for the modes)."""
+    _dev(Wp, Wp2, res_in, delta, res_out, norm_w, partial_ws, counters, best_ws)
+    a = GemvArgs()
+    rows = out.shape[0]
+    a.mode, a.rows, a.N, a.K = mode, rows, N, K
+    a.Wp, a.Wp2 = _p(Wp), _p(Wp2)
+    if x is not None:
+        xr, ldx = _rows_view(x)
+        assert xr == rows and x.shape[1] == K
+        a.x, a.ldx = x.data_ptr(), ldx
+    a.res_in, a.delta, a.res_out, a.norm_w, a.eps = _p(res_in), _p(delta), _p(res_out), _p(norm_w), float(eps)
+    orow, ldy = _rows_view(out)
+    a.y, a.ldy = out.data_ptr(), ldy
+    a.ksplit, a.partial_ws, a.counters = ksplit, _p(partial_ws), _p(counters)
+    a.temperature, a.best_ws = float(temperature), _p(best_ws)
+    if tok_out is not None:
+        assert tok_out.dtype == torch.int64 and tok_out.dim() == 1 and tok_out.shape[0] == rows
+        a.tok_out, a.tok_stride = tok_out.data_ptr(), tok_out.stride(0)
+    _check(load().fstu_gemv_packed(ctypes.byref(a), _stream()), "fstu_gemv_packed")
+    return out
 
 
 def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,

@@ -24,7 +24,9 @@ _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 class LayerDesc(ctypes.Structure):
     _fields_ = [("kind", _i), ("norm1_w", _vp), ("mlp_norm_w", _vp), ("w_gate", _vp), ("w_up", _vp), ("w_down", _vp),
                 ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_state", _vp),
-                ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp)]
+                ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp),
+                ("wp_gate", _vp), ("wp_up", _vp), ("wp_down", _vp), ("wp_m_inputs", _vp), ("wp_qkv", _vp),
+                ("wp_proj", _vp)]
 
 
 class ModelDesc(ctypes.Structure):
@@ -33,7 +35,8 @@ class ModelDesc(ctypes.Structure):
                 ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i),
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
-                ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp)]
+                ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
+                ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -58,20 +61,26 @@ class DecodeEngine:
         self.model = model
         self.cfg = cfg
         self.lib = _hip.load()
-        self.lib.fstu_decode_step.argtypes = [ctypes.POINTER(ModelDesc), _vp, _vp, ctypes.c_int64, _i, _f, _i, _f, _i,
-                                              ctypes.c_uint64, _i, _vp]
-        self.lib.fstu_decode_step.restype = _i
-        self.lib.fstu_decode_graph_create.argtypes = [ctypes.POINTER(ModelDesc), _vp, ctypes.c_int64, _vp, _f, _i, _f, _i,
-                                                      ctypes.c_uint64, _vp, ctypes.POINTER(_vp)]
-        self.lib.fstu_decode_graph_create.restype = _i
-        self.lib.fstu_decode_graph_launch.argtypes = [_vp, _vp]
-        self.lib.fstu_decode_graph_launch.restype = _i
-        self.lib.fstu_decode_graph_destroy.argtypes = [_vp]
-        self.lib.fstu_decode_graph_destroy.restype = _i
         self._keep: List[torch.Tensor] = []
         self._graph = None
+        self._packed = {}
 
     # ------------------------------------------------------------------
+    def _pack(self, w: torch.Tensor) -> torch.Tensor:
+        """MFMA-fragment-ordered copy of an (N,K) bf16 weight, rebuilt only when the weight changes."""
+        key = w.data_ptr()
+        hit = self._packed.get(key)
+        if hit is None or hit[0] != w._version:
+            hit = (w._version, _hip.pack_rows(w))
+            self._packed[key] = hit
+        return hit[1]
+
+    def _use_packed(self, B: int) -> bool:
+        cfg = self.cfg
+        d, I = cfg.n_embd, cfg.n_embd * cfg.mlp_scale
+        return (cfg.torch_dtype == torch.bfloat16 and cfg.resolved_stu_decode_mode() == "lds" and d % 128 == 0
+                and I % (128 * pick_ksplit_down(I)) == 0 and B * (d + 8) * 2 + 8192 <= 64 * 1024)
+
     def _build(self, caches, B: int, total_len: int):
         model, cfg = self.model, self.cfg
         dev = model.lm_head.weight.device
@@ -154,7 +163,22 @@ class DecodeEngine:
         m.partial = buf(m.ksplit_down, B, d, dtype=torch.float32).data_ptr()
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = self.logits.data_ptr()
-        m.best = buf(max(B, 16), dtype=torch.int64).data_ptr()
+        m.best = buf(max(B, 16) * 64, dtype=torch.int64).data_ptr()
+        if self._use_packed(B):
+            for i, layer in enumerate(model.layers):
+                ld = arr[i]
+                ld.wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
+                ld.wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
+                ld.wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
+                if isinstance(layer, STULayer):
+                    ld.wp_m_inputs = self._pack(layer.stu.m_inputs_t()).data_ptr()
+                else:
+                    ld.wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                    ld.wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
+            m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
+            m.x2, m.yd = buf(B, d).data_ptr(), buf(B, d).data_ptr()
+            m.partial_fix = buf(m.ksplit_down * ((d + 15) // 16) * 256, dtype=torch.float32).data_ptr()
+            m.counters = buf((d + 15) // 16, dtype=torch.int32).data_ptr()
         self._arr, self.desc = arr, m
         return tuple(new_caches)
 

@@ -208,6 +208,54 @@ int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ld
 int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, const void* Cm, void* y,
                    int T_steps, int Bt, int d_in, int S, int d_out, int dtype, void* stream);
 
+/* ---- decode GEMVs over packed weights ---------------------------------------
+ * Packed layout of an (N,K) bf16 row-major weight, K % 32 == 0 (fstu_pack_rows):
+ *   Wp[tile][kstep][lane][8],  tile = n/16, kstep = k/32, lane = 16*g + r,
+ *   element e of lane (r,g) = W[16*tile + r][32*kstep + 8*g + e]; rows >= N are zero.
+ * fstu_packed_elems(N,K) is the number of bf16 elements of the packed copy.
+ * fstu_gemv_packed computes, for rows <= 16 activation rows,
+ *   mode 0: y[m,n] = T(h[m,:] . W[n,:])
+ *   mode 1: y[m,i] = T( T(gelu_tanh(T(h.Wg[i]))) * T(h.Wu[i]) )        (Wp = gate, Wp2 = up)
+ *   mode 2: mode 0 with K split over `ksplit` workgroups per feature tile; the last
+ *           workgroup of a tile to finish adds the fp32 partials in slice order
+ *           (deterministic).  partial_ws: ksplit*ceil(N/16)*256 floats; counters:
+ *           ceil(N/16) uint32, zero before the first call (left zero).
+ *   mode 3: mode 0 plus the greedy pick of fstu_head_argmax; best_ws: rows*64 uint64,
+ *           zero before the first call (left zero).
+ * Activations h: if norm_w == NULL, h = x (rows,K) with row stride ldx.  Otherwise the
+ * fused prologue h = RMSNorm(T(res_in + delta)) * norm_w with res_in/delta (rows,K)
+ * dense; delta may be NULL (no add); when delta != NULL and res_out != NULL the
+ * updated residual T(res_in + delta) is written to res_out (must not alias res_in).
+ * bf16 only; K % 128 == 0 (K % (128*ksplit) == 0 in mode 2).
+ * Replaces the same reference call sites as fstu_linear_decode / fstu_glu_decode /
+ * fstu_add_rmsnorm / fstu_head_argmax. */
+typedef struct {
+  int mode;
+  int rows, N, K;
+  const void* Wp;
+  const void* Wp2;
+  const void* x;
+  int ldx;
+  const void* res_in;
+  const void* delta;
+  void* res_out;
+  const void* norm_w;
+  float eps;
+  void* y;
+  int ldy;
+  int ksplit;
+  float* partial_ws;
+  unsigned* counters;
+  float temperature;
+  void* best_ws;
+  int64_t* tok_out;
+  int64_t tok_stride;
+} fstu_gemv_args;
+
+int64_t fstu_packed_elems(int N, int K);
+int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
+int fstu_gemv_packed(const fstu_gemv_args* a, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -235,6 +283,13 @@ typedef struct {
   void* kring;              /* (B,H,kv_cap,hd) */
   void* vring;
   const float* slopes;      /* (H) */
+  /* packed copies (fstu_pack_rows) for the fused bf16 step; all NULL = not available */
+  const void* wp_gate;
+  const void* wp_up;
+  const void* wp_down;
+  const void* wp_m_inputs;  /* packed M_inputs^T */
+  const void* wp_qkv;
+  const void* wp_proj;
 } fstu_layer_desc;
 
 typedef struct {
@@ -262,7 +317,13 @@ typedef struct {
   float* partial;           /* fp32 */
   float* eo;                /* fp32 */
   void* logits;             /* (B,V) */
-  void* best;               /* B 64-bit words, zero-initialised once by the caller */
+  void* best;               /* max(B,16)*64 64-bit words, zero-initialised once by the caller */
+  /* fused bf16 step (used when wp_emb and every layer's packed copies are set) */
+  const void* wp_emb;       /* packed tied head */
+  void* x2;                 /* (B,d) second residual buffer (the stream ping-pongs x <-> x2) */
+  void* yd;                 /* (B,d) down-projection output */
+  float* partial_fix;       /* ksplit_down * ceil(d/16) * 256 floats */
+  unsigned* counters;       /* ceil(d/16) uint32, zero-initialised once */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

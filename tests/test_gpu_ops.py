@@ -119,6 +119,61 @@ def test_mlp_decode_chain(hip, dtype, rows, d, I):
         check(rd, ref, dtype, frac=0.05, atol=(2.0 ** -7 * float(down.float().abs().max())) if dtype == torch.bfloat16 else 0.0)
 
 
+def test_packed_gemv_modes_match_the_unfused_ops(hip):
+    """Packed-weight GEMVs with fused residual+RMSNorm prologue, GLU epilogue, in-kernel split-K fix-up and
+    greedy pick against the row-major ops (which are checked against the oracle above)."""
+    g = gen(20)
+    dt = torch.bfloat16
+    B, d, I, V = 8, 768, 3072, 5003
+    x = dev(torch.randn(B, d, generator=g).to(dt))
+    delta = dev(torch.randn(B, d, generator=g).to(dt))
+    nw = dev((1 + 0.2 * torch.randn(d, generator=g)).to(dt))
+    Wg, Wu = (dev((torch.randn(I, d, generator=g) / math.sqrt(d)).to(dt)) for _ in range(2))
+    Wd = dev((torch.randn(d, I, generator=g) / math.sqrt(I)).to(dt))
+    Wh = dev((torch.randn(V, d, generator=g) / math.sqrt(d)).to(dt))
+    pg, pu, pd, ph = (hip.pack_rows(w) for w in (Wg, Wu, Wd, Wh))
+    # reference chain with the unfused kernels
+    xr = x.clone()
+    h = hip.add_rmsnorm(xr, delta, nw, O.RMS_EPS_DEFAULT)
+    act_ref = hip.glu_decode(h, Wg, Wu)
+    down_ref = hip.linear_decode(act_ref, Wd)
+    logits_ref = hip.linear_decode(h, Wh)
+    # mode 1 with prologue
+    res_out = torch.zeros_like(x)
+    act = torch.empty(B, I, dtype=dt, device="cuda")
+    hip.gemv_packed(1, pg, I, d, act, Wp2=pu, res_in=x, delta=delta, res_out=res_out, norm_w=nw, eps=O.RMS_EPS_DEFAULT)
+    assert torch.equal(res_out, xr)
+    check(act, act_ref, dt, frac=0.01)
+    # prologue without delta leaves res_out untouched and equals plain norm
+    res2 = torch.full_like(x, 7.0)
+    act2 = torch.empty_like(act)
+    hip.gemv_packed(1, pg, I, d, act2, Wp2=pu, res_in=xr, res_out=res2, norm_w=nw, eps=O.RMS_EPS_DEFAULT)
+    assert torch.equal(act2, act) and bool((res2 == 7.0).all())
+    # mode 2: split-K with fix-up, twice (counters must return to zero), and unsplit
+    ws = torch.zeros(12 * 48 * 256, device="cuda")
+    cnt = torch.zeros(48, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        y = torch.empty(B, d, dtype=dt, device="cuda")
+        hip.gemv_packed(2, pd, d, I, y, x=act_ref, ksplit=12, partial_ws=ws, counters=cnt)
+        check(y, down_ref, dt, frac=0.01)
+        assert int(cnt.abs().sum()) == 0
+    y1 = torch.empty(B, d, dtype=dt, device="cuda")
+    hip.gemv_packed(2, pd, d, I, y1, x=act_ref, ksplit=1)
+    check(y1, down_ref, dt, frac=0.01)
+    # mode 0 plain (N not a multiple of 16) and mode 3 greedy pick
+    lg = torch.empty(B, V, dtype=dt, device="cuda")
+    hip.gemv_packed(0, ph, V, d, lg, x=h)
+    check(lg, logits_ref, dt, frac=0.01)
+    best = torch.zeros(16 * 64, dtype=torch.int64, device="cuda")
+    toks = torch.full((B, 2), -1, dtype=torch.int64, device="cuda")
+    lg3 = torch.empty(B, V, dtype=dt, device="cuda")
+    hip.gemv_packed(3, ph, V, d, lg3, res_in=x, delta=delta, res_out=res_out, norm_w=nw, eps=O.RMS_EPS_DEFAULT,
+                    temperature=0.9, best_ws=best, tok_out=toks[:, 1])
+    assert torch.equal(lg3, lg)
+    ref_tok = O.next_token(lg3.cpu(), temperature=0.9, do_sample=False)[:, 0]
+    assert torch.equal(toks[:, 1].cpu(), ref_tok) and int(best.abs().sum()) == 0 and bool((toks[:, 0] == -1).all())
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gelu_mul(hip, dtype):
     g = gen(5)

@@ -23,9 +23,9 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_hip.LIB_PATH)
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
-    bound = set(_hip.SIGNATURES) | {"fstu_version", "fstu_last_error", "fstu_decode_step", "fstu_prof_begin",
-                                       "fstu_prof_end", "fstu_decode_graph_create", "fstu_decode_graph_launch",
-                                       "fstu_decode_graph_destroy"}
+    # every entry point must have its argument types declared: an undeclared pointer argument would be
+    # truncated to a 32-bit int by ctypes
+    bound = set(_hip.SIGNATURES) | {"fstu_version", "fstu_last_error"}
     assert declared == bound, declared ^ bound
     assert _hip.load().fstu_version() == 100
 
