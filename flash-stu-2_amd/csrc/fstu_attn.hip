@@ -50,6 +50,28 @@ struct Partial {
   float acc[DPL];
 };
 
+// One key for an 8-lane group: score, soft-cap, ALiBi, online-softmax update.  All 8 lanes of the group call it.
+template <int DPL>
+__device__ __forceinline__ void attend_one(Partial<DPL>& P, const float* q, const float* kk, const float* vv, int j, int pos,
+                                           float scale, float softcap, float slope) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) s = fmaf(q[i], kk[i], s);
+  s += __shfl_xor(s, 1, FSTU_WAVE);
+  s += __shfl_xor(s, 2, FSTU_WAVE);
+  s += __shfl_xor(s, 4, FSTU_WAVE);
+  s *= scale;
+  if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+  s -= slope * (float)(pos - j);
+  float mn = fmaxf(P.m, s);
+  float corr = __expf(P.m - mn);
+  float p = __expf(s - mn);
+  P.l = P.l * corr + p;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) P.acc[i] = fmaf(p, vv[i], P.acc[i] * corr);
+  P.m = mn;
+}
+
 // Visits keys j = jb+u (u<U) for jb = j_first, j_first+j_step, ... < j_end.
 // kb/vb point at this lane's dims of slot 0; consecutive slots are `stride`
 // elements apart; cap > 0 maps position j to slot j % cap.
@@ -148,8 +170,9 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 // ---------------------------------------------------------------- decode
 // One workgroup per (batch, head); NWAVES*8 key groups visit 4 keys each per
 // sweep, so a 513-key window is covered in two sweeps with every load of a
-// sweep in flight at once.  With append != 0 the workgroup first stores the new
-// token's k,v (read from the qkv row) into ring slot pos % cap.
+// sweep in flight at once.  With append != 0 the workgroup stores the new token's
+// k,v (read from the qkv row) into ring slot pos % cap and attends to that key
+// straight from the qkv row, so the ring sweep covers the older keys only.
 #define SWA_U 4
 template <typename T, int HD, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64)
@@ -173,18 +196,25 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
       kring[dst] = row[d + threadIdx.x];
       vring[dst] = row[2 * d + threadIdx.x];
     }
-    __syncthreads();
   }
   float q[DPL];
   load_vec<T, DPL>(row + gl * DPL, q);
+  const bool self_grp = append && (G == NGRP - 1);   // this group also takes the new token's own key
+  float kself[DPL], vself[DPL];
+  if (self_grp) {
+    load_vec<T, DPL>(row + d + gl * DPL, kself);
+    load_vec<T, DPL>(row + 2 * d + gl * DPL, vself);
+  }
   Partial<DPL> P;
   P.m = -INFINITY;
   P.l = 0.f;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
   const int lo = max(0, pos - window);
-  attend_keys<T, DPL, SWA_U>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, q, lo + G * SWA_U, pos + 1,
-                             NGRP * SWA_U, pos, rsqrtf((float)HD), softcap, slopes[h]);
+  const float scale = rsqrtf((float)HD), slope = slopes[h];
+  attend_keys<T, DPL, SWA_U>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, q, lo + G * SWA_U,
+                             append ? pos : pos + 1, NGRP * SWA_U, pos, scale, softcap, slope);
+  if (self_grp) attend_one<DPL>(P, q, kself, vself, pos, pos, scale, softcap, slope);
   if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
 #pragma unroll
   for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];

@@ -44,6 +44,8 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
+int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
+                             int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream);
 int fstu_gemv_packed_dyn(const fstu_gemv_args* a, const int* dyn, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

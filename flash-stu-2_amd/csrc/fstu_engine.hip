@@ -189,8 +189,13 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_STU, fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
         TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
-        TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-        TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
+        if (dt == FSTU_BF16 && d % 256 == 0) {
+          TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y, d, nullptr, B,
+                                                 m->lds_S, d, d, pos, dyn, stream));
+        } else {
+          TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
+          TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
+        }
         TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       }
     } else {

@@ -9,8 +9,9 @@
 // load instruction (64 lanes x 16 B) reads 1 KB of contiguous memory and a wave
 // that walks a K range streams one contiguous block.  Rows beyond N are zero.
 //
-// Workgroup = 4 waves = one 16-feature tile x 4 K quarters (reduced through LDS
-// in fixed order).  Activations are the MFMA B operand: either read from global
+// Workgroup = 4 waves = 4 K quarters of a run of consecutive 16-feature tiles
+// (quarters reduced through LDS in fixed order; the next tile's weights are in
+// flight while the current tile is reduced and stored).  Activations are the MFMA B operand: either read from global
 // memory, or produced by the prologue into LDS:
 //   x_new = T(res_in + delta);  h = T(x_new * rsqrt(mean(x_new^2)+eps) * w)
 // (every workgroup recomputes it from the 12-24 KB of inputs; workgroup 0 also
@@ -28,29 +29,32 @@ __device__ __forceinline__ bf16x8_t gv_as_bf16x8(uint4 v) { return __builtin_bit
 
 template <int MODE, bool PRO>
 __global__ void __launch_bounds__(256)
-gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row stride in elements*/) {
-  constexpr int U = 6;  // k steps (32 wide) loaded back to back
+gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row stride in elements*/,
+                   int tpw /*consecutive tiles per workgroup*/, int ntiles) {
+  constexpr int U = 6;  // k steps (32 wide) per load batch
+  constexpr int REDF = 4 * 64 * 4 * ((MODE == GV_GLU) ? 2 : 1);   // floats of one reduction buffer
   extern __shared__ __align__(16) unsigned char smem[];
-  float* red = (float*)smem;                                            // 4*64*4 (x2 for GLU) floats
-  bf16_t* hs = (bf16_t*)(smem + ((MODE == GV_GLU) ? 8192 : 4096));      // rows x hs_ld (PRO only)
+  float* red = (float*)smem;                                        // two reduction buffers (alternating tiles)
+  bf16_t* hs = (bf16_t*)(smem + 2 * REDF * sizeof(float));          // rows x hs_ld (PRO only)
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int tile = blockIdx.x;
   const int r = lane & 15, g = lane >> 4;
   const int ksteps_total = a.K >> 5;
-  const int ksw = kw >> 5;                                              // k steps per wave
-  const int ks0 = (blockIdx.y * 4 + w) * ksw;                           // first k step of this wave
-  const uint4* wp = (const uint4*)a.Wp + ((size_t)tile * ksteps_total + ks0) * 64 + lane;
-  const uint4* wp2 = (MODE == GV_GLU) ? (const uint4*)a.Wp2 + ((size_t)tile * ksteps_total + ks0) * 64 + lane : nullptr;
+  const int ksw = kw >> 5;                                          // k steps per wave
+  const int ks0 = (blockIdx.y * 4 + w) * ksw;                       // first k step of this wave
+  const int tile0 = blockIdx.x * tpw;
+  const int tile1 = min(ntiles, tile0 + tpw);
   const bool xrow = r < a.rows;
-  floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  const uint4* wbase = (const uint4*)a.Wp + (size_t)ks0 * 64 + lane;
+  const uint4* wbase2 = (MODE == GV_GLU) ? (const uint4*)a.Wp2 + (size_t)ks0 * 64 + lane : nullptr;
+  const size_t tile_stride = (size_t)ksteps_total * 64;
 
-  // first batch of weight loads (independent of the activations)
+  // weights of the first tile's first batch: in flight while the prologue runs
   uint4 wa[U], wb[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (u < ksw) {
-      wa[u] = wp[(size_t)u * 64];
-      if (MODE == GV_GLU) wb[u] = wp2[(size_t)u * 64];
+      wa[u] = wbase[(size_t)tile0 * tile_stride + (size_t)u * 64];
+      if (MODE == GV_GLU) wb[u] = wbase2[(size_t)tile0 * tile_stride + (size_t)u * 64];
     }
   }
 
@@ -78,137 +82,175 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
       *(uint4*)(hs + (size_t)row * hs_ld + c) = xv;
     }
     __syncthreads();
-    // ---- one wave per row: statistics in a fixed order, normalise in place
+    // ---- one wave per row: statistics in a fixed order, normalise in place (16-byte LDS accesses)
     const bf16_t* nw = (const bf16_t*)a.norm_w;
     for (int row = w; row < a.rows; row += 4) {
       bf16_t* hr = hs + (size_t)row * hs_ld;
       float ss = 0.f;
-      for (int c = lane; c < a.K; c += 64) { float v = bf16_to_f32(hr[c]); ss = fmaf(v, v, ss); }
+      for (int c = lane * 8; c < a.K; c += 512) {
+        uint4 v = *(const uint4*)(hr + c);
+        unsigned vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float lo = __uint_as_float(vw[i] << 16), hi = __uint_as_float(vw[i] & 0xffff0000u);
+          ss = fmaf(lo, lo, ss);
+          ss = fmaf(hi, hi, ss);
+        }
+      }
       ss = wave_sum(ss);
       const float rstd = rsqrtf(ss / (float)a.K + a.eps);
-      for (int c = lane; c < a.K; c += 64) hr[c] = f32_to_bf16((bf16_to_f32(hr[c]) * rstd) * bf16_to_f32(nw[c]));
+      for (int c = lane * 8; c < a.K; c += 512) {
+        uint4 v = *(const uint4*)(hr + c);
+        uint4 wv = *(const uint4*)(nw + c);
+        unsigned vw[4] = {v.x, v.y, v.z, v.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float lo = (__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16);
+          float hi = (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u);
+          vw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+        }
+        *(uint4*)(hr + c) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+      }
     }
     __syncthreads();
   }
 
   const bf16_t* xg = PRO ? nullptr : (const bf16_t*)a.x + (size_t)(xrow ? r : 0) * a.ldx + ks0 * 32 + g * 8;
   const bf16_t* xl = PRO ? hs + (size_t)(xrow ? r : 0) * hs_ld + ks0 * 32 + g * 8 : nullptr;
-  for (int i0 = 0; i0 < ksw; i0 += U) {
-    uint4 xa[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (i0 + u < ksw) {
-        if (!xrow) xa[u] = make_uint4(0, 0, 0, 0);
-        else if (PRO) xa[u] = *(const uint4*)(xl + (size_t)(i0 + u) * 32);
-        else xa[u] = *(const uint4*)(xg + (size_t)(i0 + u) * 32);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (i0 + u < ksw) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv_as_bf16x8(wa[u]), gv_as_bf16x8(xa[u]), acc, 0, 0, 0);
-        if (MODE == GV_GLU)
-          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv_as_bf16x8(wb[u]), gv_as_bf16x8(xa[u]), acc2, 0, 0, 0);
-      }
-    }
-    // next batch of weights
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (i0 + U + u < ksw) {
-        wa[u] = wp[(size_t)(i0 + U + u) * 64];
-        if (MODE == GV_GLU) wb[u] = wp2[(size_t)(i0 + U + u) * 64];
-      }
-    }
-  }
 
-  // ---- reduce the 4 K quarters in fixed order
-  {
-    float* mine = red + (size_t)(w * 64 + lane) * 4;
-    constexpr int GLU_OFF = 4 * 64 * 4;
+  for (int tile = tile0; tile < tile1; ++tile) {
+    floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    const uint4* wp = wbase + (size_t)tile * tile_stride;
+    const uint4* wp2 = (MODE == GV_GLU) ? wbase2 + (size_t)tile * tile_stride : nullptr;
+    for (int i0 = 0; i0 < ksw; i0 += U) {
+      uint4 xa[U];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mine[i] = acc[i];
-      if (MODE == GV_GLU) mine[GLU_OFF + i] = acc2[i];
-    }
-    __syncthreads();
-    if (w != 0) return;
-#pragma unroll
-    for (int s = 1; s < 4; ++s) {
-      const float* o = red + (size_t)(s * 64 + lane) * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[i] += o[i];
-        if (MODE == GV_GLU) acc2[i] += o[GLU_OFF + i];
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u < ksw) {
+          if (!xrow) xa[u] = make_uint4(0, 0, 0, 0);
+          else if (PRO) xa[u] = *(const uint4*)(xl + (size_t)(i0 + u) * 32);
+          else xa[u] = *(const uint4*)(xg + (size_t)(i0 + u) * 32);
+        }
       }
-    }
-  }
-
-  if (MODE == GV_FIXUP && gridDim.y > 1) {
-    // split-K across workgroups: publish this partial tile, the last arriver adds all of them in slice order
-    const int ntiles = gridDim.x, GS = gridDim.y;
-    float* slot = a.partial_ws + (((size_t)blockIdx.y * ntiles + tile) * 64 + lane) * 4;
+      uint4 ca[U], cb[U];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) __hip_atomic_store(slot + i, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);   // the partial has reached the coherence point before the ticket is taken
-    unsigned old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(a.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __shfl(old, 0, FSTU_WAVE);
-    if (old != (unsigned)(GS - 1)) return;
-    acc = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < GS; s0 += 8) {
-      float v[8][4];
+      for (int u = 0; u < U; ++u) { ca[u] = wa[u]; if (MODE == GV_GLU) cb[u] = wb[u]; }
+      // next batch of weights (same tile, or the first batch of the next tile) goes in flight before the MFMAs
+      {
+        const bool more = i0 + U < ksw;
+        const bool next_tile = !more && (tile + 1 < tile1);
+        const uint4* np = more ? wp + (size_t)(i0 + U) * 64 : wp + tile_stride;
+        const uint4* np2 = (MODE == GV_GLU) ? (more ? wp2 + (size_t)(i0 + U) * 64 : wp2 + tile_stride) : nullptr;
+        const int lim = more ? ksw - (i0 + U) : (next_tile ? ksw : 0);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float* p = a.partial_ws + (((size_t)(s0 + k) * ntiles + tile) * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          v[k][i] = (s0 + k < GS) ? __hip_atomic_load(p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+        for (int u = 0; u < U; ++u) {
+          if (u < lim) {
+            wa[u] = np[(size_t)u * 64];
+            if (MODE == GV_GLU) wb[u] = np2[(size_t)u * 64];
+          }
+        }
       }
 #pragma unroll
-      for (int k = 0; k < 8; ++k)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] += v[k][i];
-    }
-    if (lane == 0) __hip_atomic_store(a.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  if (MODE == GV_ARGMAX) {
-    unsigned long long key = 0ull;
-    if (xrow) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int f = tile * 16 + g * 4 + i;
-        if (f < a.N) {
-          float l = DT<bf16_t>::rnd(acc[i]);
-          if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
-          l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
-          unsigned u = __float_as_uint(l);
-          u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-          unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
-          key = k > key ? k : key;
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u < ksw) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv_as_bf16x8(ca[u]), gv_as_bf16x8(xa[u]), acc, 0, 0, 0);
+          if (MODE == GV_GLU)
+            acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv_as_bf16x8(cb[u]), gv_as_bf16x8(xa[u]), acc2, 0, 0, 0);
         }
       }
     }
-    unsigned long long o = __shfl_xor(key, 16, FSTU_WAVE);
-    key = o > key ? o : key;
-    o = __shfl_xor(key, 32, FSTU_WAVE);
-    key = o > key ? o : key;
-    if (g == 0 && xrow && key != 0ull)
-      atomicMax((unsigned long long*)a.best_ws + (size_t)r * GV_SLOTS + (tile & (GV_SLOTS - 1)), key);
-  }
 
-  // D layout: lane holds features 4*g+i of batch row r
-  if (!xrow) return;
-  bf16_t* yr = (bf16_t*)a.y + (size_t)r * a.ldy;
+    // ---- reduce the 4 K quarters in fixed order (buffers alternate between tiles: one barrier per tile)
+    float* rbuf = red + (size_t)((tile - tile0) & 1) * REDF;
+    {
+      float* mine = rbuf + (size_t)(w * 64 + lane) * 4;
+      constexpr int GLU_OFF = 4 * 64 * 4;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int f = tile * 16 + g * 4 + i;
-    if (f >= a.N) continue;
-    if (MODE == GV_GLU) {
-      float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[i])));
-      yr[f] = f32_to_bf16(ge * DT<bf16_t>::rnd(acc2[i]));
-    } else {
-      yr[f] = f32_to_bf16(acc[i]);
+      for (int i = 0; i < 4; ++i) {
+        mine[i] = acc[i];
+        if (MODE == GV_GLU) mine[GLU_OFF + i] = acc2[i];
+      }
+      __syncthreads();
+      if (w != 0) continue;
+#pragma unroll
+      for (int s = 1; s < 4; ++s) {
+        const float* o = rbuf + (size_t)(s * 64 + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[i] += o[i];
+          if (MODE == GV_GLU) acc2[i] += o[GLU_OFF + i];
+        }
+      }
+    }
+
+    if (MODE == GV_FIXUP && gridDim.y > 1) {
+      // split-K across workgroups: publish this partial tile, the last arriver adds all of them in slice order
+      const int GS = gridDim.y;
+      float* slot = a.partial_ws + (((size_t)blockIdx.y * ntiles + tile) * 64 + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) __hip_atomic_store(slot + i, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);   // the partial has reached the coherence point before the ticket is taken
+      unsigned old = 0;
+      if (lane == 0) old = __hip_atomic_fetch_add(a.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = __shfl(old, 0, FSTU_WAVE);
+      if (old != (unsigned)(GS - 1)) continue;
+      acc = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < GS; s0 += 8) {
+        float v[8][4];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float* p = a.partial_ws + (((size_t)(s0 + k) * ntiles + tile) * 64 + lane) * 4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            v[k][i] = (s0 + k < GS) ? __hip_atomic_load(p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] += v[k][i];
+      }
+      if (lane == 0) __hip_atomic_store(a.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    if (MODE == GV_ARGMAX) {
+      unsigned long long key = 0ull;
+      if (xrow) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int f = tile * 16 + g * 4 + i;
+          if (f < a.N) {
+            float l = DT<bf16_t>::rnd(acc[i]);
+            if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
+            l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
+            unsigned u = __float_as_uint(l);
+            u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+            unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
+            key = k > key ? k : key;
+          }
+        }
+      }
+      unsigned long long o = __shfl_xor(key, 16, FSTU_WAVE);
+      key = o > key ? o : key;
+      o = __shfl_xor(key, 32, FSTU_WAVE);
+      key = o > key ? o : key;
+      if (g == 0 && xrow && key != 0ull)
+        atomicMax((unsigned long long*)a.best_ws + (size_t)r * GV_SLOTS + (tile & (GV_SLOTS - 1)), key);
+    }
+
+    // D layout: lane holds features 4*g+i of batch row r
+    if (xrow) {
+      bf16_t* yr = (bf16_t*)a.y + (size_t)r * a.ldy;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int f = tile * 16 + g * 4 + i;
+        if (f >= a.N) continue;
+        if (MODE == GV_GLU) {
+          float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[i])));
+          yr[f] = f32_to_bf16(ge * DT<bf16_t>::rnd(acc2[i]));
+        } else {
+          yr[f] = f32_to_bf16(acc[i]);
+        }
+      }
     }
   }
 }
@@ -227,10 +269,19 @@ __global__ void gv_argmax_finish_kernel(unsigned long long* best, int64_t* tok_o
   if (lane == 0) tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
 }
 
+static int g_target_wgs = 65535;   // tuning knob: workgroups a GEMV launch aims for
+
+extern "C" int fstu_set_gemv_target_workgroups(int n) {
+  FSTU_REQUIRE(n >= 1 && n <= 65535, FSTU_EARG, "fstu_set_gemv_target_workgroups: %d", n);
+  g_target_wgs = n;
+  return FSTU_OK;
+}
+
 template <int MODE>
-static void gv_launch(const fstu_gemv_args& a, bool pro, dim3 grid, size_t shm, int kw, int hs_ld, hipStream_t s) {
-  if (pro) hipLaunchKernelGGL((gemv_packed_kernel<MODE, true>), grid, dim3(256), shm, s, a, kw, hs_ld);
-  else hipLaunchKernelGGL((gemv_packed_kernel<MODE, false>), grid, dim3(256), shm, s, a, kw, hs_ld);
+static void gv_launch(const fstu_gemv_args& a, bool pro, dim3 grid, size_t shm, int kw, int hs_ld, int tpw, int ntiles,
+                      hipStream_t s) {
+  if (pro) hipLaunchKernelGGL((gemv_packed_kernel<MODE, true>), grid, dim3(256), shm, s, a, kw, hs_ld, tpw, ntiles);
+  else hipLaunchKernelGGL((gemv_packed_kernel<MODE, false>), grid, dim3(256), shm, s, a, kw, hs_ld, tpw, ntiles);
 }
 
 int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, const int* dyn, void* stream) {
@@ -244,7 +295,7 @@ int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, const int* dyn, void* stream)
   FSTU_REQUIRE(a.ldy >= a.N, FSTU_ESHAPE, "fstu_gemv_packed: ldy=%d < N=%d", a.ldy, a.N);
   FSTU_REQUIRE(fstu_aligned(a.Wp, 16) && fstu_aligned(a.Wp2, 16), FSTU_EALIGN, "fstu_gemv_packed: packed weights must be 16-byte aligned");
   const bool pro = a.norm_w != nullptr;
-  size_t shm = (a.mode == GV_GLU) ? 8192 : 4096;
+  size_t shm = (a.mode == GV_GLU) ? 16384 : 8192;   // two reduction buffers
   int hs_ld = 0;
   if (pro) {
     FSTU_REQUIRE(a.res_in, FSTU_ENULL, "fstu_gemv_packed: norm_w given without res_in");
@@ -262,13 +313,16 @@ int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, const int* dyn, void* stream)
   if (a.mode == GV_ARGMAX) FSTU_REQUIRE(a.best_ws && a.tok_out && a.tok_stride >= 1 && a.temperature > 0.f, FSTU_EARG, "fstu_gemv_packed: greedy pick needs best_ws, tok_out, temperature>0");
   const int ntiles = (a.N + 15) / 16;
   const int kw = a.K / (4 * gs);
-  dim3 grid(ntiles, gs);
+  // consecutive tiles per workgroup: about `g_target_wgs` workgroups in flight, so the prologue is paid once per CU
+  int tpw = (ntiles * gs + g_target_wgs - 1) / g_target_wgs;
+  if (tpw < 1) tpw = 1;
+  dim3 grid((ntiles + tpw - 1) / tpw, gs);
   hipStream_t s = (hipStream_t)stream;
   switch (a.mode) {
-    case GV_PLAIN: gv_launch<GV_PLAIN>(a, pro, grid, shm, kw, hs_ld, s); break;
-    case GV_GLU: gv_launch<GV_GLU>(a, pro, grid, shm, kw, hs_ld, s); break;
-    case GV_FIXUP: gv_launch<GV_FIXUP>(a, pro, grid, shm, kw, hs_ld, s); break;
-    default: gv_launch<GV_ARGMAX>(a, pro, grid, shm, kw, hs_ld, s); break;
+    case GV_PLAIN: gv_launch<GV_PLAIN>(a, pro, grid, shm, kw, hs_ld, tpw, ntiles, s); break;
+    case GV_GLU: gv_launch<GV_GLU>(a, pro, grid, shm, kw, hs_ld, tpw, ntiles, s); break;
+    case GV_FIXUP: gv_launch<GV_FIXUP>(a, pro, grid, shm, kw, hs_ld, tpw, ntiles, s); break;
+    default: gv_launch<GV_ARGMAX>(a, pro, grid, shm, kw, hs_ld, tpw, ntiles, s); break;
   }
   if (a.mode == GV_ARGMAX)
     hipLaunchKernelGGL(gv_argmax_finish_kernel, dim3(a.rows), dim3(64), 0, s, (unsigned long long*)a.best_ws, a.tok_out,

@@ -134,7 +134,7 @@ linear_mfma_bf16_kernel(LinArgs a) {
     key = o > key ? o : key;
     o = __shfl_xor(key, 32, FSTU_WAVE);
     key = o > key ? o : key;
-    if (tile_ok && g == 0 && r < a.rows && key != 0ull) atomicMax(a.best + r, key);
+    if (tile_ok && g == 0 && r < a.rows && key != 0ull) atomicMax(a.best + (size_t)r * 64 + (tile & 63), key);  // 64 slots per row spread the contention
   }
   if (!tile_ok) return;
   // D layout: lane holds features 4*(lane/16)+i, batch row lane%16
@@ -305,12 +305,16 @@ extern "C" int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, 
 // ---------------------------------------------------------------- head with fused greedy pick
 __global__ void argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows,
                                      const int* __restrict__ dyn) {
-  int b = threadIdx.x;
-  if (b < rows) {
-    unsigned long long k = best[b];
-    tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
-    best[b] = 0ull;
+  // one wave per row: maximum over the 64 slots, which are cleared for the next call
+  const int b = blockIdx.x, lane = threadIdx.x;
+  unsigned long long k = best[(size_t)b * 64 + lane];
+  best[(size_t)b * 64 + lane] = 0ull;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    unsigned long long t = __shfl_xor(k, o, FSTU_WAVE);
+    k = t > k ? t : k;
   }
+  if (lane == 0) tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
 }
 
 extern "C" int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
@@ -331,7 +335,7 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   if (dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1)) {
     LinArgs a{x, ldx, W, nullptr, logits, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
     launch_mfma<LIN_ARGMAX>(a, 1, (hipStream_t)stream);
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
                        tok_out, tok_stride, rows, dyn);
     FSTU_CHECK_LAUNCH("fstu_head_argmax");
     return FSTU_OK;

@@ -182,6 +182,128 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
   return FSTU_OK;
 }
 
+// ---------------------------------------------------------------- input projection + LDS-form step, one launch
+// Workgroup = one tile of 16 channels: x_proj[b, c] = T(h[b,:] . Mt[c,:]) by MFMA (K split over the 4 waves, reduced
+// in LDS), then the recurrence step of those 16 channels for every batch row.  Thread (b, jsub, cq) owns 4 channels
+// (float4) of modes jsub, jsub+8, ...; the 8 mode groups are reduced with wave shuffles.
+typedef __bf16 stu_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float stu_floatx4_t __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256)
+stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
+                       float* __restrict__ state, const float* __restrict__ a, const float* __restrict__ ce,
+                       bf16_t* __restrict__ y, int ldy, bf16_t* __restrict__ xp_out /*optional (B,d)*/, int B, int S,
+                       int d, int K, int parity, const int* __restrict__ dyn) {
+  __shared__ float red[4][64][4];
+  __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
+  if (dyn) parity = dyn[0] & 1;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x, c0 = tile * 16;
+  // ---- projection: A operand = Mt rows (channels), B operand = h rows (batch)
+  const int kw = K >> 2;                                    // k range of this wave
+  const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
+  const bool xrow = r < B;
+  const bf16_t* hp = h + (size_t)(xrow ? r : 0) * ldh + w * kw + g * 16;
+  stu_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int i0 = 0; i0 < (kw >> 6); i0 += 4) {
+    uint4 wa[4][2], xa[4][2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i0 + u < (kw >> 6)) {
+        const uint4* p = (const uint4*)(wp + (size_t)(i0 + u) * 64);
+        wa[u][0] = p[0];
+        wa[u][1] = p[1];
+        if (xrow) {
+          const uint4* q = (const uint4*)(hp + (size_t)(i0 + u) * 64);
+          xa[u][0] = q[0];
+          xa[u][1] = q[1];
+        } else {
+          xa[u][0] = make_uint4(0, 0, 0, 0);
+          xa[u][1] = make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i0 + u < (kw >> 6)) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(stu_bf16x8_t, wa[u][0]), __builtin_bit_cast(stu_bf16x8_t, xa[u][0]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(stu_bf16x8_t, wa[u][1]), __builtin_bit_cast(stu_bf16x8_t, xa[u][1]), acc, 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[w][lane][i] = acc[i];
+  __syncthreads();
+  if (w == 0) {
+    // D layout: lane holds channels 4*g+i of batch row r
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = DT<bf16_t>::rnd(((red[0][lane][i] + red[1][lane][i]) + red[2][lane][i]) + red[3][lane][i]);
+      xps[r][4 * g + i] = v;
+      if (xp_out && xrow && c0 + 4 * g + i < d) xp_out[(size_t)r * d + c0 + 4 * g + i] = f32_to_bf16(v);
+    }
+  }
+  __syncthreads();
+  // ---- recurrence step of the tile's channels
+  const int cq = threadIdx.x & 3, jsub = (threadIdx.x >> 2) & 7, bsub = threadIdx.x >> 5;
+  const int c = c0 + cq * 4;
+  for (int b = bsub; b < B; b += 8) {
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c < d) {
+      const float x0 = xps[b][cq * 4], x1 = xps[b][cq * 4 + 1], x2 = xps[b][cq * 4 + 2], x3 = xps[b][cq * 4 + 3];
+      float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
+#pragma unroll 8
+      for (int j = jsub; j < S; j += 8) {
+        float4 hv = *(float4*)(st + (size_t)j * d);
+        const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
+        const float aj = a[j];
+        hv.x = fmaf(aj, hv.x, x0);
+        hv.y = fmaf(aj, hv.y, x1);
+        hv.z = fmaf(aj, hv.z, x2);
+        hv.w = fmaf(aj, hv.w, x3);
+        *(float4*)(st + (size_t)j * d) = hv;
+        sum.x = fmaf(cj.x, hv.x, sum.x);
+        sum.y = fmaf(cj.y, hv.y, sum.y);
+        sum.z = fmaf(cj.z, hv.z, sum.z);
+        sum.w = fmaf(cj.w, hv.w, sum.w);
+      }
+    }
+    // reduce over the 8 mode groups: lanes differing in bits 2..4
+#pragma unroll
+    for (int o = 4; o <= 16; o <<= 1) {
+      sum.x += __shfl_xor(sum.x, o, FSTU_WAVE);
+      sum.y += __shfl_xor(sum.y, o, FSTU_WAVE);
+      sum.z += __shfl_xor(sum.z, o, FSTU_WAVE);
+      sum.w += __shfl_xor(sum.w, o, FSTU_WAVE);
+    }
+    if (jsub == 0 && c < d) {
+      bf16_t* yp = y + (size_t)b * ldy + c;
+      yp[0] = f32_to_bf16(2.f * sum.x);
+      yp[1] = f32_to_bf16(2.f * sum.y);
+      yp[2] = f32_to_bf16(2.f * sum.z);
+      yp[3] = f32_to_bf16(2.f * sum.w);
+    }
+  }
+}
+
+int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
+                             int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream) {
+  FSTU_REQUIRE(h && Mt && state && a && ce && y, FSTU_ENULL, "fstu_stu_inproj_step: null pointer");
+  FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
+  FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
+  FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(Mt, 16) && fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_inproj_step: pointers must be 16-byte aligned");
+  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h, ldh,
+                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, ldy, (bf16_t*)xp_out, B, S, d, K, t & 1, dyn);
+  FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
+                                    void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream) {
+  return fstu_stu_inproj_step_dyn(h, ldh, Mt, state, a, ce, y, ldy, xp_out, B, S, d, K, t, nullptr, stream);
+}
+
 // ---------------------------------------------------------------- state from history
 #define LSH_JG 4
 #define LSH_MAXJ 32

@@ -33,6 +33,7 @@ SIGNATURES = {
     "fstu_gelu_mul": [_vp, _vp, _vp, _i64, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -46,6 +47,7 @@ SIGNATURES = {
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
     "fstu_packed_elems": [_i, _i],
     "fstu_gemv_packed": [_vp, _vp],
+    "fstu_set_gemv_target_workgroups": [_i],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
@@ -243,6 +245,21 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
     return out
 
 
+def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
+                    out: Optional[torch.Tensor] = None, xp_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h (B,K) bf16, Mt = M_inputs^T (d,K): projection + recurrence step in one launch -> y (B,d)."""
+    _dev(h, Mt, state, a, ce, out, xp_out)
+    B, K = h.shape
+    d = Mt.shape[0]
+    S = a.numel()
+    assert h.dtype == Mt.dtype == torch.bfloat16 and Mt.shape[1] == K and state.shape == (B, 2, S, d)
+    if out is None:
+        out = torch.empty(B, d, dtype=h.dtype, device=h.device)
+    _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(out), d, _p(xp_out), B, S, d, K, t,
+                                       _stream()), "fstu_stu_inproj_step")
+    return out
+
+
 def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, state: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(hist, a, state)
     B, cap, d = hist.shape
@@ -341,7 +358,7 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: float = 1.0, to
 def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best_ws: torch.Tensor,
                 temperature: float = 1.0, logits: Optional[torch.Tensor] = None) -> torch.Tensor:
     """logits = x @ W^T (rows<=16) and the greedy pick per row written to out_tokens (a strided (rows,) int64 view).
-    best_ws: int64 zeros of at least `rows` elements; it is zero again when the call completes."""
+    best_ws: int64 zeros of at least rows*64 elements; it is zero again when the call completes."""
     rows, ldx = _rows_view(x)
     _dev(W, best_ws)
     N, K = W.shape
@@ -349,7 +366,7 @@ def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best
     if logits is None:
         logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
     assert out_tokens.dtype == torch.int64 and out_tokens.dim() == 1 and out_tokens.shape[0] == rows
-    assert best_ws.dtype == torch.int64 and best_ws.numel() >= rows
+    assert best_ws.dtype == torch.int64 and best_ws.numel() >= rows * 64
     _check(load().fstu_head_argmax(_p(x), ldx, _p(W), _p(logits), logits.stride(0), rows, N, K, float(temperature),
                                    _p(best_ws), out_tokens.data_ptr(), out_tokens.stride(0), _dt(x), _stream()),
            "fstu_head_argmax")

@@ -10,6 +10,7 @@ the sequence with torch.cat every step).
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import List, Optional
 
 import torch
@@ -76,6 +77,8 @@ class DecodeEngine:
         return hit[1]
 
     def _use_packed(self, B: int) -> bool:
+        if os.environ.get("FSTU_PACKED_STEP", "0") != "1":
+            return False
         cfg = self.cfg
         d, I = cfg.n_embd, cfg.n_embd * cfg.mlp_scale
         return (cfg.torch_dtype == torch.bfloat16 and cfg.resolved_stu_decode_mode() == "lds" and d % 128 == 0

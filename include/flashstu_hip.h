@@ -122,6 +122,13 @@ int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int
 int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                       int B, int S, int d, int t, int dtype, void* stream);
 
+/* Input projection and recurrence step in one launch (bf16, K % 256 == 0):
+ *   xp[b,c] = T( h[b,:] . Mt[c,:] )  with Mt = M_inputs^T (d,K) row-major, then the step of
+ * fstu_stu_step_lds on xp.  xp_out (B,d) receives xp when not NULL.
+ * Replaces `x @ M_inputs` + the convolution at flash_stu/modules/stu.py:87-98,120 for one token. */
+int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
+                         void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream);
+
 /* Builds that state from a prefilled history: for both parities p,
  *   state[b,p,j,c] = sum_{m>=0} a[j]^m * hist[b, tp-2m, c],  tp = newest index
  *   of parity p that is <= t_last.  hist is (B,cap,d). */
@@ -194,7 +201,7 @@ int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int
 /* Tied head + greedy pick in one pass: logits[m,:] = T(x[m,:] . W^T) as
  * fstu_linear_decode, and tok_out[m*tok_stride] = argmax_n clamp(T(logit/temperature))
  * with the lowest index on ties (same rule as fstu_sample with do_sample=0).
- * best_ws: `rows` 64-bit words, zero on entry and zero again on return.
+ * best_ws: rows*64 64-bit words, zero on entry and zero again on return.
  * Replaces lm_head + argmax at flash_stu/model.py:176,268-269,299. */
 int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                      float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
@@ -255,6 +262,9 @@ typedef struct {
 int64_t fstu_packed_elems(int N, int K);
 int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
 int fstu_gemv_packed(const fstu_gemv_args* a, void* stream);
+/* Tuning knob: number of workgroups a packed GEMV launch aims for (default 256 = one per CU);
+ * each workgroup then walks ceil(tiles/n) consecutive tiles. */
+int fstu_set_gemv_target_workgroups(int n);
 
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
