@@ -39,14 +39,16 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
 int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B, int H, int hd,
                          int cap, int pos, int window, float softcap, int append, const int* dyn, int dtype, void* stream);
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
-                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, const int* dyn,
+                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream);
+int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table, void* x, const void* w, void* h, int rows,
+                       int d, int vocab, float eps, int dtype, void* stream, const int* dyn);
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
                              int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream);
-int fstu_gemv_packed_dyn(const fstu_gemv_args* a, const int* dyn, void* stream);
+int fstu_gemv_packed_dyn(const fstu_gemv_args* a, int* dyn, int advance, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -217,6 +217,38 @@ extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int 
   return FSTU_OK;
 }
 
+// embedding gather fused with the first RMSNorm of the step: x[r,:] = table[id], h[r,:] = rmsnorm(x[r,:]) * w
+template <typename T>
+__global__ void __launch_bounds__(FSTU_NORM_THREADS)
+embed_rmsnorm_kernel(const int64_t* __restrict__ ids, int64_t id_stride, const T* __restrict__ table, T* __restrict__ x,
+                     const T* __restrict__ w, T* __restrict__ h, int d, int vocab, float eps, const int* __restrict__ dyn) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  int64_t id = ids[(size_t)r * id_stride + (dyn ? dyn[0] : 0)];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* src = table + (size_t)id * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += FSTU_NORM_THREADS) {
+    T raw = src[c];
+    x[(size_t)r * d + c] = raw;
+    float v = DT<T>::ld(&raw);
+    ss = fmaf(v, v, ss);
+  }
+  const float rstd = rsqrtf(block_sum_256(ss, red) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += FSTU_NORM_THREADS)
+    DT<T>::st(h + (size_t)r * d + c, (DT<T>::ld(src + c) * rstd) * DT<T>::ld(w + c));
+}
+
+int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table, void* x, const void* w, void* h, int rows,
+                       int d, int vocab, float eps, int dtype, void* stream, const int* dyn) {
+  FSTU_REQUIRE(ids && table && x && w && h, FSTU_ENULL, "fstu_embed_rmsnorm: null pointer");
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_embed_rmsnorm",
+                      hipLaunchKernelGGL(embed_rmsnorm_kernel<T>, dim3(rows), dim3(FSTU_NORM_THREADS), 0, (hipStream_t)stream,
+                                         ids, id_stride, (const T*)table, (T*)x, (const T*)w, (T*)h, d, vocab, eps, dyn));
+  FSTU_CHECK_LAUNCH("fstu_embed_rmsnorm");
+  return FSTU_OK;
+}
+
 // ---------------------------------------------------------------- gelu * up
 template <typename T>
 __global__ void gelu_mul_kernel(const T* __restrict__ g, const T* __restrict__ u, T* __restrict__ act, int64_t n) {

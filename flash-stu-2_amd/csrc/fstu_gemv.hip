@@ -255,10 +255,14 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
   }
 }
 
-__global__ void gv_argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows,
-                                        const int* __restrict__ dyn) {
-  // one wave per row: max over the slots, then clear them
-  const int b = blockIdx.x, lane = threadIdx.x;
+__global__ void __launch_bounds__(1024)
+gv_argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows, int* dyn, int advance) {
+  // one workgroup, one wave per row: max over the slots, then clear them; optionally bump the step counters
+  const int b = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = dyn ? dyn[0] : 0;
+  __syncthreads();
+  if (threadIdx.x == 0 && dyn && advance) { dyn[0] = pos + 1; dyn[1] += 1; }
+  if (b >= rows) return;
   unsigned long long k = best[(size_t)b * GV_SLOTS + lane];
   best[(size_t)b * GV_SLOTS + lane] = 0ull;
 #pragma unroll
@@ -266,7 +270,7 @@ __global__ void gv_argmax_finish_kernel(unsigned long long* best, int64_t* tok_o
     unsigned long long t = __shfl_xor(k, o, FSTU_WAVE);
     k = t > k ? t : k;
   }
-  if (lane == 0) tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
+  if (lane == 0) tok_out[(size_t)b * stride + pos] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
 }
 
 static int g_target_wgs = 65535;   // tuning knob: workgroups a GEMV launch aims for
@@ -284,7 +288,7 @@ static void gv_launch(const fstu_gemv_args& a, bool pro, dim3 grid, size_t shm, 
   else hipLaunchKernelGGL((gemv_packed_kernel<MODE, false>), grid, dim3(256), shm, s, a, kw, hs_ld, tpw, ntiles);
 }
 
-int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, const int* dyn, void* stream) {
+int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, int* dyn, int advance, void* stream) {
   FSTU_REQUIRE(ap, FSTU_ENULL, "fstu_gemv_packed: null argument block");
   const fstu_gemv_args& a = *ap;
   FSTU_REQUIRE(a.mode >= GV_PLAIN && a.mode <= GV_ARGMAX, FSTU_EARG, "fstu_gemv_packed: mode %d", a.mode);
@@ -325,13 +329,13 @@ int fstu_gemv_packed_dyn(const fstu_gemv_args* ap, const int* dyn, void* stream)
     default: gv_launch<GV_ARGMAX>(a, pro, grid, shm, kw, hs_ld, tpw, ntiles, s); break;
   }
   if (a.mode == GV_ARGMAX)
-    hipLaunchKernelGGL(gv_argmax_finish_kernel, dim3(a.rows), dim3(64), 0, s, (unsigned long long*)a.best_ws, a.tok_out,
-                       a.tok_stride, a.rows, dyn);
+    hipLaunchKernelGGL(gv_argmax_finish_kernel, dim3(1), dim3(a.rows * 64), 0, s, (unsigned long long*)a.best_ws, a.tok_out,
+                       a.tok_stride, a.rows, dyn, advance);
   FSTU_CHECK_LAUNCH("fstu_gemv_packed");
   return FSTU_OK;
 }
 
-extern "C" int fstu_gemv_packed(const fstu_gemv_args* a, void* stream) { return fstu_gemv_packed_dyn(a, nullptr, stream); }
+extern "C" int fstu_gemv_packed(const fstu_gemv_args* a, void* stream) { return fstu_gemv_packed_dyn(a, nullptr, 0, stream); }
 
 // ---------------------------------------------------------------- packing
 template <int DUMMY>

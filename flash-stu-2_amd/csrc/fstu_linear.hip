@@ -303,10 +303,15 @@ extern "C" int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, 
 }
 
 // ---------------------------------------------------------------- head with fused greedy pick
-__global__ void argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows,
-                                     const int* __restrict__ dyn) {
-  // one wave per row: maximum over the 64 slots, which are cleared for the next call
-  const int b = blockIdx.x, lane = threadIdx.x;
+__global__ void __launch_bounds__(1024)
+argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride, int rows, int* dyn, int advance) {
+  // one workgroup, one wave per row: maximum over the 64 slots, which are cleared for the next call; with
+  // `advance` the position/step counters are bumped once every row has used them
+  const int b = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = dyn ? dyn[0] : 0;
+  __syncthreads();
+  if (threadIdx.x == 0 && dyn && advance) { dyn[0] = pos + 1; dyn[1] += 1; }
+  if (b >= rows) return;
   unsigned long long k = best[(size_t)b * 64 + lane];
   best[(size_t)b * 64 + lane] = 0ull;
 #pragma unroll
@@ -314,18 +319,18 @@ __global__ void argmax_finish_kernel(unsigned long long* best, int64_t* tok_out,
     unsigned long long t = __shfl_xor(k, o, FSTU_WAVE);
     k = t > k ? t : k;
   }
-  if (lane == 0) tok_out[(size_t)b * stride + (dyn ? dyn[0] : 0)] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
+  if (lane == 0) tok_out[(size_t)b * stride + pos] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
 }
 
 extern "C" int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                                 float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
                                 void* stream) {
-  return fstu_head_argmax_dyn(x, ldx, W, logits, ldy, rows, N, K, temperature, best_ws, tok_out, tok_stride, nullptr, dtype,
-                              stream);
+  return fstu_head_argmax_dyn(x, ldx, W, logits, ldy, rows, N, K, temperature, best_ws, tok_out, tok_stride, nullptr, 0,
+                              dtype, stream);
 }
 
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
-                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, const int* dyn,
+                         float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream) {
   int rc = check_common("fstu_head_argmax", x, W, logits, ldx, rows, N, K);
   if (rc) return rc;
@@ -335,13 +340,15 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   if (dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1)) {
     LinArgs a{x, ldx, W, nullptr, logits, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
     launch_mfma<LIN_ARGMAX>(a, 1, (hipStream_t)stream);
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
-                       tok_out, tok_stride, rows, dyn);
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(rows * 64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
+                       tok_out, tok_stride, rows, dyn, advance);
     FSTU_CHECK_LAUNCH("fstu_head_argmax");
     return FSTU_OK;
   }
   rc = fstu_linear_decode(x, ldx, W, logits, ldy, rows, N, K, dtype, stream);
   if (rc) return rc;
   FSTU_REQUIRE(ldy == N, FSTU_ESHAPE, "fstu_head_argmax: this dtype/shape needs dense logits (ldy == N)");
-  return fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, dyn, dtype, stream);
+  rc = fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, dyn, dtype, stream);
+  if (rc == 0 && dyn && advance) rc = fstu_advance_dyn(dyn, stream);
+  return rc;
 }

@@ -52,8 +52,10 @@ SIGNATURES = {
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
     "fstu_decode_graph_destroy": [_vp],
+    "fstu_set_warm_workgroups": [_i],
     "fstu_prof_begin": [_i, _i],
     "fstu_prof_end": [_vp, _vp],
+    "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
 

@@ -43,6 +43,9 @@ class ModelDesc(ctypes.Structure):
 def pick_ksplit_down(I: int) -> int:
     """K split of the down projection: enough waves to fill 256 CUs while every
     slice still divides into the 64-wide k steps of the MFMA kernel."""
+    forced = int(os.environ.get("FSTU_KSPLIT_DOWN", "0"))
+    if forced > 0 and I % (forced * 64) == 0:
+        return forced
     for ks in (12, 16, 8, 6, 4, 3, 2):
         if I % (ks * 256) == 0:
             return ks

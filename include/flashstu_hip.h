@@ -354,6 +354,10 @@ int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t 
                              float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                              void* stream, void** graph_out);
 int fstu_decode_graph_launch(void* graph, void* stream);
+/* The captured graph carries a parallel branch whose kernels only read the MLP / head weights a layer is about
+ * to need (cache warm-up; `n` workgroups per kernel; default 0 = no such branch, which measured faster).  Applies to graphs created
+ * afterwards. */
+int fstu_set_warm_workgroups(int n);
 int fstu_decode_graph_destroy(void* graph);
 
 /* ---- live kernel timing (measurement aid; no counterpart in the reference) ----
@@ -366,6 +370,9 @@ int fstu_decode_graph_destroy(void* graph);
  * QKV, 7 embed/add/RMSNorm, 8 sampling.  Not thread-safe. */
 int fstu_prof_begin(int kernel_class, int max_launches);
 int fstu_prof_end(double* total_ms, int* launches);
+/* The gate/up GLU projection (fstu_glu_decode) of every layer of `m`, `reps` times back to back on `stream`
+ * between two HIP events; returns the elapsed time and launch count.  Synchronises on the second event. */
+int fstu_prof_glu_loop(const fstu_model_desc* m, int reps, double* total_ms, int* launches, void* stream);
 
 #ifdef __cplusplus
 }
