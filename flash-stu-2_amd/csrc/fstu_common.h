@@ -44,7 +44,7 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
 int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table, void* x, const void* w, void* h, int rows,
                        int d, int vocab, float eps, int dtype, void* stream, const int* dyn);
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
-                    float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream);
+                    float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
                              int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream);

@@ -332,7 +332,7 @@ __device__ __forceinline__ double block_excl_scan_d(double v, double* red, doubl
 template <typename T>
 __global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
 sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
-              int top_k, float top_p, int do_sample, uint64_t seed, int step, const int* __restrict__ dyn) {
+              int top_k, float top_p, int do_sample, uint64_t seed, int step, int row0, const int* __restrict__ dyn) {
   __shared__ SampleShared sh;
   const int b = blockIdx.x;
   if (dyn) { out += dyn[0]; step = dyn[1]; }
@@ -494,7 +494,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   double mybase = block_excl_scan_d(mysum, sh.redd, &Z);
   // counter-based uniform (splitmix64 finaliser), 24 bits
   unsigned long long z = seed * 0x9E3779B97F4A7C15ull + (unsigned long long)step * 0xBF58476D1CE4E5B9ull +
-                         (unsigned long long)b * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
+                         (unsigned long long)(b + row0) * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
   z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
   z = z ^ (z >> 31);
@@ -541,12 +541,12 @@ int fstu_advance_dyn(int* dyn, void* stream) {
 extern "C" int fstu_sample(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature,
                            int top_k, float top_p, int do_sample, uint64_t seed, int step, int dtype,
                            void* stream) {
-  return fstu_sample_dyn(logits, out, out_stride, B, V, temperature, top_k, top_p, do_sample, seed, step, nullptr, dtype,
+  return fstu_sample_dyn(logits, out, out_stride, B, V, temperature, top_k, top_p, do_sample, seed, step, 0, nullptr, dtype,
                          stream);
 }
 
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
-                    float top_p, int do_sample, uint64_t seed, int step, const int* dyn, int dtype, void* stream) {
+                    float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream) {
   FSTU_REQUIRE(logits && out, FSTU_ENULL, "fstu_sample: null pointer");
   FSTU_REQUIRE(B >= 0 && V > 0, FSTU_ESHAPE, "fstu_sample: bad shape B=%d V=%d", B, V);
   FSTU_REQUIRE(temperature > 0.f, FSTU_EARG, "fstu_sample: temperature must be > 0");
@@ -555,7 +555,7 @@ int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B,
   FSTU_DISPATCH_DTYPE(dtype, "fstu_sample",
                       hipLaunchKernelGGL(sample_kernel<T>, dim3(B), dim3(FSTU_SAMPLE_THREADS), 0, (hipStream_t)stream,
                                          (const T*)logits, out, out_stride, V, temperature, top_k, top_p, do_sample,
-                                         seed, step, dyn));
+                                         seed, step, row0, dyn));
   FSTU_CHECK_LAUNCH("fstu_sample");
   return FSTU_OK;
 }

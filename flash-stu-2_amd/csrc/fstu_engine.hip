@@ -210,7 +210,7 @@ static int decode_step_fused(const fstu_model_desc* m, const int64_t* tok_in, in
     hd.mode = 0;
     pro(hd, m->final_norm_w);
     TIMED(PC_HEAD, fstu_gemv_packed_dyn(&hd, dyn, 0, stream));
-    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dyn, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));
     if (dyn) STEP(fstu_advance_dyn(dyn, stream));
   }
   return FSTU_OK;
@@ -291,7 +291,7 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                                         tok_stride, dyn, 1, dt, stream));
   } else {
     TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
-    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, dyn, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));
     if (dyn) STEP(fstu_advance_dyn(dyn, stream));
   }
   warm_join_all((hipStream_t)stream);

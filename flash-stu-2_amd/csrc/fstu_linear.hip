@@ -348,7 +348,7 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   rc = fstu_linear_decode(x, ldx, W, logits, ldy, rows, N, K, dtype, stream);
   if (rc) return rc;
   FSTU_REQUIRE(ldy == N, FSTU_ESHAPE, "fstu_head_argmax: this dtype/shape needs dense logits (ldy == N)");
-  rc = fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, dyn, dtype, stream);
+  rc = fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, 0, dyn, dtype, stream);
   if (rc == 0 && dyn && advance) rc = fstu_advance_dyn(dyn, stream);
   return rc;
 }

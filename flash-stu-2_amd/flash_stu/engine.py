@@ -1,11 +1,15 @@
 """Decode engine behind FlashSTU.generate(): prefill through the module path,
 then one C-ABI call per token (fstu_decode_step) that launches the fused kernel
-sequence for the whole layer stack against preallocated state and workspaces.
+sequence for the whole layer stack against preallocated state and workspaces,
+or the same step captured once as a HIP graph and replayed per token.
 
 The token buffer (B, max_length) lives on the GPU for the whole loop; each step
 reads column pos and writes column pos+1, so the host never sees a token until
 generate() returns (reference loop: flash_stu/model.py:245-302, which re-allocates
 the sequence with torch.cat every step).
+
+The decode kernels take at most 16 activation rows; a larger batch runs as
+consecutive row chunks of 16 against the same weights and batch-first state.
 """
 from __future__ import annotations
 
@@ -33,7 +37,7 @@ class LayerDesc(ctypes.Structure):
 class ModelDesc(ctypes.Structure):
     _fields_ = [("dtype", _i), ("B", _i), ("d", _i), ("I", _i), ("V", _i), ("n_layers", _i), ("n_heads", _i),
                 ("head_dim", _i), ("window", _i), ("kv_cap", _i), ("L", _i), ("hist_cap", _i), ("stu_mode", _i),
-                ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i),
+                ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i), ("row0", _i),
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
@@ -55,6 +59,19 @@ def pick_ksplit_down(I: int) -> int:
     return 1
 
 
+class _Chunk:
+    """Descriptor, workspaces and graph handle of one chunk of at most 16 batch rows."""
+
+    def __init__(self, b0: int, b1: int):
+        self.b0, self.b1 = b0, b1
+        self.keep: List[torch.Tensor] = []
+        self.arr = None
+        self.desc: Optional[ModelDesc] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.graph = None
+        self.dyn: Optional[torch.Tensor] = None
+
+
 class DecodeEngine:
     HIST_NSPLIT_MAX = 16
 
@@ -65,9 +82,9 @@ class DecodeEngine:
         self.model = model
         self.cfg = cfg
         self.lib = _hip.load()
-        self._keep: List[torch.Tensor] = []
-        self._graph = None
+        self.chunks: List[_Chunk] = []
         self._packed = {}
+        self._gstream = None
 
     # ------------------------------------------------------------------
     def _pack(self, w: torch.Tensor) -> torch.Tensor:
@@ -87,18 +104,49 @@ class DecodeEngine:
         return (cfg.torch_dtype == torch.bfloat16 and cfg.resolved_stu_decode_mode() == "lds" and d % 128 == 0
                 and I % (128 * pick_ksplit_down(I)) == 0 and B * (d + 8) * 2 + 8192 <= 64 * 1024)
 
+    @property
+    def desc(self) -> ModelDesc:
+        """Descriptor of the first row chunk (the whole batch when B <= 16)."""
+        return self.chunks[0].desc
+
+    @property
+    def logits(self) -> torch.Tensor:
+        """(B,V) logits of the last eager step."""
+        return self.chunks[0].logits if len(self.chunks) == 1 else torch.cat([c.logits for c in self.chunks], 0)
+
     def _build(self, caches, B: int, total_len: int):
+        cfg = self.cfg
+        d = cfg.n_embd
+        mode = cfg.resolved_stu_decode_mode()
+        caches = list(caches)
+        if mode != "lds":                      # history buffers must hold the whole generation
+            for i, layer in enumerate(self.model.layers):
+                if isinstance(layer, STULayer):
+                    hist, state, pos = caches[i]
+                    if hist.shape[1] < total_len:
+                        bigger = hist.new_zeros(B, total_len, d)
+                        bigger[:, : hist.shape[1]] = hist
+                        caches[i] = (bigger, state, pos)
+        self.graph_end()
+        self.chunks = []
+        for b0 in range(0, B, _hip.MAX_DECODE_ROWS):
+            ch = _Chunk(b0, min(B, b0 + _hip.MAX_DECODE_ROWS))
+            self._build_chunk(ch, caches)
+            self.chunks.append(ch)
+        return tuple(caches)
+
+    def _build_chunk(self, ch: _Chunk, caches):
         model, cfg = self.model, self.cfg
         dev = model.lm_head.weight.device
         dt = cfg.torch_dtype
         d, I, V = cfg.n_embd, cfg.n_embd * cfg.mlp_scale, cfg.vocab_size
         mode = cfg.resolved_stu_decode_mode()
-        self._keep = []
-        keep = self._keep.append
+        b0, b1 = ch.b0, ch.b1
+        B = b1 - b0
+        keep = ch.keep.append
         n = len(model.layers)
         arr = (LayerDesc * n)()
         hist_cap = 0
-        new_caches = list(caches)
         for i, layer in enumerate(model.layers):
             ld = arr[i]
             ld.w_gate = layer.mlp.gate_proj.weight.data_ptr()
@@ -115,20 +163,17 @@ class DecodeEngine:
                 hist, state, pos = caches[i]
                 if mode == "lds":
                     a, ce = stu.lds_params()
-                    keep(a), keep(ce), keep(state)
-                    ld.lds_a, ld.lds_ce, ld.lds_state = a.data_ptr(), ce.data_ptr(), state.data_ptr()
+                    st = state[b0:b1]
+                    keep(a), keep(ce), keep(st)
+                    ld.lds_a, ld.lds_ce, ld.lds_state = a.data_ptr(), ce.data_ptr(), st.data_ptr()
                 else:
-                    if hist.shape[1] < total_len:
-                        bigger = hist.new_zeros(B, total_len, d)
-                        bigger[:, : hist.shape[1]] = hist
-                        hist = bigger
-                        new_caches[i] = (hist, state, pos)
-                    if hist_cap and hist.shape[1] != hist_cap:
+                    hs = hist[b0:b1]
+                    if hist_cap and hs.shape[1] != hist_cap:
                         raise RuntimeError("STU histories must share one capacity")
-                    hist_cap = hist.shape[1]
+                    hist_cap = hs.shape[1]
                     filt = stu.effective_filter()
-                    keep(filt), keep(hist)
-                    ld.filt, ld.hist = filt.data_ptr(), hist.data_ptr()
+                    keep(filt), keep(hs)
+                    ld.filt, ld.hist = filt.data_ptr(), hs.data_ptr()
             elif isinstance(layer, AttentionLayer):
                 att = layer.attn
                 ld.kind = 1
@@ -136,6 +181,7 @@ class DecodeEngine:
                 ld.w_qkv = att.c_attn.weight.data_ptr()
                 ld.w_proj = att.c_proj.weight.data_ptr()
                 kr, vr, pos = caches[i]
+                kr, vr = kr[b0:b1], vr[b0:b1]
                 keep(kr), keep(vr)
                 ld.kring, ld.vring = kr.data_ptr(), vr.data_ptr()
                 ld.slopes = att.alibi_slopes.data_ptr()
@@ -152,6 +198,7 @@ class DecodeEngine:
         m.single_branch = int(cfg.use_hankel_L)
         m.ksplit_down = pick_ksplit_down(I) if dt == torch.bfloat16 else min(8, max(1, I // 512))
         m.hist_nsplit_max = self.HIST_NSPLIT_MAX
+        m.row0 = b0
         m.eps, m.softcap = float(cfg.rms_norm_eps), float(cfg.softcap or 0.0)
         m.emb = model.lm_head.weight.data_ptr()
         m.final_norm_w = model.norm.weight.data_ptr()
@@ -161,15 +208,14 @@ class DecodeEngine:
             t = torch.zeros(*shape, dtype=dtype, device=dev)
             keep(t)
             return t
-        self.x, self.h = buf(B, d), buf(B, d)
-        self.logits = buf(B, V)
-        m.x, m.h = self.x.data_ptr(), self.h.data_ptr()
+        ch.logits = buf(B, V)
+        m.x, m.h = buf(B, d).data_ptr(), buf(B, d).data_ptr()
         m.qkv, m.attn = buf(B, 3 * d).data_ptr(), buf(B, d).data_ptr()
         m.act, m.xp, m.y = buf(B, I).data_ptr(), buf(B, d).data_ptr(), buf(B, d).data_ptr()
         m.partial = buf(m.ksplit_down, B, d, dtype=torch.float32).data_ptr()
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
-        m.logits = self.logits.data_ptr()
-        m.best = buf(max(B, 16) * 64, dtype=torch.int64).data_ptr()
+        m.logits = ch.logits.data_ptr()
+        m.best = buf(16 * 64, dtype=torch.int64).data_ptr()
         if self._use_packed(B):
             for i, layer in enumerate(model.layers):
                 ld = arr[i]
@@ -185,54 +231,63 @@ class DecodeEngine:
             m.x2, m.yd = buf(B, d).data_ptr(), buf(B, d).data_ptr()
             m.partial_fix = buf(m.ksplit_down * ((d + 15) // 16) * 256, dtype=torch.float32).data_ptr()
             m.counters = buf((d + 15) // 16, dtype=torch.int32).data_ptr()
-        self._arr, self.desc = arr, m
-        return tuple(new_caches)
+        ch.arr, ch.desc = arr, m
 
+    # ------------------------------------------------------------------ eager step
     def step(self, tokens: torch.Tensor, pos: int, temperature, top_k, top_p, do_sample, seed, step_idx):
         """Feeds tokens[:, pos], writes the sampled id to tokens[:, pos+1]."""
-        rc = self.lib.fstu_decode_step(ctypes.byref(self.desc), tokens.data_ptr() + 8 * pos,
-                                       tokens.data_ptr() + 8 * (pos + 1), tokens.stride(0), pos, float(temperature),
-                                       int(top_k) if top_k else 0, float(top_p) if top_p else 0.0, int(bool(do_sample)),
-                                       int(seed) & ((1 << 64) - 1), int(step_idx),
-                                       torch.cuda.current_stream().cuda_stream)
-        _hip._check(rc, "fstu_decode_step")
+        stride = tokens.stride(0)
+        for ch in self.chunks:
+            base = tokens.data_ptr() + 8 * (ch.b0 * stride + pos)
+            rc = self.lib.fstu_decode_step(ctypes.byref(ch.desc), base, base + 8, stride, pos, float(temperature),
+                                           int(top_k) if top_k else 0, float(top_p) if top_p else 0.0,
+                                           int(bool(do_sample)), int(seed) & ((1 << 64) - 1), int(step_idx),
+                                           torch.cuda.current_stream().cuda_stream)
+            _hip._check(rc, "fstu_decode_step")
 
     # ------------------------------------------------------------------ graph replay
     def graph_supported(self) -> bool:
         return self.cfg.resolved_stu_decode_mode() == "lds"
 
     def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed):
-        """Captures one decode step as a HIP graph on a side stream.  Each graph_step() then feeds
-        tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
+        """Captures one decode step per row chunk as a HIP graph on a side stream.  Each graph_step() then
+        feeds tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
         self.graph_end()
-        self._dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
         self._gstream = torch.cuda.Stream(device=tokens.device)
         self._gstream.wait_stream(torch.cuda.current_stream())
-        handle = _vp()
-        rc = self.lib.fstu_decode_graph_create(ctypes.byref(self.desc), tokens.data_ptr(), tokens.stride(0),
-                                               self._dyn.data_ptr(), float(temperature), int(top_k) if top_k else 0,
-                                               float(top_p) if top_p else 0.0, int(bool(do_sample)),
-                                               int(seed) & ((1 << 64) - 1), self._gstream.cuda_stream,
-                                               ctypes.byref(handle))
-        _hip._check(rc, "fstu_decode_graph_create")
-        self._graph = handle
+        stride = tokens.stride(0)
+        for ch in self.chunks:
+            ch.dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
+        self._gstream.wait_stream(torch.cuda.current_stream())
+        for ch in self.chunks:
+            handle = _vp()
+            rc = self.lib.fstu_decode_graph_create(ctypes.byref(ch.desc), tokens.data_ptr() + 8 * ch.b0 * stride, stride,
+                                                   ch.dyn.data_ptr(), float(temperature), int(top_k) if top_k else 0,
+                                                   float(top_p) if top_p else 0.0, int(bool(do_sample)),
+                                                   int(seed) & ((1 << 64) - 1), self._gstream.cuda_stream,
+                                                   ctypes.byref(handle))
+            _hip._check(rc, "fstu_decode_graph_create")
+            ch.graph = handle
         self._graph_tokens = tokens
 
     def graph_step(self):
-        _hip._check(self.lib.fstu_decode_graph_launch(self._graph, self._gstream.cuda_stream), "fstu_decode_graph_launch")
+        for ch in self.chunks:
+            _hip._check(self.lib.fstu_decode_graph_launch(ch.graph, self._gstream.cuda_stream), "fstu_decode_graph_launch")
 
     def graph_end(self):
-        if self._graph is not None:
+        live = [ch for ch in self.chunks if ch.graph is not None]
+        if live:
             torch.cuda.current_stream().wait_stream(self._gstream)
             self._gstream.synchronize()
-            self.lib.fstu_decode_graph_destroy(self._graph)
-            self._graph = None
+            for ch in live:
+                self.lib.fstu_decode_graph_destroy(ch.graph)
+                ch.graph = None
 
     # ------------------------------------------------------------------
     @torch.no_grad()
     def prefill(self, input_ids: torch.Tensor, total_len: int):
         """Runs the prompt through the module path with caches, returns the
-        logits of the last position (B,V) and prepares the step descriptor."""
+        logits of the last position (B,V) and prepares the step descriptors."""
         model = self.model
         B, P = input_ids.shape
         x = model._embed(input_ids.contiguous())
@@ -248,8 +303,6 @@ class DecodeEngine:
         if not input_ids.is_cuda:
             raise _hip.FlashSTUHipError("input_ids must be on the GPU: this model has no CPU path")
         B, P = input_ids.shape
-        if B > _hip.MAX_DECODE_ROWS:
-            raise _hip.FlashSTUHipError(f"batch {B} exceeds the decode kernels' limit of {_hip.MAX_DECODE_ROWS} rows")
         total = P + n_new
         if self.cfg.resolved_stu_decode_mode() == "history" and total > self.cfg.seq_len:
             raise ValueError(f"history-mode decode needs prompt+new tokens ({total}) <= seq_len ({self.cfg.seq_len})")

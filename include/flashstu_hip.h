@@ -312,6 +312,7 @@ typedef struct {
   int single_branch;        /* use_hankel_L */
   int ksplit_down;          /* K split of the down projection (partial holds ksplit_down*B*d floats) */
   int hist_nsplit_max;      /* eo holds hist_nsplit_max*2*B*d floats */
+  int row0;                 /* index of this descriptor's first row in the caller's batch (keys the sampling stream) */
   float eps, softcap;
   const void* emb;          /* (V,d) tied embedding / head */
   const void* final_norm_w; /* (d) */

@@ -130,7 +130,7 @@ def test_c5_shape_sampling_parity_reduced():
     from test_gpu_model import make_pair, prompt
     ocfg, w, model = make_pair(seed=2, init="healthy", mlp_scale=2, n_embd=256, n_layers=4, n_heads=2, window_size=24,
                                num_eigh=24, seq_len=256, vocab_size=2003)
-    ids = prompt(16, 20, ocfg.vocab_size, 4)
+    ids = prompt(32, 20, ocfg.vocab_size, 4)          # batch 32 as in config 5: two row chunks of 16
     ref = O.generate(w, ocfg, ids, max_length=52, temperature=0.8, top_k=40, do_sample=True, mode="stateful", seed=2)
     got = model.generate(ids.cuda(), max_length=52, temperature=0.8, top_k=40, do_sample=True, seed=2)
     assert torch.equal(got.cpu(), ref)
@@ -143,8 +143,10 @@ def test_c5_shape_bf16_lds_teacher_forced():
                                n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
                                stu_decode_mode="lds")
     P, N = 20, 60
-    ids = prompt(16, P, ocfg.vocab_size, 4)
+    ids = prompt(20, P, ocfg.vocab_size, 4)           # 16 + 4 rows
     got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
+    again = model.generate(ids.cuda(), max_length=P + N, do_sample=False)        # graph replay, chunked
+    assert torch.equal(again, got)
     ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
     err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
     assert float(err.max()) <= 2e-2
