@@ -251,9 +251,15 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   // x = embedding rows, h = norm(x) with the first layer's norm weight
   TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt,
                                     stream, dyn));
+  // The residual stream starts in m->x.  Where a layer has packed gate/up weights, its MLP norm runs as the
+  // prologue of the GLU GEMV, which writes the updated residual to the other buffer (xc <-> xo swap).
+  void* xc = m->x;
+  void* xo = m->x2;
+  const bool glu_pro = dt == FSTU_BF16 && xo != nullptr && d % 128 == 0 && (size_t)B * (d + 8) * 2 + 16384 <= 64 * 1024;
   const size_t wsz = (dt == FSTU_BF16) ? 2 : 4;
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
+    bool pending_y = false;   // m->y holds a sub-layer output not yet added to the residual stream
     // warm this layer's MLP weights while its (latency-bound) STU / attention sub-layer runs
     warm_fork((hipStream_t)stream, L.w_gate, (size_t)I * d * wsz, L.w_up, (size_t)I * d * wsz, L.w_down, (size_t)I * d * wsz);
     if (l == m->n_layers - 1) warm_fork((hipStream_t)stream, m->emb, (size_t)m->V * d * wsz, nullptr, 0, nullptr, 0);
@@ -263,7 +269,7 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, row, m->hist_cap * d, B, d, d, dt, stream));
         int ns = hist_nsplit(pos + 1, m->hist_nsplit_max);
         TIMED(PC_STU, fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
-        TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+        TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
         if (dt == FSTU_BF16 && d % 256 == 0) {
           TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y, d, nullptr, B,
@@ -272,19 +278,28 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
           TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
           TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
         }
-        TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+        pending_y = true;
       }
     } else {
       TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
                                          m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
       TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
-      TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+      pending_y = true;
     }
-    TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
+    if (pending_y && glu_pro && L.wp_gate && L.wp_up) {
+      fstu_gemv_args u = {};
+      u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
+      u.res_in = xc; u.delta = m->y; u.res_out = xo; u.norm_w = L.mlp_norm_w; u.eps = m->eps;
+      TIMED(PC_GLU, fstu_gemv_packed_dyn(&u, dyn, 0, stream));
+      void* t = xc; xc = xo; xo = t;
+    } else {
+      if (pending_y) TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+      TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
+    }
     TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
-    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
+    TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
   if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,

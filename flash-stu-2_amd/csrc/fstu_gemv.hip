@@ -59,6 +59,14 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
   }
 
   if (PRO) {
+    // norm weights of this lane's column chunks: fetched now so that their latency hides behind the first barrier
+    const bf16_t* nw = (const bf16_t*)a.norm_w;
+    uint4 nwv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int c = lane * 8 + k * 512;
+      nwv[k] = (c < a.K) ? *(const uint4*)(nw + c) : make_uint4(0, 0, 0, 0);
+    }
     // ---- x_new = res_in + delta -> LDS (and res_out), 8 elements per thread and iteration
     const int nchunk = a.K >> 3;
     const int total = a.rows * nchunk;
@@ -83,7 +91,6 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
     }
     __syncthreads();
     // ---- one wave per row: statistics in a fixed order, normalise in place (16-byte LDS accesses)
-    const bf16_t* nw = (const bf16_t*)a.norm_w;
     for (int row = w; row < a.rows; row += 4) {
       bf16_t* hr = hs + (size_t)row * hs_ld;
       float ss = 0.f;
@@ -99,9 +106,8 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
       }
       ss = wave_sum(ss);
       const float rstd = rsqrtf(ss / (float)a.K + a.eps);
-      for (int c = lane * 8; c < a.K; c += 512) {
+      auto scale_chunk = [&](int c, uint4 wv) {
         uint4 v = *(const uint4*)(hr + c);
-        uint4 wv = *(const uint4*)(nw + c);
         unsigned vw[4] = {v.x, v.y, v.z, v.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -110,7 +116,13 @@ gemv_packed_kernel(fstu_gemv_args a, int kw /*k per wave*/, int hs_ld /*LDS row 
           vw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
         }
         *(uint4*)(hr + c) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+      };
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int c = lane * 8 + k * 512;
+        if (c < a.K) scale_chunk(c, nwv[k]);
       }
+      for (int c = lane * 8 + 2048; c < a.K; c += 512) scale_chunk(c, *(const uint4*)(nw + c));
     }
     __syncthreads();
   }

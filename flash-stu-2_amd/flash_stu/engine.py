@@ -216,6 +216,14 @@ class DecodeEngine:
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = ch.logits.data_ptr()
         m.best = buf(16 * 64, dtype=torch.int64).data_ptr()
+        if (dt == torch.bfloat16 and d % 128 == 0 and B * (d + 8) * 2 + 16384 <= 64 * 1024
+                and os.environ.get("FSTU_GLU_PROLOGUE", "0") == "1"):
+            # experimental: MLP norm fused into the GLU GEMV (packed gate/up copies + a second residual buffer);
+            # measured slower than the separate norm kernel (0.494 vs 0.475 ms per step), hence off by default
+            for i, layer in enumerate(model.layers):
+                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
+                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
+            m.x2 = buf(B, d).data_ptr()
         if self._use_packed(B):
             for i, layer in enumerate(model.layers):
                 ld = arr[i]

@@ -105,7 +105,7 @@ def test_c2_dims_bf16_teacher_forced(mode, init):
     ocfg, w, model = make_pair(seed=1, init=init, dtype=torch.bfloat16, mlp_scale=4, n_embd=768, n_layers=12,
                                n_heads=12, window_size=512, num_eigh=24, seq_len=2048, vocab_size=50257,
                                stu_decode_mode=mode)
-    B, P, N = 2, 40, 40
+    B, P, N = 4, 40, 88          # 352 scored tokens
     ids = prompt(B, P, ocfg.vocab_size, 3)
     got, got_logits = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
     got, got_logits = got.cpu(), got_logits.float().cpu()
