@@ -1,0 +1,418 @@
+// Spectral convolution of the STU prefill as the reference computes it (rfft -> product -> irfft,
+// flash_stu/utils/stu_utils.py:195-246), as in-LDS complex FFTs on gfx950.
+//
+// One workgroup transforms `cols` whole columns (one (batch, channel) signal each) that live in LDS from the
+// first load to the last store: forward decimation-in-frequency passes (natural order in, digit-reversed order
+// out), a pointwise product with a filter spectrum stored in that same digit-reversed order, and the mirrored
+// decimation-in-time passes back to natural order.  No bit-reversal pass is ever needed.  A pass is a radix-16
+// (first pass: 2, 4, 8 or 16) butterfly held in registers, so a length-4096 transform touches LDS three times.
+//
+// Both sign branches come out of ONE inverse transform: with F the filter's spectrum, the minus branch
+// conv(x, (-1)^s f) has spectrum F[k + n/2], so the product X * (F[k] + i F[k + n/2]) inverts to
+// plus + i*minus (both real).  k + n/2 sits at digit-reversed position p ^ 8 because the last pass has radix 16.
+#include "fstu_common.h"
+
+namespace {
+
+typedef float2 cpx;
+
+__device__ __forceinline__ cpx cadd(cpx a, cpx b) { return make_float2(a.x + b.x, a.y + b.y); }
+__device__ __forceinline__ cpx csub(cpx a, cpx b) { return make_float2(a.x - b.x, a.y - b.y); }
+__device__ __forceinline__ cpx cmul(cpx a, cpx b) {
+  return make_float2(fmaf(a.x, b.x, -a.y * b.y), fmaf(a.x, b.y, a.y * b.x));
+}
+// a * conj(b)
+__device__ __forceinline__ cpx cmulc(cpx a, cpx b) {
+  return make_float2(fmaf(a.x, b.x, a.y * b.y), fmaf(a.y, b.x, -a.x * b.y));
+}
+__device__ __forceinline__ cpx cconj(cpx a) { return make_float2(a.x, -a.y); }
+
+// LDS index of element i of a column: one pad slot every 16 elements keeps the stride-16 accesses of the
+// last pass (and every other power-of-two stride) off a single bank.
+__device__ __forceinline__ int phys(int i) { return i + (i >> 4); }
+
+// z * exp(-2 pi i k / 16), k = 0..7, k known at compile time after unrolling
+__device__ __forceinline__ cpx mul_root16(cpx z, int k) {
+  const float s = 0.70710678118654752f, c1 = 0.92387953251128674f, s1 = 0.38268343236508977f;
+  switch (k) {
+    case 0: return z;
+    case 1: return make_float2(fmaf(c1, z.x, s1 * z.y), fmaf(c1, z.y, -s1 * z.x));
+    case 2: return make_float2((z.x + z.y) * s, (z.y - z.x) * s);
+    case 3: return make_float2(fmaf(s1, z.x, c1 * z.y), fmaf(s1, z.y, -c1 * z.x));
+    case 4: return make_float2(z.y, -z.x);
+    case 5: return make_float2(fmaf(-s1, z.x, c1 * z.y), fmaf(-s1, z.y, -c1 * z.x));
+    case 6: return make_float2((z.y - z.x) * s, -(z.x + z.y) * s);
+    default: return make_float2(fmaf(-c1, z.x, s1 * z.y), fmaf(-c1, z.y, -s1 * z.x));
+  }
+}
+
+template <int R> __device__ __forceinline__ constexpr int brev(int k) {
+  int r = 0;
+  for (int b = 1; b < R; b <<= 1) {
+    r = (r << 1) | (k & 1);
+    k >>= 1;
+  }
+  return r;
+}
+
+// In-register DFT of R points (R = 2, 4, 8, 16): input v[m] in natural order, output k left in v[brev(k)].
+template <int R> __device__ __forceinline__ void dft_inreg(cpx (&v)[R]) {
+#pragma unroll
+  for (int h = R / 2; h >= 1; h >>= 1) {
+#pragma unroll
+    for (int b0 = 0; b0 < R; b0 += 2 * h) {
+#pragma unroll
+      for (int j = 0; j < h; ++j) {
+        cpx a = v[b0 + j], b = v[b0 + j + h];
+        v[b0 + j] = cadd(a, b);
+        v[b0 + j + h] = mul_root16(csub(a, b), j * (8 / h));
+      }
+    }
+  }
+}
+
+// powers 1..R-1 of w = tw[r*ts] : the binary powers come from the table, the rest are products of two of them
+template <int R> __device__ __forceinline__ void twiddle_powers(cpx (&pw)[R], const cpx* __restrict__ tw, int e) {
+  pw[0] = make_float2(1.f, 0.f);
+  pw[1] = tw[e];
+  if (R >= 4) {
+    pw[2] = tw[2 * e];
+    pw[3] = cmul(pw[1], pw[2]);
+  }
+  if (R >= 8) {
+    pw[4] = tw[4 * e];
+    pw[5] = cmul(pw[4], pw[1]);
+    pw[6] = cmul(pw[4], pw[2]);
+    pw[7] = cmul(pw[4], pw[3]);
+  }
+  if (R >= 16) {
+    pw[8] = tw[8 * e];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) pw[8 + k] = cmul(pw[8], pw[k]);
+  }
+}
+
+// One radix-R butterfly of a pass over blocks of Nb = R*q elements (q = 1 << lq).  Forward: decimation in
+// frequency, y[k] = w^(r k) * sum_m x[m] W_R^(m k) written where x was read.  Inverse: the exact mirror.
+template <int R, bool INV>
+__device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __restrict__ tw, int u, int lq, int ts) {
+  const int q = 1 << lq;
+  const int r = u & (q - 1);
+  const int base = ((u >> lq) * R << lq) + r;
+  cpx v[R], pw[R];
+  const bool twid = lq > 0;
+  if (twid) twiddle_powers<R>(pw, tw, r * ts);
+  if (!INV) {
+#pragma unroll
+    for (int m = 0; m < R; ++m) v[m] = col[phys(base + (m << lq))];
+    dft_inreg<R>(v);
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+      cpx o = v[brev<R>(k)];
+      if (twid && k > 0) o = cmul(o, pw[k]);
+      col[phys(base + (k << lq))] = o;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+      cpx o = col[phys(base + (k << lq))];
+      if (twid && k > 0) o = cmulc(o, pw[k]);
+      v[k] = cconj(o);
+    }
+    dft_inreg<R>(v);
+#pragma unroll
+    for (int m = 0; m < R; ++m) col[phys(base + (m << lq))] = cconj(v[brev<R>(m)]);
+  }
+}
+
+template <int R, bool INV, int NT>
+__device__ __forceinline__ void run_pass(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn,
+                                         int lNb) {
+  constexpr int LR = (R == 16) ? 4 : (R == 8) ? 3 : (R == 4) ? 2 : 1;
+  const int lq = lNb - LR;           // log2 of the butterfly stride
+  const int lper = logn - LR;        // log2 of butterflies per column
+  const int ts = 1 << (logn - lNb);  // table stride: w_Nb = tw[ts]
+  const int total = cols << lper;
+  for (int w = threadIdx.x; w < total; w += NT) {
+    const int colid = w >> lper;
+    butterfly<R, INV>(lds + (size_t)colid * colstride, tw, w & ((1 << lper) - 1), lq, ts);
+  }
+  __syncthreads();
+}
+
+// logn = 4*a + rem: the first forward pass has radix 2^rem (if rem > 0), every other pass radix 16.
+template <int NT>
+__device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn) {
+  int lNb = logn;
+  const int rem = logn & 3;
+  if (rem == 1) run_pass<2, false, NT>(lds, tw, cols, colstride, logn, lNb);
+  if (rem == 2) run_pass<4, false, NT>(lds, tw, cols, colstride, logn, lNb);
+  if (rem == 3) run_pass<8, false, NT>(lds, tw, cols, colstride, logn, lNb);
+  lNb -= rem;
+  for (; lNb >= 4; lNb -= 4) run_pass<16, false, NT>(lds, tw, cols, colstride, logn, lNb);
+}
+
+template <int NT>
+__device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn) {
+  const int rem = logn & 3;
+  for (int lNb = 4; lNb <= logn - rem; lNb += 4) run_pass<16, true, NT>(lds, tw, cols, colstride, logn, lNb);
+  if (rem == 1) run_pass<2, true, NT>(lds, tw, cols, colstride, logn, logn);
+  if (rem == 2) run_pass<4, true, NT>(lds, tw, cols, colstride, logn, logn);
+  if (rem == 3) run_pass<8, true, NT>(lds, tw, cols, colstride, logn, logn);
+}
+
+// ---------------------------------------------------------------- twiddle table
+__global__ void fft_twiddle_kernel(cpx* __restrict__ tw, int n) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= n) return;
+  double s, c;
+  sincospi(-2.0 * (double)j / (double)n, &s, &c);
+  tw[j] = make_float2((float)c, (float)s);
+}
+
+// ---------------------------------------------------------------- filter spectra
+// Column j of the filter matrix (element (s, j) at filt[s*f_ls + j*f_cs], taps s < taps) -> spec[j*n + p] =
+// (F[p] + i F[p^8]) / n (both branches) or F[p] / n, p running over the digit-reversed positions.
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT)
+fft_filter_kernel(const T* __restrict__ filt, size_t f_ls, size_t f_cs, cpx* __restrict__ spec,
+                  const cpx* __restrict__ tw, int taps, int ncol_total, int n, int logn, int lcols, int both) {
+  extern __shared__ cpx fft_lds[];
+  const int cols = 1 << lcols;
+  const int colstride = n + (n >> 4);
+  const int c0 = blockIdx.x * cols;
+  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+    const int colid = idx & (cols - 1), s = idx >> lcols;
+    float v = 0.f;
+    if (s < taps && c0 + colid < ncol_total) v = DT<T>::ld(filt + (size_t)s * f_ls + (size_t)(c0 + colid) * f_cs);
+    fft_lds[(size_t)colid * colstride + phys(s)] = make_float2(v, 0.f);
+  }
+  __syncthreads();
+  fft_forward<NT>(fft_lds, tw, cols, colstride, logn);
+  const float inv_n = 1.0f / (float)n;
+  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+    const int colid = idx >> logn, p = idx & (n - 1);
+    if (c0 + colid >= ncol_total) continue;
+    const cpx* col = fft_lds + (size_t)colid * colstride;
+    cpx f = col[phys(p)];
+    if (both) {
+      const cpx g = col[phys(p ^ 8)];
+      f = make_float2(f.x - g.y, f.y + g.x);
+    }
+    spec[(size_t)(c0 + colid) * n + p] = make_float2(f.x * inv_n, f.y * inv_n);
+  }
+}
+
+// ---------------------------------------------------------------- convolution
+// x element (b, t, c) at x[b*x_sb + t*x_st + c*x_sc]; the K outputs of channel c (K = 1: per-channel spectra
+// spec[c]; K > 1: a shared bank spec[k]) go to y[b*y_sb + t*y_st + k*y_sk + c*y_sc] (and y2 likewise).
+// mode 0: y = T(T(re) + T(im));  mode 1: y = T(re);  mode 2: y = T(re), y2 = T(im).
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT)
+fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, const cpx* __restrict__ spec,
+                T* __restrict__ y, T* __restrict__ y2, size_t y_sb, size_t y_st, size_t y_sk, size_t y_sc,
+                const cpx* __restrict__ tw, int Tn, int d, int K, int n, int logn, int lcols, int mode, int xcd_remap) {
+  extern __shared__ cpx fft_lds[];
+  const int cols = 1 << lcols;
+  const int colstride = n + (n >> 4);
+  int bx = blockIdx.x;
+  if (xcd_remap) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);   // consecutive channel groups share an XCD
+  const int c0 = bx * cols;
+  const int b = blockIdx.y;
+  const int ncol = min(cols, d - c0);
+  const T* xb = x + (size_t)b * x_sb + (size_t)c0 * x_sc;
+  const bool t_fast = x_st == 1;   // time-major input: walk t with the lanes
+
+  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+    int colid, t;
+    if (t_fast) { colid = idx >> logn; t = idx & (n - 1); } else { colid = idx & (cols - 1); t = idx >> lcols; }
+    float v = 0.f;
+    if (t < Tn && colid < ncol) v = DT<T>::ld(xb + (size_t)t * x_st + (size_t)colid * x_sc);
+    fft_lds[(size_t)colid * colstride + phys(t)] = make_float2(v, 0.f);
+  }
+  __syncthreads();
+  fft_forward<NT>(fft_lds, tw, cols, colstride, logn);
+
+  const bool yt_fast = y_st == 1;
+  if (K == 1) {
+    for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+      const int colid = idx >> logn, p = idx & (n - 1);
+      if (colid >= ncol) continue;
+      cpx* e = fft_lds + (size_t)colid * colstride + phys(p);
+      *e = cmul(*e, spec[(size_t)(c0 + colid) * n + p]);
+    }
+    __syncthreads();
+    fft_inverse<NT>(fft_lds, tw, cols, colstride, logn);
+    T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc;
+    T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc : nullptr;
+    for (int idx = threadIdx.x; idx < cols * Tn; idx += NT) {
+      int colid, t;
+      if (yt_fast) { colid = idx / Tn; t = idx - colid * Tn; } else { colid = idx & (cols - 1); t = idx >> lcols; }
+      if (colid >= ncol) continue;
+      const cpx z = fft_lds[(size_t)colid * colstride + phys(t)];
+      const size_t o = (size_t)t * y_st + (size_t)colid * y_sc;
+      if (mode == 0) DT<T>::st(yb + o, DT<T>::rnd(z.x) + DT<T>::rnd(z.y));
+      else {
+        DT<T>::st(yb + o, z.x);
+        if (mode == 2) DT<T>::st(yb2 + o, z.y);
+      }
+    }
+    return;
+  }
+
+  // filter bank: keep the spectrum of the single column in registers and run one inverse per filter
+  constexpr int MAXE = 16;
+  cpx xs[MAXE];
+  const int ept = (n + NT - 1) / NT;   // host guarantees ept <= MAXE and cols == 1
+#pragma unroll
+  for (int j = 0; j < MAXE; ++j)
+    if (j < ept) {
+      const int p = threadIdx.x + j * NT;
+      xs[j] = (p < n) ? fft_lds[phys(p)] : make_float2(0.f, 0.f);
+    }
+  __syncthreads();
+  for (int k = 0; k < K; ++k) {
+    const cpx* sk = spec + (size_t)k * n;
+#pragma unroll
+    for (int j = 0; j < MAXE; ++j)
+      if (j < ept) {
+        const int p = threadIdx.x + j * NT;
+        if (p < n) fft_lds[phys(p)] = cmul(xs[j], sk[p]);
+      }
+    __syncthreads();
+    fft_inverse<NT>(fft_lds, tw, 1, colstride, logn);
+    T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk;
+    T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk : nullptr;
+    for (int t = threadIdx.x; t < Tn; t += NT) {
+      const cpx z = fft_lds[phys(t)];
+      const size_t o = (size_t)t * y_st;
+      if (mode == 0) DT<T>::st(yb + o, DT<T>::rnd(z.x) + DT<T>::rnd(z.y));
+      else {
+        DT<T>::st(yb + o, z.x);
+        if (mode == 2) DT<T>::st(yb2 + o, z.y);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+int ilog2_exact(int n) {
+  int l = 0;
+  while ((1 << l) < n) ++l;
+  return ((1 << l) == n) ? l : -1;
+}
+
+// columns per workgroup and threads per workgroup for a transform length
+void fft_shape(int logn, int ncol_total, int* lcols, int* nt) {
+  int lc = 12 - logn;           // cols * n = 4096 complex elements = 34 KB of LDS
+  if (lc < 0) lc = 0;
+  if (lc > 4) lc = 4;
+  while (lc > 0 && (1 << lc) > ncol_total) --lc;
+  *lcols = lc;
+  *nt = (logn >= 14) ? 1024 : (logn == 13 ? 512 : 256);
+}
+
+size_t fft_lds_bytes(int n, int lcols) { return (size_t)(n + (n >> 4)) * sizeof(cpx) << lcols; }
+
+template <typename K> int allow_lds(K kernel, size_t bytes, const char* name) {
+  if (bytes <= 48 * 1024) return 0;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)bytes);
+  if (e != hipSuccess) {
+    fstu_set_error("%s: %zu bytes of LDS refused: %s", name, bytes, hipGetErrorString(e));
+    return (int)e;
+  }
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int fstu_fft_length(int T_) {
+  int n = 64;
+  while (n < 2 * T_ && n < (1 << 14)) n <<= 1;
+  return (n >= 2 * T_) ? n : 0;
+}
+
+extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
+  FSTU_REQUIRE(tw, FSTU_ENULL, "fstu_fft_twiddles: null pointer");
+  const int logn = ilog2_exact(n);
+  FSTU_REQUIRE(logn >= 6 && logn <= 14, FSTU_ESHAPE, "fstu_fft_twiddles: n=%d is not a power of two in 64..16384", n);
+  hipLaunchKernelGGL(fft_twiddle_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, (cpx*)tw, n);
+  FSTU_CHECK_LAUNCH("fstu_fft_twiddles");
+  return FSTU_OK;
+}
+
+#define FFT_LAUNCH_NT(NTV, KERNEL, GRID, SHM, NAME, ...)                                             \
+  do {                                                                                               \
+    int rc__ = allow_lds(KERNEL<T, NTV>, SHM, NAME);                                                 \
+    if (rc__) return rc__;                                                                           \
+    hipLaunchKernelGGL((KERNEL<T, NTV>), GRID, dim3(NTV), SHM, (hipStream_t)stream, __VA_ARGS__);    \
+  } while (0)
+
+#define FFT_LAUNCH(NT, KERNEL, GRID, SHM, NAME, ...)                                  \
+  do {                                                                                \
+    if ((NT) == 1024) FFT_LAUNCH_NT(1024, KERNEL, GRID, SHM, NAME, __VA_ARGS__);      \
+    else if ((NT) == 512) FFT_LAUNCH_NT(512, KERNEL, GRID, SHM, NAME, __VA_ARGS__);   \
+    else FFT_LAUNCH_NT(256, KERNEL, GRID, SHM, NAME, __VA_ARGS__);                    \
+  } while (0)
+
+extern "C" int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs, float* spec, const float* tw, int taps,
+                                   int ncols, int n, int single_branch, int dtype, void* stream) {
+  FSTU_REQUIRE(filt && spec && tw, FSTU_ENULL, "fstu_stu_fft_filter: null pointer");
+  const int logn = ilog2_exact(n);
+  FSTU_REQUIRE(logn >= 6 && logn <= 14, FSTU_ESHAPE, "fstu_stu_fft_filter: n=%d is not a power of two in 64..16384", n);
+  FSTU_REQUIRE(taps >= 1 && 2 * taps <= n && ncols >= 1, FSTU_ESHAPE,
+               "fstu_stu_fft_filter: taps=%d must satisfy 1 <= taps <= n/2=%d (ncols=%d)", taps, n / 2, ncols);
+  FSTU_REQUIRE(fstu_aligned(spec, 8) && fstu_aligned(tw, 8), FSTU_EALIGN, "fstu_stu_fft_filter: spec/tw must be 8-byte aligned");
+  int lcols, nt;
+  fft_shape(logn, ncols, &lcols, &nt);
+  const size_t shm = fft_lds_bytes(n, lcols);
+  dim3 grid((ncols + (1 << lcols) - 1) >> lcols);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_fft_filter",
+                      FFT_LAUNCH(nt, fft_filter_kernel, grid, shm, "fstu_stu_fft_filter", (const T*)filt, (size_t)f_ls,
+                                 (size_t)f_cs, (cpx*)spec, (const cpx*)tw, taps, ncols, n, logn, lcols,
+                                 single_branch ? 0 : 1));
+  FSTU_CHECK_LAUNCH("fstu_stu_fft_filter");
+  return FSTU_OK;
+}
+
+static int conv_fft_launch(const char* name, const void* x, int64_t x_sb, int64_t x_st, int64_t x_sc, const float* spec,
+                           void* y, void* y2, int64_t y_sb, int64_t y_st, int64_t y_sk, int64_t y_sc, const float* tw,
+                           int B, int T_, int d, int K, int n, int mode, int dtype, void* stream) {
+  const int logn = ilog2_exact(n);
+  FSTU_REQUIRE(logn >= 6 && logn <= 14, FSTU_ESHAPE, "%s: n=%d is not a power of two in 64..16384", name, n);
+  FSTU_REQUIRE(B >= 1 && B <= 65535 && T_ >= 1 && d >= 1 && K >= 1 && 2 * T_ <= n, FSTU_ESHAPE,
+               "%s: bad shape B=%d T=%d d=%d K=%d n=%d (n >= 2T required)", name, B, T_, d, K, n);
+  FSTU_REQUIRE(fstu_aligned(spec, 8) && fstu_aligned(tw, 8), FSTU_EALIGN, "%s: spec/tw must be 8-byte aligned", name);
+  int lcols, nt;
+  fft_shape(logn, d, &lcols, &nt);
+  if (K > 1) lcols = 0;
+  FSTU_REQUIRE(K == 1 || (n + nt - 1) / nt <= 16, FSTU_ESHAPE, "%s: n=%d too long for the bank form", name, n);
+  const size_t shm = fft_lds_bytes(n, lcols);
+  const int gx = (d + (1 << lcols) - 1) >> lcols;
+  dim3 grid(gx, B);
+  const int remap = (gx % 8 == 0) ? 1 : 0;
+  FSTU_DISPATCH_DTYPE(dtype, name,
+                      FFT_LAUNCH(nt, fft_conv_kernel, grid, shm, name, (const T*)x, (size_t)x_sb, (size_t)x_st,
+                                 (size_t)x_sc, (const cpx*)spec, (T*)y, (T*)y2, (size_t)y_sb, (size_t)y_st, (size_t)y_sk,
+                                 (size_t)y_sc, (const cpx*)tw, T_, d, K, n, logn, lcols, mode, remap));
+  FSTU_CHECK_LAUNCH(name);
+  return FSTU_OK;
+}
+
+extern "C" int fstu_stu_conv_fft(const void* xp, const float* spec, void* y, const float* tw, int B, int T_, int d, int n,
+                                 int single_branch, int dtype, void* stream) {
+  FSTU_REQUIRE(xp && spec && y && tw, FSTU_ENULL, "fstu_stu_conv_fft: null pointer");
+  return conv_fft_launch("fstu_stu_conv_fft", xp, (int64_t)T_ * d, d, 1, spec, y, nullptr, (int64_t)T_ * d, d, 0, 1, tw, B,
+                         T_, d, 1, n, single_branch ? 1 : 0, dtype, stream);
+}
+
+extern "C" int fstu_stu_conv_bank_fft(const void* x, const int64_t* x_strides, const float* spec, void* u_plus,
+                                      void* u_minus, const int64_t* u_strides, const float* tw, int B, int T_, int d,
+                                      int K, int n, int dtype, void* stream) {
+  FSTU_REQUIRE(x && x_strides && spec && u_plus && u_strides && tw, FSTU_ENULL, "fstu_stu_conv_bank_fft: null pointer");
+  FSTU_REQUIRE(K >= 2, FSTU_ESHAPE, "fstu_stu_conv_bank_fft: K=%d (a bank has at least two filters)", K);
+  return conv_fft_launch("fstu_stu_conv_bank_fft", x, x_strides[0], x_strides[1], x_strides[2], spec, u_plus, u_minus,
+                         u_strides[0], u_strides[1], u_strides[2], u_strides[3], tw, B, T_, d, K, n, u_minus ? 2 : 1,
+                         dtype, stream);
+}

@@ -37,6 +37,11 @@ SIGNATURES = {
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_fft_length": [_i],
+    "fstu_fft_twiddles": [_vp, _i, _vp],
+    "fstu_stu_fft_filter": [_vp, _i64, _i64, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_conv_fft": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_conv_bank_fft": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_append": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -285,6 +290,75 @@ def stu_conv_direct(xp: torch.Tensor, filt: torch.Tensor, single_branch: bool = 
     _check(load().fstu_stu_conv_direct(_p(xp), _p(filt), _p(out), B, T, d, L, int(single_branch), _dt(xp), _stream()),
            "fstu_stu_conv_direct")
     return out
+
+
+def fft_length(T: int) -> int:
+    """Smallest supported transform length (power of two, 64..16384) with n >= 2T; 0 if T is too long."""
+    return int(load().fstu_fft_length(int(T)))
+
+
+_twiddle_cache = {}
+
+
+def fft_twiddles(n: int, device) -> torch.Tensor:
+    """exp(-2 pi i j / n) as (n, 2) fp32 on `device`, built once per (n, device)."""
+    key = (int(n), torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device())
+    tw = _twiddle_cache.get(key)
+    if tw is None:
+        tw = torch.empty(n, 2, dtype=torch.float32, device=device)
+        _check(load().fstu_fft_twiddles(_p(tw), n, _stream()), "fstu_fft_twiddles")
+        _twiddle_cache[key] = tw
+    return tw
+
+
+def stu_fft_filter(filt: torch.Tensor, n: int, taps: Optional[int] = None, single_branch: bool = False) -> torch.Tensor:
+    """Spectra (ncols, n, 2) fp32 of the columns of filt (L, ncols), cut to `taps` <= n/2 taps."""
+    _dev(filt)
+    L, ncols = filt.shape
+    taps = min(L, n // 2) if taps is None else int(taps)
+    if not 1 <= taps <= min(L, n // 2):
+        raise FlashSTUHipError(f"taps={taps} outside 1..min(L={L}, n/2={n // 2})")
+    spec = torch.empty(ncols, n, 2, dtype=torch.float32, device=filt.device)
+    _check(load().fstu_stu_fft_filter(_p(filt), ncols, 1, _p(spec), _p(fft_twiddles(n, filt.device)), taps, ncols, n,
+                                      int(single_branch), _dt(filt), _stream()), "fstu_stu_fft_filter")
+    return spec
+
+
+def stu_conv_fft(xp: torch.Tensor, spec: torch.Tensor, single_branch: bool = False,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """xp (B,T,d) convolved with the per-channel spectra spec (d,n,2) of stu_fft_filter (same single_branch)."""
+    _dev(xp, spec, out)
+    B, T, d = xp.shape
+    n = spec.shape[1]
+    if spec.shape != (d, n, 2) or spec.dtype != torch.float32:
+        raise FlashSTUHipError(f"spec must be ({d}, n, 2) float32, got {tuple(spec.shape)} {spec.dtype}")
+    if out is None:
+        out = torch.empty_like(xp)
+    _check(load().fstu_stu_conv_fft(_p(xp), _p(spec), _p(out), _p(fft_twiddles(n, xp.device)), B, T, d, n,
+                                    int(single_branch), _dt(xp), _stream()), "fstu_stu_conv_fft")
+    return out
+
+
+def stu_conv_bank_fft(x: torch.Tensor, spec: torch.Tensor, u_plus: torch.Tensor, u_minus: Optional[torch.Tensor]):
+    """x: any strided view of logical shape (B,T,d); spec (K,n,2); u_plus/u_minus: strided views of logical shape
+    (B,T,K,d), written in place.  A time stride of 1 makes the stores coalesce."""
+    for t in (x, spec, u_plus, u_minus):
+        if t is not None and not t.is_cuda:
+            raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    B, T, d = x.shape
+    K, n = spec.shape[0], spec.shape[1]
+    if not spec.is_contiguous() or spec.dtype != torch.float32 or spec.shape[2] != 2:
+        raise FlashSTUHipError("spec must be contiguous (K, n, 2) float32")
+    if tuple(u_plus.shape) != (B, T, K, d) or u_plus.dtype != x.dtype:
+        raise FlashSTUHipError(f"u_plus must have logical shape {(B, T, K, d)} and x's dtype")
+    if u_minus is not None and (tuple(u_minus.shape) != (B, T, K, d) or u_minus.stride() != u_plus.stride()
+                                or u_minus.dtype != x.dtype):
+        raise FlashSTUHipError("u_minus must match u_plus in shape, strides and dtype")
+    xs = (ctypes.c_int64 * 3)(*x.stride())
+    us = (ctypes.c_int64 * 4)(*u_plus.stride())
+    _check(load().fstu_stu_conv_bank_fft(_p(x), xs, _p(spec), _p(u_plus), _p(u_minus), us,
+                                         _p(fft_twiddles(n, x.device)), B, T, d, K, n, _dt(x), _stream()),
+           "fstu_stu_conv_bank_fft")
 
 
 def stu_conv_bank(x: torch.Tensor, phi: torch.Tensor, u_plus: torch.Tensor, u_minus: Optional[torch.Tensor]):

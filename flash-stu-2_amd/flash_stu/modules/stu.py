@@ -24,6 +24,9 @@ from .. import _hip
 from ..utils.lds_fit import fit_even_lag_lds
 
 
+FFT_MIN_T = 32     # shorter inputs take the time-domain kernel (a 64-point transform would be mostly padding)
+
+
 class STU(nn.Module):
     def __init__(self, config, phi: torch.Tensor, n: int, feature_dim: Optional[int] = None) -> None:
         super().__init__()
@@ -65,6 +68,16 @@ class STU(nn.Module):
         return self._cached("filt", (self.phi, self.M_filters),
                             lambda: torch.matmul(self.phi, self.M_filters).contiguous())
 
+    def filter_spectrum(self, n: int) -> torch.Tensor:
+        """Spectra of the convolution filters for transform length n, (d,n,2) fp32 in approx mode, (K,n,2) in
+        exact mode (the reference keeps its own phi_fft the same way, stu.py:43-53).  One length is kept."""
+        src = self.effective_filter() if self.use_approx else self.phi
+        params = (self.phi, self.M_filters) if self.use_approx else (self.phi,)
+        hit = self._derived.get("spec")
+        if hit is not None and hit[1].shape[1] != n:
+            self._derived.pop("spec")
+        return self._cached("spec", params, lambda: _hip.stu_fft_filter(src, n, single_branch=self.use_hankel_L))
+
     def m_inputs_t(self) -> torch.Tensor:
         return self._cached("mit", (self.M_inputs,), lambda: self.M_inputs.t().contiguous())
 
@@ -92,19 +105,41 @@ class STU(nn.Module):
             return _hip.linear_decode(x.reshape(B * T, d), self.m_inputs_t()).reshape(B, T, self.d_out)
         return torch.matmul(x, self.M_inputs)
 
+    def _convolve(self, xp: torch.Tensor) -> torch.Tensor:
+        """Approx-mode convolution of the projected inputs with phi_proj (stu.py:89-98,120): the FFT form of
+        the reference from FFT_MIN_T positions on, the time-domain kernel for shorter inputs and for lengths
+        beyond the longest in-LDS transform."""
+        T = xp.shape[1]
+        n = _hip.fft_length(T) if T >= FFT_MIN_T else 0
+        if n == 0:
+            return _hip.stu_conv_direct(xp, self.effective_filter(), single_branch=self.use_hankel_L)
+        return _hip.stu_conv_fft(xp, self.filter_spectrum(n), single_branch=self.use_hankel_L)
+
     def _exact_sequence(self, x: torch.Tensor) -> torch.Tensor:
-        """use_approx=False: U+-[b,t,k,i] by the time-domain kernel, one filter at a
-        time, then the (K*d_in, d_out) contractions as library GEMMs with the
-        reference's rounding points (stu.py:107-120)."""
+        """use_approx=False: U+-[b,t,k,i] for the whole filter bank (one forward transform per channel, one
+        inverse per filter), then the (K*d_in, d_out) contractions as library GEMMs with the reference's
+        rounding points (stu.py:107-120).  The FFT form writes U time-major, (B, K*d, T), which the GEMM
+        consumes as a transposed operand; x is never expanded K-fold."""
         B, T, d = x.shape
-        Up = torch.empty(B, T, self.K, d, dtype=x.dtype, device=x.device)
-        Um = None if self.use_hankel_L else torch.empty_like(Up)
-        _hip.stu_conv_bank(x, self.phi, Up, Um)
         wp, wm = self.exact_flat_weights()
-        y = torch.matmul(Up.reshape(B * T, self.K * d), wp)
+        n = _hip.fft_length(T) if T >= FFT_MIN_T else 0
+        if n == 0:
+            Up = torch.empty(B, T, self.K, d, dtype=x.dtype, device=x.device)
+            Um = None if self.use_hankel_L else torch.empty_like(Up)
+            _hip.stu_conv_bank(x, self.phi, Up, Um)
+            y = torch.matmul(Up.reshape(B * T, self.K * d), wp)
+            if Um is not None:
+                y = y + torch.matmul(Um.reshape(B * T, self.K * d), wm)
+            return y.reshape(B, T, self.d_out)
+        Up = torch.empty(B, self.K, d, T, dtype=x.dtype, device=x.device)
+        Um = None if self.use_hankel_L else torch.empty_like(Up)
+        xt = x.transpose(1, 2).contiguous().transpose(1, 2)            # time-major copy: coalesced column loads
+        _hip.stu_conv_bank_fft(xt, self.filter_spectrum(n), Up.permute(0, 3, 1, 2),
+                               None if Um is None else Um.permute(0, 3, 1, 2))
+        y = torch.matmul(Up.reshape(B, self.K * d, T).transpose(1, 2), wp)
         if Um is not None:
-            y = y + torch.matmul(Um.reshape(B * T, self.K * d), wm)
-        return y.reshape(B, T, self.d_out)
+            y = y + torch.matmul(Um.reshape(B, self.K * d, T).transpose(1, 2), wm)
+        return y
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor, past_state=None, use_cache: bool = False):
@@ -118,7 +153,7 @@ class STU(nn.Module):
                 raise ValueError(f"sequence length {T} exceeds the filter length {self.phi.shape[0]}")
             if self.use_approx:
                 xp = self._project(x)
-                y = _hip.stu_conv_direct(xp, self.effective_filter(), single_branch=self.use_hankel_L)
+                y = self._convolve(xp)
                 hist_src = xp
             else:
                 y = self._exact_sequence(x)

@@ -150,6 +150,42 @@ int fstu_stu_conv_direct(const void* xp, const void* filt, void* y, int B, int T
 int fstu_stu_conv_bank(const void* x, const void* phi, void* u_plus, void* u_minus, int B, int T, int d,
                        int L, int K, int dtype, void* stream);
 
+/* ---- STU prefill convolution, FFT form --------------------------------------
+ * The reference's own algorithm: rfft of length n, product with the filter's
+ * spectrum, irfft, first T outputs kept (flash_stu/utils/stu_utils.py:195-246).
+ * Here n is any power of two in 64..16384 with n >= 2T (fstu_fft_length gives the
+ * smallest; a circular convolution of that length never wraps into the first T
+ * outputs, so the result equals the reference's n = 2^ceil(log2(2L-1))), filters
+ * are cut to their first min(L, n/2) taps, and both sign branches come out of one
+ * complex inverse transform per channel.
+ *
+ * fstu_fft_twiddles fills tw (n complex fp32 = 2n floats) with exp(-2 pi i j / n).
+ * fstu_stu_fft_filter transforms ncols filter columns (element (s, j) at
+ *   filt[s*f_ls + j*f_cs], taps s < taps <= n/2) into spec (ncols, n) complex fp32,
+ *   scaled by 1/n, in the transform's internal frequency order; with
+ *   single_branch == 0 the spectrum of the (-1)^s branch is folded in as the
+ *   imaginary companion.  Approx mode: columns = channels of phi_proj (f_ls = d,
+ *   f_cs = 1); exact mode: columns = the K filters of phi (f_ls = K, f_cs = 1).
+ *   Replaces the rfft of v at stu_utils.py:213-214 / the cached phi_fft of
+ *   flash_stu/modules/stu.py:43-53.
+ * fstu_stu_conv_fft: y[b,t,c] = T( T(plus) + T(minus) ) (or T(plus) if
+ *   single_branch) for xp, y (B,T,d) and spec (d, n) made with the same n, tw and
+ *   single_branch.  Same contract as fstu_stu_conv_direct.
+ * fstu_stu_conv_bank_fft: the exact-mode bank, spec (K, n).  x_strides = element
+ *   strides {batch, time, channel} of x; u_strides = {batch, time, filter, channel}
+ *   of u_plus / u_minus (u_minus may be NULL).  A time stride of 1 (time-major
+ *   outputs, the transposed operand of the following contraction) gives fully
+ *   coalesced stores.  Same values as fstu_stu_conv_bank. */
+int fstu_fft_length(int T);
+int fstu_fft_twiddles(float* tw, int n, void* stream);
+int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs, float* spec, const float* tw, int taps,
+                        int ncols, int n, int single_branch, int dtype, void* stream);
+int fstu_stu_conv_fft(const void* xp, const float* spec, void* y, const float* tw, int B, int T, int d, int n,
+                      int single_branch, int dtype, void* stream);
+int fstu_stu_conv_bank_fft(const void* x, const int64_t* x_strides, const float* spec, void* u_plus, void* u_minus,
+                           const int64_t* u_strides, const float* tw, int B, int T, int d, int K, int n, int dtype,
+                           void* stream);
+
 /* ---- sliding-window attention ----------------------------------------------
  * KV ring layout: (B,H,cap,hd), absolute position j lives in slot j % cap,
  * cap >= window+1.

@@ -1,6 +1,7 @@
 """BASELINE configs 3, 4 and 5 on the GPU: parity against the CPU oracle at sizes
 the oracle finishes in seconds, plus size-independent properties at the full
 BASELINE sizes (linearity, causality, delta response, state carry)."""
+import functools
 import math
 
 import pytest
@@ -19,11 +20,17 @@ def hip():
 
 
 # ----------------------------------------------------------------- config 3
+@functools.lru_cache(maxsize=4)
+def _filters(L, K, dtype):
+    """The Hankel filters, computed once per test session (the L=8192 eigendecomposition takes a while)."""
+    return O.get_spectral_filters(L, K, dtype=dtype)
+
+
 def _exact_stu(dtype, d, L, K, seed):
     from flash_stu import STU, FlashSTUConfig
     cfg = FlashSTUConfig(n_embd=d, n_heads=1, n_layers=1, seq_len=L, num_eigh=K, use_approx=False, torch_dtype=dtype,
                          vocab_size=3)
-    phi = O.get_spectral_filters(L, K, dtype=dtype)
+    phi = _filters(L, K, dtype)
     g = torch.Generator().manual_seed(seed)
     stu = STU(cfg, phi, O.nearest_power_of_two(2 * L - 1, True))
     with torch.no_grad():
@@ -51,7 +58,7 @@ def test_c3_full_size_properties(hip):
     are linear in the input."""
     B, L, d, K = 4, 8192, 1024, 24
     dtype = torch.bfloat16
-    phi = O.get_spectral_filters(L, K, dtype=dtype).cuda()
+    phi = _filters(L, K, dtype).cuda()
     x = torch.zeros(B, L, d, dtype=dtype, device="cuda")
     x[0, 0, :] = 1.0                      # delta at t=0
     x[1, 100, 5] = 2.0                    # delayed, scaled delta in one channel
@@ -74,6 +81,53 @@ def test_c3_full_size_properties(hip):
     t, k, c = 6000, 11, 321
     ref = (phi[: t + 1, k].double().flip(0) * x[2, : t + 1, c].double()).sum()
     assert abs(float(Up[2, t, k, c]) - float(ref)) <= 2.0 ** -7 * abs(float(ref)) + 1e-6
+
+
+def test_c3_full_size_fft_bank_matches_time_domain(hip):
+    """B=4, L=8192, d=1024, K=24, bf16: the FFT bank (transform length 16384, time-major outputs) against the
+    time-domain bank kernel on the same input: at most one bf16 ulp apart, on few elements."""
+    B, L, d, K = 4, 8192, 1024, 24
+    dtype = torch.bfloat16
+    phi = _filters(L, K, dtype).cuda()
+    x = torch.randn(B, L, d, generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    Ud = torch.empty(B, L, K, d, dtype=dtype, device="cuda")
+    hip.stu_conv_bank(x, phi, Ud, None)
+    n = hip.fft_length(L)
+    assert n == 16384
+    Uf = torch.empty(B, K, d, L, dtype=dtype, device="cuda")
+    hip.stu_conv_bank_fft(x, hip.stu_fft_filter(phi, n), Uf.permute(0, 3, 1, 2), None)
+    torch.cuda.synchronize()
+    for b in range(B):                                   # compare batch by batch to bound the fp32 temporaries
+        a, r = Uf[b].permute(2, 0, 1).float(), Ud[b].float()
+        diff = (a - r).abs()
+        assert bool((diff <= r.abs() * 2.0 ** -7 + 1e-6).all())
+        assert float((diff > 0).float().mean()) < 0.02
+
+
+def test_c3_full_size_exact_mode_delta_response():
+    """The whole exact-mode operator at the BASELINE shape (FFT bank + contraction): a unit impulse in channel i
+    returns y[t] = T(T(phi[t] @ M+[:, i]) + T((-1)^t phi[t] @ M-[:, i])), and batch rows do not mix."""
+    dtype = torch.bfloat16
+    d, L, K = 1024, 8192, 24
+    stu, phi, p = _exact_stu(dtype, d, L, K, 7)
+    x = torch.zeros(4, L, d, dtype=dtype)
+    x[1, 0, 17] = 1.0
+    x[3, 5, 900] = 1.0
+    y = stu(x.cuda()).float().cpu()
+    sg = torch.ones(L, 1)
+    sg[1::2] = -1
+    for b, t0, i in ((1, 0, 17), (3, 5, 900)):
+        plus = (phi.float() @ p["M_phi_plus"][:, i, :].float()).to(dtype).float()
+        minus = ((phi.float() * sg) @ p["M_phi_minus"][:, i, :].float()).to(dtype).float()
+        ref = (plus + minus).to(dtype).float()[: L - t0]
+        got = y[b, t0:]
+        scale = float(ref.abs().max())
+        diff = (got - ref).abs()
+        assert float(diff.max()) <= 2.0 ** -6 * scale
+        assert float((diff > 0).float().mean()) < 0.05
+        if t0:
+            assert float(y[b, :t0].abs().max()) <= 1e-3 * scale
+    assert float(y[0].abs().max()) == 0.0 and float(y[2].abs().max()) == 0.0
 
 
 # ----------------------------------------------------------------- config 4

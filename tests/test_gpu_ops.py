@@ -204,6 +204,73 @@ def test_stu_conv_direct(hip, dtype, B, T, d, L):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d,L", [(2, 100, 96, 128), (1, 64, 256, 1024), (3, 120, 100, 128), (2, 17, 5, 64),
+                                     (2, 512, 64, 512), (1, 1000, 48, 1024), (1, 2048, 32, 2048), (1, 4096, 8, 4096),
+                                     (1, 3000, 4, 8192), (1, 8192, 2, 8192)])
+def test_stu_conv_fft(hip, dtype, B, T, d, L):
+    """The FFT form against the oracle's rfft/irfft convolution, every transform length 64..16384
+    (radix splits 4*16, 8*16, 16*16, 2*16*16 ... 4*16*16*16), ragged channel counts, T < L and T == L."""
+    if L <= 1024:
+        xp, filt, ref, plus = _stu_setup(dtype, B, T, d, L, 8, 6)
+    else:                                  # no eigendecomposition of a large Hankel matrix in a GPU test
+        g = gen(6)
+        filt = (torch.randn(L, d, generator=g) * torch.linspace(1, 0.02, L)[:, None] / 8).to(dtype)
+        xp = torch.randn(B, T, d, generator=g).to(dtype)
+        plus, minus = O.convolve(xp, filt, O.nearest_power_of_two(2 * L - 1, True), use_approx=True)
+        ref = plus + minus
+    n = hip.fft_length(T)
+    assert n >= 2 * T and (n == 64 or n < 4 * T)
+    atol = 2.0 ** -7 * float(plus.float().abs().max()) if dtype == torch.bfloat16 else 0.0
+    spec = hip.stu_fft_filter(dev(filt), n)
+    check(hip.stu_conv_fft(dev(xp), spec), ref, dtype, frac=0.05, atol=atol)
+    spec1 = hip.stu_fft_filter(dev(filt), n, single_branch=True)
+    check(hip.stu_conv_fft(dev(xp), spec1, single_branch=True), plus, dtype, frac=0.05)
+
+
+def test_stu_conv_fft_equals_direct_fp32(hip):
+    """Both forms of the library on the same input: equal to fp32 round-off, and a delta returns the filter."""
+    g = gen(21)
+    B, T, d, L = 2, 700, 40, 1024
+    filt = (torch.randn(L, d, generator=g) * torch.linspace(1, 0.01, L)[:, None]).float()
+    xp = torch.randn(B, T, d, generator=g)
+    xp[1] = 0
+    xp[1, 3, :] = 1.0
+    n = hip.fft_length(T)
+    yf = hip.stu_conv_fft(dev(xp), hip.stu_fft_filter(dev(filt), n, single_branch=True), single_branch=True).cpu()
+    yd = hip.stu_conv_direct(dev(xp), dev(filt), single_branch=True).cpu()
+    s = float(yd.abs().max())
+    assert float((yf - yd).abs().max()) <= 5e-6 * s
+    assert float((yf[1, 3:] - filt[: T - 3]).abs().max()) <= 5e-6 * float(filt.abs().max())
+    assert float(yf[1, :3].abs().max()) <= 5e-6 * float(filt.abs().max())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d,L,K", [(2, 100, 24, 128, 5), (1, 600, 6, 1024, 24), (1, 5000, 2, 8192, 3)])
+def test_stu_conv_bank_fft(hip, dtype, B, T, d, L, K):
+    """Exact-mode bank by FFT == the time-domain bank kernel == the oracle's convolve(use_approx=False),
+    in the (B,T,K,d) layout and in the time-major layout the contraction consumes."""
+    g = gen(22)
+    phi = O.get_spectral_filters(L, K, dtype=dtype) if L <= 1024 else \
+        (torch.randn(L, K, generator=g) * torch.linspace(1, 0.01, L)[:, None]).to(dtype)
+    x = torch.randn(B, T, d, generator=g).to(dtype)
+    n_ref = O.nearest_power_of_two(2 * L - 1, True)
+    rp, rm = O.convolve(x, phi, n_ref, use_approx=False)
+    n = hip.fft_length(T)
+    spec = hip.stu_fft_filter(dev(phi), n)
+    up = torch.empty(B, T, K, d, dtype=dtype, device="cuda")
+    um = torch.empty_like(up)
+    hip.stu_conv_bank_fft(dev(x), spec, up, um)
+    sc = float(rp.float().abs().max())
+    check(up, rp, dtype, frac=0.05, scale=sc)
+    check(um, rm, dtype, frac=0.05, scale=sc)
+    # time-major outputs (B,K,d,T) viewed as (B,T,K,d), time-major input
+    upt = torch.empty(B, K, d, T, dtype=dtype, device="cuda")
+    xt = dev(x).transpose(1, 2).contiguous().transpose(1, 2)
+    hip.stu_conv_bank_fft(xt, spec, upt.permute(0, 3, 1, 2), None)
+    assert torch.equal(upt.permute(0, 3, 1, 2), up)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("B,T,d,L,nsplit", [(2, 100, 96, 128, 3), (8, 257, 768, 512, 4), (1, 50, 100, 64, 1),
                                              (2, 128, 2048, 128, 2)])  # T <= L: the reference's FFT length assumes it
 def test_stu_step_hist(hip, dtype, B, T, d, L, nsplit):
