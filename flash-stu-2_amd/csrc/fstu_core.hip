@@ -273,6 +273,34 @@ extern "C" int fstu_gelu_mul(const void* g, const void* u, void* act, int64_t n,
   return FSTU_OK;
 }
 
+// ---------------------------------------------------------------- bias + activation
+// y[r,c] = act( T(y[r,c] + bias[c]) ), act = identity or x*sigmoid(x); bias may be null
+template <typename T>
+__global__ void bias_act_kernel(T* __restrict__ y, const T* __restrict__ bias, int64_t rows, int n, int kind) {
+  const int64_t total = rows * n;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    float v = DT<T>::ld(y + i);
+    if (bias) v = DT<T>::rnd(v + DT<T>::ld(bias + (i % n)));
+    if (kind == 1) v = v / (1.0f + expf(-v));
+    DT<T>::st(y + i, v);
+  }
+}
+
+extern "C" int fstu_bias_act(void* y, const void* bias, int64_t rows, int n, int kind, int dtype, void* stream) {
+  FSTU_REQUIRE(y, FSTU_ENULL, "fstu_bias_act: null pointer");
+  FSTU_REQUIRE(rows >= 0 && n >= 1 && (kind == 0 || kind == 1), FSTU_EARG, "fstu_bias_act: rows=%lld n=%d kind=%d", (long long)rows, n, kind);
+  if (rows == 0 || (!bias && kind == 0)) return FSTU_OK;
+  int64_t blocks = (rows * n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_bias_act",
+                      hipLaunchKernelGGL(bias_act_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                                         (T*)y, (const T*)bias, rows, n, kind));
+  FSTU_CHECK_LAUNCH("fstu_bias_act");
+  return FSTU_OK;
+}
+
 // ---------------------------------------------------------------- sampling
 // One workgroup of 1024 threads per row; the row (V logits) is re-read from
 // L2 in each pass instead of being staged.

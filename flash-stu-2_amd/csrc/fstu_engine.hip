@@ -257,6 +257,8 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   void* xo = m->x2;
   const bool glu_pro = dt == FSTU_BF16 && xo != nullptr && d % 128 == 0 && (size_t)B * (d + 8) * 2 + 16384 <= 64 * 1024;
   const size_t wsz = (dt == FSTU_BF16) ? 2 : 4;
+  const bool mlp_fused = dt == FSTU_BF16 && m->mlp_sync && m->mlp_partial &&
+                         fstu_mlp_block_plan(B, d, I, nullptr, nullptr, nullptr) == FSTU_OK;
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     bool pending_y = false;   // m->y holds a sub-layer output not yet added to the residual stream
@@ -287,6 +289,12 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
       pending_y = true;
     }
+    const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
+    if (mlp_fused && L.wp_gate && L.wp_up && L.wp_down) {
+      TIMED(PC_GLU, fstu_mlp_block(xc, pending_y ? m->y : nullptr, xc, L.mlp_norm_w, L.wp_gate, L.wp_up, L.wp_down, next_w,
+                                   m->h, m->act, m->mlp_partial, m->mlp_sync, B, d, I, m->eps, stream));
+      continue;
+    }
     if (pending_y && glu_pro && L.wp_gate && L.wp_up) {
       fstu_gemv_args u = {};
       u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
@@ -298,7 +306,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
     }
     TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
-    const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
   if (!do_sample && m->best) {

@@ -31,6 +31,7 @@ SIGNATURES = {
     "fstu_glu_decode": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_linear_decode_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_gelu_mul": [_vp, _vp, _vp, _i64, _i, _vp],
+    "fstu_bias_act": [_vp, _vp, _i64, _i, _i, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
@@ -53,6 +54,10 @@ SIGNATURES = {
     "fstu_packed_elems": [_i, _i],
     "fstu_gemv_packed": [_vp, _vp],
     "fstu_set_gemv_target_workgroups": [_i],
+    "fstu_mlp_block_sync_bytes": [],
+    "fstu_mlp_block_trace": [_vp],
+    "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
+    "fstu_mlp_block": [_vp] * 12 + [_i, _i, _i, _f, _vp],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
@@ -87,6 +92,7 @@ def load(path: Optional[str] = None):
         fn.argtypes = args
         fn.restype = ctypes.c_int
     lib.fstu_packed_elems.restype = ctypes.c_int64
+    lib.fstu_mlp_block_sync_bytes.restype = ctypes.c_size_t
     if path is None:
         _lib = lib
     return lib
@@ -218,6 +224,31 @@ def gelu_mul(g: torch.Tensor, u: torch.Tensor, out: Optional[torch.Tensor] = Non
         out = torch.empty_like(g)
     _check(load().fstu_gelu_mul(_p(g), _p(u), _p(out), g.numel(), _dt(g), _stream()), "fstu_gelu_mul")
     return out
+
+
+def bias_act(y: torch.Tensor, bias: Optional[torch.Tensor], silu: bool = False) -> torch.Tensor:
+    """In place y = act(y + bias) over the last dimension; bias may be None."""
+    _dev(y, bias)
+    n = y.shape[-1]
+    if bias is not None and (bias.shape != (n,) or bias.dtype != y.dtype):
+        raise FlashSTUHipError(f"bias must be ({n},) {y.dtype}")
+    _check(load().fstu_bias_act(_p(y), _p(bias), y.numel() // n, n, int(silu), _dt(y), _stream()), "fstu_bias_act")
+    return y
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (..., K) @ weight (N,K)^T (+ bias): the skinny GEMV kernel for up to 16 rows, a library GEMM beyond."""
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1])
+    if x2.shape[0] <= MAX_DECODE_ROWS:
+        y = linear_decode(x2.contiguous(), weight)
+        if bias is not None:
+            bias_act(y, bias)
+    elif bias is not None:
+        y = torch.addmm(bias, x2, weight.t())
+    else:
+        y = torch.matmul(x2, weight.t())
+    return y.reshape(*shape[:-1], weight.shape[0])
 
 
 def stu_step_hist(hist: torch.Tensor, filt: torch.Tensor, t: int, nsplit: int, eo: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -466,6 +497,39 @@ def pack_rows(W: torch.Tensor) -> torch.Tensor:
     out = torch.empty(lib.fstu_packed_elems(N, K), dtype=W.dtype, device=W.device)
     _check(lib.fstu_pack_rows(_p(W), _p(out), N, K, _stream()), "fstu_pack_rows")
     return out
+
+
+def mlp_block_sync_bytes() -> int:
+    return int(load().fstu_mlp_block_sync_bytes())
+
+
+def mlp_block_plan(rows: int, d: int, I: int):
+    """(grid, K split, floats of partial workspace) of the one-launch MLP sub-layer, or None if unsupported."""
+    g, ks, pf = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+    rc = load().fstu_mlp_block_plan(rows, d, I, ctypes.byref(g), ctypes.byref(ks), ctypes.byref(pf))
+    return None if rc != 0 else (g.value, ks.value, pf.value)
+
+
+def mlp_block(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torch.Tensor, wp_gate: torch.Tensor,
+              wp_up: torch.Tensor, wp_down: torch.Tensor, next_norm_w: Optional[torch.Tensor], I: int, eps: float,
+              ws: Optional[dict] = None):
+    """One launch: x <- x + delta + MLP(rmsnorm(x + delta)); returns (x, rmsnorm(x) * next_norm_w or None).
+    x is updated in place.  `ws` caches the workspaces between calls."""
+    _dev(x, delta, norm_w, wp_gate, wp_up, wp_down, next_norm_w)
+    rows, d = x.shape
+    plan = mlp_block_plan(rows, d, I)
+    if plan is None or x.dtype != torch.bfloat16:
+        raise FlashSTUHipError(f"fstu_mlp_block does not support rows={rows} d={d} I={I} dtype={x.dtype}")
+    ws = {} if ws is None else ws
+    if "sync" not in ws:
+        ws["sync"] = torch.zeros(mlp_block_sync_bytes() // 4, dtype=torch.int32, device=x.device)
+        ws["partial"] = torch.empty(plan[2], dtype=torch.float32, device=x.device)
+        ws["act"] = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    h = torch.empty_like(x) if next_norm_w is not None else None
+    _check(load().fstu_mlp_block(_p(x), _p(delta), _p(x), _p(norm_w), _p(wp_gate), _p(wp_up), _p(wp_down),
+                                 _p(next_norm_w), _p(h), _p(ws["act"]), _p(ws["partial"]), _p(ws["sync"]), rows, d, I,
+                                 float(eps), _stream()), "fstu_mlp_block")
+    return x, h
 
 
 def gemv_packed(mode: int, Wp: torch.Tensor, N: int, K: int, out: torch.Tensor, x: Optional[torch.Tensor] = None,

@@ -41,7 +41,8 @@ class ModelDesc(ctypes.Structure):
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
-                ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp)]
+                ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
+                ("mlp_partial", _vp), ("mlp_sync", _vp)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -75,10 +76,17 @@ class _Chunk:
 class DecodeEngine:
     HIST_NSPLIT_MAX = 16
 
+    @staticmethod
+    def supports(cfg) -> bool:
+        """The one-call decode step covers approx-mode STU layers without the sandwich and bias-free linears;
+        other variants decode through the layers' own state (FlashSTU.generate picks the loop)."""
+        return bool(cfg.use_approx) and not cfg.stu_enable_mlp_sandwich and not cfg.bias
+
     def __init__(self, model):
         cfg = model.config
-        if not cfg.use_approx:
-            raise NotImplementedError("the fused decode engine covers use_approx=True; use generate(use_cache=False)")
+        if not self.supports(cfg):
+            raise NotImplementedError("the fused decode engine covers use_approx=True without the STU sandwich and "
+                                      "without biases; FlashSTU.generate falls back to the per-layer state loop")
         self.model = model
         self.cfg = cfg
         self.lib = _hip.load()
@@ -224,6 +232,17 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.x2 = buf(B, d).data_ptr()
+        plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
+        if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
+            # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its
+            # workspaces).  Correct and tested, but measured slower inside the full step (0.485 vs 0.472 ms): its
+            # ~14 dependent device-scope round trips of 1.3-1.5 us each cost as much as the launches they replace
+            for i, layer in enumerate(model.layers):
+                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
+                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
+                arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
+            m.mlp_partial = buf(plan[2], dtype=torch.float32).data_ptr()
+            m.mlp_sync = buf(_hip.mlp_block_sync_bytes() // 4, dtype=torch.int32).data_ptr()
         if self._use_packed(B):
             for i, layer in enumerate(model.layers):
                 ld = arr[i]

@@ -87,6 +87,8 @@ class FlashSTU(nn.Module):
             if hasattr(module, "SCALE_INIT"):
                 self.std *= (2 * self.n_layers) ** -0.5
             torch.nn.init.normal_(module.weight, mean=0.0, std=self.std)
+            if module.bias is not None:
+                torch.nn.init.zeros_(module.bias)
         elif isinstance(module, nn.Embedding):
             torch.nn.init.normal_(module.weight, mean=0.0, std=self.std)
         elif isinstance(module, STU):
@@ -100,6 +102,9 @@ class FlashSTU(nn.Module):
         elif isinstance(module, Attention):
             torch.nn.init.xavier_normal_(module.c_attn.weight)
             torch.nn.init.xavier_normal_(module.c_proj.weight)
+            for lin in (module.c_attn, module.c_proj):
+                if lin.bias is not None:
+                    torch.nn.init.zeros_(lin.bias)
 
     @torch.no_grad()
     def load_oracle_weights(self, w: Dict[str, torch.Tensor]) -> None:
@@ -169,6 +174,8 @@ class FlashSTU(nn.Module):
                 hidden.append(x.clone())
             x, cache = self._run_layers(x, past_key_values, use_cache, hidden)
             xn = self.norm(x)
+        if kwargs.get("last_only"):        # generate() needs the newest position only (the reference computes all)
+            xn = xn[:, -1:, :].contiguous()
         logits = self._head(xn)
         loss = None
         if labels is not None:
@@ -204,12 +211,27 @@ class FlashSTU(nn.Module):
         n_new = max_length - P
         if n_new <= 0:
             return input_ids
-        if use_cache and P <= self.config.seq_len:
+        from .engine import DecodeEngine
+        if use_cache and P <= self.config.seq_len and DecodeEngine.supports(self.config):
             return self.decode_engine().generate(input_ids, n_new, temperature, top_k, top_p, do_sample, seed,
                                                  return_logits=return_logits, use_graph=kwargs.get("use_graph", True))
         tokens = torch.empty(B, max_length, dtype=torch.int64, device=input_ids.device)
         tokens[:, :P] = input_ids
         all_logits = []
+        if use_cache and max_length <= self.config.seq_len:
+            # variants the one-call decode step does not cover (exact mode, sandwich, biases): the same token loop
+            # over the layers' own decode state, one forward(use_cache=True) per token as the reference loops
+            past = None
+            for step in range(n_new):
+                cur = P + step
+                inp = tokens[:, :cur] if past is None else tokens[:, cur - 1:cur]
+                out = self.forward(inp.contiguous(), past_key_values=past, use_cache=True, last_only=True)
+                past = out.past_key_values
+                last = out.logits[:, -1, :].contiguous()
+                if return_logits:
+                    all_logits.append(last)
+                _hip.sample(last, tokens[:, cur], temperature, top_k, top_p, do_sample, seed, step)
+            return (tokens, torch.stack(all_logits, 1)) if return_logits else tokens
         for step in range(n_new):
             cur = P + step
             lo = max(0, cur - self.config.seq_len)
@@ -275,10 +297,34 @@ class FlashSTU(nn.Module):
 
     @classmethod
     def from_pretrained(cls, path: str, **kwargs) -> "FlashSTU":
+        """Loads a directory written by save_pretrained here or by the reference (config.json +
+        model.safetensors, or sharded model-*.safetensors with model.safetensors.index.json; model.py:338-366),
+        or a single training checkpoint file model_<step>.safetensors (training/distributed.py:140-148) together
+        with config=...  Only safetensors are read: nothing in a checkpoint is ever executed."""
         from safetensors.torch import load_file
-        config = kwargs.pop("config", None) or FlashSTUConfig.from_pretrained(path)
+        import json
+        if os.path.isfile(path):
+            config = kwargs.pop("config", None)
+            if config is None:
+                cj = os.path.join(os.path.dirname(path), "config.json")
+                if not os.path.exists(cj):
+                    raise ValueError("a bare .safetensors checkpoint needs config=FlashSTUConfig(...) or a config.json beside it")
+                config = FlashSTUConfig.from_pretrained(cj)
+            sd = load_file(path)
+        else:
+            config = kwargs.pop("config", None) or FlashSTUConfig.from_pretrained(path)
+            index = os.path.join(path, "model.safetensors.index.json")
+            if os.path.exists(index):
+                with open(index) as f:
+                    shards = sorted(set(json.load(f)["weight_map"].values()))
+                sd = {}
+                for sh in shards:
+                    sd.update(load_file(os.path.join(path, sh)))
+            else:
+                sd = load_file(os.path.join(path, "model.safetensors"))
         model = cls(config)
-        sd = load_file(os.path.join(path, "model.safetensors"))
+        sd = {(k[len("module."):] if k.startswith("module.") else k): v for k, v in sd.items()}   # DDP-wrapped saves
+        sd = {(k[len("_orig_mod."):] if k.startswith("_orig_mod.") else k): v for k, v in sd.items()}  # compiled saves
         if "lm_head.weight" in sd and "tok_emb.weight" not in sd:
             sd["tok_emb.weight"] = sd.pop("lm_head.weight")
         sd.pop("lm_head.weight", None)

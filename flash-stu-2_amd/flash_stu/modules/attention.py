@@ -31,12 +31,10 @@ class Attention(nn.Module):
     def __init__(self, config):
         super().__init__()
         assert config.n_embd % config.n_heads == 0
-        if config.bias:
-            raise NotImplementedError("bias=True is not supported by the HIP path")
         self.n_heads = config.n_heads
         self.head_dim = config.n_embd // config.n_heads
-        self.c_attn = nn.Linear(config.n_embd, 3 * config.n_embd, bias=False, dtype=config.torch_dtype)
-        self.c_proj = nn.Linear(config.n_embd, config.n_embd, bias=False, dtype=config.torch_dtype)
+        self.c_attn = nn.Linear(config.n_embd, 3 * config.n_embd, bias=config.bias, dtype=config.torch_dtype)
+        self.c_proj = nn.Linear(config.n_embd, config.n_embd, bias=config.bias, dtype=config.torch_dtype)
         self.c_proj.SCALE_INIT = 1
         self.register_buffer("alibi_slopes", alibi_slopes(self.n_heads), persistent=False)
         w = config.window_size
@@ -65,15 +63,9 @@ class Attention(nn.Module):
         H, hd, W = self.n_heads, self.head_dim, self.window_size
         slopes = self.alibi_slopes
         if past_key_value is None:
-            if B * T <= _hip.MAX_DECODE_ROWS:
-                qkv = _hip.linear_decode(x.reshape(B * T, d), self.c_attn.weight).reshape(B, T, 3 * d)
-            else:
-                qkv = torch.matmul(x, self.c_attn.weight.t())
+            qkv = _hip.linear(x, self.c_attn.weight, self.c_attn.bias).contiguous()
             o = _hip.swa_prefill(qkv, slopes, H, W, self.softcap)
-            if B * T <= _hip.MAX_DECODE_ROWS:
-                y = _hip.linear_decode(o.reshape(B * T, d), self.c_proj.weight).reshape(B, T, d)
-            else:
-                y = torch.matmul(o, self.c_proj.weight.t())
+            y = _hip.linear(o, self.c_proj.weight, self.c_proj.bias)
             if not use_cache:
                 return y
             cap = W + 1
@@ -87,7 +79,7 @@ class Attention(nn.Module):
             past_key_value = self._ring_from_reference_cache(*past_key_value)
         kr, vr, pos_t = past_key_value
         pos = int(pos_t[0])
-        qkv = _hip.linear_decode(x.reshape(B, d), self.c_attn.weight)
+        qkv = _hip.linear(x.reshape(B, d), self.c_attn.weight, self.c_attn.bias)
         o = _hip.swa_decode(qkv, kr, vr, slopes, pos, W, self.softcap, append=True)
-        y = _hip.linear_decode(o, self.c_proj.weight).reshape(B, 1, d)
+        y = _hip.linear(o, self.c_proj.weight, self.c_proj.bias).reshape(B, 1, d)
         return (y, (kr, vr, pos_t + 1)) if use_cache else y

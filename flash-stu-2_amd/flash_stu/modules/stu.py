@@ -46,9 +46,11 @@ class STU(nn.Module):
             self.M_phi_plus = nn.Parameter(torch.empty(self.K, self.d_in, self.d_out, dtype=dt))
             if not self.use_hankel_L:
                 self.M_phi_minus = nn.Parameter(torch.empty(self.K, self.d_in, self.d_out, dtype=dt))
-        tile = min(config.d_in_tile or self.d_in, config.d_out_tile or self.d_in)
-        if tile < self.d_in:
-            raise NotImplementedError("channel tiling (d_in_tile/d_out_tile) is not implemented on the HIP path")
+        # channel tiling (stu.py:123-191): diagonal blocks of M_inputs only, i.e. M_inputs with every entry outside
+        # the tile_size x tile_size diagonal blocks dropped; the convolution itself is per channel either way
+        self.tile_size = min(config.d_in_tile or self.d_in, config.d_out_tile or self.d_in)
+        if self.tile_size < self.d_in and not self.use_approx:
+            raise NotImplementedError("Tiling only supported for use_approx=True")
         self._derived = {}
 
     # ---- tensors derived from the parameters, rebuilt when a parameter changes
@@ -78,8 +80,18 @@ class STU(nn.Module):
             self._derived.pop("spec")
         return self._cached("spec", params, lambda: _hip.stu_fft_filter(src, n, single_branch=self.use_hankel_L))
 
+    def m_inputs_eff(self) -> torch.Tensor:
+        """M_inputs as the forward uses it: the parameter itself, or its block-diagonal part when tiling is on."""
+        if self.tile_size >= self.d_in:
+            return self.M_inputs
+
+        def build():
+            idx = torch.arange(self.d_in, device=self.M_inputs.device) // self.tile_size
+            return (self.M_inputs * (idx[:, None] == idx[None, :]).to(self.M_inputs.dtype)).contiguous()
+        return self._cached("mie", (self.M_inputs,), build)
+
     def m_inputs_t(self) -> torch.Tensor:
-        return self._cached("mit", (self.M_inputs,), lambda: self.M_inputs.t().contiguous())
+        return self._cached("mit", (self.M_inputs,), lambda: self.m_inputs_eff().t().contiguous())
 
     def lds_params(self) -> Tuple[torch.Tensor, torch.Tensor]:
         def build():
@@ -103,7 +115,7 @@ class STU(nn.Module):
         B, T, d = x.shape
         if B * T <= _hip.MAX_DECODE_ROWS:
             return _hip.linear_decode(x.reshape(B * T, d), self.m_inputs_t()).reshape(B, T, self.d_out)
-        return torch.matmul(x, self.M_inputs)
+        return torch.matmul(x, self.m_inputs_eff())
 
     def _convolve(self, xp: torch.Tensor) -> torch.Tensor:
         """Approx-mode convolution of the projected inputs with phi_proj (stu.py:89-98,120): the FFT form of

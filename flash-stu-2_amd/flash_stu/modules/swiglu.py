@@ -16,8 +16,6 @@ class MLP(nn.Module):
         self.gate_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=config.bias, dtype=dtype)
         self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=config.bias, dtype=dtype)
         self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=config.bias, dtype=dtype)
-        if config.bias:
-            raise NotImplementedError("bias=True is not supported by the HIP path")
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -26,7 +24,12 @@ class MLP(nn.Module):
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         rows = x2.shape[0]
-        if rows <= _hip.MAX_DECODE_ROWS:
+        if self.gate_proj.bias is not None:
+            g = _hip.linear(x2, self.gate_proj.weight, self.gate_proj.bias)
+            u = _hip.linear(x2, self.up_proj.weight, self.up_proj.bias)
+            act = _hip.gelu_mul(g.contiguous(), u.contiguous(), out=g)
+            out = _hip.linear(act, self.down_proj.weight, self.down_proj.bias)
+        elif rows <= _hip.MAX_DECODE_ROWS:
             act = _hip.glu_decode(x2, self.gate_proj.weight, self.up_proj.weight)
             out = _hip.linear_decode(act, self.down_proj.weight)
         else:

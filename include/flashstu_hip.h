@@ -99,6 +99,11 @@ int fstu_linear_decode_splitk(const void* x, int ldx, const void* W, float* part
  * flash_stu/modules/swiglu.py:24-26). */
 int fstu_gelu_mul(const void* g, const void* u, void* act, int64_t n, int dtype, void* stream);
 
+/* In place y[r,c] = act( T(y[r,c] + bias[c]) ) over (rows,n); bias may be NULL; kind 0: identity, 1: SiLU.
+ * The `bias=True` linears (flash_stu/modules/swiglu.py:12-20, modules/attention.py:27-36) and the SiLU of the
+ * STU sandwich (flash_stu/layers/stu_layer.py:49,84-85) on top of the bias-free GEMV kernels. */
+int fstu_bias_act(void* y, const void* bias, int64_t rows, int n, int kind, int dtype, void* stream);
+
 /* ---- STU decode step: exact history form ----------------------------------
  * hist is the (B,cap,d) history of projected inputs x_proj (model dtype), the
  * newest at time index t (0-based, t < cap); filt is the (L,d) per-channel
@@ -302,6 +307,32 @@ int fstu_gemv_packed(const fstu_gemv_args* a, void* stream);
  * each workgroup then walks ceil(tiles/n) consecutive tiles. */
 int fstu_set_gemv_target_workgroups(int n);
 
+/* ---- MLP sub-layer of one decode step in one launch (bf16) -------------------
+ *   x' = T(x_in + delta)                       (delta may be NULL)
+ *   h = rmsnorm(x') * norm_w;  act = T(gelu_tanh(T(h Wg^T))) * T(h Wu^T)
+ *   x_out = T(x' + T(act Wd^T));  h_out = rmsnorm(x_out) * next_norm_w   (h_out may be NULL)
+ * Replaces mlp_norm + MLP + residual add + the next sub-layer's norm of
+ * flash_stu/layers/stu_layer.py:93-96, flash_stu/layers/attention_layer.py:59-62
+ * and flash_stu/modules/swiglu.py:22-29 for <= 16 rows.  wp_* are fstu_pack_rows
+ * copies of gate_proj (I,d), up_proj (I,d), down_proj (d,I).  x_out may alias x_in.
+ * A persistent grid (one workgroup per CU, grid barrier in the middle): nothing
+ * else may run on the GPU at the same time.  Workspaces, owned by the caller:
+ * act_ws rows*I bf16; partial_ws and the grid size from fstu_mlp_block_plan
+ * (returns FSTU_ESHAPE when the shape is not supported: d in {256,512,768,1024,2048},
+ * I % 512 == 0); sync_ws fstu_mlp_block_sync_bytes() bytes, 128-byte aligned,
+ * zeroed once (every launch returns it to zero; word 320 is raised if a bounded
+ * spin ever timed out).
+ * fstu_mlp_block_trace: profiling hook; with a device buffer of grid*8 int64 every later launch stamps the wall
+ * clock (100 MHz ticks) of each workgroup at start, with x in LDS, after the norm prologue, after the gate/up
+ * phase, after the barrier, at the first ticket, at the second ticket and at exit (0 where a workgroup left
+ * earlier); NULL switches it off. */
+size_t fstu_mlp_block_sync_bytes(void);
+int fstu_mlp_block_trace(long long* buf);
+int fstu_mlp_block_plan(int rows, int d, int I, int* grid, int* ksplit, size_t* partial_floats);
+int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, const void* norm_w, const void* wp_gate,
+                   const void* wp_up, const void* wp_down, const void* next_norm_w, void* h_out, void* act_ws,
+                   float* partial_ws, unsigned* sync_ws, int rows, int d, int I, float eps, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -371,6 +402,10 @@ typedef struct {
   void* yd;                 /* (B,d) down-projection output */
   float* partial_fix;       /* ksplit_down * ceil(d/16) * 256 floats */
   unsigned* counters;       /* ceil(d/16) uint32, zero-initialised once */
+  /* one-launch MLP sub-layer (fstu_mlp_block), used for every layer that has wp_gate, wp_up and wp_down when both
+   * are set and the shape is supported */
+  float* mlp_partial;       /* fstu_mlp_block_plan's partial_floats */
+  unsigned* mlp_sync;       /* fstu_mlp_block_sync_bytes(), zero-initialised once */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

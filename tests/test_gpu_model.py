@@ -246,3 +246,121 @@ def test_save_and_load_pretrained_roundtrip(tmp_path):
     assert torch.equal(model.generate(ids, max_length=30, do_sample=False),
                        again.generate(ids, max_length=30, do_sample=False))
     assert again.get_num_params() == model.get_num_params()
+
+
+# ----------------------------------------------------------------- variants beyond the default configuration
+def _variant_pair(seed, dtype=torch.float32, **kw):
+    """Model with the given config variant + oracle-side restatement driven by the same state dict."""
+    from flash_stu import FlashSTU, FlashSTUConfig
+    base = dict(n_embd=128, n_layers=2, n_heads=2, window_size=16, num_eigh=8, seq_len=64, vocab_size=211,
+                mlp_scale=2, torch_dtype=dtype, use_attn=True)
+    base.update(kw)
+    torch.manual_seed(seed)
+    model = FlashSTU(FlashSTUConfig(**base))
+    with torch.no_grad():
+        for n_, p_ in model.named_parameters():
+            if n_.endswith(".bias"):
+                p_.copy_((0.1 * torch.randn(p_.shape)).to(dtype))
+            elif "M_inputs" in n_ or "M_filters" in n_:
+                p_.mul_(4.0)
+    return model
+
+
+def _ref_layer0_stu_sandwich(model, x):
+    """Oracle-side restatement of stu_layer.py:78-97 with the sandwich, from the oracle's own pieces."""
+    L = model.layers[0]
+    sd = {k: v.detach().cpu() for k, v in L.state_dict().items()}
+    cfg = model.config
+    h = O.rms_norm(x, sd["stu_norm.weight"], cfg.rms_norm_eps)
+    h = torch.nn.functional.linear(h, sd["stu_mlp_in_proj.weight"], sd.get("stu_mlp_in_proj.bias"))
+    h = torch.nn.functional.silu(h)
+    phi = model.phi.detach().cpu()
+    h = O.stu_forward(h, phi, {"M_inputs": sd["stu.M_inputs"], "M_filters": sd["stu.M_filters"]}, model.n)
+    h = torch.nn.functional.linear(h, sd["stu_mlp_out_proj.weight"], sd.get("stu_mlp_out_proj.bias"))
+    x = x + h
+    h2 = O.rms_norm(x, sd["mlp_norm.weight"], cfg.rms_norm_eps)
+    g = torch.nn.functional.gelu(torch.nn.functional.linear(h2, sd["mlp.gate_proj.weight"], sd.get("mlp.gate_proj.bias")),
+                                 approximate="tanh")
+    u = torch.nn.functional.linear(h2, sd["mlp.up_proj.weight"], sd.get("mlp.up_proj.bias"))
+    return x + torch.nn.functional.linear(g * u, sd["mlp.down_proj.weight"], sd.get("mlp.down_proj.bias"))
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_stu_sandwich_layer_matches_restatement(bias):
+    """stu_enable_mlp_sandwich (+ bias=True): the STU layer against the oracle's pieces, fp32."""
+    model = _variant_pair(11, stu_enable_mlp_sandwich=True, stu_mlp_hidden_size=192, bias=bias)
+    x = torch.randn(2, 40, 128, generator=torch.Generator().manual_seed(3))
+    ref = _ref_layer0_stu_sandwich(model, x.clone())
+    got = model.cuda().layers[0](x.cuda().clone()).cpu()
+    assert float((got - ref).abs().max()) <= 2e-4 * float(ref.abs().max())
+
+
+def test_sandwich_and_bias_generate_stateful_equals_recompute():
+    """generate() of a variant the one-call step does not cover: the per-layer state loop returns the same ids
+    as re-running the whole sequence every step."""
+    model = _variant_pair(12, stu_enable_mlp_sandwich=True, stu_mlp_hidden_size=192, bias=True).cuda()
+    ids = torch.randint(0, 211, (3, 9), generator=torch.Generator().manual_seed(5)).cuda()
+    a = model.generate(ids, max_length=30, do_sample=False, use_cache=True)
+    b = model.generate(ids, max_length=30, do_sample=False, use_cache=False)
+    assert torch.equal(a, b)
+
+
+def test_channel_tiling_is_the_block_diagonal_projection():
+    """d_in_tile/d_out_tile (stu.py:123-191): per tile x[..., i:e] @ M_inputs[i:e, i:e] and the tile's filters,
+    restated with the oracle's convolution tile by tile; decode through the engine matches recompute."""
+    model = _variant_pair(13, d_in_tile=32, d_out_tile=32)
+    stu = model.layers[0].stu
+    x = torch.randn(2, 48, 128, generator=torch.Generator().manual_seed(4))
+    phi = model.phi.detach().cpu()
+    Mi, Mf = stu.M_inputs.detach().cpu(), stu.M_filters.detach().cpu()
+    parts = []
+    for i in range(0, 128, 32):
+        plus, minus = O.convolve(x[..., i:i + 32] @ Mi[i:i + 32, i:i + 32], phi @ Mf[:, i:i + 32], model.n)
+        parts.append(plus + minus)
+    ref = torch.cat(parts, -1)
+    model = model.cuda()
+    got = model.layers[0].stu(x.cuda()).cpu()
+    assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
+    ids = torch.randint(0, 211, (2, 7), generator=torch.Generator().manual_seed(6)).cuda()
+    assert torch.equal(model.generate(ids, max_length=24, do_sample=False),
+                       model.generate(ids, max_length=24, do_sample=False, use_cache=False))
+
+
+def test_all_stu_stack_and_exact_mode_generate():
+    """use_attn=False (model.py:83-87) and use_approx=False decode: stateful loop == full recompute."""
+    for kw in (dict(use_attn=False), dict(use_approx=False, n_embd=64, n_heads=2)):
+        model = _variant_pair(14, **kw).cuda()
+        ids = torch.randint(0, 211, (2, 6), generator=torch.Generator().manual_seed(7)).cuda()
+        a = model.generate(ids, max_length=20, do_sample=False, use_cache=True)
+        b = model.generate(ids, max_length=20, do_sample=False, use_cache=False)
+        assert torch.equal(a, b), kw
+
+
+def test_checkpoint_formats(tmp_path):
+    """save_pretrained directory, a sharded directory with an index, and a bare training-style
+    model_<step>.safetensors (training/distributed.py:140-148) all load to the same logits."""
+    import json
+    from safetensors.torch import save_file
+    from flash_stu import FlashSTU
+    model = _variant_pair(15).cuda()
+    ids = torch.randint(0, 211, (2, 12), generator=torch.Generator().manual_seed(8)).cuda()
+    ref = model(ids).logits
+    d1 = tmp_path / "hf"
+    model.save_pretrained(str(d1))
+    assert torch.equal(FlashSTU.from_pretrained(str(d1)).cuda()(ids).logits, ref)
+    # sharded: split the state dict over two files + index
+    sd = {k: v.detach().cpu().contiguous() for k, v in model.state_dict().items() if k != "lm_head.weight"}
+    keys = sorted(sd)
+    d2 = tmp_path / "sharded"
+    d2.mkdir()
+    model.config.save_pretrained(str(d2))
+    half = len(keys) // 2
+    save_file({k: sd[k] for k in keys[:half]}, str(d2 / "model-00001-of-00002.safetensors"))
+    save_file({k: sd[k] for k in keys[half:]}, str(d2 / "model-00002-of-00002.safetensors"))
+    wm = {k: ("model-00001-of-00002.safetensors" if i < half else "model-00002-of-00002.safetensors") for i, k in enumerate(keys)}
+    (d2 / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": wm}))
+    assert torch.equal(FlashSTU.from_pretrained(str(d2)).cuda()(ids).logits, ref)
+    # training checkpoint: one file, DDP-style prefix, config passed in
+    f3 = tmp_path / "model_00100.safetensors"
+    save_file({"module." + k: v for k, v in sd.items()}, str(f3))
+    assert torch.equal(FlashSTU.from_pretrained(str(f3), config=model.config).cuda()(ids).logits, ref)

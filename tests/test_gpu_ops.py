@@ -482,3 +482,41 @@ def test_argument_errors_do_not_launch(hip):
     with pytest.raises(hip.FlashSTUHipError, match="ring capacity"):
         hip.swa_decode(torch.zeros(1, 384, dtype=torch.bfloat16, device="cuda"), kr, kr.clone(),
                        torch.zeros(2, device="cuda"), 3, 8, 50.0)
+
+
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 512, 2048), (8, 1024, 4096), (4, 2048, 8192)])
+def test_mlp_block_one_launch(hip, rows, d, I):
+    """The one-launch MLP sub-layer against the oracle's residual add + RMSNorm + MLP + residual add + RMSNorm,
+    launched three times on the same workspaces (its counters must return to zero)."""
+    dtype = torch.bfloat16
+    g = gen(31)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    delta = (0.5 * torch.randn(rows, d, generator=g)).to(dtype)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
+    nw2 = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
+    wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
+    x1 = x + delta
+    h = O.rms_norm(x1, nw, O.RMS_EPS_DEFAULT)
+    y = O.mlp_forward(h, {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd})
+    x2 = x1 + y
+    h2 = O.rms_norm(x2, nw2, O.RMS_EPS_DEFAULT)
+    pg, pu, pd = hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu)), hip.pack_rows(dev(wd))
+    ws = {}
+    for it in range(3):
+        xd = dev(x).clone()
+        xo, ho = hip.mlp_block(xd, dev(delta), dev(nw), pg, pu, pd, dev(nw2), I, O.RMS_EPS_DEFAULT, ws)
+        torch.cuda.synchronize()
+        assert int(ws["sync"].abs().sum()) == 0, "counters not returned to zero / spin timeout flag raised"
+        sc = float(x2.float().abs().max())
+        check(xo, x2, dtype, frac=0.10, scale=sc, atol=2.0 ** -7 * float(y.float().abs().max()))
+        err = (ho.float().cpu() - h2.float()).abs().max() / h2.float().abs().max()
+        assert float(err) <= 2e-2
+    # no delta, no trailing norm
+    xd = dev(x).clone()
+    xo, ho = hip.mlp_block(xd, None, dev(nw), pg, pu, pd, None, I, O.RMS_EPS_DEFAULT, ws)
+    h0 = O.rms_norm(x, nw, O.RMS_EPS_DEFAULT)
+    y0 = O.mlp_forward(h0, {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd})
+    assert ho is None
+    check(xo, x + y0, dtype, frac=0.10, scale=float((x + y0).float().abs().max()), atol=2.0 ** -7 * float(y0.float().abs().max()))

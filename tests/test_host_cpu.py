@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_library_exports_every_declared_symbol():
     from flash_stu import _hip
     header = open(os.path.join(ROOT, "include", "flashstu_hip.h")).read()
-    declared = set(re.findall(r"^\s*(?:int|const char\*|int64_t)\s+(fstu_\w+)\s*\(", header, flags=re.M))
+    declared = set(re.findall(r"^\s*(?:int|const char\*|int64_t|size_t)\s+(fstu_\w+)\s*\(", header, flags=re.M))
     assert {"fstu_version", "fstu_last_error", "fstu_decode_step", "fstu_swa_decode", "fstu_stu_step_lds"} <= declared
     lib = ctypes.CDLL(_hip.LIB_PATH)
     for name in sorted(declared):
