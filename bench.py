@@ -91,6 +91,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every step kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--warm-wgs", type=int, default=-1, help="workgroups of the graph's cache warm-up branch (0 = off)")
+    ap.add_argument("--pmc-calibrate", action="store_true", dest="pmc_calibrate",
+                    help="also launch the library's plain 256 MiB copy kernel 4 times (reference for traffic counters)")
     ap.add_argument("--breakdown", action="store_true", help="time every kernel class with HIP events")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -182,9 +184,20 @@ def main():
     _hip._check(lib.fstu_prof_glu_loop(ctypes.byref(eng.desc), max(4, K // 8), ctypes.byref(ms_c), ctypes.byref(n_c),
                                        torch.cuda.current_stream().cuda_stream), "fstu_prof_glu_loop")
     glu_ms, glu_n = ms_c.value, n_c.value
+    if args.pmc_calibrate:
+        a_ = torch.zeros(256 << 20, dtype=torch.uint8, device="cuda")
+        b_ = torch.empty_like(a_)
+        for _ in range(4):
+            _hip._check(lib.fstu_prof_copy(b_.data_ptr(), a_.data_ptr(), a_.numel(), torch.cuda.current_stream().cuda_stream),
+                        "fstu_prof_copy")
+        torch.cuda.synchronize()
     glu_bytes = 2 * I * d * 2 + B * d * 2 + B * I * 2          # gate+up weights, x in, act out
     glu_avg_us = glu_ms / glu_n * 1e3
     glu_gbps = glu_bytes / (glu_avg_us * 1e-6) / 1e9
+    # HBM bytes per GLU launch from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by what the same
+    # counter reads for the library's plain 256 MiB copy kernel: x2.000 and x1.000).  Measured offline for the default
+    # workload only; summary and commands in profiles/glu_c2_hbm_traffic_pmc.txt.
+    traffic = 28638208 if (cfg.n_embd, cfg.mlp_scale, B) == (768, 12, 8) else None
     out = {
         "metric": "decode tokens/sec at 1 GPU (768-d FlashSTU, bs=8) + achieved HBM GB/s",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
@@ -195,7 +208,7 @@ def main():
                    "stu_decode_mode": args.stu_mode, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
         "roofline": {"bound": "hbm", "kernel": "linear_mfma_bf16_kernel<GLU> (gate/up projection + gelu*up)",
                      "achieved": glu_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": glu_gbps / HBM_PEAK_GBPS,
-                     "traffic": None, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,
+                     "traffic": traffic, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,
                      "launches_timed": glu_n},
         "step_roofline": {"bound": "hbm", "bytes_per_step": step_bytes, "achieved": step_bytes / (ms_per_step * 1e-3) / 1e9,
                           "peak": HBM_PEAK_GBPS, "unit": "GB/s",

@@ -73,6 +73,20 @@ extern "C" int fstu_prof_glu_loop(const fstu_model_desc* m, int reps, double* to
   return rc;
 }
 
+// A plain copy of `bytes` bytes (16-byte granules): the calibration launch for hardware traffic counters, whose
+// FETCH_SIZE / WRITE_SIZE readings for this kernel are known in advance.
+__global__ void __launch_bounds__(256) prof_copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+extern "C" int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* stream) {
+  FSTU_REQUIRE(dst && src && bytes % 16 == 0 && fstu_aligned(dst, 16) && fstu_aligned(src, 16), FSTU_EARG,
+               "fstu_prof_copy: pointers and size must be 16-byte multiples");
+  hipLaunchKernelGGL(prof_copy_kernel, dim3(4096), dim3(256), 0, (hipStream_t)stream, (uint4*)dst, (const uint4*)src, bytes / 16);
+  FSTU_CHECK_LAUNCH("fstu_prof_copy");
+  return FSTU_OK;
+}
+
 #define TIMED(cls, call)                                                                        \
   do {                                                                                          \
     const bool t__ = (g_prof_class == (cls)) && g_prof_n < g_prof_cap;                          \

@@ -65,6 +65,7 @@ SIGNATURES = {
     "fstu_set_warm_workgroups": [_i],
     "fstu_prof_begin": [_i, _i],
     "fstu_prof_end": [_vp, _vp],
+    "fstu_prof_copy": [_vp, _vp, ctypes.c_size_t, _vp],
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }

@@ -444,6 +444,9 @@ int fstu_prof_begin(int kernel_class, int max_launches);
 int fstu_prof_end(double* total_ms, int* launches);
 /* The gate/up GLU projection (fstu_glu_decode) of every layer of `m`, `reps` times back to back on `stream`
  * between two HIP events; returns the elapsed time and launch count.  Synchronises on the second event. */
+/* Plain copy kernel of a known size: the reference launch against which FETCH_SIZE / WRITE_SIZE counter readings
+ * of the other kernels are scaled. */
+int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* stream);
 int fstu_prof_glu_loop(const fstu_model_desc* m, int reps, double* total_ms, int* launches, void* stream);
 
 #ifdef __cplusplus
