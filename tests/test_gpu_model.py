@@ -97,6 +97,23 @@ def _teacher_forced(w, ocfg, tokens, P):
     return logits[:, P - 1:, :]          # predictions for positions P..end
 
 
+class _wide_accumulation:
+    """Inside the block every F.linear of the oracle accumulates in float64 and rounds once to the model dtype: the
+    same specification (same rounding points) under another summation order than the CPU library's."""
+    def __enter__(self):
+        self.saved = O.F.linear
+
+        def wide(x, w, b=None):
+            y = x.double() @ w.double().t()
+            if b is not None:
+                y = y + b.double()
+            return y.to(x.dtype)
+        O.F.linear = wide
+
+    def __exit__(self, *a):
+        O.F.linear = self.saved
+
+
 @pytest.mark.parametrize("mode", ["history", "lds"])
 @pytest.mark.parametrize("init", ["healthy", "reference"])
 def test_c2_dims_bf16_teacher_forced(mode, init):
@@ -122,6 +139,16 @@ def test_c2_dims_bf16_teacher_forced(mode, init):
           f"within-one-ulp agreement {float(near):.3f}")
     assert float(near) >= 0.99
     assert float(agree) >= 0.9
+    if mode == "history" and init == "healthy":
+        # noise floor of the comparison: the oracle against itself with float64 accumulation in every linear.
+        # Two faithful evaluations of the same bf16 specification do not pick the same token every time either.
+        with _wide_accumulation():
+            ref2 = _teacher_forced(w, ocfg, got, P).float()
+        self_agree = (ref2.argmax(-1) == ref_logits.argmax(-1)).float().mean()
+        self_err = ((ref2 - ref_logits).abs().amax(-1) / ref_logits.abs().amax(-1)).max()
+        print(f"oracle vs oracle(float64 accumulation): strict agreement {float(self_agree):.3f}, "
+              f"max rel logit difference {float(self_err):.2e}")
+        assert float(agree) >= float(self_agree) - 0.03
 
 
 def test_window_wraps_the_ring_bf16():
