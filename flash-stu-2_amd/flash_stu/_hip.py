@@ -48,6 +48,8 @@ SIGNATURES = {
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_append_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "fstu_swa_prefill_ws_elems": [_i, _i, _i, _i],
+    "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
@@ -93,6 +95,7 @@ def load(path: Optional[str] = None):
         fn.argtypes = args
         fn.restype = ctypes.c_int
     lib.fstu_packed_elems.restype = ctypes.c_int64
+    lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
     lib.fstu_mlp_block_sync_bytes.restype = ctypes.c_size_t
     if path is None:
         _lib = lib
@@ -438,7 +441,8 @@ def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slop
 
 
 def swa_prefill(qkv: torch.Tensor, slopes: torch.Tensor, n_heads: int, window: int, softcap: float,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None, force_valu: bool = False) -> torch.Tensor:
+    """Prefill attention: the MFMA kernel for bf16 with head dim 64/128, the wave-per-query kernel otherwise."""
     _dev(qkv, slopes, out)
     B, T, d3 = qkv.shape
     d = d3 // 3
@@ -446,6 +450,12 @@ def swa_prefill(qkv: torch.Tensor, slopes: torch.Tensor, n_heads: int, window: i
     assert slopes.dtype == torch.float32 and slopes.numel() == n_heads
     if out is None:
         out = torch.empty(B, T, d, dtype=qkv.dtype, device=qkv.device)
+    if qkv.dtype == torch.bfloat16 and hd in (64, 128) and T >= 16 and not force_valu:
+        lib = load()
+        ws = torch.empty(lib.fstu_swa_prefill_ws_elems(B, T, n_heads, hd), dtype=qkv.dtype, device=qkv.device)
+        _check(lib.fstu_swa_prefill_mfma(_p(qkv), _p(ws), _p(out), _p(slopes), B, T, n_heads, hd, window,
+                                         float(softcap or 0.0), _stream()), "fstu_swa_prefill_mfma")
+        return out
     _check(load().fstu_swa_prefill(_p(qkv), _p(out), _p(slopes), B, T, n_heads, hd, window, float(softcap or 0.0),
                                    _dt(qkv), _stream()), "fstu_swa_prefill")
     return out

@@ -224,6 +224,14 @@ int fstu_swa_append_decode(const void* qkv, void* kring, void* vring, void* out,
 int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T, int H, int hd,
                      int window, float softcap, int dtype, void* stream);
 
+/* The same prefill attention on the matrix cores (bf16, head dim 64 or 128): S^T = K Q^T and O^T = V^T P^T as
+ * v_mfma_f32_16x16x32_bf16 tiles, 16 queries per wave, online softmax in fp32, P carried as a bf16 head plus a bf16
+ * remainder so that the second product keeps fp32-P accuracy.  vt_ws is a caller-owned workspace of
+ * fstu_swa_prefill_ws_elems(B,T,H,hd) bf16 elements that receives V transposed to (B,H,hd,Tp). */
+int64_t fstu_swa_prefill_ws_elems(int B, int T, int H, int hd);
+int fstu_swa_prefill_mfma(const void* qkv, void* vt_ws, void* out, const float* slopes, int B, int T, int H, int hd,
+                          int window, float softcap, void* stream);
+
 /* ---- sampling --------------------------------------------------------------
  * Per row of logits (B,V): l = clamp(T(logit/temperature), -1e4, 1e4); optional
  * top-k (keep every l >= k-th largest), optional top-p over the survivors

@@ -520,3 +520,23 @@ def test_mlp_block_one_launch(hip, rows, d, I):
     y0 = O.mlp_forward(h0, {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd})
     assert ho is None
     check(xo, x + y0, dtype, frac=0.10, scale=float((x + y0).float().abs().max()), atol=2.0 ** -7 * float(y0.float().abs().max()))
+
+
+@pytest.mark.parametrize("B,H,hd,W,T", [(2, 4, 64, 16, 50), (2, 12, 64, 512, 700), (1, 4, 128, 32, 100),
+                                         (1, 2, 64, 1000, 333), (1, 2, 128, 64, 17)])
+def test_swa_prefill_mfma(hip, B, H, hd, W, T):
+    """Matrix-core prefill attention (bf16): against the oracle's explicit softmax and against the wave-per-query
+    kernel; ragged T (not a multiple of the 16-query / 32-key tiles), window smaller and larger than T."""
+    dtype = torch.bfloat16
+    g = gen(40)
+    d = H * hd
+    qkv = torch.randn(B, T, 3 * d, generator=g).to(dtype)
+    slopes = O.alibi_slopes(H)
+    q, k, v = (t.reshape(B, T, H, hd) for t in torch.chunk(qkv, 3, dim=2))
+    full = O.attention_core(q, k, v, W, slopes, 50.0).reshape(B, T, d)
+    out = hip.swa_prefill(dev(qkv), dev(slopes), H, W, 50.0)
+    check(out, full, dtype, frac=0.05)
+    valu = hip.swa_prefill(dev(qkv), dev(slopes), H, W, 50.0, force_valu=True)
+    check(out, valu, dtype, frac=0.05)
+    out0 = hip.swa_prefill(dev(qkv), dev(slopes), H, W, 0.0)
+    check(out0, O.attention_core(q, k, v, W, slopes, 0.0).reshape(B, T, d), dtype, frac=0.05)
