@@ -260,10 +260,36 @@ __global__ void gelu_mul_kernel(const T* __restrict__ g, const T* __restrict__ u
   }
 }
 
+// bf16, 8 elements (16 bytes) per thread and iteration
+__global__ void __launch_bounds__(256)
+gelu_mul_bf16x8_kernel(const uint4* __restrict__ g, const uint4* __restrict__ u, uint4* __restrict__ act, int64_t n8) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < n8; i += stride) {
+    const uint4 gv = g[i], uv = u[i];
+    unsigned gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w}, ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float lo = DT<bf16_t>::rnd(gelu_tanh_f32(__uint_as_float(gw[k] << 16))) * __uint_as_float(uw[k] << 16);
+      float hi = DT<bf16_t>::rnd(gelu_tanh_f32(__uint_as_float(gw[k] & 0xffff0000u))) * __uint_as_float(uw[k] & 0xffff0000u);
+      ow[k] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+    }
+    act[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 extern "C" int fstu_gelu_mul(const void* g, const void* u, void* act, int64_t n, int dtype, void* stream) {
   FSTU_REQUIRE(g && u && act, FSTU_ENULL, "fstu_gelu_mul: null pointer");
   FSTU_REQUIRE(n >= 0, FSTU_ESHAPE, "fstu_gelu_mul: n<0");
   if (n == 0) return FSTU_OK;
+  if (dtype == FSTU_BF16 && n % 8 == 0 && fstu_aligned(g, 16) && fstu_aligned(u, 16) && fstu_aligned(act, 16)) {
+    int64_t b8 = (n / 8 + 255) / 256;
+    if (b8 > 16384) b8 = 16384;
+    hipLaunchKernelGGL(gelu_mul_bf16x8_kernel, dim3((unsigned)b8), dim3(256), 0, (hipStream_t)stream, (const uint4*)g,
+                       (const uint4*)u, (uint4*)act, n / 8);
+    FSTU_CHECK_LAUNCH("fstu_gelu_mul");
+    return FSTU_OK;
+  }
   int64_t blocks = (n + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   FSTU_DISPATCH_DTYPE(dtype, "fstu_gelu_mul",

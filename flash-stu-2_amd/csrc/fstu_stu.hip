@@ -324,10 +324,22 @@ lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__
     aj[i] = (i < per && j0 + i < S) ? a[j0 + i] : 0.f;
   }
   const T* hb = hist + (size_t)b * cap * d + c;
-  for (int tt = p; tt <= t_last; tt += 2) {
-    float x = DT<T>::ld(hb + (size_t)tt * d);
+  // 16 inputs are loaded before any is consumed, so the walk is bound by the FMA chains and not by 16x as many
+  // dependent memory latencies
+  for (int tt0 = p; tt0 <= t_last; tt0 += 32) {
+    float xs[16];
 #pragma unroll
-    for (int i = 0; i < LSH_MAXJ; ++i) h[i] = fmaf(aj[i], h[i], x);
+    for (int k = 0; k < 16; ++k) {
+      const int tt = tt0 + 2 * k;
+      xs[k] = (tt <= t_last) ? DT<T>::ld(hb + (size_t)tt * d) : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (tt0 + 2 * k <= t_last) {
+#pragma unroll
+        for (int i = 0; i < LSH_MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
+      }
+    }
   }
   float* st = state + (((size_t)b * 2 + p) * S) * d + c;
 #pragma unroll
