@@ -56,12 +56,17 @@ extern "C" int fstu_prof_glu_loop(const fstu_model_desc* m, int reps, double* to
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { fstu_set_error("fstu_prof_glu_loop: hipEventCreate failed"); return FSTU_EARG; }
   int rc = 0, n = 0;
-  for (int l = 0; l < m->n_layers && rc == 0; ++l)   // warm-up pass
-    rc = fstu_glu_decode(m->h, m->d, m->layers[l].w_gate, m->layers[l].w_up, m->act, m->I, m->B, m->I, m->d, m->dtype, stream);
+  // the same kernel the step launches for this projection
+  auto glu = [&](int l) {
+    const fstu_layer_desc& L = m->layers[l];
+    if (m->dtype == FSTU_BF16 && m->glu_packed && L.wp_gate && L.wp_up && fstu_glu_packed_supported(m->B, m->d, m->I))
+      return fstu_glu_packed(m->h, m->d, L.wp_gate, L.wp_up, m->act, m->I, m->B, m->I, m->d, stream);
+    return fstu_glu_decode(m->h, m->d, L.w_gate, L.w_up, m->act, m->I, m->B, m->I, m->d, m->dtype, stream);
+  };
+  for (int l = 0; l < m->n_layers && rc == 0; ++l) rc = glu(l);   // warm-up pass
   (void)hipEventRecord(e0, (hipStream_t)stream);
   for (int r = 0; r < reps && rc == 0; ++r)
-    for (int l = 0; l < m->n_layers && rc == 0; ++l, ++n)
-      rc = fstu_glu_decode(m->h, m->d, m->layers[l].w_gate, m->layers[l].w_up, m->act, m->I, m->B, m->I, m->d, m->dtype, stream);
+    for (int l = 0; l < m->n_layers && rc == 0; ++l, ++n) rc = glu(l);
   (void)hipEventRecord(e1, (hipStream_t)stream);
   (void)hipEventSynchronize(e1);
   float ms = 0.f;
@@ -271,6 +276,7 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   void* xo = m->x2;
   const bool glu_pro = dt == FSTU_BF16 && xo != nullptr && d % 128 == 0 && (size_t)B * (d + 8) * 2 + 16384 <= 64 * 1024;
   const size_t wsz = (dt == FSTU_BF16) ? 2 : 4;
+  const bool glu_bal = dt == FSTU_BF16 && m->glu_packed && fstu_glu_packed_supported(B, d, I);
   const bool mlp_fused = dt == FSTU_BF16 && m->mlp_sync && m->mlp_partial &&
                          fstu_mlp_block_plan(B, d, I, nullptr, nullptr, nullptr) == FSTU_OK;
   for (int l = 0; l < m->n_layers; ++l) {
@@ -317,7 +323,10 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       void* t = xc; xc = xo; xo = t;
     } else {
       if (pending_y) TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
-      TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
+      if (glu_bal && L.wp_gate && L.wp_up)
+        TIMED(PC_GLU, fstu_glu_packed(m->h, d, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
+      else
+        TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
     }
     TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));

@@ -415,6 +415,100 @@ mlp_block_kernel(MlpArgs a) {
   MLP_STAMP(7);
 }
 
+// ---------------------------------------------------------------- balanced gate/up GEMV (stand-alone launch)
+// The gate/up phase of mlp_block_kernel as a kernel of its own: one workgroup per CU, I/G features each at
+// 4-feature granularity (equal bytes per CU), every weight fragment of a workgroup in flight from the first
+// instruction, the 8 waves split K.  Input h is already normalised.
+struct GluArgs {
+  const bf16_t* h;
+  const uint4* wp_gate;
+  const uint4* wp_up;
+  bf16_t* act;
+  int rows, d, I, ldh, ldact, fpw;
+};
+
+template <int KSA>
+__global__ void __launch_bounds__(512)
+glu_balanced_kernel(GluArgs a) {
+  constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
+  __shared__ float red[DA * 8 * 512];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int wgi = blockIdx.x;
+  const bool xrow = r < a.rows;
+  // activations first (they are consumed first), then the weights
+  uint4 xa[KSA];
+  {
+    const rsrc_t rh = make_rsrc(a.h, ((size_t)(a.rows - 1) * a.ldh + a.d) * 2);
+    const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) xa[u] = buf_load16(rh, xrow ? hoff + (unsigned)u * 64u : MLP_OOB);
+  }
+  const int f0 = wgi * a.fpw, f1 = min(a.I, f0 + a.fpw);
+  const int ta0 = f0 >> 4, ta1 = (f1 > f0) ? ((f1 + 15) >> 4) : ta0;
+  const size_t tsa = (size_t)(a.d >> 5) * 64;
+  const size_t wa_bytes = (size_t)((a.I + 15) >> 4) * tsa * 16;
+  const rsrc_t rg = make_rsrc(a.wp_gate, wa_bytes), ru = make_rsrc(a.wp_up, wa_bytes);
+  const unsigned abase = ((unsigned)(w * KSA) * 64 + lane) * 16u;
+  uint4 wa[DA][KSA], wb[DA][KSA];
+  auto load_a = [&](int j, int tile) {
+    const int f = tile * 16 + r;
+    const bool ok = tile < ta1 && f >= f0 && f < f1;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) {
+      const unsigned off = ok ? abase + ((unsigned)tile * (unsigned)tsa + (unsigned)u * 64u) * 16u : MLP_OOB;
+      wa[j][u] = buf_load16(rg, off);
+      wb[j][u] = buf_load16(ru, off);
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < DA; ++j) load_a(j, ta0 + j);
+
+  for (int t0 = ta0; t0 < ta1; t0 += DA) {
+#pragma unroll
+    for (int j = 0; j < DA; ++j) {
+      floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < KSA; ++u) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
+      }
+      load_a(j, t0 + DA + j);
+      float* mine = red + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mine[i] = acc[i];
+        mine[256 + i] = acc2[i];
+      }
+    }
+    __syncthreads();
+    if (w < DA && t0 + w < ta1) {
+      const int tile = t0 + w;
+      float sg[4] = {0.f, 0.f, 0.f, 0.f}, su[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const float* o = red + (size_t)((w * 8 + s) * 2 * 64 + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          sg[i] += o[i];
+          su[i] += o[256 + i];
+        }
+      }
+      const int fb = tile * 16 + g * 4;
+      if (xrow && fb >= f0 && fb < f1) {
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
+          o[i] = ge * DT<bf16_t>::rnd(su[i]);
+        }
+        *(u64*)(a.act + (size_t)r * a.ldact + fb) = pack4_bf16(o);
+      }
+    }
+    if (t0 + DA < ta1) __syncthreads();
+  }
+}
+
 int g_cus = 0;
 long long* g_trace = nullptr;
 
@@ -499,5 +593,47 @@ extern "C" int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, 
 #undef MLP_CASE
   FSTU_REQUIRE(launched, FSTU_ESHAPE, "fstu_mlp_block: no kernel for d=%d I=%d", d, I);
   FSTU_CHECK_LAUNCH("fstu_mlp_block");
+  return FSTU_OK;
+}
+
+static int query_cus() {
+  if (g_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 0;
+    g_cus = p.multiProcessorCount;
+  }
+  return g_cus;
+}
+
+extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
+  const int ksa = d / 256;
+  return rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d % 256 == 0 && (ksa == 1 || ksa == 2 || ksa == 3 || ksa == 4 || ksa == 8) &&
+         I >= 16 && I % 4 == 0 && (size_t)I * d * 2 < 0xfff00000ull;
+}
+
+extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
+                               int I, int d, void* stream) {
+  FSTU_REQUIRE(h && wp_gate && wp_up && act, FSTU_ENULL, "fstu_glu_packed: null pointer");
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, d, I), FSTU_ESHAPE, "fstu_glu_packed: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(ldh >= d && ldh % 8 == 0 && ldact >= I && ldact % 4 == 0, FSTU_ESHAPE, "fstu_glu_packed: ldh=%d ldact=%d", ldh, ldact);
+  FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(wp_gate, 16) && fstu_aligned(wp_up, 16) && fstu_aligned(act, 8), FSTU_EALIGN,
+               "fstu_glu_packed: pointers must be 16-byte aligned");
+  int G = query_cus();
+  FSTU_REQUIRE(G > 0, FSTU_EARG, "fstu_glu_packed: no device");
+  if (G > (I + 3) / 4) G = (I + 3) / 4;
+  GluArgs a;
+  a.h = (const bf16_t*)h; a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
+  a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
+  a.fpw = (((I + G - 1) / G) + 3) & ~3;
+  hipStream_t s = (hipStream_t)stream;
+  switch (d / 256) {
+    case 1: hipLaunchKernelGGL(glu_balanced_kernel<1>, dim3(G), dim3(512), 0, s, a); break;
+    case 2: hipLaunchKernelGGL(glu_balanced_kernel<2>, dim3(G), dim3(512), 0, s, a); break;
+    case 3: hipLaunchKernelGGL(glu_balanced_kernel<3>, dim3(G), dim3(512), 0, s, a); break;
+    case 4: hipLaunchKernelGGL(glu_balanced_kernel<4>, dim3(G), dim3(512), 0, s, a); break;
+    default: hipLaunchKernelGGL(glu_balanced_kernel<8>, dim3(G), dim3(512), 0, s, a); break;
+  }
+  FSTU_CHECK_LAUNCH("fstu_glu_packed");
   return FSTU_OK;
 }

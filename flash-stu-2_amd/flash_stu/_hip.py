@@ -56,6 +56,8 @@ SIGNATURES = {
     "fstu_packed_elems": [_i, _i],
     "fstu_gemv_packed": [_vp, _vp],
     "fstu_set_gemv_target_workgroups": [_i],
+    "fstu_glu_packed_supported": [_i, _i, _i],
+    "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_mlp_block_sync_bytes": [],
     "fstu_mlp_block_trace": [_vp],
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
@@ -507,6 +509,21 @@ def pack_rows(W: torch.Tensor) -> torch.Tensor:
     lib = load()
     out = torch.empty(lib.fstu_packed_elems(N, K), dtype=W.dtype, device=W.device)
     _check(lib.fstu_pack_rows(_p(W), _p(out), N, K, _stream()), "fstu_pack_rows")
+    return out
+
+
+def glu_packed(x: torch.Tensor, wp_gate: torch.Tensor, wp_up: torch.Tensor, I: int,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gate/up projection + GLU over packed weights (rows <= 16, bf16): x (rows,d) -> act (rows,I)."""
+    _dev(wp_gate, wp_up, out)
+    rows, ldx = _rows_view(x)
+    d = x.shape[1]
+    if x.dtype != torch.bfloat16 or not load().fstu_glu_packed_supported(rows, d, I):
+        raise FlashSTUHipError(f"fstu_glu_packed does not support rows={rows} d={d} I={I} dtype={x.dtype}")
+    if out is None:
+        out = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    _check(load().fstu_glu_packed(_p(x), ldx, _p(wp_gate), _p(wp_up), _p(out), out.stride(0), rows, I, d, _stream()),
+           "fstu_glu_packed")
     return out
 
 

@@ -42,7 +42,7 @@ class ModelDesc(ctypes.Structure):
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
-                ("mlp_partial", _vp), ("mlp_sync", _vp)]
+                ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -232,6 +232,13 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.x2 = buf(B, d).data_ptr()
+        if (dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(B, d, I)
+                and os.environ.get("FSTU_GLU_PACKED", "1") == "1"):
+            # gate/up projection over packed weights, one workgroup per CU with equal bytes each
+            for i, layer in enumerate(model.layers):
+                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
+                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
+            m.glu_packed = 1
         plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
         if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
             # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its

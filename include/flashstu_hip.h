@@ -341,6 +341,15 @@ int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, const void*
                    const void* wp_up, const void* wp_down, const void* next_norm_w, void* h_out, void* act_ws,
                    float* partial_ws, unsigned* sync_ws, int rows, int d, int I, float eps, void* stream);
 
+/* Gate/up projection with the GLU epilogue over packed weights, one workgroup per CU with equal bytes each
+ * (4-feature granularity) and every weight fragment in flight from the first instruction:
+ *   act[r,f] = T( T(gelu_tanh(T(h[r,:].Wg[f,:]))) * T(h[r,:].Wu[f,:]) ),  rows <= 16, bf16.
+ * Same contract as fstu_glu_decode (flash_stu/modules/swiglu.py:23-26); wp_* from fstu_pack_rows.
+ * fstu_glu_packed_supported tells whether a shape is covered (d in {256,512,768,1024,2048}, I % 4 == 0). */
+int fstu_glu_packed_supported(int rows, int d, int I);
+int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
+                    int I, int d, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -414,6 +423,7 @@ typedef struct {
    * are set and the shape is supported */
   float* mlp_partial;       /* fstu_mlp_block_plan's partial_floats */
   unsigned* mlp_sync;       /* fstu_mlp_block_sync_bytes(), zero-initialised once */
+  int glu_packed;           /* != 0: layers with wp_gate and wp_up run their gate/up projection through fstu_glu_packed */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

@@ -579,3 +579,29 @@ def test_stu_step_lds_with_the_reference_lds_fixture(hip):
     scale = float(ref.abs().max())
     print(f"fixture LDS through the step kernel: max error {worst:.3e} of scale {scale:.3e}")
     assert worst <= 2.0 ** -8 * scale * 1.5
+
+
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (1, 256, 512), (16, 512, 1000), (5, 1024, 4096), (8, 2048, 24576),
+                                      (3, 768, 20)])
+def test_glu_packed_balanced(hip, rows, d, I):
+    """Balanced packed gate/up GEMV == the row-major GLU kernel bit for bit is not required (other K split), but both
+    must match the oracle within one bf16 ulp; ragged I (not a multiple of 16 or of the grid)."""
+    dtype = torch.bfloat16
+    g = gen(60)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    # the specification with exact (float64) accumulation and the model's rounding points
+    gate = (x.double() @ wg.double().t()).to(dtype)
+    up = (x.double() @ wu.double().t()).to(dtype)
+    ref = torch.nn.functional.gelu(gate.float(), approximate="tanh").to(dtype) * up
+    out = hip.glu_packed(dev(x), hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu)), I)
+    # act is a product of two rounded factors: a flip of gate (one ulp, stretched by gelu' <= 1.13) and a flip of up
+    # can coincide, so single elements may sit two ulps away; almost all are exact
+    def close(a, b, frac):
+        a, b = a.float().cpu(), b.float().cpu()
+        diff = (a - b).abs()
+        assert bool((diff <= b.abs() * 2.0 ** -6 + 1e-3 * 2.0 ** -7 * float(b.abs().max())).all())
+        assert float((diff > 0).float().mean()) <= frac
+    close(out, ref, 0.05)
+    close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
