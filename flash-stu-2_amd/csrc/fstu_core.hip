@@ -116,6 +116,18 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
   T* xr = x + (size_t)r * d;
   const size_t slice = (size_t)rows * d;
   float v[NG][GW];
+  // the norm weights are fetched up front: loaded after the row statistics they would add a second dependent
+  // memory round trip to a kernel that is nothing but latency
+  float wpre[NG][GW];
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int c = (threadIdx.x + i * FSTU_NORM_THREADS) * GW;
+#pragma unroll
+    for (int k = 0; k < GW; ++k) wpre[i][k] = 0.f;
+    if (y != nullptr && c < d) {
+      if (VEC) Vec4<T>::ld(w + c, wpre[i]); else wpre[i][0] = DT<T>::ld(w + c);
+    }
+  }
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NG; ++i) {
@@ -170,10 +182,9 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
   for (int i = 0; i < NG; ++i) {
     const int c = (threadIdx.x + i * FSTU_NORM_THREADS) * GW;
     if (c < d) {
-      float wv[GW], o[GW];
-      if (VEC) Vec4<T>::ld(w + c, wv); else wv[0] = DT<T>::ld(w + c);
+      float o[GW];
 #pragma unroll
-      for (int k = 0; k < GW; ++k) o[k] = (v[i][k] * rstd) * wv[k];
+      for (int k = 0; k < GW; ++k) o[k] = (v[i][k] * rstd) * wpre[i][k];
       if (VEC) Vec4<T>::st(yr + c, o); else DT<T>::st(yr + c, o[0]);
     }
   }
@@ -227,15 +238,40 @@ embed_rmsnorm_kernel(const int64_t* __restrict__ ids, int64_t id_stride, const T
   int64_t id = ids[(size_t)r * id_stride + (dyn ? dyn[0] : 0)];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + (size_t)id * d;
+  // norm weights and the embedding row are both read before the reduction (up to 8 columns per thread stay in
+  // registers), so that nothing is fetched after it
+  constexpr int PRE = 8;
+  float wv[PRE], xv[PRE];
+#pragma unroll
+  for (int k = 0; k < PRE; ++k) {
+    const int c = threadIdx.x + k * FSTU_NORM_THREADS;
+    wv[k] = (c < d) ? DT<T>::ld(w + c) : 0.f;
+  }
   float ss = 0.f;
-  for (int c = threadIdx.x; c < d; c += FSTU_NORM_THREADS) {
+#pragma unroll
+  for (int k = 0; k < PRE; ++k) {
+    const int c = threadIdx.x + k * FSTU_NORM_THREADS;
+    xv[k] = 0.f;
+    if (c < d) {
+      T raw = src[c];
+      x[(size_t)r * d + c] = raw;
+      xv[k] = DT<T>::ld(&raw);
+      ss = fmaf(xv[k], xv[k], ss);
+    }
+  }
+  for (int c = threadIdx.x + PRE * FSTU_NORM_THREADS; c < d; c += FSTU_NORM_THREADS) {
     T raw = src[c];
     x[(size_t)r * d + c] = raw;
     float v = DT<T>::ld(&raw);
     ss = fmaf(v, v, ss);
   }
   const float rstd = rsqrtf(block_sum_256(ss, red) / (float)d + eps);
-  for (int c = threadIdx.x; c < d; c += FSTU_NORM_THREADS)
+#pragma unroll
+  for (int k = 0; k < PRE; ++k) {
+    const int c = threadIdx.x + k * FSTU_NORM_THREADS;
+    if (c < d) DT<T>::st(h + (size_t)r * d + c, (xv[k] * rstd) * wv[k]);
+  }
+  for (int c = threadIdx.x + PRE * FSTU_NORM_THREADS; c < d; c += FSTU_NORM_THREADS)
     DT<T>::st(h + (size_t)r * d + c, (DT<T>::ld(src + c) * rstd) * DT<T>::ld(w + c));
 }
 

@@ -205,6 +205,26 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __re
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
   const bool xrow = r < B;
   const bf16_t* hp = h + (size_t)(xrow ? r : 0) * ldh + w * kw + g * 16;
+  // ---- the recurrence operands of this thread's first batch row go in flight before the projection: they do
+  // not depend on it, and fetched afterwards they would cost a second dependent trip to memory
+  constexpr int PJ = 8;
+  const int cq = threadIdx.x & 3, jsub = (threadIdx.x >> 2) & 7, bsub = threadIdx.x >> 5;
+  const int c = c0 + cq * 4;
+  float4 phv[PJ], pcj[PJ];
+  float paj[PJ];
+  const bool pre = bsub < B && c < d;
+  {
+    float* st = state + (((size_t)(pre ? bsub : 0) * 2 + parity) * S) * d + (pre ? c : 0);
+#pragma unroll
+    for (int k = 0; k < PJ; ++k) {
+      const int j = jsub + 8 * k;
+      if (pre && j < S) {
+        phv[k] = *(const float4*)(st + (size_t)j * d);
+        pcj[k] = *(const float4*)(ce + (size_t)j * d + c);
+        paj[k] = a[j];
+      }
+    }
+  }
   stu_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
   for (int i0 = 0; i0 < (kw >> 6); i0 += 4) {
     uint4 wa[4][2], xa[4][2];
@@ -246,15 +266,33 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __re
   }
   __syncthreads();
   // ---- recurrence step of the tile's channels
-  const int cq = threadIdx.x & 3, jsub = (threadIdx.x >> 2) & 7, bsub = threadIdx.x >> 5;
-  const int c = c0 + cq * 4;
   for (int b = bsub; b < B; b += 8) {
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c < d) {
       const float x0 = xps[b][cq * 4], x1 = xps[b][cq * 4 + 1], x2 = xps[b][cq * 4 + 2], x3 = xps[b][cq * 4 + 3];
       float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
+      int jstart = jsub;
+      if (b == bsub) {
+#pragma unroll
+        for (int k = 0; k < PJ; ++k) {
+          const int j = jsub + 8 * k;
+          if (j < S) {
+            float4 hv = phv[k];
+            hv.x = fmaf(paj[k], hv.x, x0);
+            hv.y = fmaf(paj[k], hv.y, x1);
+            hv.z = fmaf(paj[k], hv.z, x2);
+            hv.w = fmaf(paj[k], hv.w, x3);
+            *(float4*)(st + (size_t)j * d) = hv;
+            sum.x = fmaf(pcj[k].x, hv.x, sum.x);
+            sum.y = fmaf(pcj[k].y, hv.y, sum.y);
+            sum.z = fmaf(pcj[k].z, hv.z, sum.z);
+            sum.w = fmaf(pcj[k].w, hv.w, sum.w);
+          }
+        }
+        jstart = jsub + 8 * PJ;
+      }
 #pragma unroll 8
-      for (int j = jsub; j < S; j += 8) {
+      for (int j = jstart; j < S; j += 8) {
         float4 hv = *(float4*)(st + (size_t)j * d);
         const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
         const float aj = a[j];
