@@ -206,7 +206,7 @@ def main():
                                "vocab 50257, random-init bf16 seed 1, batch 8, 512-token prompt, greedy decode",
                    "mlp_scale": cfg.mlp_scale, "params": model.get_num_params(), "batch": B, "prompt": P,
                    "stu_decode_mode": args.stu_mode, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
-        "roofline": {"bound": "hbm", "kernel": "linear_mfma_bf16_kernel<GLU> (gate/up projection + gelu*up)",
+        "roofline": {"bound": "hbm", "kernel": ("glu_balanced_kernel" if getattr(eng.desc, "glu_packed", 0) else "linear_mfma_bf16_kernel<GLU>") + " (gate/up projection + gelu*up)",
                      "achieved": glu_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": glu_gbps / HBM_PEAK_GBPS,
                      "traffic": traffic, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,
                      "launches_timed": glu_n},

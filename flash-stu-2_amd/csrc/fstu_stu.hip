@@ -345,7 +345,18 @@ extern "C" int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, floa
 // ---------------------------------------------------------------- state from history
 #define LSH_JG 4
 #define LSH_MAXJ 32
-template <typename T>
+// element t of a (batch, channel) column through a raw buffer load: beyond the descriptor's range the load returns
+// zero without a branch, so a whole batch of loads sits in straight-line code and can stay in flight while the
+// previous batch is consumed
+template <typename T> __device__ __forceinline__ float lsh_load(__amdgpu_buffer_rsrc_t rs, unsigned off);
+template <> __device__ __forceinline__ float lsh_load<float>(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, 0));
+}
+template <> __device__ __forceinline__ float lsh_load<bf16_t>(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+  return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0));
+}
+
+template <typename T, int MAXJ>
 __global__ void __launch_bounds__(256)
 lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__ a, float* __restrict__ state, int S,
                            int d, int t_last, int cap) {
@@ -355,33 +366,36 @@ lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__
   const int per = (S + LSH_JG - 1) / LSH_JG;
   const int j0 = jg * per;
   if (c >= d) return;
-  float h[LSH_MAXJ], aj[LSH_MAXJ];
+  float h[MAXJ], aj[MAXJ];
 #pragma unroll
-  for (int i = 0; i < LSH_MAXJ; ++i) {
+  for (int i = 0; i < MAXJ; ++i) {
     h[i] = 0.f;
     aj[i] = (i < per && j0 + i < S) ? a[j0 + i] : 0.f;
   }
-  const T* hb = hist + (size_t)b * cap * d + c;
-  // 16 inputs are loaded before any is consumed, so the walk is bound by the FMA chains and not by 16x as many
-  // dependent memory latencies
+  // one descriptor per batch row: (t_last+1) rows of d elements
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(hist + (size_t)b * cap * d), 0, (unsigned)((size_t)(t_last + 1) * d * sizeof(T)), 0x00020000);
+  const unsigned row = (unsigned)d * (unsigned)sizeof(T), col = (unsigned)c * (unsigned)sizeof(T);
+  float xn[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) xn[k] = lsh_load<T>(rs, (unsigned)(p + 2 * k) * row + col);
   for (int tt0 = p; tt0 <= t_last; tt0 += 32) {
     float xs[16];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const int tt = tt0 + 2 * k;
-      xs[k] = (tt <= t_last) ? DT<T>::ld(hb + (size_t)tt * d) : 0.f;
-    }
+    for (int k = 0; k < 16; ++k) xs[k] = xn[k];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) xn[k] = lsh_load<T>(rs, (unsigned)(tt0 + 32 + 2 * k) * row + col);   // next batch in flight
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      if (tt0 + 2 * k <= t_last) {
+      if (tt0 + 2 * k <= t_last) {      // a step past the end must not decay the state
 #pragma unroll
-        for (int i = 0; i < LSH_MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
+        for (int i = 0; i < MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
       }
     }
   }
   float* st = state + (((size_t)b * 2 + p) * S) * d + c;
 #pragma unroll
-  for (int i = 0; i < LSH_MAXJ; ++i)
+  for (int i = 0; i < MAXJ; ++i)
     if (i < per && j0 + i < S) st[(size_t)(j0 + i) * d] = h[i];
 }
 
@@ -391,10 +405,17 @@ extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, fl
   FSTU_REQUIRE(B >= 1 && d >= 1 && S >= 1 && S <= LSH_JG * LSH_MAXJ, FSTU_ESHAPE,
                "fstu_stu_lds_state_from_hist: S=%d outside 1..%d", S, LSH_JG * LSH_MAXJ);
   FSTU_REQUIRE(t_last >= -1 && t_last < cap, FSTU_EARG, "fstu_stu_lds_state_from_hist: t_last=%d cap=%d", t_last, cap);
+  FSTU_REQUIRE((size_t)cap * d * 4 < 0xfff00000ull, FSTU_ESHAPE, "fstu_stu_lds_state_from_hist: cap*d too large for 32-bit offsets");
   dim3 grid((d + 63) / 64, B, 2);
-  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
-                      hipLaunchKernelGGL(lds_state_from_hist_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream,
-                                         (const T*)hist, a, state, S, d, t_last, cap));
+  if (S <= LSH_JG * 16) {
+    FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
+                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, 16>), grid, dim3(256), 0, (hipStream_t)stream,
+                                           (const T*)hist, a, state, S, d, t_last, cap));
+  } else {
+    FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
+                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, LSH_MAXJ>), grid, dim3(256), 0, (hipStream_t)stream,
+                                           (const T*)hist, a, state, S, d, t_last, cap));
+  }
   FSTU_CHECK_LAUNCH("fstu_stu_lds_state_from_hist");
   return FSTU_OK;
 }
