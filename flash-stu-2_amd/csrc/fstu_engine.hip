@@ -315,7 +315,11 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                                    m->h, m->act, m->mlp_partial, m->mlp_sync, B, d, I, m->eps, stream));
       continue;
     }
-    if (pending_y && glu_pro && L.wp_gate && L.wp_up) {
+    if (pending_y && glu_bal && m->x2 && L.wp_gate && L.wp_up) {
+      // residual add + mlp_norm as the prologue of the balanced gate/up launch; the stream moves to the other buffer
+      TIMED(PC_GLU, fstu_glu_packed_norm(xc, m->y, xo, L.mlp_norm_w, m->eps, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
+      void* t = xc; xc = xo; xo = t;
+    } else if (pending_y && glu_pro && L.wp_gate && L.wp_up) {
       fstu_gemv_args u = {};
       u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
       u.res_in = xc; u.delta = m->y; u.res_out = xo; u.norm_w = L.mlp_norm_w; u.eps = m->eps;

@@ -420,25 +420,44 @@ mlp_block_kernel(MlpArgs a) {
 // 4-feature granularity (equal bytes per CU), every weight fragment of a workgroup in flight from the first
 // instruction, the 8 waves split K.  Input h is already normalised.
 struct GluArgs {
-  const bf16_t* h;
+  const bf16_t* h;        // normalised input (rows x ldh); unused with the prologue
   const uint4* wp_gate;
   const uint4* wp_up;
   bf16_t* act;
   int rows, d, I, ldh, ldact, fpw;
+  // prologue (PRO): h = rmsnorm(T(x_in + delta)) * norm_w computed by every workgroup; workgroup 0 stores the sum
+  const bf16_t* x_in;
+  const bf16_t* delta;
+  bf16_t* x_out;
+  const bf16_t* norm_w;
+  float eps;
 };
 
-template <int KSA>
+template <int KSA, bool PRO>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(GluArgs a) {
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
+  constexpr int NXC = 4;
   __shared__ float red[DA * 8 * 512];
+  extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int wgi = blockIdx.x;
   const bool xrow = r < a.rows;
   // activations first (they are consumed first), then the weights
   uint4 xa[KSA];
-  {
+  uint4 xv[NXC], dv[NXC], nwv[4];
+  const int nchunk = a.d >> 3, total = a.rows * nchunk;
+  if (PRO) {
+    const rsrc_t rx = make_rsrc(a.x_in, (size_t)total * 16), rd = make_rsrc(a.delta, (size_t)total * 16);
+#pragma unroll
+    for (int j = 0; j < NXC; ++j) {
+      const unsigned q = threadIdx.x + j * 512;
+      xv[j] = buf_load16(rx, q * 16u);
+      dv[j] = buf_load16(rd, q * 16u);
+    }
+    load_norm_w(nwv, a.norm_w, a.d, lane);
+  } else {
     const rsrc_t rh = make_rsrc(a.h, ((size_t)(a.rows - 1) * a.ldh + a.d) * 2);
     const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
 #pragma unroll
@@ -463,6 +482,45 @@ glu_balanced_kernel(GluArgs a) {
   };
 #pragma unroll
   for (int j = 0; j < DA; ++j) load_a(j, ta0 + j);
+
+  if (PRO) {
+    // x' = T(x + delta) -> LDS (workgroup 0 also stores it), rows normalised in place, then this wave's B fragments
+    bf16_t* hs = (bf16_t*)glu_smem;
+    const int ld = a.d + 8;
+    auto add_chunk = [&](uint4 x4, uint4 d4) {
+      unsigned xw[4] = {x4.x, x4.y, x4.z, x4.w}, dw[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float lo = __uint_as_float(xw[i] << 16) + __uint_as_float(dw[i] << 16);
+        float hi = __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dw[i] & 0xffff0000u);
+        xw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+      }
+      return make_uint4(xw[0], xw[1], xw[2], xw[3]);
+    };
+#pragma unroll
+    for (int j = 0; j < NXC; ++j) {
+      const int q = threadIdx.x + j * 512;
+      if (q < total) {
+        const int row = q / nchunk, c = (q - row * nchunk) << 3;
+        const uint4 v = add_chunk(xv[j], dv[j]);
+        *(uint4*)(hs + (size_t)row * ld + c) = v;
+        if (wgi == 0 && a.x_out) *(uint4*)(a.x_out + (size_t)q * 8) = v;
+      }
+    }
+    for (int q = threadIdx.x + NXC * 512; q < total; q += 512) {
+      const int row = q / nchunk, c = (q - row * nchunk) << 3;
+      uint4 v = *(const uint4*)(a.x_in + (size_t)q * 8);
+      if (a.delta) v = add_chunk(v, *(const uint4*)(a.delta + (size_t)q * 8));
+      *(uint4*)(hs + (size_t)row * ld + c) = v;
+      if (wgi == 0 && a.x_out) *(uint4*)(a.x_out + (size_t)q * 8) = v;
+    }
+    __syncthreads();
+    norm_rows(hs, ld, hs, ld, a.norm_w, nwv, a.rows, a.d, a.eps, w, lane);
+    __syncthreads();
+    const bf16_t* hl = hs + (size_t)(xrow ? r : 0) * ld + (w * KSA) * 32 + g * 8;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) xa[u] = xrow ? *(const uint4*)(hl + u * 32) : make_uint4(0, 0, 0, 0);
+  }
 
   for (int t0 = ta0; t0 < ta1; t0 += DA) {
 #pragma unroll
@@ -612,6 +670,45 @@ extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
          I >= 16 && I % 4 == 0 && (size_t)I * d * 2 < 0xfff00000ull;
 }
 
+static int glu_launch(GluArgs& a, bool pro, const char* name, hipStream_t s) {
+  int G = query_cus();
+  FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
+  if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
+  a.fpw = (((a.I + G - 1) / G) + 3) & ~3;
+  const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
+#define GLU_CASE(KSA)                                                                                              \
+  case KSA:                                                                                                        \
+    if (pro) {                                                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, true>),            \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                    \
+      FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                    \
+      hipLaunchKernelGGL((glu_balanced_kernel<KSA, true>), dim3(G), dim3(512), shm, s, a);                         \
+    } else {                                                                                                       \
+      hipLaunchKernelGGL((glu_balanced_kernel<KSA, false>), dim3(G), dim3(512), 0, s, a);                          \
+    }                                                                                                              \
+    break;
+  switch (a.d / 256) {
+    GLU_CASE(1) GLU_CASE(2) GLU_CASE(3) GLU_CASE(4)
+    default:
+      if (pro) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<8, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+        FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);
+        hipLaunchKernelGGL((glu_balanced_kernel<8, true>), dim3(G), dim3(512), shm, s, a);
+      } else {
+        hipLaunchKernelGGL((glu_balanced_kernel<8, false>), dim3(G), dim3(512), 0, s, a);
+      }
+      break;
+  }
+#undef GLU_CASE
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    fstu_set_error("%s: launch failed: %s", name, hipGetErrorString(e));
+    return (int)e;
+  }
+  return FSTU_OK;
+}
+
 extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
                                int I, int d, void* stream) {
   FSTU_REQUIRE(h && wp_gate && wp_up && act, FSTU_ENULL, "fstu_glu_packed: null pointer");
@@ -619,21 +716,27 @@ extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, cons
   FSTU_REQUIRE(ldh >= d && ldh % 8 == 0 && ldact >= I && ldact % 4 == 0, FSTU_ESHAPE, "fstu_glu_packed: ldh=%d ldact=%d", ldh, ldact);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(wp_gate, 16) && fstu_aligned(wp_up, 16) && fstu_aligned(act, 8), FSTU_EALIGN,
                "fstu_glu_packed: pointers must be 16-byte aligned");
-  int G = query_cus();
-  FSTU_REQUIRE(G > 0, FSTU_EARG, "fstu_glu_packed: no device");
-  if (G > (I + 3) / 4) G = (I + 3) / 4;
-  GluArgs a;
+  GluArgs a = {};
   a.h = (const bf16_t*)h; a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
-  a.fpw = (((I + G - 1) / G) + 3) & ~3;
-  hipStream_t s = (hipStream_t)stream;
-  switch (d / 256) {
-    case 1: hipLaunchKernelGGL(glu_balanced_kernel<1>, dim3(G), dim3(512), 0, s, a); break;
-    case 2: hipLaunchKernelGGL(glu_balanced_kernel<2>, dim3(G), dim3(512), 0, s, a); break;
-    case 3: hipLaunchKernelGGL(glu_balanced_kernel<3>, dim3(G), dim3(512), 0, s, a); break;
-    case 4: hipLaunchKernelGGL(glu_balanced_kernel<4>, dim3(G), dim3(512), 0, s, a); break;
-    default: hipLaunchKernelGGL(glu_balanced_kernel<8>, dim3(G), dim3(512), 0, s, a); break;
-  }
-  FSTU_CHECK_LAUNCH("fstu_glu_packed");
-  return FSTU_OK;
+  return glu_launch(a, false, "fstu_glu_packed", (hipStream_t)stream);
+}
+
+extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
+                                    const void* wp_gate, const void* wp_up, void* act, int ldact, int rows, int I, int d,
+                                    void* stream) {
+  FSTU_REQUIRE(x_in && norm_w && wp_gate && wp_up && act, FSTU_ENULL, "fstu_glu_packed_norm: null pointer");
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, d, I), FSTU_ESHAPE, "fstu_glu_packed_norm: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(ldact >= I && ldact % 4 == 0, FSTU_ESHAPE, "fstu_glu_packed_norm: ldact=%d", ldact);
+  FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_glu_packed_norm: x_out must not alias x_in (other workgroups still read it)");
+  FSTU_REQUIRE(fstu_aligned(x_in, 16) && fstu_aligned(delta, 16) && fstu_aligned(x_out, 16) && fstu_aligned(norm_w, 16) &&
+                   fstu_aligned(wp_gate, 16) && fstu_aligned(wp_up, 16) && fstu_aligned(act, 8),
+               FSTU_EALIGN, "fstu_glu_packed_norm: pointers must be 16-byte aligned");
+  FSTU_REQUIRE((size_t)rows * (d + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_glu_packed_norm: rows*d too large for LDS");
+  GluArgs a = {};
+  a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
+  a.rows = rows; a.d = d; a.I = I; a.ldh = d; a.ldact = ldact;
+  a.x_in = (const bf16_t*)x_in; a.delta = (const bf16_t*)delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
+  a.eps = eps;
+  return glu_launch(a, true, "fstu_glu_packed_norm", (hipStream_t)stream);
 }

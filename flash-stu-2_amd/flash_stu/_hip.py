@@ -58,6 +58,7 @@ SIGNATURES = {
     "fstu_set_gemv_target_workgroups": [_i],
     "fstu_glu_packed_supported": [_i, _i, _i],
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_mlp_block_sync_bytes": [],
     "fstu_mlp_block_trace": [_vp],
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
@@ -525,6 +526,20 @@ def glu_packed(x: torch.Tensor, wp_gate: torch.Tensor, wp_up: torch.Tensor, I: i
     _check(load().fstu_glu_packed(_p(x), ldx, _p(wp_gate), _p(wp_up), _p(out), out.stride(0), rows, I, d, _stream()),
            "fstu_glu_packed")
     return out
+
+
+def glu_packed_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                    wp_gate: torch.Tensor, wp_up: torch.Tensor, I: int):
+    """(x + delta, act) with act = GLU(rmsnorm(x + delta) * norm_w): residual add, norm and gate/up in one launch."""
+    _dev(x, delta, norm_w, wp_gate, wp_up)
+    rows, d = x.shape
+    if x.dtype != torch.bfloat16 or not load().fstu_glu_packed_supported(rows, d, I):
+        raise FlashSTUHipError(f"fstu_glu_packed_norm does not support rows={rows} d={d} I={I} dtype={x.dtype}")
+    x_out = torch.empty_like(x)
+    act = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    _check(load().fstu_glu_packed_norm(_p(x), _p(delta), _p(x_out), _p(norm_w), float(eps), _p(wp_gate), _p(wp_up),
+                                       _p(act), I, rows, I, d, _stream()), "fstu_glu_packed_norm")
+    return x_out, act
 
 
 def mlp_block_sync_bytes() -> int:

@@ -239,6 +239,8 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.glu_packed = 1
+            if os.environ.get("FSTU_GLU_NORM", "1") == "1" and B * (d + 8) * 2 <= 96 * 1024:
+                m.x2 = buf(B, d).data_ptr()     # second residual buffer: the MLP norm runs as the gate/up prologue
         plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
         if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
             # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its

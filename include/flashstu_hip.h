@@ -349,6 +349,12 @@ int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, const void*
 int fstu_glu_packed_supported(int rows, int d, int I);
 int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
                     int I, int d, void* stream);
+/* The same launch with the sub-layer's residual add and mlp_norm as its prologue (stu_layer.py:93-96,
+ * attention_layer.py:59-62): x' = T(x_in + delta) (delta may be NULL), h = rmsnorm(x') * norm_w recomputed by every
+ * workgroup while its weight loads are in flight; x' is stored to x_out (may be NULL; must not alias x_in). */
+int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
+                         const void* wp_gate, const void* wp_up, void* act, int ldact, int rows, int I, int d,
+                         void* stream);
 
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of

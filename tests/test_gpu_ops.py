@@ -605,3 +605,28 @@ def test_glu_packed_balanced(hip, rows, d, I):
         assert float((diff > 0).float().mean()) <= frac
     close(out, ref, 0.05)
     close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
+
+
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192)])
+def test_glu_packed_norm_prologue(hip, rows, d, I):
+    """Residual add + RMSNorm as the prologue of the balanced gate/up launch == the separate add+norm kernel followed
+    by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored."""
+    dtype = torch.bfloat16
+    g = gen(61)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    delta = (0.5 * torch.randn(rows, d, generator=g)).to(dtype)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
+    wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    pg, pu = hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu))
+    x_out, act = hip.glu_packed_norm(dev(x), dev(delta), dev(nw), O.RMS_EPS_DEFAULT, pg, pu, I)
+    assert torch.equal(x_out.cpu(), x + delta)
+    h_ref = O.rms_norm(x + delta, nw, O.RMS_EPS_DEFAULT)
+    gate = (h_ref.double() @ wg.double().t()).to(dtype)
+    up = (h_ref.double() @ wu.double().t()).to(dtype)
+    ref = torch.nn.functional.gelu(gate.float(), approximate="tanh").to(dtype) * up
+    diff = (act.float().cpu() - ref.float()).abs()
+    assert bool((diff <= ref.float().abs() * 2.0 ** -6 + 2.0 ** -7 * 2e-2 * float(ref.float().abs().max())).all())
+    assert float((diff > 0).float().mean()) <= 0.10
+    x_out2, act2 = hip.glu_packed_norm(dev(x), None, dev(nw), O.RMS_EPS_DEFAULT, pg, pu, I)
+    assert torch.equal(x_out2.cpu(), x)
