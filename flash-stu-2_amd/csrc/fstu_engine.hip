@@ -279,6 +279,15 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   const bool glu_bal = dt == FSTU_BF16 && m->glu_packed && fstu_glu_packed_supported(B, d, I);
   const bool mlp_fused = dt == FSTU_BF16 && m->mlp_sync && m->mlp_partial &&
                          fstu_mlp_block_plan(B, d, I, nullptr, nullptr, nullptr) == FSTU_OK;
+  // Residual chain: the down projection adds straight into the residual stream (no split across workgroups) and the
+  // next sub-layer normalises it in its own prologue, so no stand-alone add+norm launch remains inside the layers.
+  bool res_chain = m->res_chain && glu_bal && m->x2 && m->stu_mode == 1 && d % 256 == 0 && !mlp_fused &&
+                   (size_t)B * (d + 8) * 2 <= 56 * 1024;
+  for (int l = 0; l < m->n_layers && res_chain; ++l) {
+    const fstu_layer_desc& L = m->layers[l];
+    res_chain = L.wp_gate && L.wp_up && L.wp_down && (L.kind == 0 || L.wp_qkv);
+  }
+  const int down_fpw = (m->down_fpw == 4 || m->down_fpw == 8 || m->down_fpw == 16) ? m->down_fpw : 8;
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     bool pending_y = false;   // m->y holds a sub-layer output not yet added to the residual stream
@@ -293,7 +302,10 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_STU, fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
         TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
-        if (dt == FSTU_BF16 && d % 256 == 0) {
+        if (res_chain) {
+          TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y,
+                                                      d, B, m->lds_S, d, d, pos, dyn, stream));
+        } else if (dt == FSTU_BF16 && d % 256 == 0) {
           TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y, d, nullptr, B,
                                                  m->lds_S, d, d, pos, dyn, stream));
         } else {
@@ -303,7 +315,10 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         pending_y = true;
       }
     } else {
-      TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
+      if (res_chain)
+        TIMED(PC_PROJ, fstu_linear_packed(xc, d, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
+      else
+        TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
                                          m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
       TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
@@ -331,6 +346,12 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_GLU, fstu_glu_packed(m->h, d, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
       else
         TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
+    }
+    if (res_chain) {
+      TIMED(PC_DOWN, fstu_down_packed_res(m->act, I, L.wp_down, xc, xc, B, d, I, down_fpw, stream));
+      if (l + 1 == m->n_layers)   // the head reads normalised rows
+        TIMED(PC_NORM, fstu_add_rmsnorm(xc, nullptr, 0, 1, 0, next_w, m->h, B, d, m->eps, dt, stream));
+      continue;
     }
     TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));

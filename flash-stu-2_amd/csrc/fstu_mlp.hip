@@ -433,7 +433,7 @@ struct GluArgs {
   float eps;
 };
 
-template <int KSA, bool PRO>
+template <int KSA, bool PRO, bool GLU>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(GluArgs a) {
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
@@ -477,7 +477,7 @@ glu_balanced_kernel(GluArgs a) {
     for (int u = 0; u < KSA; ++u) {
       const unsigned off = ok ? abase + ((unsigned)tile * (unsigned)tsa + (unsigned)u * 64u) * 16u : MLP_OOB;
       wa[j][u] = buf_load16(rg, off);
-      wb[j][u] = buf_load16(ru, off);
+      if (GLU) wb[j][u] = buf_load16(ru, off);
     }
   };
 #pragma unroll
@@ -529,14 +529,14 @@ glu_balanced_kernel(GluArgs a) {
 #pragma unroll
       for (int u = 0; u < KSA; ++u) {
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc, 0, 0, 0);
-        acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
+        if (GLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
       }
       load_a(j, t0 + DA + j);
       float* mine = red + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         mine[i] = acc[i];
-        mine[256 + i] = acc2[i];
+        if (GLU) mine[256 + i] = acc2[i];
       }
     }
     __syncthreads();
@@ -549,7 +549,7 @@ glu_balanced_kernel(GluArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           sg[i] += o[i];
-          su[i] += o[256 + i];
+          if (GLU) su[i] += o[256 + i];
         }
       }
       const int fb = tile * 16 + g * 4;
@@ -557,13 +557,99 @@ glu_balanced_kernel(GluArgs a) {
         float o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
-          o[i] = ge * DT<bf16_t>::rnd(su[i]);
+          if (GLU) {
+            float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
+            o[i] = ge * DT<bf16_t>::rnd(su[i]);
+          } else {
+            o[i] = sg[i];
+          }
         }
         *(u64*)(a.act + (size_t)r * a.ldact + fb) = pack4_bf16(o);
       }
     }
     if (t0 + DA < ta1) __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------- down projection + residual, no split across workgroups
+// x_out[r, f] = T( x_res[r, f] + T( act[r, :] . Wd[f, :] ) ): a workgroup owns `fpw` (4, 8 or 16) output features over
+// the WHOLE K range, its 8 waves split K and are reduced through LDS in wave order (deterministic), so the result is
+// complete in one launch and the next kernel can normalise it in its own prologue.  Weight and activation
+// fragments are double-buffered in registers (two chunks of CH k steps in flight per wave).
+struct DownArgs {
+  const bf16_t* act;
+  const uint4* wp_down;
+  const bf16_t* x_res;
+  bf16_t* x_out;
+  int rows, d, I, ldact, fpw;
+};
+
+template <int CH>
+__global__ void __launch_bounds__(512)
+down_res_kernel(DownArgs a) {
+  __shared__ float red[8 * 256];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const bool xrow = r < a.rows;
+  const int f0 = blockIdx.x * a.fpw, f1 = min(a.d, f0 + a.fpw);
+  const int tile = f0 >> 4;
+  const int fr = tile * 16 + r;                           // feature of this lane's A-operand row
+  const bool fok = fr >= f0 && fr < f1;
+  const int ksteps = a.I >> 5;
+  const int kpw = (ksteps + 7) >> 3;
+  const int ks_beg = w * kpw, ks_end = min(ksteps, ks_beg + kpw);
+  const size_t tsb = (size_t)ksteps * 64;
+  const rsrc_t rw = make_rsrc(a.wp_down, (size_t)((a.d + 15) >> 4) * tsb * 16);
+  const rsrc_t rx = make_rsrc(a.act, ((size_t)(a.rows - 1) * a.ldact + a.I) * 2);
+  const unsigned wbase = (unsigned)tile * (unsigned)tsb * 16u;   // byte offset of the tile (tsb 16-byte fragments per tile)
+  const unsigned wlane = (unsigned)lane * 16u;
+  const unsigned xbase = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldact + (unsigned)g * 8u) * 2u;
+  // residual of this lane's 4 output features (D layout: features tile*16 + 4g + i of row r), fetched up front
+  const int fb = tile * 16 + 4 * g;
+  const bool ook = xrow && fb >= f0 && fb < f1;
+  u64 resv = 0;
+  if (w == 0 && ook) resv = *(const u64*)(a.x_res + (size_t)r * a.d + fb);
+  uint4 wA[CH], xA[CH], wB[CH], xB[CH];
+  auto ld = [&](uint4 (&wv)[CH], uint4 (&xv)[CH], int ks0) {
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const int ks = ks0 + u;
+      const bool ok = ks < ks_end;
+      wv[u] = buf_load16(rw, (ok && fok) ? wbase + (unsigned)ks * 1024u + wlane : MLP_OOB);
+      xv[u] = buf_load16(rx, (ok && xrow) ? xbase + (unsigned)ks * 64u : MLP_OOB);
+    }
+  };
+  floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+  auto mm = [&](uint4 (&wv)[CH], uint4 (&xv)[CH]) {
+#pragma unroll
+    for (int u = 0; u < CH; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wv[u]), as_bf16x8(xv[u]), acc, 0, 0, 0);
+  };
+  ld(wA, xA, ks_beg);
+  for (int ks0 = ks_beg; ks0 < ks_end; ks0 += 2 * CH) {
+    ld(wB, xB, ks0 + CH);
+    mm(wA, xA);
+    ld(wA, xA, ks0 + 2 * CH);
+    mm(wB, xB);
+  }
+  float* mine = red + (size_t)(w * 64 + lane) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) mine[i] = acc[i];
+  __syncthreads();
+  if (w == 0 && ook) {
+    float sd[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const float* o = red + (size_t)(s * 64 + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sd[i] += o[i];
+    }
+    const unsigned lo = (unsigned)resv, hi = (unsigned)(resv >> 32);
+    const float xr[4] = {__uint_as_float(lo << 16), __uint_as_float(lo & 0xffff0000u), __uint_as_float(hi << 16),
+                         __uint_as_float(hi & 0xffff0000u)};
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = xr[i] + DT<bf16_t>::rnd(sd[i]);
+    *(u64*)(a.x_out + (size_t)r * a.d + fb) = pack4_bf16(o);
   }
 }
 
@@ -670,37 +756,41 @@ extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
          I >= 16 && I % 4 == 0 && (size_t)I * d * 2 < 0xfff00000ull;
 }
 
-static int glu_launch(GluArgs& a, bool pro, const char* name, hipStream_t s) {
+template <int KSA>
+static int glu_launch_ksa(GluArgs& a, bool pro, bool glu, int G, size_t shm, const char* name, hipStream_t s) {
+#define GLU_GO(PRO, GLUF)                                                                                        \
+  do {                                                                                                           \
+    if (shm > 0) {                                                                                               \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, PRO, GLUF>),     \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                  \
+      FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                  \
+    }                                                                                                            \
+    hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a);                    \
+  } while (0)
+  if (pro && glu) GLU_GO(true, true);
+  else if (pro) GLU_GO(true, false);
+  else if (glu) GLU_GO(false, true);
+  else GLU_GO(false, false);
+#undef GLU_GO
+  return FSTU_OK;
+}
+
+static int glu_launch(GluArgs& a, bool pro, bool glu, const char* name, hipStream_t s) {
   int G = query_cus();
   FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
   if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
   a.fpw = (((a.I + G - 1) / G) + 3) & ~3;
+  G = (a.I + a.fpw - 1) / a.fpw;
   const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
-#define GLU_CASE(KSA)                                                                                              \
-  case KSA:                                                                                                        \
-    if (pro) {                                                                                                     \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, true>),            \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                    \
-      FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                    \
-      hipLaunchKernelGGL((glu_balanced_kernel<KSA, true>), dim3(G), dim3(512), shm, s, a);                         \
-    } else {                                                                                                       \
-      hipLaunchKernelGGL((glu_balanced_kernel<KSA, false>), dim3(G), dim3(512), 0, s, a);                          \
-    }                                                                                                              \
-    break;
+  int rc;
   switch (a.d / 256) {
-    GLU_CASE(1) GLU_CASE(2) GLU_CASE(3) GLU_CASE(4)
-    default:
-      if (pro) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<8, true>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-        FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);
-        hipLaunchKernelGGL((glu_balanced_kernel<8, true>), dim3(G), dim3(512), shm, s, a);
-      } else {
-        hipLaunchKernelGGL((glu_balanced_kernel<8, false>), dim3(G), dim3(512), 0, s, a);
-      }
-      break;
+    case 1: rc = glu_launch_ksa<1>(a, pro, glu, G, shm, name, s); break;
+    case 2: rc = glu_launch_ksa<2>(a, pro, glu, G, shm, name, s); break;
+    case 3: rc = glu_launch_ksa<3>(a, pro, glu, G, shm, name, s); break;
+    case 4: rc = glu_launch_ksa<4>(a, pro, glu, G, shm, name, s); break;
+    default: rc = glu_launch_ksa<8>(a, pro, glu, G, shm, name, s); break;
   }
-#undef GLU_CASE
+  if (rc) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     fstu_set_error("%s: launch failed: %s", name, hipGetErrorString(e));
@@ -719,7 +809,7 @@ extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, cons
   GluArgs a = {};
   a.h = (const bf16_t*)h; a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
-  return glu_launch(a, false, "fstu_glu_packed", (hipStream_t)stream);
+  return glu_launch(a, false, true, "fstu_glu_packed", (hipStream_t)stream);
 }
 
 extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
@@ -738,5 +828,41 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
   a.rows = rows; a.d = d; a.I = I; a.ldh = d; a.ldact = ldact;
   a.x_in = (const bf16_t*)x_in; a.delta = (const bf16_t*)delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
   a.eps = eps;
-  return glu_launch(a, true, "fstu_glu_packed_norm", (hipStream_t)stream);
+  return glu_launch(a, true, true, "fstu_glu_packed_norm", (hipStream_t)stream);
+}
+
+// y = T(x W^T) over packed W (N,K): x given normalised (norm_w == NULL, x = h with row stride ldx) or as the residual
+// stream to normalise first (norm_w != NULL, rows dense): h = rmsnorm(x) * norm_w in the prologue.
+extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
+                                  int rows, int N, int K, void* stream) {
+  FSTU_REQUIRE(x && wp && y, FSTU_ENULL, "fstu_linear_packed: null pointer");
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N), FSTU_ESHAPE, "fstu_linear_packed: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && ldy % 4 == 0, FSTU_ESHAPE, "fstu_linear_packed: ldx=%d ldy=%d", ldx, ldy);
+  FSTU_REQUIRE(norm_w == nullptr || ldx == K, FSTU_ESHAPE, "fstu_linear_packed: the norm prologue needs dense rows");
+  FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(wp, 16) && fstu_aligned(y, 8), FSTU_EALIGN,
+               "fstu_linear_packed: pointers must be 16-byte aligned");
+  FSTU_REQUIRE(norm_w == nullptr || (size_t)rows * (K + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_linear_packed: rows*K too large for LDS");
+  GluArgs a = {};
+  a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)y;
+  a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
+  if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
+  return glu_launch(a, norm_w != nullptr, false, "fstu_linear_packed", (hipStream_t)stream);
+}
+
+extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
+                                    int d, int I, int fpw, void* stream) {
+  FSTU_REQUIRE(act && wp_down && x_res && x_out, FSTU_ENULL, "fstu_down_packed_res: null pointer");
+  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d >= 4 && d % 4 == 0 && I >= 32 && I % 32 == 0 &&
+                   (size_t)I * d * 2 < 0xfff00000ull,
+               FSTU_ESHAPE, "fstu_down_packed_res: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(fpw == 4 || fpw == 8 || fpw == 16, FSTU_EARG, "fstu_down_packed_res: fpw=%d not in {4,8,16}", fpw);
+  FSTU_REQUIRE(ldact >= I && ldact % 8 == 0, FSTU_ESHAPE, "fstu_down_packed_res: ldact=%d", ldact);
+  FSTU_REQUIRE(fstu_aligned(act, 16) && fstu_aligned(wp_down, 16) && fstu_aligned(x_res, 8) && fstu_aligned(x_out, 8),
+               FSTU_EALIGN, "fstu_down_packed_res: pointers must be 16-byte aligned");
+  DownArgs a;
+  a.act = (const bf16_t*)act; a.wp_down = (const uint4*)wp_down; a.x_res = (const bf16_t*)x_res; a.x_out = (bf16_t*)x_out;
+  a.rows = rows; a.d = d; a.I = I; a.ldact = ldact; a.fpw = fpw;
+  hipLaunchKernelGGL(down_res_kernel<9>, dim3((d + fpw - 1) / fpw), dim3(512), 0, (hipStream_t)stream, a);
+  FSTU_CHECK_LAUNCH("fstu_down_packed_res");
+  return FSTU_OK;
 }

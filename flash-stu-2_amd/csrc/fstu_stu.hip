@@ -193,9 +193,12 @@ __global__ void __launch_bounds__(256)
 stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
                        float* __restrict__ state, const float* __restrict__ a, const float* __restrict__ ce,
                        bf16_t* __restrict__ y, int ldy, bf16_t* __restrict__ xp_out /*optional (B,d)*/, int B, int S,
-                       int d, int K, int parity, const int* __restrict__ dyn) {
+                       int d, int K, int parity, const int* __restrict__ dyn,
+                       const bf16_t* __restrict__ x_res /*optional (B,K): normalise it instead of reading h*/,
+                       const bf16_t* __restrict__ norm_w, float eps) {
   __shared__ float red[4][64][4];
   __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
+  extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
   if (dyn) parity = dyn[0] & 1;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -204,7 +207,7 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __re
   const int kw = K >> 2;                                    // k range of this wave
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
   const bool xrow = r < B;
-  const bf16_t* hp = h + (size_t)(xrow ? r : 0) * ldh + w * kw + g * 16;
+  const bf16_t* hp = h + (size_t)(xrow ? r : 0) * ldh + w * kw + g * 16;   // re-pointed at LDS by the norm prologue
   // ---- the recurrence operands of this thread's first batch row go in flight before the projection: they do
   // not depend on it, and fetched afterwards they would cost a second dependent trip to memory
   constexpr int PJ = 8;
@@ -226,14 +229,66 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __re
     }
   }
   stu_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+  // first batch of projection weights in flight before the optional norm prologue
+  uint4 wa[4][2], xa[4][2];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    if (u < (kw >> 6)) {
+      const uint4* p = (const uint4*)(wp + (size_t)u * 64);
+      wa[u][0] = p[0];
+      wa[u][1] = p[1];
+    }
+  }
+  const int ldn = K + 8;
+  if (x_res) {
+    // h = rmsnorm(x_res) * norm_w for all rows into LDS (every workgroup recomputes it: B*K*2 bytes of input)
+    bf16_t* hs = (bf16_t*)inproj_smem;
+    const int nchunk = K >> 3;
+    for (int q = threadIdx.x; q < B * nchunk; q += 256) {
+      const int row = q / nchunk, c8 = (q - row * nchunk) << 3;
+      *(uint4*)(hs + (size_t)row * ldn + c8) = *(const uint4*)(x_res + (size_t)q * 8);
+    }
+    __syncthreads();
+    for (int row = w; row < B; row += 4) {
+      bf16_t* hr = hs + (size_t)row * ldn;
+      float ss = 0.f;
+      for (int c8 = lane * 8; c8 < K; c8 += 512) {
+        uint4 v = *(const uint4*)(hr + c8);
+        unsigned vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float lo = __uint_as_float(vw[i] << 16), hi = __uint_as_float(vw[i] & 0xffff0000u);
+          ss = fmaf(lo, lo, ss);
+          ss = fmaf(hi, hi, ss);
+        }
+      }
+      ss = wave_sum(ss);
+      const float rstd = rsqrtf(ss / (float)K + eps);
+      for (int c8 = lane * 8; c8 < K; c8 += 512) {
+        uint4 v = *(const uint4*)(hr + c8);
+        uint4 wv = *(const uint4*)(norm_w + c8);
+        unsigned vw[4] = {v.x, v.y, v.z, v.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float lo = (__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16);
+          float hi = (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u);
+          vw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+        }
+        *(uint4*)(hr + c8) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+      }
+    }
+    __syncthreads();
+    hp = hs + (size_t)(xrow ? r : 0) * ldn + w * kw + g * 16;
+  }
   for (int i0 = 0; i0 < (kw >> 6); i0 += 4) {
-    uint4 wa[4][2], xa[4][2];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       if (i0 + u < (kw >> 6)) {
-        const uint4* p = (const uint4*)(wp + (size_t)(i0 + u) * 64);
-        wa[u][0] = p[0];
-        wa[u][1] = p[1];
+        if (i0 > 0) {
+          const uint4* p = (const uint4*)(wp + (size_t)(i0 + u) * 64);
+          wa[u][0] = p[0];
+          wa[u][1] = p[1];
+        }
         if (xrow) {
           const uint4* q = (const uint4*)(hp + (size_t)(i0 + u) * 64);
           xa[u][0] = q[0];
@@ -325,14 +380,35 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __re
   }
 }
 
+static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
+                              float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
+                              int K, int t, const int* dyn, void* stream);
+
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
                              int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream) {
+  return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, y, ldy, xp_out, B, S, d, K, t, dyn, stream);
+}
+
+int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
+                                  const float* ce, void* y, int ldy, int B, int S, int d, int K, int t, const int* dyn,
+                                  void* stream) {
+  FSTU_REQUIRE(x_res && norm_w, FSTU_ENULL, "fstu_stu_norm_inproj_step: null pointer");
+  return inproj_step_launch(x_res, K, x_res, norm_w, eps, Mt, state, a, ce, y, ldy, nullptr, B, S, d, K, t, dyn, stream);
+}
+
+static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
+                              float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
+                              int K, int t, const int* dyn, void* stream) {
   FSTU_REQUIRE(h && Mt && state && a && ce && y, FSTU_ENULL, "fstu_stu_inproj_step: null pointer");
   FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
   FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(Mt, 16) && fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_inproj_step: pointers must be 16-byte aligned");
-  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)h, ldh,
-                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, ldy, (bf16_t*)xp_out, B, S, d, K, t & 1, dyn);
+  const size_t shm = x_res ? (size_t)B * (K + 8) * 2 : 0;
+  FSTU_REQUIRE(shm <= 56 * 1024, FSTU_ESHAPE, "fstu_stu_inproj_step: B*K too large for the norm prologue");
+  FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w must be 16-byte aligned");
+  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h, ldh,
+                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, ldy, (bf16_t*)xp_out, B, S, d, K, t & 1, dyn,
+                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps);
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
 }

@@ -59,6 +59,8 @@ SIGNATURES = {
     "fstu_glu_packed_supported": [_i, _i, _i],
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_down_packed_res": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_mlp_block_sync_bytes": [],
     "fstu_mlp_block_trace": [_vp],
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
@@ -540,6 +542,30 @@ def glu_packed_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torc
     _check(load().fstu_glu_packed_norm(_p(x), _p(delta), _p(x_out), _p(norm_w), float(eps), _p(wp_gate), _p(wp_up),
                                        _p(act), I, rows, I, d, _stream()), "fstu_glu_packed_norm")
     return x_out, act
+
+
+def linear_packed(x: torch.Tensor, wp: torch.Tensor, N: int, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0):
+    """x (rows,K) @ W^T over packed W (N,K); with norm_w, x is normalised first (rmsnorm * norm_w) in the same launch."""
+    _dev(wp, norm_w)
+    rows, ldx = _rows_view(x)
+    K = x.shape[1]
+    out = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    _check(load().fstu_linear_packed(_p(x), ldx, _p(norm_w), float(eps), _p(wp), _p(out), N, rows, N, K, _stream()),
+           "fstu_linear_packed")
+    return out
+
+
+def down_packed_res(act: torch.Tensor, wp_down: torch.Tensor, x_res: torch.Tensor, fpw: int = 8,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x_res + act @ Wd^T over packed Wd (d,I), complete in one launch; `out` may be x_res itself."""
+    _dev(act, wp_down, x_res, out)
+    rows, I = act.shape
+    d = x_res.shape[1]
+    if out is None:
+        out = torch.empty_like(x_res)
+    _check(load().fstu_down_packed_res(_p(act), I, _p(wp_down), _p(x_res), _p(out), rows, d, I, fpw, _stream()),
+           "fstu_down_packed_res")
+    return out
 
 
 def mlp_block_sync_bytes() -> int:

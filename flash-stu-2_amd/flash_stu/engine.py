@@ -42,7 +42,8 @@ class ModelDesc(ctypes.Structure):
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
-                ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i)]
+                ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
+                ("down_fpw", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -241,6 +242,17 @@ class DecodeEngine:
             m.glu_packed = 1
             if os.environ.get("FSTU_GLU_NORM", "1") == "1" and B * (d + 8) * 2 <= 96 * 1024:
                 m.x2 = buf(B, d).data_ptr()     # second residual buffer: the MLP norm runs as the gate/up prologue
+                if mode == "lds" and d % 256 == 0 and os.environ.get("FSTU_RES_CHAIN", "0") == "1":
+                    # opt-in: down projection adds into the residual stream, the next sub-layer normalises in its
+                    # prologue (12 launches fewer).  Measured slower, 0.503 vs 0.454 ms per step: the down projection
+                    # without a split across workgroups takes 5 us longer than the split-K kernel and the norm
+                    # prologues add 2.8 us to each consumer, more than the removed add+norm launches cost
+                    for i, layer in enumerate(model.layers):
+                        arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
+                        if isinstance(layer, AttentionLayer):
+                            arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                    m.res_chain = 1
+                    m.down_fpw = int(os.environ.get("FSTU_DOWN_FPW", "8"))
         plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
         if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
             # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its

@@ -356,6 +356,18 @@ int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const
                          const void* wp_gate, const void* wp_up, void* act, int ldact, int rows, int I, int d,
                          void* stream);
 
+/* y = T(x W^T) over packed W (N,K) with the same balanced launch; with norm_w != NULL, x is the residual stream
+ * (dense rows) and h = rmsnorm(x) * norm_w is formed in the prologue (the sub-layer norm of stu_layer.py:81 /
+ * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, rows <= 16, bf16. */
+int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
+                       int rows, int N, int K, void* stream);
+/* Down projection with the residual add, complete in one launch (no split across workgroups):
+ *   x_out[r,f] = T( x_res[r,f] + T( act[r,:] . Wd[f,:] ) )      (swiglu.py:27 + the x.add_ of stu_layer.py:96)
+ * wp_down = fstu_pack_rows of down_proj (d,I); a workgroup owns fpw (4, 8 or 16) output features over the whole K range.
+ * x_out may alias x_res. */
+int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
+                         int d, int I, int fpw, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -430,6 +442,10 @@ typedef struct {
   float* mlp_partial;       /* fstu_mlp_block_plan's partial_floats */
   unsigned* mlp_sync;       /* fstu_mlp_block_sync_bytes(), zero-initialised once */
   int glu_packed;           /* != 0: layers with wp_gate and wp_up run their gate/up projection through fstu_glu_packed */
+  int res_chain;            /* != 0 (needs glu_packed, x2, lds mode, wp_down everywhere and wp_qkv on attention layers): the
+                               down projection adds into the residual stream (fstu_down_packed_res) and the next
+                               sub-layer normalises it in its prologue; no stand-alone add+norm launch inside the layers */
+  int down_fpw;             /* output features per workgroup of that down projection: 4, 8 (default) or 16 */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

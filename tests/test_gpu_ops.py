@@ -630,3 +630,37 @@ def test_glu_packed_norm_prologue(hip, rows, d, I):
     assert float((diff > 0).float().mean()) <= 0.10
     x_out2, act2 = hip.glu_packed_norm(dev(x), None, dev(nw), O.RMS_EPS_DEFAULT, pg, pu, I)
     assert torch.equal(x_out2.cpu(), x)
+
+
+@pytest.mark.parametrize("rows,d,I,fpw", [(8, 768, 9216, 8), (8, 768, 9216, 4), (3, 256, 512, 16), (16, 1024, 4096, 8),
+                                          (5, 100, 800, 4)])
+def test_down_packed_res(hip, rows, d, I, fpw):
+    """Down projection + residual add in one launch against the float64-accumulated specification."""
+    dtype = torch.bfloat16
+    g = gen(62)
+    act = torch.randn(rows, I, generator=g).to(dtype)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
+    y = (act.double() @ wd.double().t()).to(dtype)
+    ref = x + y
+    out = hip.down_packed_res(dev(act), hip.pack_rows(dev(wd)), dev(x), fpw)
+    check(out, ref, dtype, frac=0.05, atol=2.0 ** -8 * float(y.float().abs().max()))
+    xin = dev(x).clone()
+    hip.down_packed_res(dev(act), hip.pack_rows(dev(wd)), xin, fpw, out=xin)          # in place
+    assert torch.equal(xin, out)
+
+
+@pytest.mark.parametrize("rows,K,N", [(8, 768, 2304), (8, 768, 768), (4, 256, 96), (16, 1024, 3072)])
+def test_linear_packed_with_and_without_norm(hip, rows, K, N):
+    dtype = torch.bfloat16
+    g = gen(63)
+    x = torch.randn(rows, K, generator=g).to(dtype)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(dtype)
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    wp = hip.pack_rows(dev(W))
+    ref = (x.double() @ W.double().t()).to(dtype)
+    check(hip.linear_packed(dev(x), wp, N), ref, dtype, frac=0.05)
+    h = O.rms_norm(x, nw, O.RMS_EPS_DEFAULT)
+    refn = (h.double() @ W.double().t()).to(dtype)
+    check(hip.linear_packed(dev(x), wp, N, dev(nw), O.RMS_EPS_DEFAULT), refn, dtype, frac=0.10,
+          atol=2.0 ** -7 * 0.05 * float(refn.float().abs().max()))
