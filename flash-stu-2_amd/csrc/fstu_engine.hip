@@ -317,11 +317,16 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     } else {
       if (res_chain)
         TIMED(PC_PROJ, fstu_linear_packed(xc, d, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
+      else if (glu_bal && L.wp_qkv)
+        TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else
         TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
                                          m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
-      TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
+      if (glu_bal && L.wp_proj)
+        TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
+      else
+        TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
       pending_y = true;
     }
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;

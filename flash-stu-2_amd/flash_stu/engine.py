@@ -240,6 +240,11 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.glu_packed = 1
+            if os.environ.get("FSTU_PACKED_QKV", "0") == "1":
+                for i, layer in enumerate(model.layers):
+                    if isinstance(layer, AttentionLayer):
+                        arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                        arr[i].wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
             if os.environ.get("FSTU_GLU_NORM", "1") == "1" and B * (d + 8) * 2 <= 96 * 1024:
                 m.x2 = buf(B, d).data_ptr()     # second residual buffer: the MLP norm runs as the gate/up prologue
                 if mode == "lds" and d % 256 == 0 and os.environ.get("FSTU_RES_CHAIN", "0") == "1":

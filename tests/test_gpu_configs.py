@@ -204,3 +204,21 @@ def test_c5_shape_bf16_lds_teacher_forced():
     ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
     err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
     assert float(err.max()) <= 2e-2
+
+
+@pytest.mark.parametrize("d,heads", [(1024, 8), (2048, 16)])
+def test_c5_width_bf16_step_kernels(d, heads):
+    """Config 5's widths through the whole one-call step (head dim 128, d=2048 takes the 8-k-step variants of the
+    balanced gate/up kernel and its norm prologue): two layers, bf16, logits against the teacher-forced oracle."""
+    from test_gpu_model import make_pair, prompt, _teacher_forced
+    ocfg, w, model = make_pair(seed=4, init="healthy", dtype=torch.bfloat16, mlp_scale=4, n_embd=d, n_layers=2,
+                               n_heads=heads, window_size=32, num_eigh=24, seq_len=128, vocab_size=1511,
+                               stu_decode_mode="lds")
+    P, N = 12, 28
+    ids = prompt(8, P, ocfg.vocab_size, 6)
+    got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
+    again = model.generate(ids.cuda(), max_length=P + N, do_sample=False)        # graph replay
+    assert torch.equal(again, got)
+    ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
+    err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
+    assert float(err.max()) <= 2e-2
