@@ -141,12 +141,12 @@ def main():
         eng.graph_begin(tokens, pos, pos - P + 1, 1.0, None, None, False, 0)
         for _ in range(W):
             eng.graph_step()
-        eng._gstream.synchronize()
+        eng.graph_sync()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(K):
             eng.graph_step()
-        eng._gstream.synchronize()
+        eng.graph_sync()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         eng.graph_end()

@@ -72,6 +72,7 @@ class _Chunk:
         self.logits: Optional[torch.Tensor] = None
         self.graph = None
         self.dyn: Optional[torch.Tensor] = None
+        self.stream = None
 
 
 class DecodeEngine:
@@ -94,6 +95,7 @@ class DecodeEngine:
         self.chunks: List[_Chunk] = []
         self._packed = {}
         self._gstream = None
+        self._gstreams = []
 
     # ------------------------------------------------------------------
     def _pack(self, w: torch.Tensor) -> torch.Tensor:
@@ -303,21 +305,26 @@ class DecodeEngine:
         return self.cfg.resolved_stu_decode_mode() == "lds"
 
     def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed):
-        """Captures one decode step per row chunk as a HIP graph on a side stream.  Each graph_step() then
-        feeds tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
+        """Captures one decode step per row chunk as a HIP graph, each chunk on a side stream of its own: the chunks
+        are independent (own workspaces, state rows and device-side position), so their graphs run concurrently and
+        the second chunk finds the layer's weights, which the first has just streamed, in the Infinity Cache.  Each
+        graph_step() then feeds tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
         self.graph_end()
-        self._gstream = torch.cuda.Stream(device=tokens.device)
-        self._gstream.wait_stream(torch.cuda.current_stream())
+        concurrent = os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1" and os.environ.get("FSTU_FUSED_MLP", "0") != "1"
+        n_streams = len(self.chunks) if concurrent else 1
+        self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
         stride = tokens.stride(0)
         for ch in self.chunks:
             ch.dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
-        self._gstream.wait_stream(torch.cuda.current_stream())
-        for ch in self.chunks:
+        for st in self._gstreams:
+            st.wait_stream(torch.cuda.current_stream())
+        for i, ch in enumerate(self.chunks):
             handle = _vp()
+            ch.stream = self._gstreams[i % n_streams]
             rc = self.lib.fstu_decode_graph_create(ctypes.byref(ch.desc), tokens.data_ptr() + 8 * ch.b0 * stride, stride,
                                                    ch.dyn.data_ptr(), float(temperature), int(top_k) if top_k else 0,
                                                    float(top_p) if top_p else 0.0, int(bool(do_sample)),
-                                                   int(seed) & ((1 << 64) - 1), self._gstream.cuda_stream,
+                                                   int(seed) & ((1 << 64) - 1), ch.stream.cuda_stream,
                                                    ctypes.byref(handle))
             _hip._check(rc, "fstu_decode_graph_create")
             ch.graph = handle
@@ -325,13 +332,19 @@ class DecodeEngine:
 
     def graph_step(self):
         for ch in self.chunks:
-            _hip._check(self.lib.fstu_decode_graph_launch(ch.graph, self._gstream.cuda_stream), "fstu_decode_graph_launch")
+            _hip._check(self.lib.fstu_decode_graph_launch(ch.graph, ch.stream.cuda_stream), "fstu_decode_graph_launch")
+
+    def graph_sync(self):
+        """Blocks until every chunk's replay stream has drained."""
+        for st in self._gstreams:
+            st.synchronize()
 
     def graph_end(self):
         live = [ch for ch in self.chunks if ch.graph is not None]
         if live:
-            torch.cuda.current_stream().wait_stream(self._gstream)
-            self._gstream.synchronize()
+            for st in self._gstreams:
+                torch.cuda.current_stream().wait_stream(st)
+                st.synchronize()
             for ch in live:
                 self.lib.fstu_decode_graph_destroy(ch.graph)
                 ch.graph = None
