@@ -182,6 +182,78 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
   return FSTU_OK;
 }
 
+// ---------------------------------------------------------------- exact mode: filter-bank step on the recurrence state
+// One token of use_approx=False (flash_stu/modules/stu.py:99-120) without re-running the convolution: the two parity
+// banks of state hold h_j = sum_m a_j^m x[t' - 2m] of the raw inputs; with ce/co (S,K) fitted to the even / odd lags
+// of every filter phi_k,
+//   E_k = sum_j ce[j,k] h_j[bank of t],  O_k = sum_j co[j,k] h_j[other bank]   (lag 2m+1 reaches x[t-1-2m])
+//   U+[b,k,c] = T(E_k + O_k),  U-[b,k,c] = T(E_k - O_k)
+// Thread = one (batch, channel); the fitted weights sit in LDS; state traffic is coalesced along the channels.
+#define BANK_MAXK 32
+template <typename T>
+__global__ void __launch_bounds__(256)
+stu_bank_step_kernel(float* __restrict__ state, const T* __restrict__ x, int ldx, const float* __restrict__ a,
+                     const float* __restrict__ ce, const float* __restrict__ co, T* __restrict__ up, T* __restrict__ um,
+                     int S, int d, int K, int parity, const int* __restrict__ dyn) {
+  extern __shared__ float bank_smem[];   // a (S), ce (S*K), co (S*K)
+  float* sa = bank_smem;
+  float* sce = sa + S;
+  float* sco = sce + (size_t)S * K;
+  if (dyn) parity = dyn[0] & 1;
+  for (int i = threadIdx.x; i < S; i += 256) sa[i] = a[i];
+  for (int i = threadIdx.x; i < S * K; i += 256) {
+    sce[i] = ce[i];
+    sco[i] = co ? co[i] : 0.f;
+  }
+  __syncthreads();
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= d) return;
+  const float xv = DT<T>::ld(x + (size_t)b * ldx + c);
+  float* sp = state + (((size_t)b * 2 + parity) * S) * d + c;
+  const float* sq = state + (((size_t)b * 2 + (1 - parity)) * S) * d + c;
+  float E[BANK_MAXK], O[BANK_MAXK];
+#pragma unroll
+  for (int k = 0; k < BANK_MAXK; ++k) E[k] = O[k] = 0.f;
+  for (int j = 0; j < S; ++j) {
+    const float hp = fmaf(sa[j], sp[(size_t)j * d], xv);
+    sp[(size_t)j * d] = hp;
+    const float hq = sq[(size_t)j * d];
+    const float* cej = sce + (size_t)j * K;
+    const float* coj = sco + (size_t)j * K;
+#pragma unroll
+    for (int k = 0; k < BANK_MAXK; ++k) {
+      if (k < K) {
+        E[k] = fmaf(cej[k], hp, E[k]);
+        O[k] = fmaf(coj[k], hq, O[k]);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < BANK_MAXK; ++k) {
+    if (k < K) {
+      DT<T>::st(up + ((size_t)b * K + k) * d + c, E[k] + O[k]);
+      if (um) DT<T>::st(um + ((size_t)b * K + k) * d + c, E[k] - O[k]);
+    }
+  }
+}
+
+extern "C" int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, const float* a, const float* ce, const float* co,
+                                      void* u_plus, void* u_minus, int B, int S, int d, int K, int t, int dtype,
+                                      void* stream) {
+  FSTU_REQUIRE(state && x && a && ce && u_plus, FSTU_ENULL, "fstu_stu_bank_step_lds: null pointer");
+  FSTU_REQUIRE(B >= 1 && B <= 65535 && S >= 1 && d >= 1 && K >= 1 && K <= BANK_MAXK && ldx >= d && t >= 0, FSTU_ESHAPE,
+               "fstu_stu_bank_step_lds: bad shape B=%d S=%d d=%d K=%d (K <= %d)", B, S, d, K, BANK_MAXK);
+  const size_t shm = (size_t)(S + 2 * S * K) * sizeof(float);
+  FSTU_REQUIRE(shm <= 60 * 1024, FSTU_ESHAPE, "fstu_stu_bank_step_lds: S*K too large for LDS");
+  dim3 grid((d + 255) / 256, B);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_bank_step_lds",
+                      hipLaunchKernelGGL(stu_bank_step_kernel<T>, grid, dim3(256), shm, (hipStream_t)stream, state, (const T*)x,
+                                         ldx, a, ce, co, (T*)u_plus, (T*)u_minus, S, d, K, t & 1, (const int*)nullptr));
+  FSTU_CHECK_LAUNCH("fstu_stu_bank_step_lds");
+  return FSTU_OK;
+}
+
 // ---------------------------------------------------------------- input projection + LDS-form step, one launch
 // Workgroup = one tile of 16 channels: x_proj[b, c] = T(h[b,:] . Mt[c,:]) by MFMA (K split over the 4 waves, reduced
 // in LDS), then the recurrence step of those 16 channels for every batch row.  Thread (b, jsub, cq) owns 4 channels

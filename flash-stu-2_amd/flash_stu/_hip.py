@@ -34,6 +34,7 @@ SIGNATURES = {
     "fstu_bias_act": [_vp, _vp, _i64, _i, _i, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -318,6 +319,21 @@ def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, st
     _check(load().fstu_stu_lds_state_from_hist(_p(hist), _p(a), _p(state), B, S, d, t_last, cap, _dt(hist), _stream()),
            "fstu_stu_lds_state_from_hist")
     return state
+
+
+def stu_bank_step_lds(state: torch.Tensor, x: torch.Tensor, a: torch.Tensor, ce: torch.Tensor,
+                      co: Optional[torch.Tensor], t: int):
+    """Exact-mode decode step on the recurrence state: returns (U+, U- or None), each (B,K,d) in x's dtype."""
+    _dev(state, a, ce, co)
+    B, ldx = _rows_view(x)
+    d = x.shape[1]
+    S, K = ce.shape
+    assert state.shape == (B, 2, S, d) and state.dtype == torch.float32 and a.shape == (S,)
+    up = torch.empty(B, K, d, dtype=x.dtype, device=x.device)
+    um = torch.empty_like(up) if co is not None else None
+    _check(load().fstu_stu_bank_step_lds(_p(state), _p(x), ldx, _p(a), _p(ce), _p(co), _p(up), _p(um), B, S, d, K, int(t),
+                                         _dt(x), _stream()), "fstu_stu_bank_step_lds")
+    return up, um
 
 
 def stu_conv_direct(xp: torch.Tensor, filt: torch.Tensor, single_branch: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -101,9 +101,14 @@ class FlashSTUConfig:
     def resolved_stu_decode_mode(self) -> str:
         if self.stu_decode_mode != "auto":
             return self.stu_decode_mode
-        if self.use_hankel_L or not self.use_approx:
+        bf16 = self.torch_dtype == torch.bfloat16
+        if not self.use_approx:
+            # exact mode decodes on the recurrence state of the raw inputs when the filters can be split into equal
+            # even / odd lag halves and fit the bank kernel; otherwise it re-evaluates the bank over the history
+            return "lds" if (bf16 and self.seq_len % 2 == 0 and self.num_eigh <= 32) else "history"
+        if self.use_hankel_L:
             return "history"
-        return "lds" if self.torch_dtype == torch.bfloat16 else "history"
+        return "lds" if bf16 else "history"
 
     # -- serialisation (config.json, HF style)
     def to_dict(self) -> Dict[str, Any]:

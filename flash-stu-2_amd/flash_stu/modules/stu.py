@@ -65,6 +65,11 @@ class STU(nn.Module):
     def decode_mode(self) -> str:
         return self.config.resolved_stu_decode_mode()
 
+    def _exact_lds_ok(self) -> bool:
+        """Exact mode can decode on the recurrence state when asked for explicitly (stu_decode_mode='lds'), the
+        filter length is even (equal pole grids for the even and odd lags) and K fits the bank kernel."""
+        return (not self.use_approx and self.decode_mode() == "lds" and self.phi.shape[0] % 2 == 0 and self.K <= 32)
+
     def effective_filter(self) -> torch.Tensor:
         """phi_proj = phi @ M_filters, (L,d) in the model dtype (stu.py:88)."""
         return self._cached("filt", (self.phi, self.M_filters),
@@ -100,6 +105,28 @@ class STU(nn.Module):
             dev = self.M_filters.device
             return a.to(dev), ce.to(dev).contiguous()
         return self._cached("lds", (self.phi, self.M_filters), build)
+
+    def bank_lds_params(self):
+        """Exact mode: poles a (S) and output weights ce, co (S,K) fitted to the even / odd lags of the filters."""
+        def build():
+            S = self.config.stu_lds_state_dim
+            phi = self.phi
+            a, ce, e1 = fit_even_lag_lds(phi[0::2], S)
+            a2, co, e2 = fit_even_lag_lds(phi[1::2], S)       # odd lags: read from the other parity bank
+            if phi.shape[0] % 2 == 0 and not torch.equal(a, a2):
+                raise RuntimeError("pole grids of the even and odd lags differ")
+            self.lds_fit_error = max(e1, e2)
+            dev = phi.device
+            return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
+        return self._cached("banklds", (self.phi,), build)
+
+    def exact_flat_weights_t(self):
+        """(d_out, K*d_in) copies of M_phi_plus / M_phi_minus for the skinny GEMVs of a decode step."""
+        def build():
+            wp, wm = self.exact_flat_weights()
+            return wp.t().contiguous(), (wm.t().contiguous() if wm is not None else None)
+        params = (self.M_phi_plus,) + (() if self.use_hankel_L else (self.M_phi_minus,))
+        return self._cached("flat_t", params, build)
 
     def exact_flat_weights(self):
         def build():
@@ -183,8 +210,8 @@ class STU(nn.Module):
     def _state_from_sequence(self, src: torch.Tensor):
         B, T, d = src.shape
         pos = torch.full((B,), T, dtype=torch.int64)
-        if self.use_approx and self.decode_mode() == "lds":
-            a, _ = self.lds_params()
+        if self.decode_mode() == "lds" and (self.use_approx or self._exact_lds_ok()):
+            a = self.lds_params()[0] if self.use_approx else self.bank_lds_params()[0]
             state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1)
             return (src.new_empty(B, 0, d), state, pos)
         cap = max(self.config.seq_len, T)
@@ -200,6 +227,16 @@ class STU(nn.Module):
             a, ce = self.lds_params()
             xp = _hip.linear_decode(x, self.m_inputs_t())
             y = _hip.stu_step_lds(state, xp, a, ce, pos)
+            return y, (hist, state, pos_t + 1)
+        if not self.use_approx and state.numel() > 0:
+            # exact mode on the recurrence state: U+- for all K filters, then the two contractions as skinny GEMVs
+            a, ce, co = self.bank_lds_params()
+            up, um = _hip.stu_bank_step_lds(state, x, a, ce, co, pos)
+            wpt, wmt = self.exact_flat_weights_t()
+            if self.use_hankel_L:
+                y = _hip.linear(up.reshape(B, -1), wpt)
+            else:
+                y = _hip.linear(up.reshape(B, -1), wpt) + _hip.linear(um.reshape(B, -1), wmt)
             return y, (hist, state, pos_t + 1)
         if pos >= hist.shape[1]:
             hist = torch.cat([hist, torch.zeros_like(hist)], dim=1)

@@ -127,6 +127,14 @@ int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int
 int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                       int B, int S, int d, int t, int dtype, void* stream);
 
+/* Exact mode (use_approx=False) on the same two-bank state, fed with the raw inputs x (B,d): after advancing the bank
+ * of parity t&1,  E_k = sum_j ce[j,k] h_j[that bank],  O_k = sum_j co[j,k] h_j[other bank]  and
+ *   u_plus[b,k,c] = T(E_k + O_k),  u_minus[b,k,c] = T(E_k - O_k)   (u_minus / co may be NULL: single branch)
+ * with ce, co (S,K) fitted to the even / odd lags of the K filters.  Outputs are (B,K,d); the contraction with
+ * M_phi_plus / M_phi_minus (flash_stu/modules/stu.py:107-120) follows as two skinny GEMVs.  K <= 32. */
+int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, const float* a, const float* ce, const float* co,
+                           void* u_plus, void* u_minus, int B, int S, int d, int K, int t, int dtype, void* stream);
+
 /* Input projection and recurrence step in one launch (bf16, K % 256 == 0):
  *   xp[b,c] = T( h[b,:] . Mt[c,:] )  with Mt = M_inputs^T (d,K) row-major, then the step of
  * fstu_stu_step_lds on xp.  xp_out (B,d) receives xp when not NULL.

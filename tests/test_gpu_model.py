@@ -391,3 +391,22 @@ def test_checkpoint_formats(tmp_path):
     f3 = tmp_path / "model_00100.safetensors"
     save_file({"module." + k: v for k, v in sd.items()}, str(f3))
     assert torch.equal(FlashSTU.from_pretrained(str(f3), config=model.config).cuda()(ids).logits, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_exact_mode_decode_on_the_recurrence_state(dtype):
+    """use_approx=False with stu_decode_mode='lds': one decode step per token on the bank state gives the logits of
+    a full recompute to the fit's accuracy (fp32) / within the bf16 tolerance, and mostly the same greedy ids."""
+    model = _variant_pair(16, dtype=dtype, use_approx=False, n_embd=64, n_heads=2, stu_decode_mode="lds").cuda()
+    assert model.layers[0].stu._exact_lds_ok()
+    ids = torch.randint(0, 211, (3, 10), generator=torch.Generator().manual_seed(9)).cuda()
+    out = model(ids[:, :6], use_cache=True)
+    past = out.past_key_values
+    worst = 0.0
+    for t in range(6, 10):
+        step = model(ids[:, t:t + 1], past_key_values=past, use_cache=True)
+        past = step.past_key_values
+        full = model(ids[:, :t + 1]).logits[:, -1]
+        rel = float((step.logits[:, -1].float() - full.float()).abs().max() / full.float().abs().max())
+        worst = max(worst, rel)
+    assert worst <= (2e-3 if dtype == torch.float32 else 2e-2), worst

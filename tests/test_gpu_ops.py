@@ -664,3 +664,32 @@ def test_linear_packed_with_and_without_norm(hip, rows, K, N):
     refn = (h.double() @ W.double().t()).to(dtype)
     check(hip.linear_packed(dev(x), wp, N, dev(nw), O.RMS_EPS_DEFAULT), refn, dtype, frac=0.10,
           atol=2.0 ** -7 * 0.05 * float(refn.float().abs().max()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stu_bank_step_lds(hip, dtype):
+    """Exact-mode step on the recurrence state == a float64 evaluation of the same recurrence and output maps, and ==
+    the oracle's exact-mode filter-bank convolution when ce/co are fitted to the filters."""
+    from flash_stu.utils.lds_fit import fit_even_lag_lds
+    g = gen(70)
+    B, d, K, S, L, T = 2, 96, 6, 64, 128, 60
+    phi = torch.tensor(O.get_spectral_filters_f64(L, K))
+    a, ce, _ = fit_even_lag_lds(phi[0::2], S)
+    a2, co, _ = fit_even_lag_lds(phi[1::2], S)
+    assert torch.equal(a, a2)
+    x = torch.randn(B, T, d, generator=g).to(dtype)
+    rp, rm = O.convolve(x, phi.to(dtype), O.nearest_power_of_two(2 * L - 1, True), use_approx=False)   # (B,T,K,d)
+    state = torch.zeros(B, 2, S, d, device="cuda")
+    st64 = torch.zeros(B, 2, S, d, dtype=torch.float64)
+    worst = 0.0
+    for t in range(T):
+        up, um = hip.stu_bank_step_lds(state, dev(x[:, t].contiguous()), dev(a), dev(ce), dev(co), t)
+        p = t & 1
+        st64[:, p] = st64[:, p] * a.double()[None, :, None] + x[:, t].double()[:, None, :]
+        E = torch.einsum("jk,bjc->bkc", ce.double(), st64[:, p])
+        Od = torch.einsum("jk,bjc->bkc", co.double(), st64[:, 1 - p])
+        check(up, (E + Od).to(dtype), dtype, frac=0.05, scale=float(rp.float().abs().max()))
+        check(um, (E - Od).to(dtype), dtype, frac=0.05, scale=float(rp.float().abs().max()))
+        worst = max(worst, float((up.float().cpu() - rp[:, t].float()).abs().max()), float((um.float().cpu() - rm[:, t].float()).abs().max()))
+    tol = 1e-3 if dtype == torch.float32 else 2.0 ** -7
+    assert worst <= tol * float(rp.float().abs().max()), worst
