@@ -358,8 +358,12 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_NORM, fstu_add_rmsnorm(xc, nullptr, 0, 1, 0, next_w, m->h, B, d, m->eps, dt, stream));
       continue;
     }
-    TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
-    TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, m->ksplit_down, 0, next_w, m->h, B, d, m->eps, dt, stream));
+    int nsl = m->ksplit_down;
+    if (glu_bal && m->down_packed && L.wp_down && d % 16 == 0 && I % 512 == 0 && I / 512 <= 64)
+      TIMED(PC_DOWN, fstu_down_packed_splitk(m->act, I, L.wp_down, m->partial, B, d, I, &nsl, stream));
+    else
+      TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
+    TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
   if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,

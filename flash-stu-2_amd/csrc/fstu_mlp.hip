@@ -653,6 +653,77 @@ down_res_kernel(DownArgs a) {
   }
 }
 
+// ---------------------------------------------------------------- balanced split-K down projection (stand-alone launch)
+// partial[chunk][row][feature] (fp32 slices, the layout fstu_add_rmsnorm sums): workgroup (tile group, K chunk) as in
+// phase B of mlp_block_kernel, every weight fragment and the activations of the chunk in flight from the first
+// instruction, the 8 waves split the chunk's k steps and are reduced through LDS in wave order.
+struct DownSkArgs {
+  const bf16_t* act;
+  const uint4* wp_down;
+  float* partial;      // KS x rows x d
+  int rows, d, I, ldact, KS, tpw, tiles_out, kch;
+};
+
+template <int KSB>
+__global__ void __launch_bounds__(512)
+down_splitk_balanced_kernel(DownSkArgs a) {
+  constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : 2);
+  __shared__ float red[DB * 8 * 256];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const bool xrow = r < a.rows;
+  const int chunk = blockIdx.x % a.KS, tgrp = blockIdx.x / a.KS;
+  const int tb0 = tgrp * a.tpw, tb1 = min(a.tiles_out, tb0 + a.tpw);
+  const int ksb0 = w * KSB;
+  const int nks = max(0, min(KSB, a.kch - ksb0));
+  const size_t tsb = (size_t)(a.I >> 5) * 64;
+  // activations of this wave's k steps first, then the weights
+  const rsrc_t rx = make_rsrc(a.act, ((size_t)(a.rows - 1) * a.ldact + a.I) * 2);
+  const unsigned xbase = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldact + (unsigned)(chunk * a.kch + ksb0) * 32u + (unsigned)g * 8u) * 2u;
+  uint4 xb[KSB];
+#pragma unroll
+  for (int u = 0; u < KSB; ++u) xb[u] = buf_load16(rx, (xrow && u < nks) ? xbase + (unsigned)u * 64u : MLP_OOB);
+  const rsrc_t rdn = make_rsrc(a.wp_down, (size_t)a.tiles_out * tsb * 16);
+  const unsigned bbase = ((unsigned)(chunk * a.kch + ksb0) * 64 + lane) * 16u;
+  uint4 wd[DB][KSB];
+  auto load_b = [&](int j, int tile) {
+#pragma unroll
+    for (int u = 0; u < KSB; ++u)
+      wd[j][u] = buf_load16(rdn, (u < nks && tile < tb1) ? bbase + ((unsigned)tile * (unsigned)tsb + (unsigned)u * 64u) * 16u : MLP_OOB);
+  };
+#pragma unroll
+  for (int j = 0; j < DB; ++j) load_b(j, tb0 + j);
+  for (int t0 = tb0; t0 < tb1; t0 += DB) {
+#pragma unroll
+    for (int j = 0; j < DB; ++j) {
+      floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < KSB; ++u)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc, 0, 0, 0);
+      load_b(j, t0 + DB + j);
+      float* mine = red + (size_t)((j * 8 + w) * 64 + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[i] = acc[i];
+    }
+    __syncthreads();
+    if (w < DB && t0 + w < tb1) {
+      const int tile = t0 + w;
+      float sd[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const float* o = red + (size_t)((w * 8 + s) * 64 + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sd[i] += o[i];
+      }
+      // D layout: features tile*16 + 4g + i of batch row r
+      const int fb = tile * 16 + 4 * g;
+      if (xrow && fb < a.d)
+        *(float4*)(a.partial + ((size_t)chunk * a.rows + r) * a.d + fb) = make_float4(sd[0], sd[1], sd[2], sd[3]);
+    }
+    if (t0 + DB < tb1) __syncthreads();
+  }
+}
+
 int g_cus = 0;
 long long* g_trace = nullptr;
 
@@ -864,5 +935,42 @@ extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_d
   a.rows = rows; a.d = d; a.I = I; a.ldact = ldact; a.fpw = fpw;
   hipLaunchKernelGGL(down_res_kernel<9>, dim3((d + fpw - 1) / fpw), dim3(512), 0, (hipStream_t)stream, a);
   FSTU_CHECK_LAUNCH("fstu_down_packed_res");
+  return FSTU_OK;
+}
+
+// Balanced split-K down projection: partial (ksplit, rows, d) fp32 slices, summed by fstu_add_rmsnorm(delta_mode 1).
+// Returns the number of slices through *ksplit_out (16, the K chunks of the launch).
+extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
+                                       int* ksplit_out, void* stream) {
+  FSTU_REQUIRE(act && wp_down && partial, FSTU_ENULL, "fstu_down_packed_splitk: null pointer");
+  const int KS = 16;
+  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d >= 16 && d % 16 == 0 && I >= KS * 32 && I % (KS * 32) == 0 &&
+                   (size_t)I * d * 2 < 0xfff00000ull,
+               FSTU_ESHAPE, "fstu_down_packed_splitk: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(ldact >= I && ldact % 8 == 0, FSTU_ESHAPE, "fstu_down_packed_splitk: ldact=%d", ldact);
+  FSTU_REQUIRE(fstu_aligned(act, 16) && fstu_aligned(wp_down, 16) && fstu_aligned(partial, 16), FSTU_EALIGN,
+               "fstu_down_packed_splitk: pointers must be 16-byte aligned");
+  int cus = query_cus();
+  FSTU_REQUIRE(cus > 0, FSTU_EARG, "fstu_down_packed_splitk: no device");
+  DownSkArgs a;
+  a.act = (const bf16_t*)act; a.wp_down = (const uint4*)wp_down; a.partial = partial;
+  a.rows = rows; a.d = d; a.I = I; a.ldact = ldact; a.KS = KS; a.tiles_out = d / 16; a.kch = I / 32 / KS;
+  int ngroups = cus / KS;
+  if (ngroups < 1) ngroups = 1;
+  if (ngroups > a.tiles_out) ngroups = a.tiles_out;
+  a.tpw = (a.tiles_out + ngroups - 1) / ngroups;
+  ngroups = (a.tiles_out + a.tpw - 1) / a.tpw;
+  const int ksb = (a.kch + 7) / 8;
+  FSTU_REQUIRE(ksb <= 8, FSTU_ESHAPE, "fstu_down_packed_splitk: I=%d too large", I);
+  dim3 grid(ngroups * KS);
+  hipStream_t s = (hipStream_t)stream;
+  if (ksb <= 1) hipLaunchKernelGGL(down_splitk_balanced_kernel<1>, grid, dim3(512), 0, s, a);
+  else if (ksb == 2) hipLaunchKernelGGL(down_splitk_balanced_kernel<2>, grid, dim3(512), 0, s, a);
+  else if (ksb == 3) hipLaunchKernelGGL(down_splitk_balanced_kernel<3>, grid, dim3(512), 0, s, a);
+  else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a);
+  else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a);
+  else hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a);
+  FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
+  if (ksplit_out) *ksplit_out = KS;
   return FSTU_OK;
 }

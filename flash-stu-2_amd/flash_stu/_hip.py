@@ -62,6 +62,7 @@ SIGNATURES = {
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_res": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_down_packed_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
     "fstu_mlp_block_sync_bytes": [],
     "fstu_mlp_block_trace": [_vp],
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
@@ -582,6 +583,18 @@ def down_packed_res(act: torch.Tensor, wp_down: torch.Tensor, x_res: torch.Tenso
     _check(load().fstu_down_packed_res(_p(act), I, _p(wp_down), _p(x_res), _p(out), rows, d, I, fpw, _stream()),
            "fstu_down_packed_res")
     return out
+
+
+def down_packed_splitk(act: torch.Tensor, wp_down: torch.Tensor, d: int) -> torch.Tensor:
+    """Balanced split-K down projection: returns the fp32 slices (16, rows, d); their sum in slice order is the result."""
+    _dev(act, wp_down)
+    rows, I = act.shape
+    partial = torch.empty(16, rows, d, dtype=torch.float32, device=act.device)
+    ks = ctypes.c_int(0)
+    _check(load().fstu_down_packed_splitk(_p(act), I, _p(wp_down), _p(partial), rows, d, I, ctypes.byref(ks), _stream()),
+           "fstu_down_packed_splitk")
+    assert ks.value == 16
+    return partial
 
 
 def mlp_block_sync_bytes() -> int:

@@ -43,7 +43,7 @@ class ModelDesc(ctypes.Structure):
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
                 ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
-                ("down_fpw", _i)]
+                ("down_fpw", _i), ("down_packed", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -223,7 +223,7 @@ class DecodeEngine:
         m.x, m.h = buf(B, d).data_ptr(), buf(B, d).data_ptr()
         m.qkv, m.attn = buf(B, 3 * d).data_ptr(), buf(B, d).data_ptr()
         m.act, m.xp, m.y = buf(B, I).data_ptr(), buf(B, d).data_ptr(), buf(B, d).data_ptr()
-        m.partial = buf(m.ksplit_down, B, d, dtype=torch.float32).data_ptr()
+        m.partial = buf(max(m.ksplit_down, 16), B, d, dtype=torch.float32).data_ptr()
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = ch.logits.data_ptr()
         m.best = buf(16 * 64, dtype=torch.int64).data_ptr()
@@ -242,6 +242,10 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.glu_packed = 1
+            if os.environ.get("FSTU_DOWN_PACKED", "1") == "1" and I % 512 == 0 and d % 16 == 0:
+                for i, layer in enumerate(model.layers):
+                    arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
+                m.down_packed = 1
             if os.environ.get("FSTU_PACKED_QKV", "0") == "1":
                 for i, layer in enumerate(model.layers):
                     if isinstance(layer, AttentionLayer):

@@ -376,6 +376,12 @@ int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, co
 int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
                          int d, int I, int fpw, void* stream);
 
+/* Split-K form of the down projection over packed weights, one workgroup per CU: partial receives 16 fp32 slices
+ * (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1, nslices 16) sums in slice order; *ksplit_out = 16.
+ * d % 16 == 0, I % 512 == 0, rows <= 16, bf16.  Same values as fstu_linear_decode_splitk up to the summation order. */
+int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
+                            int* ksplit_out, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -454,6 +460,8 @@ typedef struct {
                                down projection adds into the residual stream (fstu_down_packed_res) and the next
                                sub-layer normalises it in its prologue; no stand-alone add+norm launch inside the layers */
   int down_fpw;             /* output features per workgroup of that down projection: 4, 8 (default) or 16 */
+  int down_packed;          /* != 0: layers with wp_down use fstu_down_packed_splitk (16 slices: partial must hold
+                               max(ksplit_down,16)*B*d floats) */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

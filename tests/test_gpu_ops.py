@@ -693,3 +693,16 @@ def test_stu_bank_step_lds(hip, dtype):
         worst = max(worst, float((up.float().cpu() - rp[:, t].float()).abs().max()), float((um.float().cpu() - rm[:, t].float()).abs().max()))
     tol = 1e-3 if dtype == torch.float32 else 2.0 ** -7
     assert worst <= tol * float(rp.float().abs().max()), worst
+
+
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 24576), (5, 48, 1024)])
+def test_down_packed_splitk(hip, rows, d, I):
+    """Balanced split-K down projection: the 16 slices sum to the float64-accumulated product."""
+    dtype = torch.bfloat16
+    g = gen(64)
+    act = torch.randn(rows, I, generator=g).to(dtype)
+    wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
+    ref = act.double() @ wd.double().t()
+    part = hip.down_packed_splitk(dev(act), hip.pack_rows(dev(wd)), d)
+    got = part.double().sum(0).cpu()
+    assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
