@@ -51,6 +51,9 @@ int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* stat
 int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
                                   const float* ce, void* y, int ldy, int B, int S, int d, int K, int t, const int* dyn,
                                   void* stream);
+int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                                float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
+                                void* stream);
 int fstu_gemv_packed_dyn(const fstu_gemv_args* a, int* dyn, int advance, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

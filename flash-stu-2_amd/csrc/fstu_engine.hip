@@ -365,7 +365,10 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
-  if (!do_sample && m->best) {
+  if (!do_sample && m->best && glu_bal && m->head_packed && m->wp_emb && fstu_glu_packed_supported(B, d, m->V)) {
+    TIMED(PC_HEAD, fstu_head_packed_argmax_dyn(m->h, d, m->wp_emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
+                                               tok_stride, dyn, 1, stream));
+  } else if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
                                         tok_stride, dyn, 1, dt, stream));
   } else {

@@ -322,6 +322,13 @@ argmax_finish_kernel(unsigned long long* best, int64_t* tok_out, int64_t stride,
   if (lane == 0) tok_out[(size_t)b * stride + pos] = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
 }
 
+int fstu_argmax_finish_launch(void* best_ws, int64_t* tok_out, int64_t tok_stride, int rows, int* dyn, int advance, void* stream) {
+  hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(rows * 64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
+                     tok_out, tok_stride, rows, dyn, advance);
+  FSTU_CHECK_LAUNCH("argmax_finish");
+  return FSTU_OK;
+}
+
 extern "C" int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                                 float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
                                 void* stream) {

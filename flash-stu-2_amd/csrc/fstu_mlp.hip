@@ -431,11 +431,16 @@ struct GluArgs {
   bf16_t* x_out;
   const bf16_t* norm_w;
   float eps;
+  // EPI 2: greedy pick fused into the epilogue (packed (value key << 32 | ~index) maxima into 64 slots per row)
+  unsigned long long* best_ws;
+  float temperature;
 };
 
-template <int KSA, bool PRO, bool GLU>
+// EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus the greedy-pick maxima
+template <int KSA, bool PRO, int EPI>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(GluArgs a) {
+  constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
   __shared__ float red[DA * 8 * 512];
@@ -553,18 +558,49 @@ glu_balanced_kernel(GluArgs a) {
         }
       }
       const int fb = tile * 16 + g * 4;
-      if (xrow && fb >= f0 && fb < f1) {
-        float o[4];
+      float o[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (GLU) {
-            float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
-            o[i] = ge * DT<bf16_t>::rnd(su[i]);
-          } else {
-            o[i] = sg[i];
+      for (int i = 0; i < 4; ++i) {
+        if (GLU) {
+          float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
+          o[i] = ge * DT<bf16_t>::rnd(su[i]);
+        } else {
+          o[i] = sg[i];
+        }
+      }
+      const bool grp_ok = xrow && fb >= f0 && fb < f1;
+      if (grp_ok) {
+        bf16_t* yr = a.act + (size_t)r * a.ldact + fb;
+        if (fb + 4 <= f1 && (a.ldact & 3) == 0) {
+          *(u64*)yr = pack4_bf16(o);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (fb + i < f1) yr[i] = f32_to_bf16(o[i]);
+        }
+      }
+      if (EPI == 2) {
+        unsigned long long key = 0ull;
+        if (grp_ok) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int f = fb + i;
+            if (f < f1) {
+              float l = DT<bf16_t>::rnd(o[i]);
+              if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
+              l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
+              unsigned u = __float_as_uint(l);
+              u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+              unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
+              key = k > key ? k : key;
+            }
           }
         }
-        *(u64*)(a.act + (size_t)r * a.ldact + fb) = pack4_bf16(o);
+        unsigned long long ok2 = __shfl_xor(key, 16, FSTU_WAVE);
+        key = ok2 > key ? ok2 : key;
+        ok2 = __shfl_xor(key, 32, FSTU_WAVE);
+        key = ok2 > key ? ok2 : key;
+        if (g == 0 && xrow && key != 0ull) atomicMax(a.best_ws + (size_t)r * 64 + (tile & 63), key);
       }
     }
     if (t0 + DA < ta1) __syncthreads();
@@ -824,11 +860,11 @@ static int query_cus() {
 extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
   const int ksa = d / 256;
   return rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d % 256 == 0 && (ksa == 1 || ksa == 2 || ksa == 3 || ksa == 4 || ksa == 8) &&
-         I >= 16 && I % 4 == 0 && (size_t)I * d * 2 < 0xfff00000ull;
+         I >= 16 && (size_t)I * d * 2 < 0xfff00000ull;
 }
 
 template <int KSA>
-static int glu_launch_ksa(GluArgs& a, bool pro, bool glu, int G, size_t shm, const char* name, hipStream_t s) {
+static int glu_launch_ksa(GluArgs& a, bool pro, int epi, int G, size_t shm, const char* name, hipStream_t s) {
 #define GLU_GO(PRO, GLUF)                                                                                        \
   do {                                                                                                           \
     if (shm > 0) {                                                                                               \
@@ -838,15 +874,16 @@ static int glu_launch_ksa(GluArgs& a, bool pro, bool glu, int G, size_t shm, con
     }                                                                                                            \
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a);                    \
   } while (0)
-  if (pro && glu) GLU_GO(true, true);
-  else if (pro) GLU_GO(true, false);
-  else if (glu) GLU_GO(false, true);
-  else GLU_GO(false, false);
+  if (pro && epi == 0) GLU_GO(true, 0);
+  else if (pro) GLU_GO(true, 1);
+  else if (epi == 0) GLU_GO(false, 0);
+  else if (epi == 1) GLU_GO(false, 1);
+  else GLU_GO(false, 2);
 #undef GLU_GO
   return FSTU_OK;
 }
 
-static int glu_launch(GluArgs& a, bool pro, bool glu, const char* name, hipStream_t s) {
+static int glu_launch(GluArgs& a, bool pro, int epi, const char* name, hipStream_t s) {
   int G = query_cus();
   FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
   if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
@@ -855,11 +892,11 @@ static int glu_launch(GluArgs& a, bool pro, bool glu, const char* name, hipStrea
   const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
   int rc;
   switch (a.d / 256) {
-    case 1: rc = glu_launch_ksa<1>(a, pro, glu, G, shm, name, s); break;
-    case 2: rc = glu_launch_ksa<2>(a, pro, glu, G, shm, name, s); break;
-    case 3: rc = glu_launch_ksa<3>(a, pro, glu, G, shm, name, s); break;
-    case 4: rc = glu_launch_ksa<4>(a, pro, glu, G, shm, name, s); break;
-    default: rc = glu_launch_ksa<8>(a, pro, glu, G, shm, name, s); break;
+    case 1: rc = glu_launch_ksa<1>(a, pro, epi, G, shm, name, s); break;
+    case 2: rc = glu_launch_ksa<2>(a, pro, epi, G, shm, name, s); break;
+    case 3: rc = glu_launch_ksa<3>(a, pro, epi, G, shm, name, s); break;
+    case 4: rc = glu_launch_ksa<4>(a, pro, epi, G, shm, name, s); break;
+    default: rc = glu_launch_ksa<8>(a, pro, epi, G, shm, name, s); break;
   }
   if (rc) return rc;
   hipError_t e = hipGetLastError();
@@ -880,7 +917,7 @@ extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, cons
   GluArgs a = {};
   a.h = (const bf16_t*)h; a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
-  return glu_launch(a, false, true, "fstu_glu_packed", (hipStream_t)stream);
+  return glu_launch(a, false, 0, "fstu_glu_packed", (hipStream_t)stream);
 }
 
 extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
@@ -899,7 +936,7 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
   a.rows = rows; a.d = d; a.I = I; a.ldh = d; a.ldact = ldact;
   a.x_in = (const bf16_t*)x_in; a.delta = (const bf16_t*)delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
   a.eps = eps;
-  return glu_launch(a, true, true, "fstu_glu_packed_norm", (hipStream_t)stream);
+  return glu_launch(a, true, 0, "fstu_glu_packed_norm", (hipStream_t)stream);
 }
 
 // y = T(x W^T) over packed W (N,K): x given normalised (norm_w == NULL, x = h with row stride ldx) or as the residual
@@ -917,7 +954,7 @@ extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, fl
   a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)y;
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
   if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
-  return glu_launch(a, norm_w != nullptr, false, "fstu_linear_packed", (hipStream_t)stream);
+  return glu_launch(a, norm_w != nullptr, 1, "fstu_linear_packed", (hipStream_t)stream);
 }
 
 extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
@@ -973,4 +1010,32 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
   if (ksplit_out) *ksplit_out = KS;
   return FSTU_OK;
+}
+
+// Tied head with the greedy pick over packed weights: logits (rows, ldy) and, through best_ws (rows*64 64-bit words,
+// zero between calls) and the finish launch, the index of the largest logit per row (lowest index on ties).
+int fstu_argmax_finish_launch(void* best_ws, int64_t* tok_out, int64_t tok_stride, int rows, int* dyn, int advance, void* stream);
+
+int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                                float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
+                                void* stream) {
+  FSTU_REQUIRE(x && wp && logits && best_ws && tok_out, FSTU_ENULL, "fstu_head_packed_argmax: null pointer");
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N), FSTU_ESHAPE, "fstu_head_packed_argmax: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && tok_stride >= 1 && temperature > 0.f, FSTU_EARG,
+               "fstu_head_packed_argmax: bad ldx / ldy / stride / temperature");
+  FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(wp, 16) && fstu_aligned(logits, 2) && fstu_aligned(best_ws, 8), FSTU_EALIGN,
+               "fstu_head_packed_argmax: pointers must be 16-byte aligned");
+  GluArgs a = {};
+  a.h = (const bf16_t*)x; a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)logits;
+  a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy;
+  a.best_ws = (unsigned long long*)best_ws; a.temperature = temperature;
+  int rc = glu_launch(a, false, 2, "fstu_head_packed_argmax", (hipStream_t)stream);
+  if (rc) return rc;
+  return fstu_argmax_finish_launch(best_ws, tok_out, tok_stride, rows, dyn, advance, stream);
+}
+
+extern "C" int fstu_head_packed_argmax(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                                       float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, void* stream) {
+  return fstu_head_packed_argmax_dyn(x, ldx, wp, logits, ldy, rows, N, K, temperature, best_ws, tok_out, tok_stride, nullptr, 0,
+                                     stream);
 }

@@ -53,6 +53,7 @@ SIGNATURES = {
     "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
+    "fstu_head_packed_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _vp],
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
     "fstu_packed_elems": [_i, _i],
     "fstu_gemv_packed": [_vp, _vp],
@@ -595,6 +596,19 @@ def down_packed_splitk(act: torch.Tensor, wp_down: torch.Tensor, d: int) -> torc
            "fstu_down_packed_splitk")
     assert ks.value == 16
     return partial
+
+
+def head_packed_argmax(x: torch.Tensor, wp: torch.Tensor, N: int, temperature: float, best_ws: torch.Tensor,
+                       tok_out: torch.Tensor):
+    """Tied head over packed weights + greedy pick: returns logits (rows,N); tok_out (rows,) int64 receives the ids."""
+    _dev(wp, best_ws)
+    rows, ldx = _rows_view(x)
+    K = x.shape[1]
+    logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    assert tok_out.dtype == torch.int64 and tok_out.is_cuda and tok_out.dim() == 1 and tok_out.shape[0] == rows
+    _check(load().fstu_head_packed_argmax(_p(x), ldx, _p(wp), _p(logits), N, rows, N, K, float(temperature), _p(best_ws),
+                                          tok_out.data_ptr(), tok_out.stride(0), _stream()), "fstu_head_packed_argmax")
+    return logits
 
 
 def mlp_block_sync_bytes() -> int:

@@ -43,7 +43,7 @@ class ModelDesc(ctypes.Structure):
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
                 ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
-                ("down_fpw", _i), ("down_packed", _i)]
+                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -246,6 +246,9 @@ class DecodeEngine:
                 for i, layer in enumerate(model.layers):
                     arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
                 m.down_packed = 1
+            if os.environ.get("FSTU_HEAD_PACKED", "0") == "1":     # measured 3 us slower than the row-major head kernel
+                m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
+                m.head_packed = 1
             if os.environ.get("FSTU_PACKED_QKV", "0") == "1":
                 for i, layer in enumerate(model.layers):
                     if isinstance(layer, AttentionLayer):

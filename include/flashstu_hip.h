@@ -382,6 +382,13 @@ int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const 
 int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
                             int* ksplit_out, void* stream);
 
+/* Tied head + greedy pick over packed weights (fstu_pack_rows of the (V,d) embedding), one workgroup per CU:
+ * logits (rows,ldy) and tok_out[b*tok_stride] = argmax_v logits[b,v] (lowest index on ties) after dividing by
+ * temperature and clamping to +-1e4 in the model dtype, as fstu_head_argmax (model.py:176,267-271,299).
+ * best_ws: rows*64 64-bit words, zero before the first call (left zero by every call). */
+int fstu_head_packed_argmax(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                            float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, void* stream);
+
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
  * the input token, the layer stack against its decode state, final norm, tied
@@ -462,6 +469,7 @@ typedef struct {
   int down_fpw;             /* output features per workgroup of that down projection: 4, 8 (default) or 16 */
   int down_packed;          /* != 0: layers with wp_down use fstu_down_packed_splitk (16 slices: partial must hold
                                max(ksplit_down,16)*B*d floats) */
+  int head_packed;          /* != 0 and wp_emb set: the greedy path runs the tied head through fstu_head_packed_argmax */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

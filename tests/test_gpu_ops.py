@@ -706,3 +706,27 @@ def test_down_packed_splitk(hip, rows, d, I):
     part = hip.down_packed_splitk(dev(act), hip.pack_rows(dev(wd)), d)
     got = part.double().sum(0).cpu()
     assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("rows,K,N,temp", [(8, 768, 50257, 1.0), (3, 256, 1001, 0.7), (16, 1024, 4099, 1.0)])
+def test_head_packed_argmax(hip, rows, K, N, temp):
+    """Packed tied head + greedy pick: logits equal to the row-major head kernel's within a bf16 ulp, ids equal to the
+    argmax (lowest index on ties) of its own logits after temperature and clamp; ragged vocabulary sizes."""
+    dtype = torch.bfloat16
+    g = gen(65)
+    x = torch.randn(rows, K, generator=g).to(dtype)
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    best = torch.zeros(16 * 64, dtype=torch.int64, device="cuda")
+    tok = torch.zeros(rows, dtype=torch.int64, device="cuda")
+    logits = hip.head_packed_argmax(dev(x), hip.pack_rows(dev(W)), N, temp, best, tok)
+    ref = (x.double() @ W.double().t()).to(dtype)
+    check(logits, ref, dtype, frac=0.05)
+    l = logits.cpu()
+    if temp != 1.0:
+        l = (l / temp)
+    l = torch.clamp(l, -1e4, 1e4)
+    assert torch.equal(tok.cpu(), l.float().argmax(-1))
+    assert int(best.abs().sum()) == 0
+    tok2 = torch.zeros_like(tok)
+    hip.head_packed_argmax(dev(x), hip.pack_rows(dev(W)), N, temp, best, tok2)      # slots were left clean
+    assert torch.equal(tok2, tok)
