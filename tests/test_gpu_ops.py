@@ -730,3 +730,49 @@ def test_head_packed_argmax(hip, rows, K, N, temp):
     tok2 = torch.zeros_like(tok)
     hip.head_packed_argmax(dev(x), hip.pack_rows(dev(W)), N, temp, best, tok2)      # slots were left clean
     assert torch.equal(tok2, tok)
+
+
+def test_kernels_against_committed_known_answers(hip):
+    """The HIP kernels against tests/golden/kat_small.npz (first-principles float64 vectors, made by
+    tests/golden/make_fixtures.py without any oracle code): both convolution forms, decode and prefill attention,
+    the dense LDS loop and the top-k / top-p survivor sets of the sampler."""
+    import os
+    import numpy as np
+    k = np.load(os.path.join(os.path.dirname(__file__), "golden", "kat_small.npz"))
+    f32 = lambda a: torch.tensor(a, dtype=torch.float32)
+    # convolution: time-domain and FFT form, both branches (mode: single branch = plus; sum = plus + minus)
+    x, f = f32(k["conv_x"])[None], f32(k["conv_f"])
+    plus, both = f32(k["conv_plus"]), f32(k["conv_plus"] + k["conv_minus"])
+    assert float((hip.stu_conv_direct(dev(x), dev(f), single_branch=True)[0].cpu() - plus).abs().max()) < 2e-5
+    assert float((hip.stu_conv_direct(dev(x), dev(f))[0].cpu() - both).abs().max()) < 4e-5
+    n = hip.fft_length(12)
+    assert float((hip.stu_conv_fft(dev(x), hip.stu_fft_filter(dev(f), n, single_branch=True), single_branch=True)[0].cpu()
+                  - plus).abs().max()) < 2e-5
+    assert float((hip.stu_conv_fft(dev(x), hip.stu_fft_filter(dev(f), n))[0].cpu() - both).abs().max()) < 4e-5
+    # attention: prefill kernel and ring decode of the last position
+    q, kk, v = (f32(k[n_]) for n_ in ("att_q", "att_k", "att_v"))          # (T,H,hd)
+    T, H, hd = q.shape
+    qkv = torch.cat([q.reshape(T, H * hd), kk.reshape(T, H * hd), v.reshape(T, H * hd)], dim=1)[None].contiguous()
+    slopes = O.alibi_slopes(H)
+    out = hip.swa_prefill(dev(qkv), dev(slopes), H, 3, 50.0)[0].cpu().reshape(T, H, hd)
+    assert float((out - f32(k["att_out"])).abs().max()) < 5e-6
+    kr = torch.zeros(1, H, 4, hd, device="cuda")
+    vr = torch.zeros_like(kr)
+    hip.kv_fill(dev(qkv[:, : T - 1].contiguous()), kr, vr, 0)
+    o = hip.swa_decode(dev(qkv[:, T - 1].contiguous()), kr, vr, dev(slopes), T - 1, 3, 50.0, append=True)
+    assert float((o.cpu().reshape(H, hd) - f32(k["att_out"])[T - 1]).abs().max()) < 5e-6
+    # dense LDS loop
+    h = torch.zeros(2, 5, device="cuda")
+    y = hip.lds_steps(h, dev(f32(k["lds_x"])), dev(f32(k["lds_A"])), dev(f32(k["lds_B"])), dev(f32(k["lds_C"])))
+    assert float((y.cpu() - f32(k["lds_y"])).abs().max()) < 5e-6
+    # sampler survivor sets: with many seeds every draw must land inside the set, and every member gets drawn
+    lg = f32(k["samp_logits"])
+    for kw, keep in ((dict(top_k=3), k["samp_topk_keep"]), (dict(top_p=0.8), k["samp_topp_keep"])):
+        seen = np.zeros_like(keep)
+        for seed in range(300):
+            out_ids = torch.zeros(2, dtype=torch.int64, device="cuda")
+            hip.sample(dev(lg), out_ids, 1.0, kw.get("top_k"), kw.get("top_p"), True, seed, 0)
+            for b, t in enumerate(out_ids.cpu().tolist()):
+                assert keep[b, t], (kw, b, t)
+                seen[b, t] = True
+        assert np.array_equal(seen, keep)

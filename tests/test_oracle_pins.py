@@ -369,3 +369,33 @@ def test_decode_step_bytes_matches_worked_example():
                          mlp_scale=12)
     b = O.decode_step_bytes(cfg, 8, 2048, state_dim=160)
     assert abs(b / 1e6 - 749.8) < 3.0
+
+
+# ----------------------------------------------------------------- committed known-answer vectors
+def _kat():
+    return np.load(os.path.join(GOLD, "kat_small.npz"))
+
+
+def test_kat_filters_convolution_attention_lds_sampling():
+    """The oracle against tests/golden/kat_small.npz (first-principles float64 loops, tests/golden/make_fixtures.py)."""
+    k = _kat()
+    for name, L, K in (("phi_L8_K3", 8, 3), ("phi_L64_K6", 64, 6)):
+        phi = np.asarray(O.get_spectral_filters_f64(L, K))
+        ref = k[name]
+        for c in range(K):                                    # eigenvector sign is a convention
+            err = min(np.abs(phi[:, c] - ref[:, c]).max(), np.abs(phi[:, c] + ref[:, c]).max())
+            assert err < 1e-9
+    x = torch.tensor(k["conv_x"], dtype=torch.float32)[None]
+    f = torch.tensor(k["conv_f"], dtype=torch.float32)
+    plus, minus = O.convolve(x, f, O.nearest_power_of_two(2 * 12 - 1, True), use_approx=True)
+    assert np.abs(plus[0].numpy() - k["conv_plus"]).max() < 2e-5
+    assert np.abs(minus[0].numpy() - k["conv_minus"]).max() < 2e-5
+    q, kk, v = (torch.tensor(k[n], dtype=torch.float32)[None] for n in ("att_q", "att_k", "att_v"))
+    out = O.attention_core(q, kk, v, 3, O.alibi_slopes(4), 50.0)
+    assert np.abs(out[0].numpy() - k["att_out"]).max() < 2e-6
+    y, _ = O.lds_sequence(torch.tensor(k["lds_x"], dtype=torch.float32), torch.tensor(k["lds_A"], dtype=torch.float32),
+                          torch.tensor(k["lds_B"], dtype=torch.float32), torch.tensor(k["lds_C"], dtype=torch.float32))
+    assert np.abs(y.numpy() - k["lds_y"]).max() < 2e-6
+    lg = torch.tensor(k["samp_logits"], dtype=torch.float32)
+    assert np.array_equal(torch.isfinite(O.filter_logits(lg, top_k=3)).numpy(), k["samp_topk_keep"])
+    assert np.array_equal(torch.isfinite(O.filter_logits(lg, top_p=0.8)).numpy(), k["samp_topp_keep"])
