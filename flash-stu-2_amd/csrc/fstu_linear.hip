@@ -35,9 +35,12 @@ struct LinArgs {
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
 
+// The arguments are passed one by one (not as a struct) so that the command processor can preload them into SGPRs.
 template <int KSW, int MODE>
 __global__ void __launch_bounds__(256)
-linear_mfma_bf16_kernel(LinArgs a) {
+linear_mfma_bf16_kernel(const void* x, const void* W, const void* W2, void* y, unsigned long long* best, int ldx, int ldy,
+                        int rows, int N, int K, int kw, float temperature) {
+  const LinArgs a{x, ldx, W, W2, y, ldy, rows, N, K, kw, best, temperature};
   constexpr int RT = 4 / KSW;
   constexpr int U = 4;  // k steps (of 64) whose loads are issued back to back
   __shared__ float red[(KSW > 1) ? 4 * 64 * 4 * ((MODE == LIN_GLU) ? 2 : 1) : 1];
@@ -231,9 +234,9 @@ static int launch_mfma(LinArgs a, int ksplit, hipStream_t s) {
   int tiles = (a.N + 15) / 16;
   int rt = 4 / ksw;
   dim3 grid((tiles + rt - 1) / rt, ksplit);
-  if (ksw == 4) hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, MODE>), grid, dim3(256), 0, s, a);
-  else if (ksw == 2) hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, MODE>), grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, MODE>), grid, dim3(256), 0, s, a);
+  if (ksw == 4) hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
+  else if (ksw == 2) hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
+  else hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
   return 0;
 }
 

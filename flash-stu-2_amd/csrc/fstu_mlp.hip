@@ -437,9 +437,16 @@ struct GluArgs {
 };
 
 // EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus the greedy-pick maxima
+// (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
 template <int KSA, bool PRO, int EPI>
 __global__ void __launch_bounds__(512)
-glu_balanced_kernel(GluArgs a) {
+glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
+                    const bf16_t* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
+                    int fpw, float eps, float temperature, unsigned long long* best_ws) {
+  GluArgs a;
+  a.h = h; a.wp_gate = wp_gate; a.wp_up = wp_up; a.act = act; a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
+  a.fpw = fpw; a.x_in = x_in; a.delta = delta; a.x_out = x_out; a.norm_w = norm_w; a.eps = eps; a.best_ws = best_ws;
+  a.temperature = temperature;
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
@@ -702,7 +709,9 @@ struct DownSkArgs {
 
 template <int KSB>
 __global__ void __launch_bounds__(512)
-down_splitk_balanced_kernel(DownSkArgs a) {
+down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* partial, int rows, int d, int I, int ldact, int KS,
+                            int tpw, int tiles_out, int kch) {
+  const DownSkArgs a{act, wp_down, partial, rows, d, I, ldact, KS, tpw, tiles_out, kch};
   constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : 2);
   __shared__ float red[DB * 8 * 256];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -872,7 +881,9 @@ static int glu_launch_ksa(GluArgs& a, bool pro, int epi, int G, size_t shm, cons
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                  \
       FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                  \
     }                                                                                                            \
-    hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a);                    \
+    hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,    \
+                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.temperature, a.best_ws); \
+                    \
   } while (0)
   if (pro && epi == 0) GLU_GO(true, 0);
   else if (pro) GLU_GO(true, 1);
@@ -1001,12 +1012,12 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   FSTU_REQUIRE(ksb <= 8, FSTU_ESHAPE, "fstu_down_packed_splitk: I=%d too large", I);
   dim3 grid(ngroups * KS);
   hipStream_t s = (hipStream_t)stream;
-  if (ksb <= 1) hipLaunchKernelGGL(down_splitk_balanced_kernel<1>, grid, dim3(512), 0, s, a);
-  else if (ksb == 2) hipLaunchKernelGGL(down_splitk_balanced_kernel<2>, grid, dim3(512), 0, s, a);
-  else if (ksb == 3) hipLaunchKernelGGL(down_splitk_balanced_kernel<3>, grid, dim3(512), 0, s, a);
-  else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a);
-  else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a);
-  else hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a);
+  if (ksb <= 1) hipLaunchKernelGGL(down_splitk_balanced_kernel<1>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb == 2) hipLaunchKernelGGL(down_splitk_balanced_kernel<2>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb == 3) hipLaunchKernelGGL(down_splitk_balanced_kernel<3>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
   if (ksplit_out) *ksplit_out = KS;
   return FSTU_OK;
