@@ -177,7 +177,8 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 template <typename T, int HD, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64)
 swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__ out, const float* __restrict__ slopes,
-                  int H, int cap, int pos, int window, float softcap, int append, const int* __restrict__ dyn) {
+                  const int* __restrict__ dyn /* early in the list: within the preloaded argument dwords */, int H, int cap,
+                  int pos, int window, float softcap, int append) {
   constexpr int DPL = HD / 8;
   constexpr int NGRP = NWAVES * 8;
   if (dyn) pos = dyn[0];
@@ -261,7 +262,7 @@ int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, c
   const int nkeys = dyn ? window + 1 : (pos < window ? pos : window) + 1;
 #define SWA_LAUNCH(HD, NW)                                                                                      \
   hipLaunchKernelGGL((swa_decode_kernel<T, HD, NW>), dim3(H, B), dim3(NW * 64), 0, s, (const T*)qkv, (T*)kring, \
-                     (T*)vring, (T*)out, slopes, H, cap, pos, window, softcap, append, dyn)
+                     (T*)vring, (T*)out, slopes, dyn, H, cap, pos, window, softcap, append)
   FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_decode", {
     if (hd == 32) { if (nkeys > 128) SWA_LAUNCH(32, 16); else SWA_LAUNCH(32, 4); }
     else if (hd == 64) { if (nkeys > 128) SWA_LAUNCH(64, 16); else SWA_LAUNCH(64, 4); }

@@ -231,8 +231,9 @@ extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int 
 // embedding gather fused with the first RMSNorm of the step: x[r,:] = table[id], h[r,:] = rmsnorm(x[r,:]) * w
 template <typename T>
 __global__ void __launch_bounds__(FSTU_NORM_THREADS)
-embed_rmsnorm_kernel(const int64_t* __restrict__ ids, int64_t id_stride, const T* __restrict__ table, T* __restrict__ x,
-                     const T* __restrict__ w, T* __restrict__ h, int d, int vocab, float eps, const int* __restrict__ dyn) {
+embed_rmsnorm_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, T* __restrict__ x,
+                     const T* __restrict__ w, T* __restrict__ h, const int* __restrict__ dyn, int64_t id_stride, int d,
+                     int vocab, float eps) {
   __shared__ float red[4];
   const int r = blockIdx.x;
   int64_t id = ids[(size_t)r * id_stride + (dyn ? dyn[0] : 0)];
@@ -280,7 +281,7 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
   FSTU_REQUIRE(ids && table && x && w && h, FSTU_ENULL, "fstu_embed_rmsnorm: null pointer");
   FSTU_DISPATCH_DTYPE(dtype, "fstu_embed_rmsnorm",
                       hipLaunchKernelGGL(embed_rmsnorm_kernel<T>, dim3(rows), dim3(FSTU_NORM_THREADS), 0, (hipStream_t)stream,
-                                         ids, id_stride, (const T*)table, (T*)x, (const T*)w, (T*)h, d, vocab, eps, dyn));
+                                         ids, (const T*)table, (T*)x, (const T*)w, (T*)h, dyn, id_stride, d, vocab, eps));
   FSTU_CHECK_LAUNCH("fstu_embed_rmsnorm");
   return FSTU_OK;
 }

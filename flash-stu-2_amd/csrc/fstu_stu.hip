@@ -262,10 +262,11 @@ typedef __bf16 stu_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float stu_floatx4_t __attribute__((ext_vector_type(4)));
 
 __global__ void __launch_bounds__(256)
-stu_inproj_step_kernel(const bf16_t* __restrict__ h, int ldh, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
+stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
                        float* __restrict__ state, const float* __restrict__ a, const float* __restrict__ ce,
-                       bf16_t* __restrict__ y, int ldy, bf16_t* __restrict__ xp_out /*optional (B,d)*/, int B, int S,
-                       int d, int K, int parity, const int* __restrict__ dyn,
+                       bf16_t* __restrict__ y, const int* __restrict__ dyn, int parity /* pointers and the parity first:
+                       these are the kernel-argument dwords the command processor preloads */, int ldh, int ldy,
+                       bf16_t* __restrict__ xp_out /*optional (B,d)*/, int B, int S, int d, int K,
                        const bf16_t* __restrict__ x_res /*optional (B,K): normalise it instead of reading h*/,
                        const bf16_t* __restrict__ norm_w, float eps) {
   __shared__ float red[4][64][4];
@@ -478,8 +479,8 @@ static int inproj_step_launch(const void* h, int ldh, const void* x_res, const v
   const size_t shm = x_res ? (size_t)B * (K + 8) * 2 : 0;
   FSTU_REQUIRE(shm <= 56 * 1024, FSTU_ESHAPE, "fstu_stu_inproj_step: B*K too large for the norm prologue");
   FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w must be 16-byte aligned");
-  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h, ldh,
-                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, ldy, (bf16_t*)xp_out, B, S, d, K, t & 1, dyn,
+  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,
+                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,
                      (const bf16_t*)x_res, (const bf16_t*)norm_w, eps);
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
