@@ -191,13 +191,13 @@ def main():
             _hip._check(lib.fstu_prof_copy(b_.data_ptr(), a_.data_ptr(), a_.numel(), torch.cuda.current_stream().cuda_stream),
                         "fstu_prof_copy")
         torch.cuda.synchronize()
-    glu_bytes = 2 * I * d * 2 + B * d * 2 + B * I * 2          # gate+up weights, x in, act out
+    glu_bytes = 2 * I * d * 2 + B * d * 2 + B * I * 2          # gate+up weights, x in, act out (the fused prologue adds 3*B*d*2 + d*2 bytes: 0.1 %)
     glu_avg_us = glu_ms / glu_n * 1e3
     glu_gbps = glu_bytes / (glu_avg_us * 1e-6) / 1e9
     # HBM bytes per GLU launch from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by what the same
     # counter reads for the library's plain 256 MiB copy kernel: x2.000 and x1.000).  Measured offline for the default
     # workload only; summary and commands in profiles/glu_c2_hbm_traffic_pmc.txt.
-    traffic = 28638208 if (cfg.n_embd, cfg.mlp_scale, B) == (768, 12, 8) else None
+    traffic = 32097280 if (cfg.n_embd, cfg.mlp_scale, B) == (768, 12, 8) else None
     out = {
         "metric": "decode tokens/sec at 1 GPU (768-d FlashSTU, bs=8) + achieved HBM GB/s",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
@@ -206,7 +206,10 @@ def main():
                                "vocab 50257, random-init bf16 seed 1, batch 8, 512-token prompt, greedy decode",
                    "mlp_scale": cfg.mlp_scale, "params": model.get_num_params(), "batch": B, "prompt": P,
                    "stu_decode_mode": args.stu_mode, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
-        "roofline": {"bound": "hbm", "kernel": ("glu_balanced_kernel" if getattr(eng.desc, "glu_packed", 0) else "linear_mfma_bf16_kernel<GLU>") + " (gate/up projection + gelu*up)",
+        "roofline": {"bound": "hbm", "kernel": ("glu_balanced_kernel<PRO> (residual add + mlp_norm + gate/up projection + gelu*up)"
+                                if getattr(eng.desc, "glu_packed", 0) and eng.desc.x2 else
+                                "glu_balanced_kernel (gate/up projection + gelu*up)" if getattr(eng.desc, "glu_packed", 0)
+                                else "linear_mfma_bf16_kernel<GLU> (gate/up projection + gelu*up)"),
                      "achieved": glu_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": glu_gbps / HBM_PEAK_GBPS,
                      "traffic": traffic, "bytes_per_launch": glu_bytes, "avg_launch_us": glu_avg_us,
                      "launches_timed": glu_n},

@@ -59,8 +59,11 @@ extern "C" int fstu_prof_glu_loop(const fstu_model_desc* m, int reps, double* to
   // the same kernel the step launches for this projection
   auto glu = [&](int l) {
     const fstu_layer_desc& L = m->layers[l];
-    if (m->dtype == FSTU_BF16 && m->glu_packed && L.wp_gate && L.wp_up && fstu_glu_packed_supported(m->B, m->d, m->I))
+    if (m->dtype == FSTU_BF16 && m->glu_packed && L.wp_gate && L.wp_up && fstu_glu_packed_supported(m->B, m->d, m->I)) {
+      if (m->x2)   // as in the step: residual add + mlp_norm as the prologue
+        return fstu_glu_packed_norm(m->x, m->y, m->x2, L.mlp_norm_w, m->eps, L.wp_gate, L.wp_up, m->act, m->I, m->B, m->I, m->d, stream);
       return fstu_glu_packed(m->h, m->d, L.wp_gate, L.wp_up, m->act, m->I, m->B, m->I, m->d, stream);
+    }
     return fstu_glu_decode(m->h, m->d, L.w_gate, L.w_up, m->act, m->I, m->B, m->I, m->d, m->dtype, stream);
   };
   for (int l = 0; l < m->n_layers && rc == 0; ++l) rc = glu(l);   // warm-up pass
