@@ -63,12 +63,14 @@ typedef unsigned short bf16_t;  // raw bf16 bits
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((unsigned)v) << 16); }
 
-// round-to-nearest-even; NaN stays NaN
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+// round-to-nearest-even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32, two values per instruction).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
+// (lo, hi) -> two bf16 in one word, lo in the low half
+__device__ __forceinline__ unsigned pack2_bf16(float lo, float hi) {
+  typedef float fstu_f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 fstu_bf16x2 __attribute__((ext_vector_type(2)));
+  fstu_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, fstu_bf16x2));
 }
 
 template <typename T> struct DT;

@@ -70,9 +70,31 @@ __device__ __forceinline__ uint4 buf_load16(rsrc_t rs, unsigned off) {
 }
 
 __device__ __forceinline__ u64 pack4_bf16(const float* v) {
-  unsigned lo = (unsigned)f32_to_bf16(v[0]) | ((unsigned)f32_to_bf16(v[1]) << 16);
-  unsigned hi = (unsigned)f32_to_bf16(v[2]) | ((unsigned)f32_to_bf16(v[3]) << 16);
-  return (u64)lo | ((u64)hi << 32);
+  return (u64)pack2_bf16(v[0], v[1]) | ((u64)pack2_bf16(v[2], v[3]) << 32);
+}
+
+// sum over each aligned group of 32 lanes, returned in every lane of the group (four DPP steps inside a row of 16
+// lanes, one swizzle across the two rows)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+  v += dpp_f32<0xB1>(v);    // quad_perm [1,0,3,2]
+  v += dpp_f32<0x4E>(v);    // quad_perm [2,3,0,1]
+  v += dpp_f32<0x141>(v);   // row_half_mirror
+  v += dpp_f32<0x140>(v);   // row_mirror
+  v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));   // lane ^ 16
+  return v;
+}
+
+// tanh-approximated GELU with tanh(t) = 1 - 2 / (exp(2t) + 1) on the hardware exp and reciprocal: absolute error of
+// 1 + tanh about 1e-7, far below the bf16 rounding that follows
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float e = __builtin_amdgcn_exp2f(2.8853900817779268f * inner);   // exp(2 inner)
+  const float th = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return 0.5f * x * (1.0f + th);
 }
 
 // rows of `src` (LDS, bf16, stride ld) -> T((v * rstd) * w) into dst (stride ld_dst); wave per row.
@@ -438,6 +460,13 @@ struct GluArgs {
 
 // EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus the greedy-pick maxima
 // (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
+#ifdef FSTU_GLU_TRACE
+__device__ long long glu_trace_buf[256 * 8];
+#define GLU_STAMP(k) do { if (threadIdx.x == 0 && blockIdx.x < 256) glu_trace_buf[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+#else
+#define GLU_STAMP(k) do { } while (0)
+#endif
+
 template <int KSA, bool PRO, int EPI>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
@@ -450,31 +479,19 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
+  GLU_STAMP(0);
+#ifdef FSTU_GLU_TRACE
+  if (threadIdx.x == 0 && blockIdx.x == 0) glu_trace_buf[255 * 8 + 7] = (long long)__builtin_amdgcn_s_getpc();
+#endif
   __shared__ float red[DA * 8 * 512];
   extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int wgi = blockIdx.x;
   const bool xrow = r < a.rows;
-  // activations first (they are consumed first), then the weights
   uint4 xa[KSA];
-  uint4 xv[NXC], dv[NXC], nwv[4];
   const int nchunk = a.d >> 3, total = a.rows * nchunk;
-  if (PRO) {
-    const rsrc_t rx = make_rsrc(a.x_in, (size_t)total * 16), rd = make_rsrc(a.delta, (size_t)total * 16);
-#pragma unroll
-    for (int j = 0; j < NXC; ++j) {
-      const unsigned q = threadIdx.x + j * 512;
-      xv[j] = buf_load16(rx, q * 16u);
-      dv[j] = buf_load16(rd, q * 16u);
-    }
-    load_norm_w(nwv, a.norm_w, a.d, lane);
-  } else {
-    const rsrc_t rh = make_rsrc(a.h, ((size_t)(a.rows - 1) * a.ldh + a.d) * 2);
-    const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
-#pragma unroll
-    for (int u = 0; u < KSA; ++u) xa[u] = buf_load16(rh, xrow ? hoff + (unsigned)u * 64u : MLP_OOB);
-  }
+  // weight addressing
   const int f0 = wgi * a.fpw, f1 = min(a.I, f0 + a.fpw);
   const int ta0 = f0 >> 4, ta1 = (f1 > f0) ? ((f1 + 15) >> 4) : ta0;
   const size_t tsa = (size_t)(a.d >> 5) * 64;
@@ -492,43 +509,127 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       if (GLU) wb[j][u] = buf_load16(ru, off);
     }
   };
+  // a tile beyond the workgroup's range is skipped by a uniform branch: a load of nothing still costs its address cycles
+  auto load_first = [&]() {
 #pragma unroll
-  for (int j = 0; j < DA; ++j) load_a(j, ta0 + j);
+    for (int j = 0; j < DA; ++j)
+      if (ta0 + j < ta1) load_a(j, ta0 + j);
+  };
+  // same, but only the last tile is conditional: loads issued earlier keep an exact position in the load counter
+  auto load_first_exact = [&]() {
+#pragma unroll
+    for (int j = 0; j < DA; ++j)
+      if (j < DA - 1 || ta0 + j < ta1) load_a(j, ta0 + j);
+  };
+#ifndef FSTU_GLU_ORDER
+#define FSTU_GLU_ORDER 1
+#endif
 
-  if (PRO) {
-    // x' = T(x + delta) -> LDS (workgroup 0 also stores it), rows normalised in place, then this wave's B fragments
+  if (!PRO) {
+    // activations first (they are consumed first), then the weights
+    const rsrc_t rh = make_rsrc(a.h, ((size_t)(a.rows - 1) * a.ldh + a.d) * 2);
+    const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) xa[u] = buf_load16(rh, xrow ? hoff + (unsigned)u * 64u : MLP_OOB);
+    load_first();
+  } else {
+    // x' = T(x + delta) (workgroup 0 also stores it), h = T((x' * rstd) * w) into LDS, then this wave's B fragments.
+    // The 24 KB of x and delta are requested and consumed BEFORE the weights are requested: they return at
+    // idle-memory latency instead of queueing behind every workgroup's weight stream, nothing the norm needs is
+    // left behind the weight loads in the load counter, and the second half of the norm runs while the weights
+    // arrive.
     bf16_t* hs = (bf16_t*)glu_smem;
     const int ld = a.d + 8;
-    auto add_chunk = [&](uint4 x4, uint4 d4) {
+    __shared__ float ss_part[NXC * 16];
+    const rsrc_t rx = make_rsrc(a.x_in, (size_t)total * 16), rd = make_rsrc(a.delta, (size_t)total * 16);
+    const rsrc_t rn = make_rsrc(a.norm_w, (size_t)a.d * 2);
+    auto add_chunk = [&](uint4 x4, uint4 d4, float& ss) {
       unsigned xw[4] = {x4.x, x4.y, x4.z, x4.w}, dw[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float lo = __uint_as_float(xw[i] << 16) + __uint_as_float(dw[i] << 16);
-        float hi = __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dw[i] & 0xffff0000u);
-        xw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+        xw[i] = pack2_bf16(__uint_as_float(xw[i] << 16) + __uint_as_float(dw[i] << 16),
+                           __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dw[i] & 0xffff0000u));
+        const float lo = __uint_as_float(xw[i] << 16), hi = __uint_as_float(xw[i] & 0xffff0000u);
+        ss = fmaf(lo, lo, ss);
+        ss = fmaf(hi, hi, ss);
       }
       return make_uint4(xw[0], xw[1], xw[2], xw[3]);
     };
+    if ((nchunk & 31) == 0 && total <= NXC * 512) {
+      // a row is a whole number of 32-lane groups: thread q owns chunk q of the (rows x nchunk) grid from load to store
+      uint4 xv[NXC], dv[NXC], nv[NXC];
+      int rowj[NXC];
+      const float inv_nc = 1.0f / (float)nchunk;
 #pragma unroll
-    for (int j = 0; j < NXC; ++j) {
-      const int q = threadIdx.x + j * 512;
-      if (q < total) {
+      for (int j = 0; j < NXC; ++j) {
+        if (j * 512 >= total) continue;   // uniform
+        const int q = threadIdx.x + j * 512;
+        rowj[j] = (int)(((float)q + 0.5f) * inv_nc);
+        xv[j] = buf_load16(rx, (unsigned)q * 16u);     // beyond the last chunk: zeros
+        dv[j] = buf_load16(rd, (unsigned)q * 16u);     // no delta: zeros
+        nv[j] = buf_load16(rn, (unsigned)(q - rowj[j] * nchunk) * 16u);
+      }
+      if (FSTU_GLU_ORDER == 1) load_first_exact();
+#pragma unroll
+      for (int j = 0; j < NXC; ++j) {
+        if (j * 512 >= total) continue;
+        const int q = threadIdx.x + j * 512;
+        float ss = 0.f;
+        xv[j] = add_chunk(xv[j], dv[j], ss);
+        ss = half_wave_sum(ss);
+        if ((lane & 31) == 0) ss_part[q >> 5] = ss;
+        if (wgi == 0 && a.x_out && q < total) *(uint4*)(a.x_out + (size_t)q * 8) = xv[j];
+      }
+      if (FSTU_GLU_ORDER == 0) {
+#pragma unroll
+        for (int j = 0; j < NXC; ++j)
+          if (j * 512 < total) asm volatile("" ::"v"(nv[j].x), "v"(nv[j].y), "v"(nv[j].z), "v"(nv[j].w));   // arrived
+        __builtin_amdgcn_sched_barrier(0);
+        if (blockIdx.x < 255) GLU_STAMP(6);
+        load_first();
+        if (blockIdx.x < 255) GLU_STAMP(7);
+      }
+      __syncthreads();
+      GLU_STAMP(1);
+      const int gpr = nchunk >> 5;
+      const float inv_d = 1.0f / (float)a.d;
+#pragma unroll
+      for (int j = 0; j < NXC; ++j) {
+        if (j * 512 >= total) continue;
+        const int q = threadIdx.x + j * 512;
+        if (q < total) {
+          float ss = 0.f;
+          const float* sp = ss_part + rowj[j] * gpr;
+          for (int i = 0; i < gpr; ++i) ss += sp[i];
+          const float rstd = rsqrtf(ss * inv_d + a.eps);
+          unsigned vw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {nv[j].x, nv[j].y, nv[j].z, nv[j].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            vw[i] = pack2_bf16((__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
+                               (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
+          }
+          *(uint4*)(hs + (size_t)rowj[j] * ld + (size_t)(q - rowj[j] * nchunk) * 8) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+        }
+      }
+    } else {
+      // any other shape: wave per row
+      uint4 nwv[4];
+      load_norm_w(nwv, a.norm_w, a.d, lane);
+      for (int q = threadIdx.x; q < total; q += 512) {
         const int row = q / nchunk, c = (q - row * nchunk) << 3;
-        const uint4 v = add_chunk(xv[j], dv[j]);
+        float ss = 0.f;
+        uint4 v = *(const uint4*)(a.x_in + (size_t)q * 8);
+        if (a.delta) v = add_chunk(v, *(const uint4*)(a.delta + (size_t)q * 8), ss);
         *(uint4*)(hs + (size_t)row * ld + c) = v;
         if (wgi == 0 && a.x_out) *(uint4*)(a.x_out + (size_t)q * 8) = v;
       }
-    }
-    for (int q = threadIdx.x + NXC * 512; q < total; q += 512) {
-      const int row = q / nchunk, c = (q - row * nchunk) << 3;
-      uint4 v = *(const uint4*)(a.x_in + (size_t)q * 8);
-      if (a.delta) v = add_chunk(v, *(const uint4*)(a.delta + (size_t)q * 8));
-      *(uint4*)(hs + (size_t)row * ld + c) = v;
-      if (wgi == 0 && a.x_out) *(uint4*)(a.x_out + (size_t)q * 8) = v;
+      __builtin_amdgcn_sched_barrier(0);
+      load_first();
+      __syncthreads();
+      norm_rows(hs, ld, hs, ld, a.norm_w, nwv, a.rows, a.d, a.eps, w, lane);
     }
     __syncthreads();
-    norm_rows(hs, ld, hs, ld, a.norm_w, nwv, a.rows, a.d, a.eps, w, lane);
-    __syncthreads();
+    GLU_STAMP(2);
     const bf16_t* hl = hs + (size_t)(xrow ? r : 0) * ld + (w * KSA) * 32 + g * 8;
 #pragma unroll
     for (int u = 0; u < KSA; ++u) xa[u] = xrow ? *(const uint4*)(hl + u * 32) : make_uint4(0, 0, 0, 0);
@@ -537,13 +638,14 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
   for (int t0 = ta0; t0 < ta1; t0 += DA) {
 #pragma unroll
     for (int j = 0; j < DA; ++j) {
+      if (t0 + j >= ta1) continue;   // uniform
       floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int u = 0; u < KSA; ++u) {
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc, 0, 0, 0);
         if (GLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
       }
-      load_a(j, t0 + DA + j);
+      if (t0 + DA + j < ta1) load_a(j, t0 + DA + j);   // uniform: a load of nothing still costs its address cycles
       float* mine = red + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -552,37 +654,44 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       }
     }
     __syncthreads();
-    if (w < DA && t0 + w < ta1) {
-      const int tile = t0 + w;
-      float sg[4] = {0.f, 0.f, 0.f, 0.f}, su[4] = {0.f, 0.f, 0.f, 0.f};
+    GLU_STAMP(3);
+    // reduction over the 8 K slices and the epilogue: wave w takes half a tile (two of a lane's four features)
+    if ((w >> 1) < DA && t0 + (w >> 1) < ta1) {
+      const int jt = w >> 1, hf = (w & 1) * 2;
+      const int tile = t0 + jt;
+      float sg[2] = {0.f, 0.f}, su[2] = {0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        const float* o = red + (size_t)((w * 8 + s) * 2 * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          sg[i] += o[i];
-          if (GLU) su[i] += o[256 + i];
+        const float* o = red + (size_t)((jt * 8 + s) * 2 * 64 + lane) * 4 + hf;
+        const float2 pg = *(const float2*)o;
+        sg[0] += pg.x;
+        sg[1] += pg.y;
+        if (GLU) {
+          const float2 pu = *(const float2*)(o + 256);
+          su[0] += pu.x;
+          su[1] += pu.y;
         }
       }
-      const int fb = tile * 16 + g * 4;
-      float o[4];
+      const int fb = tile * 16 + g * 4 + hf;
+      float o[2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 2; ++i) {
         if (GLU) {
-          float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
+          float ge = DT<bf16_t>::rnd(gelu_tanh_fast(DT<bf16_t>::rnd(sg[i])));
           o[i] = ge * DT<bf16_t>::rnd(su[i]);
         } else {
           o[i] = sg[i];
         }
       }
+      // the workgroup's range starts and ends on a multiple of four features, so a pair is inside it or outside it
       const bool grp_ok = xrow && fb >= f0 && fb < f1;
       if (grp_ok) {
         bf16_t* yr = a.act + (size_t)r * a.ldact + fb;
-        if (fb + 4 <= f1 && (a.ldact & 3) == 0) {
-          *(u64*)yr = pack4_bf16(o);
+        if (fb + 2 <= f1 && (a.ldact & 1) == 0) {
+          *(unsigned*)yr = pack2_bf16(o[0], o[1]);
         } else {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < 2; ++i)
             if (fb + i < f1) yr[i] = f32_to_bf16(o[i]);
         }
       }
@@ -590,7 +699,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         unsigned long long key = 0ull;
         if (grp_ok) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
+          for (int i = 0; i < 2; ++i) {
             const int f = fb + i;
             if (f < f1) {
               float l = DT<bf16_t>::rnd(o[i]);
@@ -612,7 +721,28 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     }
     if (t0 + DA < ta1) __syncthreads();
   }
+  GLU_STAMP(4);
 }
+
+#ifdef FSTU_GLU_TRACE
+__global__ void __launch_bounds__(256) touch_kernel(const uint4* p, unsigned n16, unsigned* sink) {
+  unsigned acc = 0;
+  for (unsigned i = threadIdx.x; i < n16; i += 256) {
+    uint4 v = p[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x12345679u) sink[0] = acc;
+}
+}  // namespace
+extern "C" int fstu_glu_trace(long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(glu_trace_buf), sizeof(long long) * 256 * 8);
+}
+extern "C" int fstu_touch(unsigned long long addr, unsigned bytes, void* sink, hipStream_t s) {
+  hipLaunchKernelGGL(touch_kernel, dim3(256), dim3(256), 0, s, (const uint4*)addr, bytes / 16, (unsigned*)sink);
+  return (int)hipGetLastError();
+}
+namespace {
+#endif
 
 // ---------------------------------------------------------------- down projection + residual, no split across workgroups
 // x_out[r, f] = T( x_res[r, f] + T( act[r, :] . Wd[f, :] ) ): a workgroup owns `fpw` (4, 8 or 16) output features over
