@@ -50,18 +50,40 @@ struct Partial {
   float acc[DPL];
 };
 
+// sum over each aligned group of 8 lanes, returned in every lane of the group (DPP, no LDS traffic)
+template <int CTRL>
+__device__ __forceinline__ float swa_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float group8_sum(float v) {
+  v += swa_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+  v += swa_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+  v += swa_dpp<0x141>(v);   // row_half_mirror: the other quad of the 8
+  return v;
+}
+
+// softcap * tanh(s / softcap).  FAST (bf16 models): tanh(t) = 1 - 2 / (exp(2t) + 1) on the hardware exp2 and
+// reciprocal, absolute error about 1e-7 * softcap, far below the bf16 rounding of the operands; the fp32 parity
+// path keeps tanhf.
+template <bool FAST>
+__device__ __forceinline__ float soft_cap(float s, float softcap, float inv_cap2l) {
+  if (FAST) {
+    const float e = __builtin_amdgcn_exp2f(s * inv_cap2l);   // exp(2 s / softcap)
+    return softcap - (2.0f * softcap) * __builtin_amdgcn_rcpf(e + 1.0f);
+  }
+  return softcap * tanhf(s / softcap);
+}
+
 // One key for an 8-lane group: score, soft-cap, ALiBi, online-softmax update.  All 8 lanes of the group call it.
-template <int DPL>
+template <int DPL, bool FAST>
 __device__ __forceinline__ void attend_one(Partial<DPL>& P, const float* q, const float* kk, const float* vv, int j, int pos,
                                            float scale, float softcap, float slope) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) s = fmaf(q[i], kk[i], s);
-  s += __shfl_xor(s, 1, FSTU_WAVE);
-  s += __shfl_xor(s, 2, FSTU_WAVE);
-  s += __shfl_xor(s, 4, FSTU_WAVE);
+  s = group8_sum(s);
   s *= scale;
-  if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+  if (softcap > 0.f) s = soft_cap<FAST>(s, softcap, 2.8853900817779268f / softcap);
   s -= slope * (float)(pos - j);
   float mn = fmaxf(P.m, s);
   float corr = __expf(P.m - mn);
@@ -74,20 +96,26 @@ __device__ __forceinline__ void attend_one(Partial<DPL>& P, const float* q, cons
 
 // Visits keys j = jb+u (u<U) for jb = j_first, j_first+j_step, ... < j_end.
 // kb/vb point at this lane's dims of slot 0; consecutive slots are `stride`
-// elements apart; cap > 0 maps position j to slot j % cap.
-template <typename T, int DPL, int U>
-__device__ __forceinline__ void attend_keys(Partial<DPL>& P, const T* kb, const T* vb, size_t stride, int cap,
-                                            const float* q, int j_first, int j_end, int j_step, int pos, float scale,
-                                            float softcap, float slope) {
+// elements apart.  cap > 0: a ring, key j_lo sits in slot slot_lo (= j_lo % cap, computed once by the caller) and
+// key j in slot_lo + (j - j_lo), wrapped once (j - j_lo < cap).  cap == 0: key j sits in slot j.
+template <typename T, int DPL, int U, bool FAST>
+__device__ __forceinline__ void attend_keys(Partial<DPL>& P, const T* kb, const T* vb, size_t stride, int cap, int j_lo,
+                                            int slot_lo, const float* q, int j_first, int j_end, int j_step, int pos,
+                                            float scale, float softcap, float slope) {
+  const float inv_cap2l = softcap > 0.f ? 2.8853900817779268f / softcap : 0.f;
   for (int jb = j_first; jb < j_end; jb += j_step) {
     float kk[U][DPL], vv[U][DPL];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int j = jb + u;
       if (j < j_end) {
-        size_t slot = cap > 0 ? (size_t)(j % cap) : (size_t)j;
-        load_vec<T, DPL>(kb + slot * stride, kk[u]);
-        load_vec<T, DPL>(vb + slot * stride, vv[u]);
+        int slot = j;
+        if (cap > 0) {
+          slot = slot_lo + (j - j_lo);
+          slot = slot >= cap ? slot - cap : slot;
+        }
+        load_vec<T, DPL>(kb + (size_t)slot * stride, kk[u]);
+        load_vec<T, DPL>(vb + (size_t)slot * stride, vv[u]);
       }
     }
 #pragma unroll
@@ -99,12 +127,10 @@ __device__ __forceinline__ void attend_keys(Partial<DPL>& P, const T* kb, const 
 #pragma unroll
         for (int i = 0; i < DPL; ++i) s = fmaf(q[i], kk[u][i], s);
       }
-      s += __shfl_xor(s, 1, FSTU_WAVE);
-      s += __shfl_xor(s, 2, FSTU_WAVE);
-      s += __shfl_xor(s, 4, FSTU_WAVE);
+      s = group8_sum(s);
       if (valid) {
         s *= scale;
-        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        if (softcap > 0.f) s = soft_cap<FAST>(s, softcap, inv_cap2l);
         s -= slope * (float)(pos - j);
         float mn = fmaxf(P.m, s);
         float corr = __expf(P.m - mn);
@@ -211,23 +237,45 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   P.l = 0.f;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
+  constexpr bool FAST = sizeof(T) == 2;
   const int lo = max(0, pos - window);
   const float scale = rsqrtf((float)HD), slope = slopes[h];
-  attend_keys<T, DPL, SWA_U>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, q, lo + G * SWA_U,
-                             append ? pos : pos + 1, NGRP * SWA_U, pos, scale, softcap, slope);
-  if (self_grp) attend_one<DPL>(P, q, kself, vself, pos, pos, scale, softcap, slope);
+  attend_keys<T, DPL, SWA_U, FAST>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, lo, lo % cap, q,
+                                   lo + G * SWA_U, append ? pos : pos + 1, NGRP * SWA_U, pos, scale, softcap, slope);
+  if (self_grp) attend_one<DPL, FAST>(P, q, kself, vself, pos, pos, scale, softcap, slope);
   if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
 #pragma unroll
   for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];
   __syncthreads();
+  // merge in two stages: every wave folds its own 8 groups (lane = one output dim), then the first HD threads fold
+  // the NWAVES wave partials
+  __shared__ float wm[NWAVES], wl[NWAVES];
+  __shared__ float wacc[NWAVES][HD];
+  for (int i = lane; i < HD; i += 64) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) M = fmaxf(M, sm[w * 8 + g]);
+    float Lsum = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      const float e = (sm[w * 8 + g] == -INFINITY) ? 0.f : __expf(sm[w * 8 + g] - M);
+      Lsum = fmaf(sl[w * 8 + g], e, Lsum);
+      o = fmaf(sacc[w * 8 + g][i], e, o);
+    }
+    wacc[w][i] = o;
+    if (i == 0) { wm[w] = M; wl[w] = Lsum; }
+  }
+  __syncthreads();
   if (threadIdx.x < HD) {
     float M = -INFINITY;
-    for (int g = 0; g < NGRP; ++g) M = fmaxf(M, sm[g]);
+#pragma unroll
+    for (int g = 0; g < NWAVES; ++g) M = fmaxf(M, wm[g]);
     float Lsum = 0.f, o = 0.f;
-    for (int g = 0; g < NGRP; ++g) {
-      float e = __expf(sm[g] - M);
-      Lsum = fmaf(sl[g], e, Lsum);
-      o = fmaf(sacc[g][threadIdx.x], e, o);
+#pragma unroll
+    for (int g = 0; g < NWAVES; ++g) {
+      const float e = (wm[g] == -INFINITY) ? 0.f : __expf(wm[g] - M);
+      Lsum = fmaf(wl[g], e, Lsum);
+      o = fmaf(wacc[g][threadIdx.x], e, o);
     }
     DT<T>::st(out + (size_t)b * d + h * HD + threadIdx.x, o / Lsum);
   }
@@ -311,8 +359,8 @@ swa_prefill_kernel(const T* __restrict__ qkv, T* __restrict__ out, const float* 
     const T* row0 = qkv + (size_t)b * Tn * 3 * d + h * HD + gl * DPL;
     load_vec<T, DPL>(row0 + (size_t)t * 3 * d, q);
     const int lo = max(0, t - window);
-    attend_keys<T, DPL, SWA_U>(P, row0 + d, row0 + 2 * d, (size_t)3 * d, 0, q, lo + grp * SWA_U, t + 1, 8 * SWA_U, t,
-                               rsqrtf((float)HD), softcap, slopes[h]);
+    attend_keys<T, DPL, SWA_U, sizeof(T) == 2>(P, row0 + d, row0 + 2 * d, (size_t)3 * d, 0, 0, 0, q, lo + grp * SWA_U, t + 1,
+                                               8 * SWA_U, t, rsqrtf((float)HD), softcap, slopes[h]);
   }
   if (gl == 0) { sm[w][grp] = P.m; sl[w][grp] = P.l; }
 #pragma unroll

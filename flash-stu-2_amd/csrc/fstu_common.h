@@ -86,15 +86,32 @@ template <> struct DT<bf16_t> {
 };
 
 // ---------------------------------------------------------------- wave ops
+// All-lane reductions of a 64-wide wave, every lane active: four DPP steps inside a row of 16 lanes, one swizzle
+// across the two rows of a half, two lane reads across the halves (no LDS round trips).
+template <int CTRL>
+__device__ __forceinline__ float fstu_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float fstu_swz16(float v) {   // value of lane ^ 16
+  return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, FSTU_WAVE);
-  return v;
+  v += fstu_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+  v += fstu_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+  v += fstu_dpp<0x141>(v);   // row_half_mirror
+  v += fstu_dpp<0x140>(v);   // row_mirror
+  v += fstu_swz16(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) +
+         __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, FSTU_WAVE));
-  return v;
+  v = fmaxf(v, fstu_dpp<0xB1>(v));
+  v = fmaxf(v, fstu_dpp<0x4E>(v));
+  v = fmaxf(v, fstu_dpp<0x141>(v));
+  v = fmaxf(v, fstu_dpp<0x140>(v));
+  v = fmaxf(v, fstu_swz16(v));
+  return fmaxf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)),
+               __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)));
 }
 
 // tanh-approximated GELU as torch evaluates it in fp32

@@ -866,34 +866,44 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
     for (int u = 0; u < KSB; ++u)
       wd[j][u] = buf_load16(rdn, (u < nks && tile < tb1) ? bbase + ((unsigned)tile * (unsigned)tsb + (unsigned)u * 64u) * 16u : MLP_OOB);
   };
+  // waves beyond the chunk's k steps and tiles beyond the group's range are skipped by uniform branches: a load of
+  // nothing still costs its address cycles
+  const bool active = nks > 0;
+  const int nact = min(8, (a.kch + KSB - 1) / KSB);
+  if (active) {
 #pragma unroll
-  for (int j = 0; j < DB; ++j) load_b(j, tb0 + j);
+    for (int j = 0; j < DB; ++j)
+      if (tb0 + j < tb1) load_b(j, tb0 + j);
+  }
   for (int t0 = tb0; t0 < tb1; t0 += DB) {
+    if (active) {
 #pragma unroll
-    for (int j = 0; j < DB; ++j) {
-      floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < DB; ++j) {
+        if (t0 + j >= tb1) continue;
+        floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int u = 0; u < KSB; ++u)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc, 0, 0, 0);
-      load_b(j, t0 + DB + j);
-      float* mine = red + (size_t)((j * 8 + w) * 64 + lane) * 4;
+        for (int u = 0; u < KSB; ++u)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc, 0, 0, 0);
+        if (t0 + DB + j < tb1) load_b(j, t0 + DB + j);
+        float* mine = red + (size_t)((j * 8 + w) * 64 + lane) * 4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) mine[i] = acc[i];
+        for (int i = 0; i < 4; ++i) mine[i] = acc[i];
+      }
     }
     __syncthreads();
-    if (w < DB && t0 + w < tb1) {
-      const int tile = t0 + w;
-      float sd[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const float* o = red + (size_t)((w * 8 + s) * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) sd[i] += o[i];
+    // reduction over the K slices of the active waves: wave w takes half a tile (two of a lane's four features)
+    if ((w >> 1) < DB && t0 + (w >> 1) < tb1) {
+      const int jt = w >> 1, hf = (w & 1) * 2;
+      const int tile = t0 + jt;
+      float sd[2] = {0.f, 0.f};
+      for (int s = 0; s < nact; ++s) {
+        const float2 o = *(const float2*)(red + (size_t)((jt * 8 + s) * 64 + lane) * 4 + hf);
+        sd[0] += o.x;
+        sd[1] += o.y;
       }
       // D layout: features tile*16 + 4g + i of batch row r
-      const int fb = tile * 16 + 4 * g;
-      if (xrow && fb < a.d)
-        *(float4*)(a.partial + ((size_t)chunk * a.rows + r) * a.d + fb) = make_float4(sd[0], sd[1], sd[2], sd[3]);
+      const int fb = tile * 16 + 4 * g + hf;
+      if (xrow && fb < a.d) *(float2*)(a.partial + ((size_t)chunk * a.rows + r) * a.d + fb) = make_float2(sd[0], sd[1]);
     }
     if (t0 + DB < tb1) __syncthreads();
   }

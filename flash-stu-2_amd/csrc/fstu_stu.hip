@@ -435,20 +435,27 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
         sum.w = fmaf(cj.w, hv.w, sum.w);
       }
     }
-    // reduce over the 8 mode groups: lanes differing in bits 2..4
-#pragma unroll
-    for (int o = 4; o <= 16; o <<= 1) {
-      sum.x += __shfl_xor(sum.x, o, FSTU_WAVE);
-      sum.y += __shfl_xor(sum.y, o, FSTU_WAVE);
-      sum.z += __shfl_xor(sum.z, o, FSTU_WAVE);
-      sum.w += __shfl_xor(sum.w, o, FSTU_WAVE);
-    }
+    // reduce over the 8 mode groups (lanes differing in bits 2..4): two rotations inside the row of 16 lanes, one
+    // swizzle across the two rows
+    auto grp_sum = [](float v) {
+      v += fstu_dpp<0x124>(v);   // row_ror:4
+      v += fstu_dpp<0x128>(v);   // row_ror:8
+      return v + fstu_swz16(v);
+    };
+    sum.x = grp_sum(sum.x);
+    sum.y = grp_sum(sum.y);
+    sum.z = grp_sum(sum.z);
+    sum.w = grp_sum(sum.w);
     if (jsub == 0 && c < d) {
       bf16_t* yp = y + (size_t)b * ldy + c;
-      yp[0] = f32_to_bf16(2.f * sum.x);
-      yp[1] = f32_to_bf16(2.f * sum.y);
-      yp[2] = f32_to_bf16(2.f * sum.z);
-      yp[3] = f32_to_bf16(2.f * sum.w);
+      if ((ldy & 3) == 0) {
+        *(uint2*)yp = make_uint2(pack2_bf16(2.f * sum.x, 2.f * sum.y), pack2_bf16(2.f * sum.z, 2.f * sum.w));
+      } else {
+        yp[0] = f32_to_bf16(2.f * sum.x);
+        yp[1] = f32_to_bf16(2.f * sum.y);
+        yp[2] = f32_to_bf16(2.f * sum.z);
+        yp[3] = f32_to_bf16(2.f * sum.w);
+      }
     }
   }
 }
