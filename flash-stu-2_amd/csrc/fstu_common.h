@@ -48,6 +48,9 @@ int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B,
 int fstu_advance_dyn(int* dyn, void* stream);
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
                              int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream);
+int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
+                                 const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
+                                 int d, int K, int t, const int* dyn, void* stream);
 int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
                                   const float* ce, void* y, int ldy, int B, int S, int d, int K, int t, const int* dyn,
                                   void* stream);

@@ -291,6 +291,16 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     res_chain = L.wp_gate && L.wp_up && L.wp_down && (L.kind == 0 || L.wp_qkv);
   }
   const int down_fpw = (m->down_fpw == 4 || m->down_fpw == 8 || m->down_fpw == 16) ? m->down_fpw : 8;
+  // Merged norms: the down projection leaves 4 split-K slices and the first projection of the NEXT layer adds them
+  // to the residual stream and normalises it in its own prologue, so the add+norm launch between two layers is gone
+  // (the one in front of the head stays).
+  bool merge_norm = m->merge_norm && glu_bal && m->down_packed && m->x2 && m->stu_mode == 1 && d % 256 == 0 && !mlp_fused &&
+                    !res_chain && (size_t)B * (d / 8) <= 1024 && I % 128 == 0 && I / 128 <= 96;
+  for (int l = 0; l < m->n_layers && merge_norm; ++l) {
+    const fstu_layer_desc& L = m->layers[l];
+    merge_norm = L.wp_gate && L.wp_up && L.wp_down && (L.kind == 0 || L.wp_qkv);
+  }
+  bool pending_slices = false;   // m->partial holds 4 slices of the previous layer's MLP output, not yet added
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     bool pending_y = false;   // m->y holds a sub-layer output not yet added to the residual stream
@@ -305,7 +315,12 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_STU, fstu_stu_step_hist(L.hist, L.filt, m->eo, B, d, pos, m->hist_cap, m->L, ns, dt, stream));
         TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->eo, 2, ns, m->single_branch, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
       } else {
-        if (res_chain) {
+        if (pending_slices) {
+          TIMED(PC_STU, fstu_stu_res_inproj_step_dyn(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a,
+                                                     L.lds_ce, m->y, d, B, m->lds_S, d, d, pos, dyn, stream));
+          void* t = xc; xc = xo; xo = t;
+          pending_slices = false;
+        } else if (res_chain) {
           TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y,
                                                       d, B, m->lds_S, d, d, pos, dyn, stream));
         } else if (dt == FSTU_BF16 && d % 256 == 0) {
@@ -318,7 +333,12 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         pending_y = true;
       }
     } else {
-      if (res_chain)
+      if (pending_slices) {
+        TIMED(PC_PROJ, fstu_linear_packed_res(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d,
+                                              stream));
+        void* t = xc; xc = xo; xo = t;
+        pending_slices = false;
+      } else if (res_chain)
         TIMED(PC_PROJ, fstu_linear_packed(xc, d, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else if (glu_bal && L.wp_qkv)
         TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
@@ -361,11 +381,22 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_NORM, fstu_add_rmsnorm(xc, nullptr, 0, 1, 0, next_w, m->h, B, d, m->eps, dt, stream));
       continue;
     }
-    int nsl = m->ksplit_down;
+    if (merge_norm) {
+      int nsl = 4;
+      TIMED(PC_DOWN, fstu_down_packed_splitk(m->act, I, L.wp_down, m->partial, B, d, I, &nsl, stream));
+      if (l + 1 == m->n_layers)   // the head reads normalised rows
+        TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
+      else
+        pending_slices = true;
+      continue;
+    }
+    int nsl = 16;
     if (glu_bal && m->down_packed && L.wp_down && d % 16 == 0 && I % 512 == 0 && I / 512 <= 64)
       TIMED(PC_DOWN, fstu_down_packed_splitk(m->act, I, L.wp_down, m->partial, B, d, I, &nsl, stream));
-    else
+    else {
+      nsl = m->ksplit_down;
       TIMED(PC_DOWN, fstu_linear_decode_splitk(m->act, I, L.w_down, m->partial, B, d, I, m->ksplit_down, dt, stream));
+    }
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
   if (!do_sample && m->best && glu_bal && m->head_packed && m->wp_emb && fstu_glu_packed_supported(B, d, m->V)) {

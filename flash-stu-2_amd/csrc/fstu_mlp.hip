@@ -18,6 +18,7 @@
 //            and returns every counter to zero, so the launch can be replayed from a graph.
 // Every spin is bounded; a timeout raises a flag in the sync block and the kernel still exits.
 #include "fstu_common.h"
+#include "fstu_prologue.h"
 
 namespace {
 
@@ -448,11 +449,13 @@ struct GluArgs {
   bf16_t* act;
   int rows, d, I, ldh, ldact, fpw;
   // prologue (PRO): h = rmsnorm(T(x_in + delta)) * norm_w computed by every workgroup; workgroup 0 stores the sum
+  // (PRO 2: delta = up to 4 fp32 split-K slices of (rows x d), summed in order and rounded before the add)
   const bf16_t* x_in;
-  const bf16_t* delta;
+  const void* delta;
   bf16_t* x_out;
   const bf16_t* norm_w;
   float eps;
+  int nslices;
   // EPI 2: greedy pick fused into the epilogue (packed (value key << 32 | ~index) maxima into 64 slots per row)
   unsigned long long* best_ws;
   float temperature;
@@ -467,15 +470,15 @@ __device__ long long glu_trace_buf[256 * 8];
 #define GLU_STAMP(k) do { } while (0)
 #endif
 
-template <int KSA, bool PRO, int EPI>
+template <int KSA, int PRO, int EPI>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
-                    const bf16_t* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
-                    int fpw, float eps, float temperature, unsigned long long* best_ws) {
+                    const void* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
+                    int fpw, float eps, float temperature, unsigned long long* best_ws, int nslices) {
   GluArgs a;
   a.h = h; a.wp_gate = wp_gate; a.wp_up = wp_up; a.act = act; a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
   a.fpw = fpw; a.x_in = x_in; a.delta = delta; a.x_out = x_out; a.norm_w = norm_w; a.eps = eps; a.best_ws = best_ws;
-  a.temperature = temperature;
+  a.temperature = temperature; a.nslices = nslices;
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
@@ -540,9 +543,6 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     // arrive.
     bf16_t* hs = (bf16_t*)glu_smem;
     const int ld = a.d + 8;
-    __shared__ float ss_part[NXC * 16];
-    const rsrc_t rx = make_rsrc(a.x_in, (size_t)total * 16), rd = make_rsrc(a.delta, (size_t)total * 16);
-    const rsrc_t rn = make_rsrc(a.norm_w, (size_t)a.d * 2);
     auto add_chunk = [&](uint4 x4, uint4 d4, float& ss) {
       unsigned xw[4] = {x4.x, x4.y, x4.z, x4.w}, dw[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
@@ -555,63 +555,19 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       }
       return make_uint4(xw[0], xw[1], xw[2], xw[3]);
     };
-    if ((nchunk & 31) == 0 && total <= NXC * 512) {
-      // a row is a whole number of 32-lane groups: thread q owns chunk q of the (rows x nchunk) grid from load to store
-      uint4 xv[NXC], dv[NXC], nv[NXC];
-      int rowj[NXC];
-      const float inv_nc = 1.0f / (float)nchunk;
-#pragma unroll
-      for (int j = 0; j < NXC; ++j) {
-        if (j * 512 >= total) continue;   // uniform
-        const int q = threadIdx.x + j * 512;
-        rowj[j] = (int)(((float)q + 0.5f) * inv_nc);
-        xv[j] = buf_load16(rx, (unsigned)q * 16u);     // beyond the last chunk: zeros
-        dv[j] = buf_load16(rd, (unsigned)q * 16u);     // no delta: zeros
-        nv[j] = buf_load16(rn, (unsigned)(q - rowj[j] * nchunk) * 16u);
-      }
-      if (FSTU_GLU_ORDER == 1) load_first_exact();
-#pragma unroll
-      for (int j = 0; j < NXC; ++j) {
-        if (j * 512 >= total) continue;
-        const int q = threadIdx.x + j * 512;
-        float ss = 0.f;
-        xv[j] = add_chunk(xv[j], dv[j], ss);
-        ss = half_wave_sum(ss);
-        if ((lane & 31) == 0) ss_part[q >> 5] = ss;
-        if (wgi == 0 && a.x_out && q < total) *(uint4*)(a.x_out + (size_t)q * 8) = xv[j];
-      }
-      if (FSTU_GLU_ORDER == 0) {
-#pragma unroll
-        for (int j = 0; j < NXC; ++j)
-          if (j * 512 < total) asm volatile("" ::"v"(nv[j].x), "v"(nv[j].y), "v"(nv[j].z), "v"(nv[j].w));   // arrived
-        __builtin_amdgcn_sched_barrier(0);
-        if (blockIdx.x < 255) GLU_STAMP(6);
-        load_first();
-        if (blockIdx.x < 255) GLU_STAMP(7);
-      }
+    typedef NormPrologue<512, PRO == 2 ? 2 : NXC, PRO == 2 ? 4 : 0> Pro;
+    if (Pro::supported(a.rows, a.d)) {
+      // the activations are requested first and the weights right behind them; x' and the row statistics are formed
+      // as soon as the activations are there, the scaling runs while the rest of the weights arrive
+      __shared__ float ss_part[Pro::NPART];
+      Pro pro;
+      pro.issue(a.x_in, a.delta, a.nslices, a.norm_w, a.rows, a.d);
+      load_first_exact();
+      pro.reduce(ss_part, wgi == 0 ? a.x_out : nullptr, a.rows, a.d);
       __syncthreads();
       GLU_STAMP(1);
-      const int gpr = nchunk >> 5;
-      const float inv_d = 1.0f / (float)a.d;
-#pragma unroll
-      for (int j = 0; j < NXC; ++j) {
-        if (j * 512 >= total) continue;
-        const int q = threadIdx.x + j * 512;
-        if (q < total) {
-          float ss = 0.f;
-          const float* sp = ss_part + rowj[j] * gpr;
-          for (int i = 0; i < gpr; ++i) ss += sp[i];
-          const float rstd = rsqrtf(ss * inv_d + a.eps);
-          unsigned vw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {nv[j].x, nv[j].y, nv[j].z, nv[j].w};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            vw[i] = pack2_bf16((__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
-                               (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
-          }
-          *(uint4*)(hs + (size_t)rowj[j] * ld + (size_t)(q - rowj[j] * nchunk) * 8) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-        }
-      }
-    } else {
+      pro.scale(ss_part, hs, ld, a.rows, a.d, a.eps);
+    } else if (PRO == 1) {
       // any other shape: wave per row
       uint4 nwv[4];
       load_norm_w(nwv, a.norm_w, a.d, lane);
@@ -619,7 +575,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         const int row = q / nchunk, c = (q - row * nchunk) << 3;
         float ss = 0.f;
         uint4 v = *(const uint4*)(a.x_in + (size_t)q * 8);
-        if (a.delta) v = add_chunk(v, *(const uint4*)(a.delta + (size_t)q * 8), ss);
+        if (a.delta) v = add_chunk(v, *(const uint4*)((const bf16_t*)a.delta + (size_t)q * 8), ss);
         *(uint4*)(hs + (size_t)row * ld + c) = v;
         if (wgi == 0 && a.x_out) *(uint4*)(a.x_out + (size_t)q * 8) = v;
       }
@@ -842,7 +798,7 @@ __global__ void __launch_bounds__(512)
 down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* partial, int rows, int d, int I, int ldact, int KS,
                             int tpw, int tiles_out, int kch) {
   const DownSkArgs a{act, wp_down, partial, rows, d, I, ldact, KS, tpw, tiles_out, kch};
-  constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : 2);
+  constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : (KSB <= 8 ? 2 : 1));
   __shared__ float red[DB * 8 * 256];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -1013,7 +969,7 @@ extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
 }
 
 template <int KSA>
-static int glu_launch_ksa(GluArgs& a, bool pro, int epi, int G, size_t shm, const char* name, hipStream_t s) {
+static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const char* name, hipStream_t s) {
 #define GLU_GO(PRO, GLUF)                                                                                        \
   do {                                                                                                           \
     if (shm > 0) {                                                                                               \
@@ -1022,19 +978,20 @@ static int glu_launch_ksa(GluArgs& a, bool pro, int epi, int G, size_t shm, cons
       FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                  \
     }                                                                                                            \
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,    \
-                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.temperature, a.best_ws); \
+                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.temperature, a.best_ws, a.nslices); \
                     \
   } while (0)
-  if (pro && epi == 0) GLU_GO(true, 0);
-  else if (pro) GLU_GO(true, 1);
-  else if (epi == 0) GLU_GO(false, 0);
-  else if (epi == 1) GLU_GO(false, 1);
-  else GLU_GO(false, 2);
+  if (pro == 2) GLU_GO(2, 1);
+  else if (pro && epi == 0) GLU_GO(1, 0);
+  else if (pro) GLU_GO(1, 1);
+  else if (epi == 0) GLU_GO(0, 0);
+  else if (epi == 1) GLU_GO(0, 1);
+  else GLU_GO(0, 2);
 #undef GLU_GO
   return FSTU_OK;
 }
 
-static int glu_launch(GluArgs& a, bool pro, int epi, const char* name, hipStream_t s) {
+static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_t s) {
   int G = query_cus();
   FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
   if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
@@ -1068,7 +1025,7 @@ extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, cons
   GluArgs a = {};
   a.h = (const bf16_t*)h; a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
-  return glu_launch(a, false, 0, "fstu_glu_packed", (hipStream_t)stream);
+  return glu_launch(a, 0, 0, "fstu_glu_packed", (hipStream_t)stream);
 }
 
 extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
@@ -1085,9 +1042,9 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
   GluArgs a = {};
   a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = d; a.ldact = ldact;
-  a.x_in = (const bf16_t*)x_in; a.delta = (const bf16_t*)delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
+  a.x_in = (const bf16_t*)x_in; a.delta = delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
   a.eps = eps;
-  return glu_launch(a, true, 0, "fstu_glu_packed_norm", (hipStream_t)stream);
+  return glu_launch(a, 1, 0, "fstu_glu_packed_norm", (hipStream_t)stream);
 }
 
 // y = T(x W^T) over packed W (N,K): x given normalised (norm_w == NULL, x = h with row stride ldx) or as the residual
@@ -1105,7 +1062,29 @@ extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, fl
   a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)y;
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
   if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
-  return glu_launch(a, norm_w != nullptr, 1, "fstu_linear_packed", (hipStream_t)stream);
+  return glu_launch(a, norm_w != nullptr ? 1 : 0, 1, "fstu_linear_packed", (hipStream_t)stream);
+}
+
+// y = T(h W^T) with h = rmsnorm(x') * norm_w and x' = T(x_in + T(sum of nslices fp32 slices)): the add+norm launch
+// between a split-K projection and the next projection, folded into the latter.  x' is stored to x_out by one
+// workgroup (x_out must not alias x_in: the other workgroups still read it).
+extern "C" int fstu_linear_packed_res(const void* x_in, const float* partial, int nslices, void* x_out, const void* norm_w,
+                                      float eps, const void* wp, void* y, int ldy, int rows, int N, int K, void* stream) {
+  FSTU_REQUIRE(x_in && partial && x_out && norm_w && wp && y, FSTU_ENULL, "fstu_linear_packed_res: null pointer");
+  FSTU_REQUIRE((fstu_glu_packed_supported(rows, K, N) && NormPrologue<512, 2, 4>::supported(rows, K)), FSTU_ESHAPE,
+               "fstu_linear_packed_res: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(nslices >= 1 && nslices <= 4, FSTU_EARG, "fstu_linear_packed_res: nslices=%d outside 1..4", nslices);
+  FSTU_REQUIRE(ldy >= N && ldy % 4 == 0, FSTU_ESHAPE, "fstu_linear_packed_res: ldy=%d", ldy);
+  FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_linear_packed_res: x_out must not alias x_in");
+  FSTU_REQUIRE(fstu_aligned(x_in, 16) && fstu_aligned(partial, 16) && fstu_aligned(x_out, 16) && fstu_aligned(norm_w, 16) &&
+                   fstu_aligned(wp, 16) && fstu_aligned(y, 8),
+               FSTU_EALIGN, "fstu_linear_packed_res: pointers must be 16-byte aligned");
+  FSTU_REQUIRE((size_t)rows * (K + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_linear_packed_res: rows*K too large for LDS");
+  GluArgs a = {};
+  a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)y;
+  a.rows = rows; a.d = K; a.I = N; a.ldh = K; a.ldact = ldy; a.eps = eps;
+  a.x_in = (const bf16_t*)x_in; a.delta = partial; a.nslices = nslices; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
+  return glu_launch(a, 2, 1, "fstu_linear_packed_res", (hipStream_t)stream);
 }
 
 extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
@@ -1129,9 +1108,11 @@ extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_d
 // Balanced split-K down projection: partial (ksplit, rows, d) fp32 slices, summed by fstu_add_rmsnorm(delta_mode 1).
 // Returns the number of slices through *ksplit_out (16, the K chunks of the launch).
 extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
-                                       int* ksplit_out, void* stream) {
+                                       int* ksplit_io, void* stream) {
   FSTU_REQUIRE(act && wp_down && partial, FSTU_ENULL, "fstu_down_packed_splitk: null pointer");
-  const int KS = 16;
+  // *ksplit_io on entry: the number of K slices wanted (4, 8 or 16; anything else: 16); on return: the number written
+  const int want = ksplit_io ? *ksplit_io : 16;
+  const int KS = (want == 4 || want == 8) ? want : 16;
   FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d >= 16 && d % 16 == 0 && I >= KS * 32 && I % (KS * 32) == 0 &&
                    (size_t)I * d * 2 < 0xfff00000ull,
                FSTU_ESHAPE, "fstu_down_packed_splitk: unsupported shape rows=%d d=%d I=%d", rows, d, I);
@@ -1149,7 +1130,7 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   a.tpw = (a.tiles_out + ngroups - 1) / ngroups;
   ngroups = (a.tiles_out + a.tpw - 1) / a.tpw;
   const int ksb = (a.kch + 7) / 8;
-  FSTU_REQUIRE(ksb <= 8, FSTU_ESHAPE, "fstu_down_packed_splitk: I=%d too large", I);
+  FSTU_REQUIRE(ksb <= 12, FSTU_ESHAPE, "fstu_down_packed_splitk: I=%d too large", I);
   dim3 grid(ngroups * KS);
   hipStream_t s = (hipStream_t)stream;
   if (ksb <= 1) hipLaunchKernelGGL(down_splitk_balanced_kernel<1>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
@@ -1157,9 +1138,10 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   else if (ksb == 3) hipLaunchKernelGGL(down_splitk_balanced_kernel<3>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb <= 8) hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else hipLaunchKernelGGL(down_splitk_balanced_kernel<12>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
-  if (ksplit_out) *ksplit_out = KS;
+  if (ksplit_io) *ksplit_io = KS;
   return FSTU_OK;
 }
 

@@ -3,6 +3,7 @@
 // prefilled history into recurrence state, the time-domain prefill
 // convolution, and the dense LDS step of mini_stu.
 #include "fstu_common.h"
+#include "fstu_prologue.h"
 
 // ---------------------------------------------------------------- history step
 // Lags are rows of the (lag, channel) plane; a workgroup walks a contiguous
@@ -268,7 +269,9 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
                        these are the kernel-argument dwords the command processor preloads */, int ldh, int ldy,
                        bf16_t* __restrict__ xp_out /*optional (B,d)*/, int B, int S, int d, int K,
                        const bf16_t* __restrict__ x_res /*optional (B,K): normalise it instead of reading h*/,
-                       const bf16_t* __restrict__ norm_w, float eps) {
+                       const bf16_t* __restrict__ norm_w, float eps,
+                       const float* __restrict__ slices /*optional, with x_res: up to 4 fp32 (B,K) slices added first*/,
+                       int nslices, bf16_t* __restrict__ x_out /*receives x_res + T(sum of slices); not x_res itself*/) {
   __shared__ float red[4][64][4];
   __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
   extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
@@ -276,6 +279,11 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int tile = blockIdx.x, c0 = tile * 16;
+  // residual update + norm in the prologue: its loads go first, they head the kernel's critical path
+  typedef NormPrologue<256, 4, 4> Pro;
+  Pro pro;
+  const bool merged = x_res != nullptr && slices != nullptr;
+  if (merged) pro.issue(x_res, slices, nslices, norm_w, B, K);
   // ---- projection: A operand = Mt rows (channels), B operand = h rows (batch)
   const int kw = K >> 2;                                    // k range of this wave
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
@@ -313,7 +321,15 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     }
   }
   const int ldn = K + 8;
-  if (x_res) {
+  if (merged) {
+    bf16_t* hs = (bf16_t*)inproj_smem;
+    __shared__ float ss_part[Pro::NPART];
+    pro.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
+    __syncthreads();
+    pro.scale(ss_part, hs, ldn, B, K, eps);
+    __syncthreads();
+    hp = hs + (size_t)(xrow ? r : 0) * ldn + w * kw + g * 16;
+  } else if (x_res) {
     // h = rmsnorm(x_res) * norm_w for all rows into LDS (every workgroup recomputes it: B*K*2 bytes of input)
     bf16_t* hs = (bf16_t*)inproj_smem;
     const int nchunk = K >> 3;
@@ -462,7 +478,8 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
 
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
                               float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
-                              int K, int t, const int* dyn, void* stream);
+                              int K, int t, const int* dyn, void* stream, const float* slices = nullptr, int nslices = 0,
+                              void* x_out = nullptr);
 
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
                              int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream) {
@@ -476,9 +493,23 @@ int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float e
   return inproj_step_launch(x_res, K, x_res, norm_w, eps, Mt, state, a, ce, y, ldy, nullptr, B, S, d, K, t, dyn, stream);
 }
 
+// x' = x_in + T(sum of nslices <= 4 fp32 slices) goes to x_out, h = rmsnorm(x') * norm_w feeds the projection: the
+// add+norm launch between the previous layer's down projection and this layer, folded into this kernel
+int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
+                                 const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
+                                 int d, int K, int t, const int* dyn, void* stream) {
+  FSTU_REQUIRE(x_in && slices && x_out && norm_w, FSTU_ENULL, "fstu_stu_res_inproj_step: null pointer");
+  FSTU_REQUIRE(nslices >= 1 && nslices <= 4, FSTU_EARG, "fstu_stu_res_inproj_step: nslices=%d outside 1..4", nslices);
+  FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_stu_res_inproj_step: x_out must not alias x_in");
+  FSTU_REQUIRE((NormPrologue<256, 4, 4>::supported(B, K)), FSTU_ESHAPE, "fstu_stu_res_inproj_step: B=%d K=%d not supported", B, K);
+  FSTU_REQUIRE(fstu_aligned(slices, 16) && fstu_aligned(x_out, 16), FSTU_EALIGN, "fstu_stu_res_inproj_step: pointers must be 16-byte aligned");
+  return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, y, ldy, nullptr, B, S, d, K, t, dyn, stream, slices,
+                            nslices, x_out);
+}
+
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
                               float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
-                              int K, int t, const int* dyn, void* stream) {
+                              int K, int t, const int* dyn, void* stream, const float* slices, int nslices, void* x_out) {
   FSTU_REQUIRE(h && Mt && state && a && ce && y, FSTU_ENULL, "fstu_stu_inproj_step: null pointer");
   FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
   FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
@@ -488,9 +519,16 @@ static int inproj_step_launch(const void* h, int ldh, const void* x_res, const v
   FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w must be 16-byte aligned");
   hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,
                      (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,
-                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps);
+                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out);
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
+}
+
+extern "C" int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w,
+                                        float eps, const void* Mt, float* state, const float* a, const float* ce, void* y,
+                                        int ldy, int B, int S, int d, int K, int t, void* stream) {
+  return fstu_stu_res_inproj_step_dyn(x_in, slices, nslices, x_out, norm_w, eps, Mt, state, a, ce, y, ldy, B, S, d, K, t, nullptr,
+                                      stream);
 }
 
 extern "C" int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,

@@ -36,6 +36,7 @@ SIGNATURES = {
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -62,6 +63,7 @@ SIGNATURES = {
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_linear_packed_res": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_res": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
     "fstu_mlp_block_sync_bytes": [],
@@ -308,6 +310,22 @@ def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: t
     _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(out), d, _p(xp_out), B, S, d, K, t,
                                        _stream()), "fstu_stu_inproj_step")
     return out
+
+
+def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tensor, eps: float, Mt: torch.Tensor,
+                        state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int):
+    """(x', y): x' = x + bf16(sum of the fp32 slices); y = projection + recurrence step of rmsnorm(x') * norm_w."""
+    _dev(x, partial, norm_w, Mt, state, a, ce)
+    B, K = x.shape
+    d = Mt.shape[0]
+    S = a.numel()
+    assert x.dtype == Mt.dtype == torch.bfloat16 and partial.dtype == torch.float32 and state.shape == (B, 2, S, d)
+    x_out = torch.empty_like(x)
+    y = torch.empty(B, d, dtype=x.dtype, device=x.device)
+    _check(load().fstu_stu_res_inproj_step(_p(x), _p(partial), partial.shape[0], _p(x_out), _p(norm_w), float(eps), _p(Mt),
+                                           _p(state), _p(a), _p(ce), _p(y), d, B, S, d, K, t, _stream()),
+           "fstu_stu_res_inproj_step")
+    return x_out, y
 
 
 def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, state: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -586,16 +604,29 @@ def down_packed_res(act: torch.Tensor, wp_down: torch.Tensor, x_res: torch.Tenso
     return out
 
 
-def down_packed_splitk(act: torch.Tensor, wp_down: torch.Tensor, d: int) -> torch.Tensor:
-    """Balanced split-K down projection: returns the fp32 slices (16, rows, d); their sum in slice order is the result."""
+def down_packed_splitk(act: torch.Tensor, wp_down: torch.Tensor, d: int, ksplit: int = 16) -> torch.Tensor:
+    """Balanced split-K down projection: returns the fp32 slices (ksplit, rows, d); their sum in slice order is the
+    result.  ksplit: 4, 8 or 16."""
     _dev(act, wp_down)
     rows, I = act.shape
-    partial = torch.empty(16, rows, d, dtype=torch.float32, device=act.device)
-    ks = ctypes.c_int(0)
+    partial = torch.empty(ksplit, rows, d, dtype=torch.float32, device=act.device)
+    ks = ctypes.c_int(ksplit)
     _check(load().fstu_down_packed_splitk(_p(act), I, _p(wp_down), _p(partial), rows, d, I, ctypes.byref(ks), _stream()),
            "fstu_down_packed_splitk")
-    assert ks.value == 16
+    assert ks.value == ksplit
     return partial
+
+
+def linear_packed_res(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tensor, eps: float, wp: torch.Tensor, N: int):
+    """(x', y): x' = x + bf16(sum of the fp32 slices), y = (rmsnorm(x') * norm_w) @ W^T over packed W, one launch."""
+    _dev(x, partial, norm_w, wp)
+    rows, K = x.shape
+    ns = partial.shape[0]
+    x_out = torch.empty_like(x)
+    y = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    _check(load().fstu_linear_packed_res(_p(x), _p(partial), ns, _p(x_out), _p(norm_w), float(eps), _p(wp), _p(y), N, rows,
+                                         N, K, _stream()), "fstu_linear_packed_res")
+    return x_out, y
 
 
 def head_packed_argmax(x: torch.Tensor, wp: torch.Tensor, N: int, temperature: float, best_ws: torch.Tensor,

@@ -43,7 +43,7 @@ class ModelDesc(ctypes.Structure):
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
                 ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
-                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i)]
+                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i), ("merge_norm", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -267,6 +267,14 @@ class DecodeEngine:
                             arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
                     m.res_chain = 1
                     m.down_fpw = int(os.environ.get("FSTU_DOWN_FPW", "8"))
+                elif (mode == "lds" and d % 256 == 0 and m.down_packed and B * (d // 8) <= 1024 and I % 128 == 0
+                      and os.environ.get("FSTU_MERGE_NORM", "1") == "1"):
+                    # the add+norm between two layers runs as the prologue of the next layer's first projection
+                    # (the down projection leaves 4 split-K slices for it): one launch less per layer
+                    for i, layer in enumerate(model.layers):
+                        if isinstance(layer, AttentionLayer):
+                            arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                    m.merge_norm = 1
         plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
         if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
             # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its

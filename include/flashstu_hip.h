@@ -142,6 +142,14 @@ int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, const float* a,
 int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
                          void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream);
 
+/* The same launch with the residual update and the RMSNorm of its input as the prologue
+ * (flash_stu/layers/stu_layer.py:78-82 after the previous layer's :93-97): x' = T(x_in + T(sum of nslices <= 4 fp32
+ * (B,K) slices)) goes to x_out (not x_in itself), h = rmsnorm(x') * norm_w feeds the projection.  K % 256 == 0,
+ * B*K/8 <= 1024. */
+int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
+                             const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
+                             int d, int K, int t, void* stream);
+
 /* Builds that state from a prefilled history: for both parities p,
  *   state[b,p,j,c] = sum_{m>=0} a[j]^m * hist[b, tp-2m, c],  tp = newest index
  *   of parity p that is <= t_last.  hist is (B,cap,d). */
@@ -376,11 +384,20 @@ int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, co
 int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
                          int d, int I, int fpw, void* stream);
 
-/* Split-K form of the down projection over packed weights, one workgroup per CU: partial receives 16 fp32 slices
- * (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1, nslices 16) sums in slice order; *ksplit_out = 16.
- * d % 16 == 0, I % 512 == 0, rows <= 16, bf16.  Same values as fstu_linear_decode_splitk up to the summation order. */
+/* Split-K form of the down projection over packed weights (reference: flash_stu/modules/swiglu.py:22-29, down_proj):
+ * partial receives *ksplit_io fp32 slices (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1) or the norm prologue of
+ * the next projection sums in slice order.  *ksplit_io on entry: slices wanted (4, 8 or 16; anything else: 16); on
+ * return: slices written.  d % 16 == 0, I % (32 * slices) == 0, rows <= 16, bf16.  Same values as
+ * fstu_linear_decode_splitk up to the summation order. */
 int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
-                            int* ksplit_out, void* stream);
+                            int* ksplit_io, void* stream);
+
+/* y = T(h W^T) over packed W (N,K) with h = rmsnorm(x') * norm_w, x' = T(x_in + T(sum of nslices <= 4 fp32 slices)):
+ * the residual add + RMSNorm between the MLP of one layer and the first projection of the next
+ * (flash_stu/layers/stu_layer.py:93-97 followed by attention_layer.py:53-57), folded into that projection.  x' goes to
+ * x_out (must not alias x_in).  K % 256 == 0, rows*K/8 <= 1024, rows <= 16, bf16. */
+int fstu_linear_packed_res(const void* x_in, const float* partial, int nslices, void* x_out, const void* norm_w, float eps,
+                           const void* wp, void* y, int ldy, int rows, int N, int K, void* stream);
 
 /* Tied head + greedy pick over packed weights (fstu_pack_rows of the (V,d) embedding), one workgroup per CU:
  * logits (rows,ldy) and tok_out[b*tok_stride] = argmax_v logits[b,v] (lowest index on ties) after dividing by
@@ -470,6 +487,10 @@ typedef struct {
   int down_packed;          /* != 0: layers with wp_down use fstu_down_packed_splitk (16 slices: partial must hold
                                max(ksplit_down,16)*B*d floats) */
   int head_packed;          /* != 0 and wp_emb set: the greedy path runs the tied head through fstu_head_packed_argmax */
+  int merge_norm;           /* != 0 (needs glu_packed, down_packed, x2, lds mode, wp_gate/up/down everywhere and wp_qkv on
+                               attention layers, B*d <= 8192): the down projection leaves 4 split-K slices and the next
+                               layer's first projection adds and normalises them in its prologue
+                               (fstu_stu_res_inproj_step / fstu_linear_packed_res); one add+norm launch less per layer */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

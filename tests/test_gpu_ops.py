@@ -339,6 +339,30 @@ def test_stu_inproj_step_equals_projection_then_step(hip):
         assert float((st1 - st2).abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("B,ns", [(8, 4), (3, 2), (1, 1)])
+def test_stu_res_inproj_step_equals_add_norm_then_step(hip, B, ns):
+    """Split-K slices + residual + RMSNorm as the prologue of the projection+step launch == fstu_add_rmsnorm followed
+    by the plain launch: the residual bit for bit, the output up to the summation order of the row statistics."""
+    g = gen(22)
+    S, d = 64, 768
+    a = dev((0.5 + 0.49 * torch.rand(S, generator=g)).float())
+    ce = dev((torch.randn(S, d, generator=g) / S).float())
+    Mt = dev((torch.randn(d, d, generator=g) / math.sqrt(d)).bfloat16())
+    nw = dev((1 + 0.1 * torch.randn(d, generator=g)).bfloat16())
+    st1 = dev(torch.randn(B, 2, S, d, generator=g))
+    st2 = st1.clone()
+    for t in range(4):
+        x = dev(torch.randn(B, d, generator=g).bfloat16())
+        part = dev(0.3 * torch.randn(ns, B, d, generator=g))
+        x_ref = x.clone()
+        h = hip.add_rmsnorm(x_ref, part, nw, O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ns)
+        y_ref = hip.stu_inproj_step(h, Mt, st1, a, ce, t)
+        x_out, y = hip.stu_res_inproj_step(x, part, nw, O.RMS_EPS_DEFAULT, Mt, st2, a, ce, t)
+        assert torch.equal(x_out, x_ref)
+        check(y, y_ref, torch.bfloat16, frac=0.05)
+        assert float((st1 - st2).abs().max()) <= 2.0 ** -7 * float(st1.abs().max())
+
+
 @pytest.mark.parametrize("L", [128, 1024])
 def test_stu_step_lds_tracks_the_convolution(hip, L):
     """With poles/weights fitted to the effective filter, the recurrence
@@ -650,6 +674,27 @@ def test_down_packed_res(hip, rows, d, I, fpw):
     assert torch.equal(xin, out)
 
 
+@pytest.mark.parametrize("rows,K,N,ns", [(8, 768, 2304, 4), (4, 256, 96, 3), (2, 1024, 3072, 1)])
+def test_linear_packed_res_equals_add_norm_then_linear(hip, rows, K, N, ns):
+    dtype = torch.bfloat16
+    g = gen(64)
+    x = dev(torch.randn(rows, K, generator=g).to(dtype))
+    part = dev(0.3 * torch.randn(ns, rows, K, generator=g))
+    nw = dev((1 + 0.1 * torch.randn(K, generator=g)).to(dtype))
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    wp = hip.pack_rows(dev(W))
+    x_ref = x.clone()
+    h = hip.add_rmsnorm(x_ref, part, nw, O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ns)
+    y_ref = hip.linear_packed(h, wp, N)
+    x_out, y = hip.linear_packed_res(x, part, nw, O.RMS_EPS_DEFAULT, wp, N)
+    assert torch.equal(x_out, x_ref)
+    check(y, y_ref, dtype, frac=0.05)
+    # against the float64-accumulated specification
+    xs = x.cpu() + part.cpu().sum(0).to(dtype)
+    ref = (O.rms_norm(xs, nw.cpu(), O.RMS_EPS_DEFAULT).double() @ W.double().t()).to(dtype)
+    check(y, ref, dtype, frac=0.05, atol=2.0 ** -8 * float(ref.float().abs().max()))
+
+
 @pytest.mark.parametrize("rows,K,N", [(8, 768, 2304), (8, 768, 768), (4, 256, 96), (16, 1024, 3072)])
 def test_linear_packed_with_and_without_norm(hip, rows, K, N):
     dtype = torch.bfloat16
@@ -695,15 +740,16 @@ def test_stu_bank_step_lds(hip, dtype):
     assert worst <= tol * float(rp.float().abs().max()), worst
 
 
-@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 24576), (5, 48, 1024)])
-def test_down_packed_splitk(hip, rows, d, I):
-    """Balanced split-K down projection: the 16 slices sum to the float64-accumulated product."""
+@pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8)])
+def test_down_packed_splitk(hip, rows, d, I, ks):
+    """Balanced split-K down projection: the 4, 8 or 16 slices sum to the float64-accumulated product."""
     dtype = torch.bfloat16
     g = gen(64)
     act = torch.randn(rows, I, generator=g).to(dtype)
     wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
     ref = act.double() @ wd.double().t()
-    part = hip.down_packed_splitk(dev(act), hip.pack_rows(dev(wd)), d)
+    part = hip.down_packed_splitk(dev(act), hip.pack_rows(dev(wd)), d, ks)
+    assert part.shape[0] == ks
     got = part.double().sum(0).cpu()
     assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
 
