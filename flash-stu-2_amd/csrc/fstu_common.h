@@ -38,6 +38,10 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream);
 int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B, int H, int hd,
                          int cap, int pos, int window, float softcap, int append, const int* dyn, int dtype, void* stream);
+int fstu_swa_qkv_decode_dyn(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
+                            const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
+                            const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
+                            const int* dyn, void* stream);
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                          float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream);

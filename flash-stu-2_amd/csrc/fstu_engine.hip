@@ -333,7 +333,22 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         pending_y = true;
       }
     } else {
-      if (pending_slices) {
+      // QKV projection inside the attention launch: every (row, head) workgroup forms its own q, k, v
+      const bool swa_fused = m->swa_fused && dt == FSTU_BF16 && L.wp_qkv && m->head_dim == 64 && d % 256 == 0 && d <= 768 &&
+                             !res_chain;
+      if (swa_fused) {
+        if (pending_slices) {
+          TIMED(PC_SWA, fstu_swa_qkv_decode_dyn(nullptr, xc, m->partial, 4, xo, L.norm1_w, m->eps, L.wp_qkv, L.kring, L.vring,
+                                                m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos, m->window,
+                                                m->softcap, dyn, stream));
+          void* t = xc; xc = xo; xo = t;
+          pending_slices = false;
+        } else {
+          TIMED(PC_SWA, fstu_swa_qkv_decode_dyn(m->h, nullptr, nullptr, 0, nullptr, nullptr, 0.f, L.wp_qkv, L.kring, L.vring,
+                                                m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos, m->window,
+                                                m->softcap, dyn, stream));
+        }
+      } else if (pending_slices) {
         TIMED(PC_PROJ, fstu_linear_packed_res(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d,
                                               stream));
         void* t = xc; xc = xo; xo = t;
@@ -344,8 +359,9 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else
         TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
-      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
-                                         m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
+      if (!swa_fused)
+        TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
+                                           m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
       if (glu_bal && L.wp_proj)
         TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
       else

@@ -49,6 +49,7 @@ SIGNATURES = {
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_append_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "fstu_swa_qkv_decode": [_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_prefill_ws_elems": [_i, _i, _i, _i],
     "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
@@ -479,6 +480,24 @@ def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slop
     _check(fn(_p(qkv), _p(kring), _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window,
               float(softcap or 0.0), _dt(qkv), _stream()), "fstu_swa_decode")
     return out
+
+
+def swa_qkv_decode(wp_qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slopes: torch.Tensor, pos: int,
+                   window: int, softcap: float, h: Optional[torch.Tensor] = None, x: Optional[torch.Tensor] = None,
+                   partial: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0):
+    """QKV projection + ring append + one-token attention in one launch.  Give h (B,d) normalised rows, or x (B,d)
+    with norm_w (and optionally partial (ns,B,d) fp32 slices to add first).  Returns out (B,d), or (x', out)."""
+    _dev(wp_qkv, kring, vring, slopes, h, x, partial, norm_w)
+    src = h if h is not None else x
+    B, d = src.shape
+    _, H, cap, hd = kring.shape
+    out = torch.empty(B, d, dtype=src.dtype, device=src.device)
+    x_out = torch.empty_like(x) if x is not None else None
+    ns = 0 if partial is None else partial.shape[0]
+    _check(load().fstu_swa_qkv_decode(_p(h), _p(x), _p(partial), ns, _p(x_out), _p(norm_w), float(eps), _p(wp_qkv), _p(kring),
+                                      _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window, float(softcap), _stream()),
+           "fstu_swa_qkv_decode")
+    return out if x is None else (x_out, out)
 
 
 def swa_prefill(qkv: torch.Tensor, slopes: torch.Tensor, n_heads: int, window: int, softcap: float,

@@ -236,6 +236,16 @@ int fstu_swa_append_decode(const void* qkv, void* kring, void* vring, void* out,
                            int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
                            void* stream);
 
+/* QKV projection + ring append + decode in one launch (reference: flash_stu/modules/attention.py:66-105 for one new
+ * token): every (batch row, head) workgroup forms its own q, k, v = h W_qkv^T from the packed weight (fstu_pack_rows of
+ * c_attn.weight (3d,d)).  h is given (h_in, (B,d) normalised rows; x_in NULL) or formed here from the residual stream
+ * (h_in NULL): x' = T(x_in + T(sum of nslices <= 4 fp32 (B,d) slices)), h = rmsnorm(x') * norm_w
+ * (attention_layer.py:53-57); x' goes to x_out (not x_in itself).  Head dim 64, d % 256 == 0, d <= 768, bf16. */
+int fstu_swa_qkv_decode(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
+                        const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
+                        const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
+                        void* stream);
+
 /* Prefill form: qkv (B,T,3*H*hd), positions 0..T-1, out (B,T,H*hd). */
 int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T, int H, int hd,
                      int window, float softcap, int dtype, void* stream);
@@ -491,6 +501,8 @@ typedef struct {
                                attention layers, B*d <= 8192): the down projection leaves 4 split-K slices and the next
                                layer's first projection adds and normalises them in its prologue
                                (fstu_stu_res_inproj_step / fstu_linear_packed_res); one add+norm launch less per layer */
+  int swa_fused;            /* != 0 (bf16, head dim 64, width <= 768, wp_qkv set): the QKV projection runs inside the
+                               attention launch (fstu_swa_qkv_decode), together with the merged add+norm when merge_norm */
 } fstu_model_desc;
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next

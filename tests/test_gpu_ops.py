@@ -546,6 +546,42 @@ def test_mlp_block_one_launch(hip, rows, d, I):
     check(xo, x + y0, dtype, frac=0.10, scale=float((x + y0).float().abs().max()), atol=2.0 ** -7 * float(y0.float().abs().max()))
 
 
+@pytest.mark.parametrize("B,H,W,ns", [(8, 12, 512, 4), (3, 4, 16, 2), (2, 8, 40, 0)])
+def test_swa_qkv_decode_equals_projection_then_decode(hip, B, H, W, ns):
+    """QKV projection (+ split-K slices, residual and RMSNorm in front of it) inside the attention launch == the
+    separate launches: add+norm, packed QKV projection, append+decode.  Ring and residual bit for bit; the output up
+    to the K split of the projection.  Several positions, the ring wrapping in the small cases."""
+    dtype = torch.bfloat16
+    g = gen(71)
+    hd, d, cap = 64, H * 64, W + 1
+    Wqkv = (torch.randn(3 * d, d, generator=g) / math.sqrt(d)).to(dtype)
+    wp = hip.pack_rows(dev(Wqkv))
+    nw = dev((1 + 0.1 * torch.randn(d, generator=g)).to(dtype))
+    slopes = dev(torch.tensor([0.25 * 2.0 ** (-(h + 1) * 8.0 / H) for h in range(H)], dtype=torch.float32))
+    kr1 = dev((0.5 * torch.randn(B, H, cap, hd, generator=g)).to(dtype))
+    vr1 = dev(torch.randn(B, H, cap, hd, generator=g).to(dtype))
+    kr2, vr2, kr3, vr3 = kr1.clone(), vr1.clone(), kr1.clone(), vr1.clone()
+    for pos in (W + 7, W + 8, 3 * W + 1):
+        x = dev(torch.randn(B, d, generator=g).to(dtype))
+        part = dev(0.3 * torch.randn(ns, B, d, generator=g)) if ns else None
+        x_ref = x.clone()
+        h = (hip.add_rmsnorm(x_ref, part, nw, O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ns) if ns
+             else hip.add_rmsnorm(x_ref, None, nw, O.RMS_EPS_DEFAULT))
+        qkv = hip.linear_packed(h, wp, 3 * d)
+        ref = hip.swa_decode(qkv, kr1, vr1, slopes, pos, W, 50.0, append=True)
+        x_out, out = hip.swa_qkv_decode(wp, kr2, vr2, slopes, pos, W, 50.0, x=x, partial=part, norm_w=nw,
+                                        eps=O.RMS_EPS_DEFAULT)
+        assert torch.equal(x_out, x_ref)
+        out_h = hip.swa_qkv_decode(wp, kr3, vr3, slopes, pos, W, 50.0, h=h)
+        for o in (out, out_h):
+            check(o, ref, dtype, frac=0.10, atol=2.0 ** -8 * float(ref.float().abs().max()))
+        # the appended keys / values: equal up to a rounding flip of the projection
+        for a, b_ in ((kr2, kr1), (vr2, vr1), (kr3, kr1), (vr3, vr1)):
+            dk = (a.float() - b_.float()).abs()
+            assert float(dk.max()) <= 2.0 ** -7 * float(b_.float().abs().max())
+            assert float((dk > 0).float().mean()) <= 1e-3
+
+
 @pytest.mark.parametrize("B,H,hd,W,T", [(2, 4, 64, 16, 50), (2, 12, 64, 512, 700), (1, 4, 128, 32, 100),
                                          (1, 2, 64, 1000, 333), (1, 2, 128, 64, 17)])
 def test_swa_prefill_mfma(hip, B, H, hd, W, T):
