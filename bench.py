@@ -96,8 +96,8 @@ def main():
     ap.add_argument("--breakdown", action="store_true", help="time every kernel class with HIP events")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (batch-sharded decode needs no exchange; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (decode shards by batch: every GPU would hold the full weights "
+              "and its own sequences, with no exchange); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import ctypes
     import torch
