@@ -238,6 +238,13 @@ static int decode_step_fused(const fstu_model_desc* m, const int64_t* tok_in, in
   return FSTU_OK;
 }
 
+// While a graph is captured for one parity of the position, the STU launches get that parity as a plain argument
+// instead of reading the device-side position first: their state addresses then depend on nothing, which takes one
+// dependent trip to memory (about 1 us) off each of them.  -1: no override.
+static thread_local int g_stu_parity = -1;
+static inline const int* stu_dyn(const int* dyn) { return g_stu_parity >= 0 ? nullptr : dyn; }
+static inline int stu_pos(int pos) { return g_stu_parity >= 0 ? g_stu_parity : pos; }
+
 // dyn == nullptr: pos/step come from the host arguments.  dyn != nullptr (graph capture): every position-dependent
 // kernel reads {pos, step} from that device int[2]; tok_in/tok_out are then the bases of token columns 0 and 1.
 static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
@@ -317,18 +324,18 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       } else {
         if (pending_slices) {
           TIMED(PC_STU, fstu_stu_res_inproj_step_dyn(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a,
-                                                     L.lds_ce, m->y, d, B, m->lds_S, d, d, pos, dyn, stream));
+                                                     L.lds_ce, m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
           void* t = xc; xc = xo; xo = t;
           pending_slices = false;
         } else if (res_chain) {
           TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y,
-                                                      d, B, m->lds_S, d, d, pos, dyn, stream));
+                                                      d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
         } else if (dt == FSTU_BF16 && d % 256 == 0) {
           TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y, d, nullptr, B,
-                                                 m->lds_S, d, d, pos, dyn, stream));
+                                                 m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
         } else {
           TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-          TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
+          TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, stu_pos(pos), stu_dyn(dyn), dt, stream));
         }
         pending_y = true;
       }
@@ -439,9 +446,10 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
 
 // ---------------------------------------------------------------- one step as a replayable HIP graph
 struct fstu_graph {
-  hipGraph_t graph;
-  hipGraphExec_t exec;
+  hipGraph_t graph[2];       // one per parity of the position (the second is null when the model has no STU state)
+  hipGraphExec_t exec[2];
   WarmCtx* warm;
+  long long next_pos;        // position the next launch will process
 };
 
 static void warm_destroy(WarmCtx* w) {
@@ -459,10 +467,11 @@ extern "C" int fstu_set_warm_workgroups(int n) {
   return FSTU_OK;
 }
 
-extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn,
+extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn, int pos0,
                                         float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                                         void* stream, void** graph_out) {
   FSTU_REQUIRE(m && tokens && dyn && graph_out && stream, FSTU_ENULL, "fstu_decode_graph_create: null pointer (a non-default stream is required)");
+  FSTU_REQUIRE(pos0 >= 0, FSTU_EARG, "fstu_decode_graph_create: pos0=%d", pos0);
   hipStream_t s = (hipStream_t)stream;
   WarmCtx* warm = nullptr;
   if (g_warm_wgs > 0 && m->n_layers + 1 <= 64) {
@@ -477,35 +486,44 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
       }
     }
   }
-  hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
-  if (e != hipSuccess) { warm_destroy(warm); fstu_set_error("fstu_decode_graph_create: begin capture: %s", hipGetErrorString(e)); return (int)e; }
-  g_warm = warm;
-  int rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
-  g_warm = nullptr;
-  hipGraph_t g = nullptr;
-  e = hipStreamEndCapture(s, &g);
-  if (rc != 0) { if (g) (void)hipGraphDestroy(g); warm_destroy(warm); return rc; }
-  if (e != hipSuccess) { warm_destroy(warm); fstu_set_error("fstu_decode_graph_create: end capture: %s", hipGetErrorString(e)); return (int)e; }
-  hipGraphExec_t ge = nullptr;
-  e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
-  if (e != hipSuccess) { (void)hipGraphDestroy(g); warm_destroy(warm); fstu_set_error("fstu_decode_graph_create: instantiate: %s", hipGetErrorString(e)); return (int)e; }
-  fstu_graph* h = new fstu_graph{g, ge, warm};
+  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0};
+  // one graph per parity of the position: the STU launches of each carry their parity as an argument
+  const int ngraphs = (m->stu_mode == 1 && warm == nullptr) ? 2 : 1;
+  for (int par = 0; par < ngraphs; ++par) {
+    hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: begin capture: %s", hipGetErrorString(e)); return (int)e; }
+    g_warm = warm;
+    g_stu_parity = ngraphs == 2 ? par : -1;
+    int rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
+    g_stu_parity = -1;
+    g_warm = nullptr;
+    e = hipStreamEndCapture(s, &h->graph[par]);
+    if (rc != 0) { fstu_decode_graph_destroy(h); return rc; }
+    if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: end capture: %s", hipGetErrorString(e)); return (int)e; }
+    e = hipGraphInstantiate(&h->exec[par], h->graph[par], nullptr, nullptr, 0);
+    if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: instantiate: %s", hipGetErrorString(e)); return (int)e; }
+  }
   *graph_out = h;
   return FSTU_OK;
 }
 
 extern "C" int fstu_decode_graph_launch(void* graph, void* stream) {
   FSTU_REQUIRE(graph, FSTU_ENULL, "fstu_decode_graph_launch: null graph");
-  hipError_t e = hipGraphLaunch(((fstu_graph*)graph)->exec, (hipStream_t)stream);
+  fstu_graph* h = (fstu_graph*)graph;
+  const int par = h->exec[1] ? (int)(h->next_pos & 1) : 0;
+  hipError_t e = hipGraphLaunch(h->exec[par], (hipStream_t)stream);
   if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_launch: %s", hipGetErrorString(e)); return (int)e; }
+  h->next_pos += 1;
   return FSTU_OK;
 }
 
 extern "C" int fstu_decode_graph_destroy(void* graph) {
   if (!graph) return FSTU_OK;
   fstu_graph* h = (fstu_graph*)graph;
-  (void)hipGraphExecDestroy(h->exec);
-  (void)hipGraphDestroy(h->graph);
+  for (int par = 0; par < 2; ++par) {
+    if (h->exec[par]) (void)hipGraphExecDestroy(h->exec[par]);
+    if (h->graph[par]) (void)hipGraphDestroy(h->graph[par]);
+  }
   warm_destroy(h->warm);
   delete h;
   return FSTU_OK;

@@ -346,7 +346,7 @@ class DecodeEngine:
             handle = _vp()
             ch.stream = self._gstreams[i % n_streams]
             rc = self.lib.fstu_decode_graph_create(ctypes.byref(ch.desc), tokens.data_ptr() + 8 * ch.b0 * stride, stride,
-                                                   ch.dyn.data_ptr(), float(temperature), int(top_k) if top_k else 0,
+                                                   ch.dyn.data_ptr(), int(pos), float(temperature), int(top_k) if top_k else 0,
                                                    float(top_p) if top_p else 0.0, int(bool(do_sample)),
                                                    int(seed) & ((1 << 64) - 1), ch.stream.cuda_stream,
                                                    ctypes.byref(handle))
