@@ -69,6 +69,15 @@ __device__ __forceinline__ uint4 buf_load16(rsrc_t rs, unsigned off) {
   u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+// the same for data read exactly once (weights): non-temporal, so that the stream does not push the activations, the
+// norm weights and the kernels' own code out of the L2
+#ifndef FSTU_WEIGHT_AUX
+#define FSTU_WEIGHT_AUX 2
+#endif
+__device__ __forceinline__ uint4 buf_load16_stream(rsrc_t rs, unsigned off) {
+  u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, FSTU_WEIGHT_AUX);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 __device__ __forceinline__ u64 pack4_bf16(const float* v) {
   return (u64)pack2_bf16(v[0], v[1]) | ((u64)pack2_bf16(v[2], v[3]) << 32);
@@ -518,8 +527,8 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
 #pragma unroll
     for (int u = 0; u < KSA; ++u) {
       const unsigned off = ok ? abase + ((unsigned)tile * (unsigned)tsa + (unsigned)u * 64u) * 16u : MLP_OOB;
-      wa[j][u] = buf_load16(rg, off);
-      if (GLU) wb[j][u] = buf_load16(ru, off);
+      wa[j][u] = buf_load16_stream(rg, off);
+      if (GLU) wb[j][u] = buf_load16_stream(ru, off);
     }
   };
   // a tile beyond the workgroup's range is skipped by a uniform branch: a load of nothing still costs its address cycles
@@ -830,7 +839,7 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
   auto load_b = [&](int j, int tile) {
 #pragma unroll
     for (int u = 0; u < KSB; ++u)
-      wd[j][u] = buf_load16(rdn, (u < nks && tile < tb1) ? bbase + ((unsigned)tile * (unsigned)tsb + (unsigned)u * 64u) * 16u : MLP_OOB);
+      wd[j][u] = buf_load16_stream(rdn, (u < nks && tile < tb1) ? bbase + ((unsigned)tile * (unsigned)tsb + (unsigned)u * 64u) * 16u : MLP_OOB);
   };
   // waves beyond the chunk's k steps and tiles beyond the group's range are skipped by uniform branches: a load of
   // nothing still costs its address cycles
