@@ -1013,10 +1013,11 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
 static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_t s) {
   int G = query_cus();
   FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
-  // FSTU_GLU_BY8=1 deals features in groups of 8 (no 128-byte line shared between two workgroups: HBM traffic of the
-  // gate/up launch 1.00x instead of 1.125x the algorithmic bytes), at the price of workgroups of 32 and 40 features
-  // instead of 36 each; measured 0.363 vs 0.361 ms per decode step, so groups of 4 stay the default
-  static const bool by4 = [] { const char* e = getenv("FSTU_GLU_BY8"); return !(e && e[0] == '1'); }();
+  // Features are dealt out in groups of 8: no 128-byte line is shared between two workgroups (HBM traffic of the
+  // gate/up launch 1.00x the algorithmic bytes instead of 1.125x with groups of 4), at the price of workgroups of 32
+  // and 40 features instead of 36 each.  Measured 0.3305 vs 0.3326 ms per decode step; FSTU_GLU_BY4=1 brings the
+  // groups of 4 back.
+  static const bool by4 = [] { const char* e = getenv("FSTU_GLU_BY4"); return e && e[0] == '1'; }();
   if (by4) {
     if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
     a.fpw = (((a.I + G - 1) / G) + 3) & ~3;
