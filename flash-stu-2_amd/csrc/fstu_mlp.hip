@@ -1017,7 +1017,8 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
   // gate/up launch 1.00x the algorithmic bytes instead of 1.125x with groups of 4), at the price of workgroups of 32
   // and 40 features instead of 36 each.  Measured 0.3305 vs 0.3326 ms per decode step; FSTU_GLU_BY4=1 brings the
   // groups of 4 back.
-  static const bool by4 = [] { const char* e = getenv("FSTU_GLU_BY4"); return e && e[0] == '1'; }();
+  const char* by4_env = getenv("FSTU_GLU_BY4");   // read at every launch: a graph keeps what it was captured with
+  const bool by4 = by4_env && by4_env[0] == '1';
   if (by4) {
     if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
     a.fpw = (((a.I + G - 1) / G) + 3) & ~3;

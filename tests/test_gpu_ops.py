@@ -667,10 +667,13 @@ def test_glu_packed_balanced(hip, rows, d, I):
     close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
 
 
+@pytest.mark.parametrize("by4", ["0", "1"])
 @pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192)])
-def test_glu_packed_norm_prologue(hip, rows, d, I):
+def test_glu_packed_norm_prologue(hip, rows, d, I, monkeypatch, by4):
     """Residual add + RMSNorm as the prologue of the balanced gate/up launch == the separate add+norm kernel followed
-    by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored."""
+    by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored.  Features dealt to the
+    workgroups in groups of 8 (default) and of 4."""
+    monkeypatch.setenv("FSTU_GLU_BY4", by4)
     dtype = torch.bfloat16
     g = gen(61)
     x = torch.randn(rows, d, generator=g).to(dtype)
