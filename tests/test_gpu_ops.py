@@ -668,7 +668,8 @@ def test_glu_packed_balanced(hip, rows, d, I):
 
 
 @pytest.mark.parametrize("by4", ["0", "1"])
-@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192)])
+@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192),
+                                      (16, 2048, 4096)])     # the last: more chunks than threads x 4, wave-per-row norm
 def test_glu_packed_norm_prologue(hip, rows, d, I, monkeypatch, by4):
     """Residual add + RMSNorm as the prologue of the balanced gate/up launch == the separate add+norm kernel followed
     by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored.  Features dealt to the
