@@ -89,6 +89,8 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph-steps", type=int, default=8, dest="graph_steps",
+                    help="decode steps captured per HIP graph (used when it divides --steps and --warmup)")
     ap.add_argument("--no-graph", action="store_true", help="launch every step kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--warm-wgs", type=int, default=-1, help="workgroups of the graph's cache warm-up branch (0 = off)")
     ap.add_argument("--pmc-calibrate", action="store_true", dest="pmc_calibrate",
@@ -138,13 +140,14 @@ def main():
     use_graph = eng.graph_supported() and not args.no_graph
     if use_graph:
         # one decode step captured once; every replay reads its position from device memory
-        eng.graph_begin(tokens, pos, pos - P + 1, 1.0, None, None, False, 0)
-        for _ in range(W):
+        S = args.graph_steps if (W % args.graph_steps == 0 and K % args.graph_steps == 0) else 1
+        eng.graph_begin(tokens, pos, pos - P + 1, 1.0, None, None, False, 0, steps_per_graph=S)
+        for _ in range(W // S):
             eng.graph_step()
         eng.graph_sync()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(K):
+        for _ in range(K // S):
             eng.graph_step()
         eng.graph_sync()
         torch.cuda.synchronize()

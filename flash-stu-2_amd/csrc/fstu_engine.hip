@@ -449,7 +449,8 @@ struct fstu_graph {
   hipGraph_t graph[2];       // one per parity of the position (the second is null when the model has no STU state)
   hipGraphExec_t exec[2];
   WarmCtx* warm;
-  long long next_pos;        // position the next launch will process
+  long long next_pos;        // position the next launch will process first
+  int nsteps;                // decode steps per launch
 };
 
 static void warm_destroy(WarmCtx* w) {
@@ -468,10 +469,10 @@ extern "C" int fstu_set_warm_workgroups(int n) {
 }
 
 extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn, int pos0,
-                                        float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                                        int nsteps, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                                         void* stream, void** graph_out) {
   FSTU_REQUIRE(m && tokens && dyn && graph_out && stream, FSTU_ENULL, "fstu_decode_graph_create: null pointer (a non-default stream is required)");
-  FSTU_REQUIRE(pos0 >= 0, FSTU_EARG, "fstu_decode_graph_create: pos0=%d", pos0);
+  FSTU_REQUIRE(pos0 >= 0 && nsteps >= 1 && nsteps <= 64, FSTU_EARG, "fstu_decode_graph_create: pos0=%d nsteps=%d (1..64)", pos0, nsteps);
   hipStream_t s = (hipStream_t)stream;
   WarmCtx* warm = nullptr;
   if (g_warm_wgs > 0 && m->n_layers + 1 <= 64) {
@@ -486,15 +487,21 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
       }
     }
   }
-  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0};
-  // one graph per parity of the position: the STU launches of each carry their parity as an argument
-  const int ngraphs = (m->stu_mode == 1 && warm == nullptr) ? 2 : 1;
-  for (int par = 0; par < ngraphs; ++par) {
+  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0, nsteps};
+  // One graph per parity of the first position: the STU launches carry their parity as an argument.  A graph of an
+  // even number of steps always starts on the parity of pos0, so the other one is not captured.
+  const bool baked = m->stu_mode == 1 && warm == nullptr;
+  for (int par = 0; par < 2; ++par) {
+    if (!baked && par == 1) break;
+    if (baked && (nsteps & 1) == 0 && par != (pos0 & 1)) continue;
     hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: begin capture: %s", hipGetErrorString(e)); return (int)e; }
     g_warm = warm;
-    g_stu_parity = ngraphs == 2 ? par : -1;
-    int rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
+    int rc = 0;
+    for (int st = 0; st < nsteps && rc == 0; ++st) {
+      g_stu_parity = baked ? ((par + st) & 1) : -1;
+      rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
+    }
     g_stu_parity = -1;
     g_warm = nullptr;
     e = hipStreamEndCapture(s, &h->graph[par]);
@@ -510,10 +517,11 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
 extern "C" int fstu_decode_graph_launch(void* graph, void* stream) {
   FSTU_REQUIRE(graph, FSTU_ENULL, "fstu_decode_graph_launch: null graph");
   fstu_graph* h = (fstu_graph*)graph;
-  const int par = h->exec[1] ? (int)(h->next_pos & 1) : 0;
+  int par = (int)(h->next_pos & 1);
+  if (!h->exec[par]) par ^= 1;   // position-independent graph, or an even number of steps per graph
   hipError_t e = hipGraphLaunch(h->exec[par], (hipStream_t)stream);
   if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_launch: %s", hipGetErrorString(e)); return (int)e; }
-  h->next_pos += 1;
+  h->next_pos += h->nsteps;
   return FSTU_OK;
 }
 

@@ -72,7 +72,7 @@ SIGNATURES = {
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
     "fstu_mlp_block": [_vp] * 12 + [_i, _i, _i, _f, _vp],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
-    "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _i, _f, _i, _f, _i, _u64, _vp, _vp],
+    "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _i, _i, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
     "fstu_decode_graph_destroy": [_vp],
     "fstu_set_warm_workgroups": [_i],

@@ -328,12 +328,17 @@ class DecodeEngine:
     def graph_supported(self) -> bool:
         return self.cfg.resolved_stu_decode_mode() == "lds"
 
-    def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed):
+    GRAPH_STEPS = 8     # decode steps per graph launch in generate() (the launch of a graph costs several microseconds)
+
+    def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed,
+                    steps_per_graph: int = 1):
         """Captures one decode step per row chunk as a HIP graph, each chunk on a side stream of its own: the chunks
         are independent (own workspaces, state rows and device-side position), so their graphs run concurrently and
         the second chunk finds the layer's weights, which the first has just streamed, in the Infinity Cache.  Each
-        graph_step() then feeds tokens[:, pos], writes tokens[:, pos+1] and advances pos on the device."""
+        graph_step() then runs steps_per_graph decode steps: each feeds tokens[:, pos], writes tokens[:, pos+1] and
+        advances pos on the device."""
         self.graph_end()
+        self.graph_steps = int(steps_per_graph)
         concurrent = os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1" and os.environ.get("FSTU_FUSED_MLP", "0") != "1"
         n_streams = len(self.chunks) if concurrent else 1
         self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
@@ -346,7 +351,8 @@ class DecodeEngine:
             handle = _vp()
             ch.stream = self._gstreams[i % n_streams]
             rc = self.lib.fstu_decode_graph_create(ctypes.byref(ch.desc), tokens.data_ptr() + 8 * ch.b0 * stride, stride,
-                                                   ch.dyn.data_ptr(), int(pos), float(temperature), int(top_k) if top_k else 0,
+                                                   ch.dyn.data_ptr(), int(pos), self.graph_steps, float(temperature),
+                                                   int(top_k) if top_k else 0,
                                                    float(top_p) if top_p else 0.0, int(bool(do_sample)),
                                                    int(seed) & ((1 << 64) - 1), ch.stream.cuda_stream,
                                                    ctypes.byref(handle))
@@ -402,10 +408,18 @@ class DecodeEngine:
         _hip.sample(logits, tokens[:, P], temperature, top_k, top_p, do_sample, seed, 0)
         all_logits = [logits.clone()] if return_logits else None
         if use_graph and not return_logits and self.graph_supported() and n_new > 2:
-            self.graph_begin(tokens, P, 1, temperature, top_k, top_p, do_sample, seed)
+            todo, pos, S = n_new - 1, P, self.GRAPH_STEPS
             try:
-                for s in range(1, n_new):
-                    self.graph_step()
+                if todo >= 4 * S:       # long runs: S steps per graph launch, the remainder one by one
+                    self.graph_begin(tokens, pos, pos - P + 1, temperature, top_k, top_p, do_sample, seed, steps_per_graph=S)
+                    for _ in range(todo // S):
+                        self.graph_step()
+                    pos += (todo // S) * S
+                    todo -= (todo // S) * S
+                if todo > 0:
+                    self.graph_begin(tokens, pos, pos - P + 1, temperature, top_k, top_p, do_sample, seed)
+                    for _ in range(todo):
+                        self.graph_step()
             finally:
                 self.graph_end()
             return tokens

@@ -521,9 +521,11 @@ int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in, int64_t* t
  * recorded).  pos0 is the value the caller stores in dyn[0] before the first launch: with the recurrence STU state
  * two graphs are captured, one per parity of the position (their STU launches carry the parity as an argument
  * instead of reading dyn first), and launch n replays the one for pos0 + n; a caller that rewrites dyn[0] creates a
- * new graph.  No counterpart in the reference. */
+ * new graph.  nsteps (1..64) consecutive decode steps are captured into one graph, so that one launch produces
+ * nsteps tokens per sequence (the cost of starting a graph is paid once per nsteps tokens).  No counterpart in the
+ * reference. */
 int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn, int pos0,
-                             float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
+                             int nsteps, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                              void* stream, void** graph_out);
 int fstu_decode_graph_launch(void* graph, void* stream);
 /* The captured graph carries a parallel branch whose kernels only read the MLP / head weights a layer is about
