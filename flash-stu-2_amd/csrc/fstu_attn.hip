@@ -201,6 +201,15 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 // k,v (read from the qkv row) into ring slot pos % cap and attends to that key
 // straight from the qkv row, so the ring sweep covers the older keys only.
 #define SWA_U 4
+#ifdef FSTU_GLU_TRACE
+__device__ long long swa_trace_buf[96 * 8];
+#define SWA_STAMP(k) do { if (threadIdx.x == 0) swa_trace_buf[(blockIdx.y * gridDim.x + blockIdx.x) % 96 * 8 + (k)] = wall_clock64(); } while (0)
+extern "C" int fstu_swa_trace(long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(swa_trace_buf), sizeof(long long) * 96 * 8);
+}
+#else
+#define SWA_STAMP(k) do { } while (0)
+#endif
 template <typename T, int HD, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64)
 swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__ out, const float* __restrict__ slopes,
@@ -208,9 +217,8 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
                   int pos, int window, float softcap, int append) {
   constexpr int DPL = HD / 8;
   constexpr int NGRP = NWAVES * 8;
+  SWA_STAMP(0);
   if (dyn) pos = dyn[0];
-  __shared__ float sm[NGRP], sl[NGRP];
-  __shared__ float sacc[NGRP][HD];
   const int h = blockIdx.x, b = blockIdx.y;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int grp = lane >> 3, gl = lane & 7;
@@ -229,44 +237,98 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   load_vec<T, DPL>(row + gl * DPL, q);
   const bool self_grp = append && (G == NGRP - 1);   // this group also takes the new token's own key
   float kself[DPL], vself[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) { kself[i] = 0.f; vself[i] = 0.f; }
   if (self_grp) {
     load_vec<T, DPL>(row + d + gl * DPL, kself);
     load_vec<T, DPL>(row + 2 * d + gl * DPL, vself);
   }
-  Partial<DPL> P;
-  P.m = -INFINITY;
-  P.l = 0.f;
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
+  // Every wave keeps ONE running maximum for its 8 key groups (wave-wide max of the scores of an iteration), so the
+  // groups of a wave merge by plain sums across lanes; only the NWAVES wave partials go through LDS.
   constexpr bool FAST = sizeof(T) == 2;
   const int lo = max(0, pos - window);
   const float scale = rsqrtf((float)HD), slope = slopes[h];
-  attend_keys<T, DPL, SWA_U, FAST>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, lo, lo % cap, q,
-                                   lo + G * SWA_U, append ? pos : pos + 1, NGRP * SWA_U, pos, scale, softcap, slope);
-  if (self_grp) attend_one<DPL, FAST>(P, q, kself, vself, pos, pos, scale, softcap, slope);
-  if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
+  const float inv_cap2l = softcap > 0.f ? 2.8853900817779268f / softcap : 0.f;
+  const int j_end = append ? pos : pos + 1, slot_lo = lo % cap;
+  const T* kb = kring + hbase + gl * DPL;
+  const T* vb = vring + hbase + gl * DPL;
+  float M = -INFINITY, l = 0.f, acc[DPL];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];
-  __syncthreads();
-  // merge in two stages: every wave folds its own 8 groups (lane = one output dim), then the first HD threads fold
-  // the NWAVES wave partials
+  for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+  auto score = [&](const float* kk, int j) {
+    float sc = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) sc = fmaf(q[i], kk[i], sc);
+    sc = group8_sum(sc) * scale;
+    if (softcap > 0.f) sc = soft_cap<FAST>(sc, softcap, inv_cap2l);
+    return sc - slope * (float)(pos - j);
+  };
+  // wave-uniform loop: the wave's first group decides whether the wave has keys left
+  for (int base = lo + w * 8 * SWA_U; base < j_end; base += NGRP * SWA_U) {
+    const int jb = base + grp * SWA_U;
+    float kk[SWA_U][DPL], vv[SWA_U][DPL];
+    // no branch around the loads (a key beyond the range re-reads the last valid one and gets weight 0): all loads
+    // of the iteration stay in flight together
+#pragma unroll
+    for (int u = 0; u < SWA_U; ++u) {
+      const int j = min(jb + u, j_end - 1);
+      int slot = slot_lo + (j - lo);
+      slot = slot >= cap ? slot - cap : slot;
+      load_vec<T, DPL>(kb + (size_t)slot * HD, kk[u]);
+      load_vec<T, DPL>(vb + (size_t)slot * HD, vv[u]);
+    }
+    float sc[SWA_U], mit = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < SWA_U; ++u) {
+      const float v = score(kk[u], jb + u);
+      sc[u] = (jb + u < j_end) ? v : -INFINITY;
+      mit = fmaxf(mit, sc[u]);
+    }
+    const float Mn = fmaxf(M, wave_max(mit));     // finite: the wave's first key is valid
+    const float corr = __expf(M - Mn);
+    float psum = 0.f, p[SWA_U];
+#pragma unroll
+    for (int u = 0; u < SWA_U; ++u) { p[u] = __expf(sc[u] - Mn); psum += p[u]; }
+    l = fmaf(l, corr, psum);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      float a = acc[i] * corr;
+#pragma unroll
+      for (int u = 0; u < SWA_U; ++u) a = fmaf(p[u], vv[u][i], a);
+      acc[i] = a;
+    }
+    M = Mn;
+  }
+  SWA_STAMP(1);
+  if (append && w == NWAVES - 1) {     // the new token's own key, taken by the last group of the last wave
+    const float v = score(kself, pos);
+    const float ss = self_grp ? v : -INFINITY;
+    const float Mn = fmaxf(M, wave_max(ss));
+    const float corr = __expf(M - Mn);
+    const float ps = __expf(ss - Mn);
+    l = fmaf(l, corr, ps);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc[i] = fmaf(ps, vself[i], acc[i] * corr);
+    M = Mn;
+  }
+  // the wave's 8 groups share M: sums across the lanes 8, 16 and 32 apart
+  auto xsum = [](float v) {
+    v += fstu_dpp<0x128>(v);          // row_ror:8
+    v += fstu_swz16(v);
+    return v + __shfl_xor(v, 32, FSTU_WAVE);
+  };
+  l = xsum(l);
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) acc[i] = xsum(acc[i]);
   __shared__ float wm[NWAVES], wl[NWAVES];
   __shared__ float wacc[NWAVES][HD];
-  for (int i = lane; i < HD; i += 64) {
-    float M = -INFINITY;
+  if (lane < 8) {
 #pragma unroll
-    for (int g = 0; g < 8; ++g) M = fmaxf(M, sm[w * 8 + g]);
-    float Lsum = 0.f, o = 0.f;
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      const float e = (sm[w * 8 + g] == -INFINITY) ? 0.f : __expf(sm[w * 8 + g] - M);
-      Lsum = fmaf(sl[w * 8 + g], e, Lsum);
-      o = fmaf(sacc[w * 8 + g][i], e, o);
-    }
-    wacc[w][i] = o;
-    if (i == 0) { wm[w] = M; wl[w] = Lsum; }
+    for (int i = 0; i < DPL; ++i) wacc[w][gl * DPL + i] = acc[i];
+    if (lane == 0) { wm[w] = M; wl[w] = l; }
   }
   __syncthreads();
+  SWA_STAMP(3);
   if (threadIdx.x < HD) {
     float M = -INFINITY;
 #pragma unroll
@@ -280,6 +342,7 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
     }
     DT<T>::st(out + (size_t)b * d + h * HD + threadIdx.x, o / Lsum);
   }
+  SWA_STAMP(4);
 }
 
 static int check_swa(const char* name, int H, int hd, int window, const void* slopes) {
