@@ -226,23 +226,18 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   const int d = H * HD;
   const T* row = qkv + (size_t)b * 3 * d + h * HD;
   const size_t hbase = ((size_t)b * H + h) * cap * HD;
-  if (append) {
-    if (threadIdx.x < HD) {
-      size_t dst = hbase + (size_t)(pos % cap) * HD + threadIdx.x;
-      kring[dst] = row[d + threadIdx.x];
-      vring[dst] = row[2 * d + threadIdx.x];
-    }
-  }
+  // the ring append: element `at` of the new key and value, read now by the last HD threads (no branch: the other
+  // threads re-read element 0) and stored after everything else; slot pos % cap is not among the slots the sweep reads
+  const int at = (int)threadIdx.x - (NWAVES * 64 - HD);
+  const T app_k = row[d + max(at, 0)], app_v = row[2 * d + max(at, 0)];
   float q[DPL];
   load_vec<T, DPL>(row + gl * DPL, q);
   const bool self_grp = append && (G == NGRP - 1);   // this group also takes the new token's own key
+  // every group reads the new token's key and value (no branch, so nothing waits for them before the ring loads are
+  // out); only the last group of the last wave gives them a weight
   float kself[DPL], vself[DPL];
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) { kself[i] = 0.f; vself[i] = 0.f; }
-  if (self_grp) {
-    load_vec<T, DPL>(row + d + gl * DPL, kself);
-    load_vec<T, DPL>(row + 2 * d + gl * DPL, vself);
-  }
+  load_vec<T, DPL>(row + d + gl * DPL, kself);
+  load_vec<T, DPL>(row + 2 * d + gl * DPL, vself);
   // Every wave keeps ONE running maximum for its 8 key groups (wave-wide max of the scores of an iteration), so the
   // groups of a wave merge by plain sums across lanes; only the NWAVES wave partials go through LDS.
   constexpr bool FAST = sizeof(T) == 2;
@@ -341,6 +336,11 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
       o = fmaf(wacc[g][threadIdx.x], e, o);
     }
     DT<T>::st(out + (size_t)b * d + h * HD + threadIdx.x, o / Lsum);
+  }
+  if (append && at >= 0) {
+    const size_t dst = hbase + (size_t)(pos % cap) * HD + at;
+    kring[dst] = app_k;
+    vring[dst] = app_v;
   }
   SWA_STAMP(4);
 }
