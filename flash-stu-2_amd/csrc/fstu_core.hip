@@ -1,6 +1,7 @@
 // Error reporting, embedding gather, fused residual + RMSNorm, GELU-gate and
 // the sampling kernel.  All bandwidth-bound, one workgroup per row.
 #include "fstu_common.h"
+#include "fstu_prologue.h"
 #include <string.h>
 
 // ---------------------------------------------------------------- errors
@@ -71,6 +72,9 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
 
 template <typename T> struct Vec4;
 template <> struct Vec4<float> {
+  typedef float4 raw_t;
+  static __device__ __forceinline__ raw_t ldraw(const float* p) { return *(const float4*)p; }
+  static __device__ __forceinline__ void cvt(raw_t v, float* o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
   static __device__ __forceinline__ void ld(const float* p, float* o) {
     float4 v = *(const float4*)p;
     o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
@@ -78,6 +82,12 @@ template <> struct Vec4<float> {
   static __device__ __forceinline__ void st(float* p, const float* v) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
 };
 template <> struct Vec4<bf16_t> {
+  typedef uint2 raw_t;
+  static __device__ __forceinline__ raw_t ldraw(const bf16_t* p) { return *(const uint2*)p; }
+  static __device__ __forceinline__ void cvt(raw_t v, float* o) {
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
   static __device__ __forceinline__ void ld(const bf16_t* p, float* o) {
     uint2 v = *(const uint2*)p;
     o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
@@ -96,11 +106,15 @@ template <> struct Vec4<bf16_t> {
 __device__ __forceinline__ void sum_slices4(const float* p, size_t stride, int n, float* out) {
   float4 tot = make_float4(0, 0, 0, 0);
   for (int s0 = 0; s0 < n; s0 += 16) {
+    // no branch around the loads: a slice index beyond n re-reads the last slice and is added with weight 0
     float4 v[16];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) v[k] = (s0 + k < n) ? *(const float4*)(p + (size_t)(s0 + k) * stride) : make_float4(0, 0, 0, 0);
+    for (int k = 0; k < 16; ++k) v[k] = *(const float4*)(p + (size_t)min(s0 + k, n - 1) * stride);
 #pragma unroll
-    for (int k = 0; k < 16; ++k) { tot.x += v[k].x; tot.y += v[k].y; tot.z += v[k].z; tot.w += v[k].w; }
+    for (int k = 0; k < 16; ++k) {
+      const float m = (s0 + k < n) ? 1.f : 0.f;
+      tot.x = fmaf(m, v[k].x, tot.x); tot.y = fmaf(m, v[k].y, tot.y); tot.z = fmaf(m, v[k].z, tot.z); tot.w = fmaf(m, v[k].w, tot.w);
+    }
   }
   out[0] = tot.x; out[1] = tot.y; out[2] = tot.z; out[3] = tot.w;
 }
@@ -122,11 +136,11 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
 #pragma unroll
   for (int i = 0; i < NG; ++i) {
     const int c = (threadIdx.x + i * FSTU_NORM_THREADS) * GW;
-#pragma unroll
-    for (int k = 0; k < GW; ++k) wpre[i][k] = 0.f;
-    if (y != nullptr && c < d) {
-      if (VEC) Vec4<T>::ld(w + c, wpre[i]); else wpre[i][0] = DT<T>::ld(w + c);
-    }
+    // no branch around the load (a branch with a zero on its other side makes the kernel wait for the load at once):
+    // threads beyond the row re-read column 0, and without y the row itself stands in for the weights
+    const T* wsrc = (y != nullptr) ? w : (const T*)xr;
+    const int cw = c < d ? c : 0;
+    if (VEC) Vec4<T>::ld(wsrc + cw, wpre[i]); else wpre[i][0] = DT<T>::ld(wsrc + cw);
   }
   float ss = 0.f;
 #pragma unroll
@@ -136,7 +150,11 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
     for (int k = 0; k < GW; ++k) v[i][k] = 0.f;
     if (c < d) {
       float xv[GW], dv[GW];
-      if (VEC) Vec4<T>::ld(xr + c, xv); else xv[0] = DT<T>::ld(xr + c);
+      // the row is requested here and converted only after the delta loads are out: a conversion in between would
+      // make the kernel wait for the row before it requests the slices
+      typename Vec4<T>::raw_t xraw = {};
+      T xraw1 = 0;
+      if (VEC) xraw = Vec4<T>::ldraw(xr + c); else xraw1 = xr[c];
       if (delta != nullptr) {
         if (delta_mode == 0) {
           const T* dp = (const T*)delta + (size_t)r * d + c;
@@ -166,9 +184,12 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
           for (int k = 0; k < GW; ++k)
             dv[k] = single_branch ? DT<T>::rnd(e[k] + o[k]) : DT<T>::rnd(DT<T>::rnd(e[k] + o[k]) + DT<T>::rnd(e[k] - o[k]));
         }
+        if (VEC) Vec4<T>::cvt(xraw, xv); else xv[0] = DT<T>::ld(&xraw1);
 #pragma unroll
         for (int k = 0; k < GW; ++k) xv[k] = DT<T>::rnd(xv[k] + dv[k]);
         if (VEC) Vec4<T>::st(xr + c, xv); else DT<T>::st(xr + c, xv[0]);
+      } else {
+        if (VEC) Vec4<T>::cvt(xraw, xv); else xv[0] = DT<T>::ld(&xraw1);
       }
 #pragma unroll
       for (int k = 0; k < GW; ++k) { v[i][k] = xv[k]; ss += xv[k] * xv[k]; }
@@ -239,6 +260,33 @@ embed_rmsnorm_kernel(const int64_t* __restrict__ ids, const T* __restrict__ tabl
   int64_t id = ids[(size_t)r * id_stride + (dyn ? dyn[0] : 0)];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + (size_t)id * d;
+  if (sizeof(T) == 2 && (d & 7) == 0 && d <= 8 * FSTU_NORM_THREADS &&
+      (((uintptr_t)table | (uintptr_t)w | (uintptr_t)x | (uintptr_t)h) & 15) == 0) {
+    // bf16 rows of up to 2048 channels: a thread owns one chunk of 8 channels; both loads sit in straight-line code
+    // (a lane beyond the row reads zeros through the buffer descriptor), so one wait covers them
+    const int nchunk = d >> 3, q = threadIdx.x;
+    const uint4 wv4 = fstu_buf_load16(fstu_make_rsrc(w, (size_t)d * 2), (unsigned)q * 16u);
+    const uint4 xv4 = fstu_buf_load16(fstu_make_rsrc(src, (size_t)d * 2), (unsigned)q * 16u);
+    const unsigned xw[4] = {xv4.x, xv4.y, xv4.z, xv4.w}, ww[4] = {wv4.x, wv4.y, wv4.z, wv4.w};
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = __uint_as_float(xw[i] << 16), hi = __uint_as_float(xw[i] & 0xffff0000u);
+      ss = fmaf(lo, lo, ss);
+      ss = fmaf(hi, hi, ss);
+    }
+    if (q < nchunk) *(uint4*)((bf16_t*)x + (size_t)r * d + q * 8) = xv4;
+    const float rstd = rsqrtf(block_sum_256(ss, red) / (float)d + eps);
+    if (q < nchunk) {
+      unsigned o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o[i] = pack2_bf16((__uint_as_float(xw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
+                          (__uint_as_float(xw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
+      *(uint4*)((bf16_t*)h + (size_t)r * d + q * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    return;
+  }
   // norm weights and the embedding row are both read before the reduction (up to 8 columns per thread stay in
   // registers), so that nothing is fetched after it
   constexpr int PRE = 8;
