@@ -17,6 +17,7 @@
 //            (deterministic), forms x'' and stores it; the last workgroup of all normalises x'' into h_next
 //            and returns every counter to zero, so the launch can be replayed from a graph.
 // Every spin is bounded; a timeout raises a flag in the sync block and the kernel still exits.
+#include <type_traits>
 #include "fstu_common.h"
 #include "fstu_prologue.h"
 
@@ -565,8 +566,10 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       }
       return make_uint4(xw[0], xw[1], xw[2], xw[3]);
     };
-    typedef NormPrologue<512, PRO == 2 ? 2 : NXC, PRO == 2 ? 4 : 0> Pro;
-    if (Pro::supported(a.rows, a.d)) {
+    // the lean prologue, instantiated for the exact number of chunks per thread so that it is one straight line
+    auto lean = [&](auto nxc_tag) {
+      constexpr int NX = decltype(nxc_tag)::value;
+      typedef NormPrologue<512, NX, PRO == 2 ? 4 : 0> Pro;
       // the activations are requested first; x' and the row statistics are formed as soon as they are there, the
       // scaling runs while the weights arrive
       __shared__ float ss_part[Pro::NPART];
@@ -578,6 +581,8 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       // end of the 28 MB (measured: 4.9 us instead of 2 us after the first instruction).  Only the last tile is
       // conditional, so that the norm weights, requested earlier, keep an exact position in the load counter.
       load_a(0, ta0);
+      asm volatile("" ::: "memory");   // the loads above are neither sunk below the branches of the reduction
+      __builtin_amdgcn_sched_barrier(0);   // nor overtaken by its arithmetic (which waits for the activations)
       pro.reduce(ss_part, wgi == 0 ? a.x_out : nullptr, a.rows, a.d);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -586,6 +591,14 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       __syncthreads();
       GLU_STAMP(1);
       pro.scale(ss_part, hs, ld, a.rows, a.d, a.eps);
+    };
+    constexpr int NXMAX = PRO == 2 ? 2 : NXC;
+    if (total <= 512 && (nchunk & 31) == 0) {
+      lean(std::integral_constant<int, 1>{});
+    } else if (total <= 1024 && (nchunk & 31) == 0) {
+      lean(std::integral_constant<int, 2>{});
+    } else if (NXMAX >= 4 && total <= 2048 && (nchunk & 31) == 0) {
+      lean(std::integral_constant<int, NXMAX>{});
     } else if (PRO == 1) {
       // any other shape: wave per row
       uint4 nwv[4];

@@ -43,6 +43,8 @@ struct NormPrologue {
   uint4 sv[NSV];
   int rowj[NXC];
 
+  // the caller picks the smallest NXC with rows * d/8 <= NXC * NT: every j below then has chunks to do, and the code
+  // is one straight line (lanes beyond the last chunk read zeros and store nothing)
   static __host__ __device__ bool supported(int rows, int d) {
     return d % 256 == 0 && rows >= 1 && (long long)rows * (d / 8) <= (long long)NXC * NT;
   }
@@ -57,7 +59,6 @@ struct NormPrologue {
     const float inv_nc = 1.0f / (float)nchunk;
 #pragma unroll
     for (int j = 0; j < NXC; ++j) {
-      if (j * NT >= total) continue;   // uniform
       const int q = threadIdx.x + j * NT;
       rowj[j] = (int)(((float)q + 0.5f) * inv_nc);
       xv[j] = fstu_buf_load16(rx, (unsigned)q * 16u);     // beyond the last chunk: zeros
@@ -81,7 +82,6 @@ struct NormPrologue {
     const int nchunk = d >> 3, total = rows * nchunk;
 #pragma unroll
     for (int j = 0; j < NXC; ++j) {
-      if (j * NT >= total) continue;
       const int q = threadIdx.x + j * NT;
       unsigned xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
       float ss = 0.f;
@@ -117,11 +117,10 @@ struct NormPrologue {
   }
 
   // the norm weights have arrived (keeps later loads of the caller from having to be waited for with them)
-  __device__ __forceinline__ void pin_weights(int rows, int d) {
-    const int total = rows * (d >> 3);
+  __device__ __forceinline__ void pin_weights() {
 #pragma unroll
     for (int j = 0; j < NXC; ++j)
-      if (j * NT < total) asm volatile("" ::"v"(nv[j].x), "v"(nv[j].y), "v"(nv[j].z), "v"(nv[j].w));
+      asm volatile("" ::"v"(nv[j].x), "v"(nv[j].y), "v"(nv[j].z), "v"(nv[j].w));
   }
 
   // phase 3 (after a __syncthreads()): h rows into LDS, row stride ld elements
@@ -130,7 +129,6 @@ struct NormPrologue {
     const float inv_d = 1.0f / (float)d;
 #pragma unroll
     for (int j = 0; j < NXC; ++j) {
-      if (j * NT >= total) continue;
       const int q = threadIdx.x + j * NT;
       if (q < total) {
         float ss = 0.f;

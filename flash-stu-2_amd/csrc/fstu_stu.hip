@@ -291,9 +291,14 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   const int tile = blockIdx.x, c0 = tile * 16;
   // residual update + norm in the prologue: its loads go first, they head the kernel's critical path
   typedef NormPrologue<256, 4, 4> Pro;
+  typedef NormPrologue<256, 3, 4> Pro3;   // exact for rows * K / 8 <= 768: one straight line without idle chunks
   Pro pro;
+  Pro3 pro3;
   const bool merged = x_res != nullptr && slices != nullptr;
-  if (merged) pro.issue(x_res, slices, nslices, norm_w, B, K);
+  const bool exact3 = B * (K >> 3) <= 768;
+  if (merged) {
+    if (exact3) pro3.issue(x_res, slices, nslices, norm_w, B, K); else pro.issue(x_res, slices, nslices, norm_w, B, K);
+  }
   // ---- projection: A operand = Mt rows (channels), B operand = h rows (batch)
   const int kw = K >> 2;                                    // k range of this wave
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
@@ -334,10 +339,11 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   if (merged) {
     bf16_t* hs = (bf16_t*)inproj_smem;
     __shared__ float ss_part[Pro::NPART];
-    pro.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
+    if (exact3) pro3.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
+    else pro.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
     __syncthreads();
     STU_STAMP(1);
-    pro.scale(ss_part, hs, ldn, B, K, eps);
+    if (exact3) pro3.scale(ss_part, hs, ldn, B, K, eps); else pro.scale(ss_part, hs, ldn, B, K, eps);
     __syncthreads();
     STU_STAMP(2);
     hp = hs + (size_t)(xrow ? r : 0) * ldn + w * kw + g * 16;
