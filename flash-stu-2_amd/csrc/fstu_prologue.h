@@ -116,6 +116,16 @@ struct NormPrologue {
     }
   }
 
+  // Makes the loaded values opaque at this point of the program: arithmetic of reduce() that depends on a single load
+  // (the first term of a slice sum) can then not be hoisted to the loads, where its wait would stall whatever the
+  // caller issues between issue() and reduce().
+  __device__ __forceinline__ void pin_loads() {
+    if (NS > 0) {
+#pragma unroll
+      for (int k = 0; k < NSV; ++k) asm volatile("" : "+v"(sv[k].x), "+v"(sv[k].y), "+v"(sv[k].z), "+v"(sv[k].w));
+    }
+  }
+
   // the norm weights have arrived (keeps later loads of the caller from having to be waited for with them)
   __device__ __forceinline__ void pin_weights() {
 #pragma unroll

@@ -289,16 +289,13 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int tile = blockIdx.x, c0 = tile * 16;
-  // residual update + norm in the prologue: its loads go first, they head the kernel's critical path
+  // residual update + norm in the prologue
   typedef NormPrologue<256, 4, 4> Pro;
   typedef NormPrologue<256, 3, 4> Pro3;   // exact for rows * K / 8 <= 768: one straight line without idle chunks
   Pro pro;
   Pro3 pro3;
   const bool merged = x_res != nullptr && slices != nullptr;
   const bool exact3 = B * (K >> 3) <= 768;
-  if (merged) {
-    if (exact3) pro3.issue(x_res, slices, nslices, norm_w, B, K); else pro.issue(x_res, slices, nslices, norm_w, B, K);
-  }
   // ---- projection: A operand = Mt rows (channels), B operand = h rows (batch)
   const int kw = K >> 2;                                    // k range of this wave
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
@@ -316,12 +313,12 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     float* st = state + (((size_t)(pre ? bsub : 0) * 2 + parity) * S) * d + (pre ? c : 0);
 #pragma unroll
     for (int k = 0; k < PJ; ++k) {
-      const int j = jsub + 8 * k;
-      if (pre && j < S) {
-        phv[k] = *(const float4*)(st + (size_t)j * d);
-        pcj[k] = *(const float4*)(ce + (size_t)j * d + c);
-        paj[k] = a[j];
-      }
+      // branch-free (out-of-range lanes and modes re-read a valid element and ignore it): a conditional load would
+      // reach its use through a copy, and the copy's wait would hold back every load issued after it
+      const int j = min(jsub + 8 * k, S - 1);
+      phv[k] = *(const float4*)(st + (size_t)j * d);
+      pcj[k] = *(const float4*)(ce + (size_t)j * d + (pre ? c : 0));
+      paj[k] = a[j];
     }
   }
   stu_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -336,6 +333,12 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     }
   }
   const int ldn = K + 8;
+  // The prologue's loads go last: the compiler starts their arithmetic (and so their waits) right behind them, and
+  // loads issued after that point would cost a second trip to memory.  The loads above return first anyway.
+  __builtin_amdgcn_sched_barrier(0);
+  if (merged) {
+    if (exact3) pro3.issue(x_res, slices, nslices, norm_w, B, K); else pro.issue(x_res, slices, nslices, norm_w, B, K);
+  }
   if (merged) {
     bf16_t* hs = (bf16_t*)inproj_smem;
     __shared__ float ss_part[Pro::NPART];
