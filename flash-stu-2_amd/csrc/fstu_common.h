@@ -45,6 +45,10 @@ int fstu_swa_qkv_decode_dyn(const void* h_in, const void* x_in, const float* sli
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                          float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream);
+bool fstu_finish_embed_supported(int rows, int d, const void* table, const void* x, const void* w, const void* h);
+int fstu_finish_embed_rmsnorm(void* best_ws, int64_t* tok_out, int64_t tok_stride, const void* table, void* x, const void* w,
+                              void* h, int* dyn, int rows, int d, int vocab, float eps, void* stream);
+bool fstu_head_argmax_fused_pick(const void* x, int ldx, const void* W, int K, int dtype);
 int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table, void* x, const void* w, void* h, int rows,
                        int d, int vocab, float eps, int dtype, void* stream, const int* dyn);
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,

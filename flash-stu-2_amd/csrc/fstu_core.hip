@@ -334,6 +334,84 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
   return FSTU_OK;
 }
 
+// ---------------------------------------------------------------- greedy pick of one step finished inside the next step's first launch
+// The head of a greedy step leaves 64 packed maxima per row ((key << 32) | ~index).  Inside a graph of several steps the
+// launch that would reduce them, store the token and advance the device-side position is followed at once by the
+// next step's embedding + norm launch, which needs nothing but that token: both are one launch here.  One
+// workgroup, one wave per row (so the position is read by every wave before thread 0 advances it); a lane owns
+// chunks lane, lane+64, ... (8 channels each) of its row.
+__global__ void __launch_bounds__(1024)
+finish_embed_rmsnorm_kernel(unsigned long long* __restrict__ best, int64_t* __restrict__ tok_out, int64_t stride,
+                            const bf16_t* __restrict__ table, bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                            bf16_t* __restrict__ h, int* __restrict__ dyn, int d, int vocab, float eps) {
+  constexpr int NCH = 4;   // d <= 2048
+  const int b = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = dyn[0];
+  unsigned long long k = best[(size_t)b * 64 + lane];
+  uint4 wv[NCH], xv[NCH];
+  const fstu_rsrc_t rw = fstu_make_rsrc(w, (size_t)d * 2);
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) wv[j] = fstu_buf_load16(rw, (unsigned)(lane + 64 * j) * 16u);
+  best[(size_t)b * 64 + lane] = 0ull;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    unsigned long long t = __shfl_xor(k, o, FSTU_WAVE);
+    k = t > k ? t : k;
+  }
+  int64_t id = (int64_t)(0xffffffffu - (unsigned)(k & 0xffffffffull));
+  __syncthreads();
+  if (threadIdx.x == 0) { dyn[0] = pos + 1; dyn[1] += 1; }
+  if (lane == 0) tok_out[(size_t)b * stride + pos] = id;
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const fstu_rsrc_t rx = fstu_make_rsrc(table + (size_t)id * d, (size_t)d * 2);
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) xv[j] = fstu_buf_load16(rx, (unsigned)(lane + 64 * j) * 16u);
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const unsigned xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = __uint_as_float(xw[i] << 16), hi = __uint_as_float(xw[i] & 0xffff0000u);
+      ss = fmaf(lo, lo, ss);
+      ss = fmaf(hi, hi, ss);
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(ss) / (float)d + eps);
+  const int nchunk = d >> 3;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int q = lane + 64 * j;
+    if (q < nchunk) {
+      const unsigned xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+      unsigned o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o[i] = pack2_bf16((__uint_as_float(xw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
+                          (__uint_as_float(xw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
+      *(uint4*)(x + (size_t)b * d + q * 8) = xv[j];
+      *(uint4*)(h + (size_t)b * d + q * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
+bool fstu_finish_embed_supported(int rows, int d, const void* table, const void* x, const void* w, const void* h) {
+  return rows >= 1 && rows <= 16 && (d & 7) == 0 && d <= 2048 &&
+         (((uintptr_t)table | (uintptr_t)w | (uintptr_t)x | (uintptr_t)h) & 15) == 0;
+}
+
+int fstu_finish_embed_rmsnorm(void* best_ws, int64_t* tok_out, int64_t tok_stride, const void* table, void* x, const void* w,
+                              void* h, int* dyn, int rows, int d, int vocab, float eps, void* stream) {
+  FSTU_REQUIRE(best_ws && tok_out && table && x && w && h && dyn, FSTU_ENULL, "fstu_finish_embed_rmsnorm: null pointer");
+  FSTU_REQUIRE(fstu_finish_embed_supported(rows, d, table, x, w, h), FSTU_ESHAPE,
+               "fstu_finish_embed_rmsnorm: rows=%d d=%d unsupported (rows <= 16, d %% 8 == 0, d <= 2048, 16-byte aligned)", rows, d);
+  hipLaunchKernelGGL(finish_embed_rmsnorm_kernel, dim3(1), dim3(rows * 64), 0, (hipStream_t)stream,
+                     (unsigned long long*)best_ws, tok_out, tok_stride, (const bf16_t*)table, (bf16_t*)x, (const bf16_t*)w,
+                     (bf16_t*)h, dyn, d, vocab, eps);
+  FSTU_CHECK_LAUNCH("fstu_finish_embed_rmsnorm");
+  return FSTU_OK;
+}
+
 // ---------------------------------------------------------------- gelu * up
 template <typename T>
 __global__ void gelu_mul_kernel(const T* __restrict__ g, const T* __restrict__ u, T* __restrict__ act, int64_t n) {

@@ -245,6 +245,16 @@ static thread_local int g_stu_parity = -1;
 static inline const int* stu_dyn(const int* dyn) { return g_stu_parity >= 0 ? nullptr : dyn; }
 static inline int stu_pos(int pos) { return g_stu_parity >= 0 ? g_stu_parity : pos; }
 
+// Inside a graph of several greedy steps the reduction of one step's packed maxima (token store, position advance) and
+// the next step's embedding + norm are one launch.  g_chain_prev: this step starts with that launch; g_chain_next:
+// this step's head leaves its maxima for the next step.
+static thread_local bool g_chain_prev = false, g_chain_next = false;
+static bool chain_ok(const fstu_model_desc* m, int do_sample, const int* dyn) {
+  return dyn && !do_sample && m->best && m->dtype == FSTU_BF16 && !m->head_packed && !fused_available(m) &&
+         fstu_head_argmax_fused_pick(m->h, m->d, m->emb, m->d, m->dtype) &&
+         fstu_finish_embed_supported(m->B, m->d, m->emb, m->x, m->layers[0].norm1_w, m->h);
+}
+
 // dyn == nullptr: pos/step come from the host arguments.  dyn != nullptr (graph capture): every position-dependent
 // kernel reads {pos, step} from that device int[2]; tok_in/tok_out are then the bases of token columns 0 and 1.
 static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
@@ -278,8 +288,13 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   if (fused_available(m))
     return decode_step_fused(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
   // x = embedding rows, h = norm(x) with the first layer's norm weight
-  TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt,
-                                    stream, dyn));
+  const bool chain = chain_ok(m, do_sample, dyn);
+  if (chain && g_chain_prev)
+    TIMED(PC_NORM, fstu_finish_embed_rmsnorm(m->best, tok_out, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, dyn, B, d,
+                                             m->V, m->eps, stream));
+  else
+    TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt,
+                                      stream, dyn));
   // The residual stream starts in m->x.  Where a layer has packed gate/up weights, its MLP norm runs as the
   // prologue of the GLU GEMV, which writes the updated residual to the other buffer (xc <-> xo swap).
   void* xc = m->x;
@@ -427,7 +442,7 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                                                tok_stride, dyn, 1, stream));
   } else if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
-                                        tok_stride, dyn, 1, dt, stream));
+                                        tok_stride, dyn, (chain && g_chain_next) ? -1 : 1, dt, stream));
   } else {
     TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
     TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));
@@ -500,9 +515,12 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
     int rc = 0;
     for (int st = 0; st < nsteps && rc == 0; ++st) {
       g_stu_parity = baked ? ((par + st) & 1) : -1;
+      g_chain_prev = st > 0;
+      g_chain_next = st + 1 < nsteps;
       rc = decode_step_impl(m, tokens, tokens + 1, tok_stride, 0, temperature, top_k, top_p, do_sample, seed, 0, dyn, stream);
     }
     g_stu_parity = -1;
+    g_chain_prev = g_chain_next = false;
     g_warm = nullptr;
     e = hipStreamEndCapture(s, &h->graph[par]);
     if (rc != 0) { fstu_decode_graph_destroy(h); return rc; }

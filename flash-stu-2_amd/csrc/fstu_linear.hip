@@ -339,6 +339,11 @@ extern "C" int fstu_head_argmax(const void* x, int ldx, const void* W, void* log
                               dtype, stream);
 }
 
+// true when fstu_head_argmax takes the path that leaves packed maxima in the workspace (and so can defer their reduction)
+bool fstu_head_argmax_fused_pick(const void* x, int ldx, const void* W, int K, int dtype) {
+  return dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1);
+}
+
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                          float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream) {
@@ -350,8 +355,10 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   if (dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1)) {
     LinArgs a{x, ldx, W, nullptr, logits, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
     launch_mfma<LIN_ARGMAX>(a, 1, (hipStream_t)stream);
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(rows * 64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
-                       tok_out, tok_stride, rows, dyn, advance);
+    // advance < 0: the caller's next launch reduces the maxima itself (fstu_finish_embed_rmsnorm)
+    if (advance >= 0)
+      hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(rows * 64), 0, (hipStream_t)stream, (unsigned long long*)best_ws,
+                         tok_out, tok_stride, rows, dyn, advance);
     FSTU_CHECK_LAUNCH("fstu_head_argmax");
     return FSTU_OK;
   }
