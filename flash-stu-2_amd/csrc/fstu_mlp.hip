@@ -1182,6 +1182,7 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   else if (ksb <= 8) hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+  else if (ksb == 9) hipLaunchKernelGGL(down_splitk_balanced_kernel<9>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   else hipLaunchKernelGGL(down_splitk_balanced_kernel<12>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
   if (ksplit_io) *ksplit_io = KS;
