@@ -31,7 +31,7 @@ def build_model(args, torch):
     from flash_stu import FlashSTU, FlashSTUConfig
     cfg = FlashSTUConfig(n_embd=768, n_layers=12, n_heads=12, window_size=512, num_eigh=24, seq_len=2048,
                          vocab_size=50257, mlp_scale=args.mlp_scale, torch_dtype=torch.bfloat16,
-                         stu_decode_mode=args.stu_mode)
+                         stu_decode_mode=args.stu_mode, stu_prefill_mode=args.stu_prefill)
     torch.manual_seed(1)
     model = FlashSTU(cfg).cuda().eval()
     return cfg, model
@@ -86,6 +86,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--mlp-scale", type=int, default=12, dest="mlp_scale")
     ap.add_argument("--stu-mode", default="lds", choices=["lds", "history"], dest="stu_mode")
+    ap.add_argument("--stu-prefill", default="fft", choices=["fft", "scan"], dest="stu_prefill",
+                    help="prompt pass of the STU layers: the reference's FFT convolution, or the distilled recurrence as a scan")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -208,7 +210,7 @@ def main():
         "config": {"workload": "BASELINE config 2: FlashSTU 768-d/12-layer/12-head, window 512, K=24, seq_len 2048, "
                                "vocab 50257, random-init bf16 seed 1, batch 8, 512-token prompt, greedy decode",
                    "mlp_scale": cfg.mlp_scale, "params": model.get_num_params(), "batch": B, "prompt": P,
-                   "stu_decode_mode": args.stu_mode, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
+                   "stu_decode_mode": args.stu_mode, "stu_prefill_mode": args.stu_prefill, "hip_graph": bool(use_graph), "stu_state_dim": S if args.stu_mode == "lds" else None},
         "roofline": {"bound": "hbm", "kernel": ("glu_balanced_kernel<PRO> (residual add + mlp_norm + gate/up projection + gelu*up)"
                                 if getattr(eng.desc, "glu_packed", 0) and eng.desc.x2 else
                                 "glu_balanced_kernel (gate/up projection + gelu*up)" if getattr(eng.desc, "glu_packed", 0)

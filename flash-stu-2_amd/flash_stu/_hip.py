@@ -37,6 +37,7 @@ SIGNATURES = {
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_scan_lds": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -296,6 +297,29 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
     _check(load().fstu_stu_step_lds(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
            "fstu_stu_step_lds")
     return out
+
+
+def stu_scan_lds(xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, state: Optional[torch.Tensor] = None,
+                 t_start: int = 0, out: Optional[torch.Tensor] = None):
+    """xp (B,T,d) -> (y (B,T,d), state fp32 (B,2,S,d)): the recurrence step over a whole sequence in one launch.
+    state=None starts from zero; a given state is continued in place (t_start = position of xp[:, 0])."""
+    _dev(a, ce, state)
+    if not xp.is_cuda or (out is not None and not out.is_cuda):
+        raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    B, T, d = xp.shape          # batch and token strides are passed on: slices along time need no copy
+    S = a.numel()
+    assert a.dtype == torch.float32 and ce.dtype == torch.float32 and ce.shape == (S, d) and ce.is_contiguous()
+    assert xp.stride(2) == 1
+    carry = state is not None
+    if state is None:
+        state = torch.empty(B, 2, S, d, dtype=torch.float32, device=xp.device)
+    assert state.shape == (B, 2, S, d) and state.dtype == torch.float32 and state.is_contiguous()
+    if out is None:
+        out = torch.empty(B, T, d, dtype=xp.dtype, device=xp.device)
+    assert out.shape == xp.shape and out.dtype == xp.dtype and out.stride(2) == 1
+    _check(load().fstu_stu_scan_lds(_p(xp), xp.stride(0), xp.stride(1), _p(a), _p(ce), _p(state), _p(out), out.stride(0),
+                                    out.stride(1), B, T, S, d, t_start, int(carry), _dt(xp), _stream()), "fstu_stu_scan_lds")
+    return out, state
 
 
 def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,

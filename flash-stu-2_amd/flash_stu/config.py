@@ -47,6 +47,7 @@ class FlashSTUConfig:
         rms_norm_eps: float = RMS_NORM_EPS,
         stu_decode_mode: str = "auto",       # "history" (exact), "lds" (distilled recurrence), "auto": lds for bf16
         stu_lds_state_dim: int = 64,
+        stu_prefill_mode: str = "fft",       # "fft": the reference's convolution; "scan": the distilled recurrence over the prompt
         **kwargs: Any,
     ):
         self.bsz = bsz
@@ -87,6 +88,9 @@ class FlashSTUConfig:
             raise ValueError(f"stu_decode_mode must be auto|history|lds, got {stu_decode_mode!r}")
         self.stu_decode_mode = stu_decode_mode
         self.stu_lds_state_dim = stu_lds_state_dim
+        if stu_prefill_mode not in ("fft", "scan"):
+            raise ValueError(f"stu_prefill_mode must be fft|scan, got {stu_prefill_mode!r}")
+        self.stu_prefill_mode = stu_prefill_mode
         self.use_return_dict = kwargs.pop("return_dict", True)
         self.output_hidden_states = kwargs.pop("output_hidden_states", False)
         for k, v in kwargs.items():          # unknown keys are kept, as PretrainedConfig does

@@ -137,6 +137,13 @@ class STU(nn.Module):
         params = (self.M_phi_plus,) + (() if self.use_hankel_L else (self.M_phi_minus,))
         return self._cached("flat", params, build)
 
+    def _scan_prefill(self) -> bool:
+        """stu_prefill_mode='scan': approx mode with both sign branches only (the recurrence is fitted to the even
+        lags of the two-branch filter), 16-byte aligned rows."""
+        esz = 8 if self.M_inputs.dtype == torch.bfloat16 else 4
+        return (getattr(self.config, "stu_prefill_mode", "fft") == "scan" and not self.use_hankel_L
+                and self.d_out % esz == 0)
+
     # ---- full-sequence evaluation
     def _project(self, x: torch.Tensor) -> torch.Tensor:
         B, T, d = x.shape
@@ -190,6 +197,16 @@ class STU(nn.Module):
         if past_state is None:
             if T > self.phi.shape[0]:
                 raise ValueError(f"sequence length {T} exceeds the filter length {self.phi.shape[0]}")
+            if self.use_approx and self._scan_prefill():
+                # the distilled recurrence over the whole prompt: outputs and the decode state in one launch
+                xp = self._project(x)
+                a, ce = self.lds_params()
+                y, state = _hip.stu_scan_lds(xp, a, ce)
+                if not use_cache:
+                    return y
+                if self.decode_mode() == "lds":
+                    return y, (xp.new_empty(B, 0, self.d_out), state, torch.full((B,), T, dtype=torch.int64))
+                return y, self._state_from_sequence(xp)
             if self.use_approx:
                 xp = self._project(x)
                 y = self._convolve(xp)

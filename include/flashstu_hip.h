@@ -150,6 +150,18 @@ int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices,
                              const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
                              int d, int K, int t, void* stream);
 
+/* The step of fstu_stu_step_lds applied to T consecutive positions t_start .. t_start+T-1 in one launch (scan form
+ * of the prefill: no FFT, no history buffer): y[b,t,c] for every position and the state after the last one.
+ * xp, y are (B,T,d) with element strides (x_bstride, x_tstride, 1) / (y_bstride, y_tstride, 1), rows 16-byte aligned;
+ * carry 0 starts from a zero state (state is output only), carry 1 continues from the state given.  S <= 128.
+ * The final state equals T calls of fstu_stu_step_lds bit for bit; the outputs differ from theirs only by the order
+ * of the sum over the S modes.  Sequence counterpart of the reference's scan, mini_stu/stu_lds.py:17-68 (Triton
+ * lds_scan_kernel) and :279-338 (FixedDiagonalLDS.forward), merged with the approx-mode contraction of
+ * flash_stu/modules/stu.py:87-98,120. */
+int fstu_stu_scan_lds(const void* xp, int64_t x_bstride, int64_t x_tstride, const float* a, const float* ce,
+                      float* state, void* y, int64_t y_bstride, int64_t y_tstride, int B, int T, int S, int d,
+                      int t_start, int carry, int dtype, void* stream);
+
 /* Builds that state from a prefilled history: for both parities p,
  *   state[b,p,j,c] = sum_{m>=0} a[j]^m * hist[b, tp-2m, c],  tp = newest index
  *   of parity p that is <= t_last.  hist is (B,cap,d). */

@@ -17,7 +17,7 @@ def make_pair(seed=0, init="healthy", **kw):
     """(oracle cfg, oracle weights, device model) sharing the same tensors."""
     from flash_stu import FlashSTU, FlashSTUConfig
     dt = kw.pop("dtype", torch.float32)
-    extra = {k: kw.pop(k) for k in ("stu_decode_mode", "stu_lds_state_dim") if k in kw}
+    extra = {k: kw.pop(k) for k in ("stu_decode_mode", "stu_lds_state_dim", "stu_prefill_mode") if k in kw}
     ocfg = O.OracleConfig(dtype=dt, **kw)
     w = O.init_weights(ocfg, seed=seed, mode=init)
     cfg = FlashSTUConfig(n_embd=ocfg.n_embd, n_heads=ocfg.n_heads, n_layers=ocfg.n_layers, seq_len=ocfg.seq_len,
@@ -90,6 +90,31 @@ def test_graph_replay_equals_eager_steps(do_sample):
         got = model.generate(ids, use_graph=True, **kw)
         assert torch.equal(got, eager)
     del junk
+
+
+@pytest.mark.parametrize("dtype,mode", [(torch.bfloat16, "lds"), (torch.float32, "lds"), (torch.float32, "history")])
+def test_scan_prefill_against_oracle_and_fft_prefill(dtype, mode):
+    """stu_prefill_mode='scan' (the distilled recurrence over the prompt instead of the FFT convolution): prompt logits
+    within the model-dtype tolerance of the oracle's, the decode state it leaves equal to the one the FFT path
+    builds (same recurrence over the same projected inputs), and generation continues from it."""
+    kw = dict(seed=5, init="healthy", dtype=dtype, mlp_scale=2, n_embd=128, n_layers=4, n_heads=2, window_size=16,
+              num_eigh=8, seq_len=256, vocab_size=701, stu_decode_mode=mode)
+    ocfg, w, fft = make_pair(**kw)
+    _, _, scan = make_pair(stu_prefill_mode="scan", **kw)
+    ids = prompt(2, 150, ocfg.vocab_size, 4)
+    ref, _ = O.model_forward(w, ocfg, ids)
+    a = fft(ids.cuda(), use_cache=True)
+    b = scan(ids.cuda(), use_cache=True)
+    scale = float(ref.abs().max())
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-3      # fp32: the fit error of the 64-mode recurrence (about 1e-4 per layer)
+    assert float((b.logits.float().cpu() - ref.float()).abs().max()) <= tol * scale
+    assert float((b.logits.float() - a.logits.float()).abs().max()) <= tol * scale
+    if mode == "lds":
+        for ca, cb in zip(a.past_key_values, b.past_key_values):
+            if len(ca) == 3 and ca[0].dim() == 3 and ca[0].shape[1] == 0:     # STU entry: (empty hist, state, pos)
+                assert float((ca[1] - cb[1]).abs().max()) <= 2e-2 * float(ca[1].abs().max())
+    out = scan.generate(ids.cuda(), max_length=170, do_sample=False)
+    assert out.shape == (2, 170) and torch.equal(out[:, :150].cpu(), ids)
 
 
 def _teacher_forced(w, ocfg, tokens, P):

@@ -320,6 +320,49 @@ def test_stu_step_lds_recurrence(hip, dtype):
     assert float((st2.cpu().double() - h64).abs().max()) < 1e-4 * float(h64.abs().max())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,S,d,T,t_start", [(3, 64, 256, 41, 0), (2, 64, 768, 512, 0), (2, 40, 200, 37, 5), (1, 128, 64, 130, 1),
+                                             (2, 64, 128, 1, 3), (2, 8, 72, 16, 0)])
+def test_stu_scan_lds_equals_steps_and_float64(hip, dtype, B, S, d, T, t_start):
+    """The whole-sequence recurrence: outputs equal a float64 evaluation of the recurrence, the final state equals
+    T single-token steps bit for bit; ragged channel counts, odd start positions, S not a multiple of 8, and a
+    sequence continued from a carried state in two pieces of odd length."""
+    g = gen(8)
+    a = (0.5 + 0.49 * torch.rand(S, generator=g)).float()
+    ce = (torch.randn(S, d, generator=g) / S).float()
+    xs = torch.randn(B, T, d, generator=g).to(dtype)
+    h64 = torch.zeros(B, 2, S, d, dtype=torch.float64)
+    ref = torch.zeros(B, T, d, dtype=torch.float64)
+    for t in range(T):
+        p = (t_start + t) & 1
+        h64[:, p] = a.double()[None, :, None] * h64[:, p] + xs[:, t].double()[:, None, :]
+        ref[:, t] = 2 * (ce.double()[None] * h64[:, p]).sum(1)
+    ad, ced, xd = dev(a), dev(ce), dev(xs)
+    y, st = hip.stu_scan_lds(xd, ad, ced, t_start=t_start)
+    check(y, ref.to(dtype), dtype, frac=0.05, scale=float(ref.abs().max()))
+    assert float((st.cpu().double() - h64).abs().max()) <= 1e-4 * float(h64.abs().max())
+    if T <= 64:
+        step_state = torch.zeros(B, 2, S, d, device="cuda")
+        ys = [hip.stu_step_lds(step_state, xd[:, t].contiguous(), ad, ced, t_start + t) for t in range(T)]
+        assert torch.equal(st, step_state)
+        check(y, torch.stack(ys, 1).float().cpu().to(dtype), dtype, frac=0.05, scale=float(ref.abs().max()))
+    if T >= 3:
+        cut = (T // 2) | 1
+        y1, st1 = hip.stu_scan_lds(xd[:, :cut], ad, ced, t_start=t_start)
+        y2, st2 = hip.stu_scan_lds(xd[:, cut:], ad, ced, state=st1, t_start=t_start + cut)
+        assert st2.data_ptr() == st1.data_ptr()
+        assert torch.equal(torch.cat([y1, y2], 1), y) and torch.equal(st2, st)
+
+
+def test_stu_scan_lds_rejects_bad_arguments(hip):
+    a = torch.full((200,), 0.9, device="cuda")
+    x = torch.zeros(1, 4, 64, device="cuda")
+    with pytest.raises(RuntimeError):
+        hip.stu_scan_lds(x, a, torch.zeros(200, 64, device="cuda"))          # S > 128
+    with pytest.raises(RuntimeError):
+        hip.stu_scan_lds(torch.zeros(1, 4, 66, device="cuda", dtype=torch.bfloat16), a[:8], torch.zeros(8, 66, device="cuda"))
+
+
 def test_stu_inproj_step_equals_projection_then_step(hip):
     g = gen(21)
     B, S, d = 8, 64, 768
