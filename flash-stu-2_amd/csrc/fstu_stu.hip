@@ -640,38 +640,41 @@ extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, fl
 // ---------------------------------------------------------------- whole-sequence recurrence (scan form of the prefill)
 // The decode step of fstu_stu_step_lds applied to T consecutive positions in one launch: outputs for every position and
 // the state after the last one, without an FFT and without a history buffer (sequence counterpart of
-// mini_stu/stu_lds.py:17-68,279-338).  Workgroup = (64 channels, batch row); lane = channel; the 8 waves split the modes,
-// wave w keeps modes [w*MW, (w+1)*MW) of both parity banks in registers for the whole sequence.  Time runs in blocks
-// of 16 positions: the block's inputs are staged in LDS once (the next block's are in flight meanwhile), every wave
-// steps its modes through the block and leaves one partial output per position in LDS, then the 8 partials are
-// summed in wave order.  Per mode the update is the same fmaf as the decode step, so the final state equals T decode
-// steps bit for bit; the outputs differ from them only by the order of the sum over modes.
-#define SCAN_TB 16
+// mini_stu/stu_lds.py:17-68,279-338).  The two parity banks are independent recurrences (even positions only touch
+// the even bank), so they advance side by side: workgroup = (32 channels, batch row), lane = (parity, channel), and
+// one pass of the loop steps an even and an odd position.  The 8 waves split the modes; wave w keeps modes
+// [w*MW, (w+1)*MW) of its lanes' bank in registers for the whole sequence.  Time runs in blocks of 32 positions: the
+// block's inputs are staged in LDS once (the next block's are in flight meanwhile), every wave steps its modes
+// through the block and leaves one partial output per position in LDS, then the 8 partials are summed in wave order.
+// Per mode the update is the same fmaf as the decode step, so the final state equals T decode steps bit for bit;
+// the outputs differ from them only by the order of the sum over modes.
+#define SCAN_TB 32
+#define SCAN_CH 32
 template <typename T, int MW>
 __global__ void __launch_bounds__(512)
 stu_scan_lds_kernel(const T* __restrict__ xp, long long sxb, long long sxt, const float* __restrict__ a,
                     const float* __restrict__ ce, float* __restrict__ state, T* __restrict__ y, long long syb,
                     long long syt, int Tn, int S, int d, int t_start, int carry) {
-  __shared__ __align__(16) T xs[SCAN_TB * 64];
-  __shared__ float part[8][SCAN_TB][64];
+  __shared__ __align__(16) T xs[SCAN_TB * SCAN_CH];
+  __shared__ float part[8][SCAN_TB * SCAN_CH];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int b = blockIdx.y, c0 = blockIdx.x * 64, c = c0 + lane;
+  const int ch = lane & 31, hp = lane >> 5;      // hp: parity of the position inside this call
+  const int b = blockIdx.y, c0 = blockIdx.x * SCAN_CH, c = c0 + ch;
   const bool cok = c < d;
   const int cc = cok ? c : d - 1;
-  const int sp = t_start & 1;           // logical bank lb holds the physical bank lb ^ sp
-  float h[2][MW], aj[MW], cj[MW];
+  const int bank = hp ^ (t_start & 1);           // the state bank this lane advances
+  float h[MW], aj[MW], cj[MW];
 #pragma unroll
   for (int m = 0; m < MW; ++m) {
     const int j = w * MW + m;
     const bool jok = j < S;
     aj[m] = jok ? a[j] : 0.f;
     cj[m] = jok ? ce[(size_t)j * d + cc] : 0.f;
-#pragma unroll
-    for (int lb = 0; lb < 2; ++lb)
-      h[lb][m] = (carry && jok) ? state[(((size_t)b * 2 + (lb ^ sp)) * S + j) * d + cc] : 0.f;
+    h[m] = (carry && jok) ? state[(((size_t)b * 2 + bank) * S + j) * d + cc] : 0.f;
   }
-  // input tile: SCAN_TB rows of 64 channels, one 16-byte piece per thread (bf16: the first 256 threads)
-  constexpr int PIECES = SCAN_TB * 64 * (int)sizeof(T) / 16, PPR = 64 * (int)sizeof(T) / 16, EPP = 16 / (int)sizeof(T);
+  // input tile: SCAN_TB rows of SCAN_CH channels, one 16-byte piece per loading thread
+  constexpr int PIECES = SCAN_TB * SCAN_CH * (int)sizeof(T) / 16, PPR = SCAN_CH * (int)sizeof(T) / 16,
+                EPP = 16 / (int)sizeof(T);
   const int prow = threadIdx.x / PPR, pcol = (threadIdx.x % PPR) * EPP;
   const bool ploader = threadIdx.x < PIECES && c0 + pcol < d;
   auto load_tile = [&](int t0) {
@@ -681,29 +684,30 @@ stu_scan_lds_kernel(const T* __restrict__ xp, long long sxb, long long sxt, cons
   };
   uint4 xr = load_tile(0);
   for (int t0 = 0; t0 < Tn; t0 += SCAN_TB) {
-    if (threadIdx.x < PIECES) *(uint4*)(xs + prow * 64 + pcol) = xr;
+    if (threadIdx.x < PIECES) *(uint4*)(xs + prow * SCAN_CH + pcol) = xr;
     __syncthreads();
     xr = load_tile(t0 + SCAN_TB);
 #pragma unroll
-    for (int k = 0; k < SCAN_TB; ++k) {
+    for (int i = 0; i < SCAN_TB / 2; ++i) {
+      // position 2i + hp of the block: element 64 i + lane of the tile
       float p = 0.f;
-      if (t0 + k < Tn) {   // uniform; a step past the end must not decay the state
-        const float x = DT<T>::ld(xs + k * 64 + lane);
+      if (t0 + 2 * i + hp < Tn) {   // a step past the end must not decay the state
+        const float x = DT<T>::ld(xs + 64 * i + lane);
 #pragma unroll
         for (int m = 0; m < MW; ++m) {
-          h[k & 1][m] = fmaf(aj[m], h[k & 1][m], x);
-          p = fmaf(cj[m], h[k & 1][m], p);
+          h[m] = fmaf(aj[m], h[m], x);
+          p = fmaf(cj[m], h[m], p);
         }
       }
-      part[w][k][lane] = p;
+      part[w][64 * i + lane] = p;
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < SCAN_TB / 8; ++i) {
-      const int k = w + 8 * i;
+    for (int i = 0; i < SCAN_TB / 16; ++i) {
+      const int e = (w * (SCAN_TB / 16) + i) * 64 + lane, k = e >> 5;   // tile element: position k, channel ch
       float sum = 0.f;
 #pragma unroll
-      for (int ww = 0; ww < 8; ++ww) sum += part[ww][k][lane];
+      for (int ww = 0; ww < 8; ++ww) sum += part[ww][e];
       if (cok && t0 + k < Tn) DT<T>::st(y + (size_t)b * syb + (size_t)(t0 + k) * syt + c, 2.f * sum);
     }
   }
@@ -711,10 +715,7 @@ stu_scan_lds_kernel(const T* __restrict__ xp, long long sxb, long long sxt, cons
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
       const int j = w * MW + m;
-      if (j < S) {
-#pragma unroll
-        for (int lb = 0; lb < 2; ++lb) state[(((size_t)b * 2 + (lb ^ sp)) * S + j) * d + c] = h[lb][m];
-      }
+      if (j < S) state[(((size_t)b * 2 + bank) * S + j) * d + c] = h[m];
     }
   }
 }
@@ -730,7 +731,7 @@ extern "C" int fstu_stu_scan_lds(const void* xp, int64_t x_bstride, int64_t x_ts
                "fstu_stu_scan_lds: input rows must be 16-byte aligned (d and strides multiples of %d elements)", epp);
   FSTU_REQUIRE(x_tstride >= d && y_tstride >= d, FSTU_EARG, "fstu_stu_scan_lds: token stride below d");
   if (len == 0 && carry) return FSTU_OK;
-  dim3 grid((d + 63) / 64, B);
+  dim3 grid((d + SCAN_CH - 1) / SCAN_CH, B);
   hipStream_t s = (hipStream_t)stream;
   if (S <= 64) {
     FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_scan_lds",
