@@ -1038,6 +1038,10 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
     G = (a.I + a.fpw - 1) / a.fpw;
   } else {
     if (G > (a.I + 7) / 8) G = (a.I + 7) / 8;
+    // a plain projection narrower than 16 features per CU (QKV at d = 768: 2304 features) gets one whole tile per
+    // workgroup rather than half tiles on every CU: every workgroup repeats the norm prologue, and its operands come
+    // out of one L2 per XCD (0.3113 -> 0.3105 ms per decode step)
+    if (epi != 0 && G > (a.I + 15) / 16) G = (a.I + 15) / 16;
     a.fpw = 0;
   }
   const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
