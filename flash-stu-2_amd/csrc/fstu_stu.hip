@@ -119,8 +119,8 @@ extern "C" int fstu_stu_step_hist(const void* hist, const void* filt, float* eo,
 template <typename T>
 __global__ void __launch_bounds__(256)
 stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
-                    const float* __restrict__ ce, T* __restrict__ y, int ldy, int S, int d, int parity,
-                    const int* __restrict__ dyn) {
+                    const float* __restrict__ ce, const float* __restrict__ co /*optional: weights of the other bank*/,
+                    float scale, T* __restrict__ y, int ldy, int S, int d, int parity, const int* __restrict__ dyn) {
   __shared__ float sh[LDS_JG][32][4];
   if (dyn) parity = dyn[0] & 1;
   const int b = blockIdx.y;
@@ -148,6 +148,19 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
       acc[2] = fmaf(cj.z, h.z, acc[2]);
       acc[3] = fmaf(cj.w, h.w, acc[3]);
     }
+    if (co) {
+      // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (not advanced here)
+      const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
+#pragma unroll 4
+      for (int j = jg; j < S; j += LDS_JG) {
+        const float4 h = *(const float4*)(so + (size_t)j * d);
+        const float4 oj = *(const float4*)(co + (size_t)j * d + c);
+        acc[0] = fmaf(oj.x, h.x, acc[0]);
+        acc[1] = fmaf(oj.y, h.y, acc[1]);
+        acc[2] = fmaf(oj.z, h.z, acc[2]);
+        acc[3] = fmaf(oj.w, h.w, acc[3]);
+      }
+    }
   }
 #pragma unroll
   for (int v = 0; v < 4; ++v) sh[jg][q][v] = acc[v];
@@ -158,7 +171,7 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < LDS_JG; ++g) s += sh[g][q][v];
-      DT<T>::st(y + (size_t)b * ldy + c + v, 2.0f * s);
+      DT<T>::st(y + (size_t)b * ldy + c + v, scale * s);
     }
   }
 }
@@ -168,8 +181,26 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
   return fstu_stu_step_lds_dyn(state, xp, ldxp, a, ce, y, ldy, B, S, d, t, nullptr, dtype, stream);
 }
 
+static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                               float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
+                               void* stream);
+
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
+  return stu_step_lds_launch(state, xp, ldxp, a, ce, nullptr, 2.0f, y, ldy, B, S, d, t, dyn, dtype, stream);
+}
+
+extern "C" int fstu_stu_step_lds_single(float* state, const void* xp, int ldxp, const float* a, const float* ce,
+                                        const float* co, void* y, int ldy, int B, int S, int d, int t, int dtype,
+                                        void* stream) {
+  FSTU_REQUIRE(co, FSTU_ENULL, "fstu_stu_step_lds_single: null pointer");
+  FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_single: co must be 16-byte aligned");
+  return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, nullptr, dtype, stream);
+}
+
+static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                               float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
+                               void* stream) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
   FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
@@ -178,7 +209,7 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
   dim3 grid((d / 4 + 31) / 32, B);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
                       hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
-                                         (const T*)xp, ldxp, a, ce, (T*)y, ldy, S, d, t & 1, dyn));
+                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn));
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }

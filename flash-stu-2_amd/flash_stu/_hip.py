@@ -34,6 +34,7 @@ SIGNATURES = {
     "fstu_bias_act": [_vp, _vp, _i64, _i, _i, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_single": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -282,9 +283,10 @@ def stu_step_hist(hist: torch.Tensor, filt: torch.Tensor, t: int, nsplit: int, e
 
 
 def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d)."""
-    _dev(state, a, ce)
+                 out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d).  With co (S,d), the single-branch form:
+    y = ce . bank(t) + co . other bank (use_hankel_L), without the factor 2 of the two sign branches."""
+    _dev(state, a, ce, co)
     B, two, S, d = state.shape
     assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
     assert a.numel() == S and ce.shape == (S, d)
@@ -294,6 +296,11 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
         out = torch.empty(B, d, dtype=xp.dtype, device=xp.device)
     orow, ldy = _rows_view(out)
     assert orow == B and out.dtype == xp.dtype
+    if co is not None:
+        assert co.dtype == torch.float32 and co.shape == (S, d)
+        _check(load().fstu_stu_step_lds_single(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), _p(out), ldy, B, S, d, t,
+                                               _dt(xp), _stream()), "fstu_stu_step_lds_single")
+        return out
     _check(load().fstu_stu_step_lds(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
            "fstu_stu_step_lds")
     return out

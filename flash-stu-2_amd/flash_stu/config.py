@@ -111,7 +111,8 @@ class FlashSTUConfig:
             # even / odd lag halves and fit the bank kernel; otherwise it re-evaluates the bank over the history
             return "lds" if (bf16 and self.seq_len % 2 == 0 and self.num_eigh <= 32) else "history"
         if self.use_hankel_L:
-            return "history"
+            # one branch over all lags: even lags from the bank of the token's parity, odd lags from the other bank
+            return "lds" if (bf16 and self.seq_len % 2 == 0) else "history"
         return "lds" if bf16 else "history"
 
     # -- serialisation (config.json, HF style)

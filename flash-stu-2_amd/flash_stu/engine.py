@@ -82,6 +82,8 @@ class DecodeEngine:
     def supports(cfg) -> bool:
         """The one-call decode step covers approx-mode STU layers without the sandwich and bias-free linears;
         other variants decode through the layers' own state (FlashSTU.generate picks the loop)."""
+        if cfg.use_hankel_L and cfg.resolved_stu_decode_mode() == "lds":
+            return False     # single-branch filters on the recurrence state: the odd lags read the other bank
         return bool(cfg.use_approx) and not cfg.stu_enable_mlp_sandwich and not cfg.bias
 
     def __init__(self, model):

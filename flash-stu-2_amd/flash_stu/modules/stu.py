@@ -63,7 +63,10 @@ class STU(nn.Module):
         return hit[1]
 
     def decode_mode(self) -> str:
-        return self.config.resolved_stu_decode_mode()
+        mode = self.config.resolved_stu_decode_mode()
+        if mode == "lds" and self.use_approx and self.use_hankel_L and self.phi.shape[0] % 2 != 0:
+            return "history"     # the single-branch recurrence needs equally long even- and odd-lag halves
+        return mode
 
     def _exact_lds_ok(self) -> bool:
         """Exact mode can decode on the recurrence state when asked for explicitly (stu_decode_mode='lds'), the
@@ -105,6 +108,24 @@ class STU(nn.Module):
             dev = self.M_filters.device
             return a.to(dev), ce.to(dev).contiguous()
         return self._cached("lds", (self.phi, self.M_filters), build)
+
+    def lds_single_params(self):
+        """use_hankel_L (one branch over all lags): poles a (S) and per-channel weights ce, co (S,d) fitted to the
+        even / odd lags of the effective filter; the odd lags read the other parity bank."""
+        def build():
+            S = self.config.stu_lds_state_dim
+            f = self.effective_filter()
+            a, ce, e1 = fit_even_lag_lds(f[0::2], S)
+            a2, co, e2 = fit_even_lag_lds(f[1::2], S)
+            if not torch.equal(a, a2):
+                raise RuntimeError("pole grids of the even and odd lags differ")
+            self.lds_fit_error = max(e1, e2)
+            dev = self.M_filters.device
+            return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
+        return self._cached("ldssingle", (self.phi, self.M_filters), build)
+
+    def _single_lds_ok(self) -> bool:
+        return self.use_approx and self.use_hankel_L and self.phi.shape[0] % 2 == 0
 
     def bank_lds_params(self):
         """Exact mode: poles a (S) and output weights ce, co (S,K) fitted to the even / odd lags of the filters."""
@@ -228,7 +249,8 @@ class STU(nn.Module):
         B, T, d = src.shape
         pos = torch.full((B,), T, dtype=torch.int64)
         if self.decode_mode() == "lds" and (self.use_approx or self._exact_lds_ok()):
-            a = self.lds_params()[0] if self.use_approx else self.bank_lds_params()[0]
+            a = (self.lds_single_params()[0] if self._single_lds_ok() else
+                 self.lds_params()[0] if self.use_approx else self.bank_lds_params()[0])
             state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1)
             return (src.new_empty(B, 0, d), state, pos)
         cap = max(self.config.seq_len, T)
@@ -241,9 +263,13 @@ class STU(nn.Module):
         pos = int(pos_t[0])
         B, d = x.shape
         if self.use_approx and state.numel() > 0:
-            a, ce = self.lds_params()
             xp = _hip.linear_decode(x, self.m_inputs_t())
-            y = _hip.stu_step_lds(state, xp, a, ce, pos)
+            if self.use_hankel_L:
+                a, ce, co = self.lds_single_params()
+                y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co)
+            else:
+                a, ce = self.lds_params()
+                y = _hip.stu_step_lds(state, xp, a, ce, pos)
             return y, (hist, state, pos_t + 1)
         if not self.use_approx and state.numel() > 0:
             # exact mode on the recurrence state: U+- for all K filters, then the two contractions as skinny GEMVs

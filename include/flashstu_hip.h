@@ -127,6 +127,13 @@ int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int
 int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                       int B, int S, int d, int t, int dtype, void* stream);
 
+/* The same step for the single-branch filters of use_hankel_L=True (flash_stu/utils/stu_utils.py:22-25,229-246:
+ * one convolution over ALL lags, no sign branch): ce (S,d) is fitted to the even lags and weighs the bank of parity
+ * t&1 after its advance, co (S,d) is fitted to the odd lags and weighs the other bank (lag 2m+1 reaches position
+ * t-1-2m):  y[b,c] = T( sum_j ce[j,c]*h_j[bank t&1] + sum_j co[j,c]*h_j[other bank] ). */
+int fstu_stu_step_lds_single(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                             void* y, int ldy, int B, int S, int d, int t, int dtype, void* stream);
+
 /* Exact mode (use_approx=False) on the same two-bank state, fed with the raw inputs x (B,d): after advancing the bank
  * of parity t&1,  E_k = sum_j ce[j,k] h_j[that bank],  O_k = sum_j co[j,k] h_j[other bank]  and
  *   u_plus[b,k,c] = T(E_k + O_k),  u_minus[b,k,c] = T(E_k - O_k)   (u_minus / co may be NULL: single branch)

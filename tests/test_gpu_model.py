@@ -117,6 +117,23 @@ def test_scan_prefill_against_oracle_and_fft_prefill(dtype, mode):
     assert out.shape == (2, 170) and torch.equal(out[:, :150].cpu(), ids)
 
 
+def test_hankel_L_decodes_on_the_recurrence_state():
+    """use_hankel_L=True in bf16 decodes on the two-bank recurrence state (even lags from the token's bank, odd lags
+    from the other one): logits of the stateful loop within the bf16 tolerance of the oracle teacher-forced on the
+    same tokens, and of the cache-free loop."""
+    ocfg, w, model = make_pair(seed=6, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=128, n_layers=4,
+                               n_heads=2, window_size=16, num_eigh=8, seq_len=128, vocab_size=503, use_hankel_L=True)
+    assert model.config.resolved_stu_decode_mode() == "lds"
+    P, N = 20, 40
+    ids = prompt(2, P, ocfg.vocab_size, 3)
+    got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
+    ref = _teacher_forced(w, ocfg, got.cpu(), P)
+    scale = float(ref.float().abs().max())
+    assert float((gl.float().cpu() - ref.float()).abs().max()) <= 2e-2 * scale
+    _, gl2 = model.generate(ids.cuda(), max_length=P + 8, do_sample=False, use_cache=False, return_logits=True)
+    assert float((gl2.float() - gl[:, :8].float()).abs().max()) <= 2e-2 * scale
+
+
 def _teacher_forced(w, ocfg, tokens, P):
     logits, _ = O.model_forward(w, ocfg, tokens[:, :-1])
     return logits[:, P - 1:, :]          # predictions for positions P..end

@@ -425,6 +425,33 @@ def test_stu_step_lds_tracks_the_convolution(hip, L):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_stu_step_lds_single_branch(hip, dtype):
+    """use_hankel_L on the recurrence state: even lags from the bank of the token's parity, odd lags from the other
+    bank.  The kernel equals a float64 evaluation of that recurrence, and with weights fitted to the even / odd
+    halves of a filter it tracks the oracle's single-branch convolution."""
+    B, d, L, K, S = 2, 128, 128, 8, 64
+    xp, filt, _, plus = _stu_setup(dtype, B, L, d, L, K, 9)
+    a, ce, _ = _fit_lds(filt.double()[0::2], S)
+    a2, co, _ = _fit_lds(filt.double()[1::2], S)
+    assert torch.equal(a, a2)
+    state = torch.zeros(B, 2, S, d, device="cuda")
+    h64 = torch.zeros(B, 2, S, d, dtype=torch.float64)
+    ad, ced, cod = dev(a), dev(ce), dev(co)
+    worst = 0.0
+    for t in range(L):
+        y = hip.stu_step_lds(state, dev(xp[:, t].contiguous()), ad, ced, t, co=cod)
+        p = t & 1
+        h64[:, p] = a.double()[None, :, None] * h64[:, p] + xp[:, t].double()[:, None, :]
+        ref = (ce.double()[None] * h64[:, p]).sum(1) + (co.double()[None] * h64[:, p ^ 1]).sum(1)
+        # the two bank sums cancel in part: fp32 error relative to the larger of them, not to their sum
+        check(y, ref.to(dtype), dtype, frac=0.12, scale=float(ref.abs().max()), atol=2.0 ** -10 * float(ref.abs().max()))
+        worst = max(worst, float((y.float().cpu() - plus[:, t].float()).abs().max()))
+    assert float((state.cpu().double() - h64).abs().max()) < 1e-4 * float(h64.abs().max())
+    tol = 1e-3 if dtype == torch.float32 else 2.0 ** -6
+    assert worst < tol * float(plus.float().abs().max()), worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("B,H,hd,W,T", [(2, 4, 64, 16, 50), (8, 12, 64, 512, 600), (1, 16, 128, 32, 40),
                                          (2, 2, 32, 7, 20)])
 def test_swa_ring_decode_and_prefill(hip, dtype, B, H, hd, W, T):
