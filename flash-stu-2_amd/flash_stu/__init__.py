@@ -5,6 +5,6 @@ from .config import FlashSTUConfig
 from .model import FlashSTU
 from .modules.attention import Attention
 from .modules.stu import STU
-from .utils.stu_utils import get_spectral_filters
+from .utils.stu_utils import convolve, get_spectral_filters
 
-__all__ = ["FlashSTU", "FlashSTUConfig", "FlashSTUBlock", "STU", "Attention", "get_spectral_filters"]
+__all__ = ["FlashSTU", "FlashSTUConfig", "FlashSTUBlock", "STU", "Attention", "get_spectral_filters", "convolve"]

@@ -208,6 +208,21 @@ class STU(nn.Module):
             y = y + torch.matmul(Um.reshape(B, self.K * d, T).transpose(1, 2), wm)
         return y
 
+    def forward_differentiable(self, x: torch.Tensor) -> torch.Tensor:
+        """Training-side forward of the approx-mode STU (stu.py:81-98,120) under autograd: the two projections are
+        library GEMMs, the convolution between them is the HIP kernel with its own backward
+        (flash_stu.utils.stu_utils.convolve), so gradients reach x, M_inputs and M_filters.  No decode state."""
+        from ..utils.stu_utils import convolve, nearest_power_of_two
+        if not self.use_approx:
+            raise NotImplementedError("forward_differentiable covers use_approx=True")
+        if self.tile_size < self.d_in:
+            raise NotImplementedError("forward_differentiable does not cover d_in_tile / d_out_tile")
+        x_proj = x @ self.M_inputs
+        phi_proj = self.phi @ self.M_filters
+        n = nearest_power_of_two(2 * self.phi.shape[0] - 1, round_up=True)
+        plus, minus = convolve(x_proj, phi_proj, n, use_approx=True, return_both=not self.use_hankel_L)
+        return plus if self.use_hankel_L else plus + minus
+
     @torch.no_grad()
     def forward(self, x: torch.Tensor, past_state=None, use_cache: bool = False):
         """x (B,T,d).  Without past_state the whole sequence is convolved from

@@ -134,6 +134,35 @@ def test_hankel_L_decodes_on_the_recurrence_state():
     assert float((gl2.float() - gl[:, :8].float()).abs().max()) <= 2e-2 * scale
 
 
+@pytest.mark.parametrize("hankel", [False, True])
+def test_stu_forward_differentiable_gradients(hankel):
+    """Training-side forward of the approx-mode STU under autograd: output equal to the inference forward, gradients
+    of x, M_inputs and M_filters equal to autograd through the oracle's stu_forward (fp32)."""
+    from flash_stu import STU, FlashSTUConfig
+    L, K, d, B, T = 64, 8, 32, 2, 50
+    cfg = FlashSTUConfig(n_embd=d, n_heads=2, n_layers=2, seq_len=L, num_eigh=K, vocab_size=11, torch_dtype=torch.float32,
+                         use_hankel_L=hankel)
+    phi = torch.tensor(O.get_spectral_filters_f64(L, K, hankel)).float()
+    n = O.nearest_power_of_two(2 * L - 1, True)
+    g = torch.Generator().manual_seed(17)
+    Mi, Mf = torch.randn(d, d, generator=g) / d ** 0.5, torch.randn(K, d, generator=g) / K ** 0.5
+    x, wgt = torch.randn(B, T, d, generator=g), torch.randn(B, T, d, generator=g)
+    stu = STU(cfg, phi.cuda(), n).cuda()
+    with torch.no_grad():
+        stu.M_inputs.copy_(Mi)
+        stu.M_filters.copy_(Mf)
+    xd = x.cuda().requires_grad_(True)
+    y = stu.forward_differentiable(xd)
+    assert float((y.detach() - stu(x.cuda())).abs().max()) <= 2e-5 * float(y.detach().abs().max())
+    (y * wgt.cuda()).sum().backward()
+    xo = x.clone().requires_grad_(True)
+    p = {"M_inputs": Mi.clone().requires_grad_(True), "M_filters": Mf.clone().requires_grad_(True)}
+    ref = O.stu_forward(xo, phi, p, n, use_approx=True, use_hankel_L=hankel)
+    (ref * wgt).sum().backward()
+    for got, want in ((xd.grad, xo.grad), (stu.M_inputs.grad, p["M_inputs"].grad), (stu.M_filters.grad, p["M_filters"].grad)):
+        assert float((got.cpu() - want).abs().max()) <= 2e-4 * float(want.abs().max())
+
+
 def _teacher_forced(w, ocfg, tokens, P):
     logits, _ = O.model_forward(w, ocfg, tokens[:, :-1])
     return logits[:, P - 1:, :]          # predictions for positions P..end

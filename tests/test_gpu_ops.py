@@ -289,6 +289,54 @@ def test_stu_step_hist(hip, dtype, B, T, d, L, nsplit):
         check(x, ref[:, t], dtype, frac=0.05, scale=float(ref.abs().max()), atol=atol)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d,L", [(2, 100, 96, 128), (1, 20, 8, 64), (2, 64, 40, 64)])
+def test_convolve_operator_matches_oracle(hip, dtype, B, T, d, L):
+    """flash_stu.utils.stu_utils.convolve with the reference's signature: both branches, one branch, exact mode."""
+    from flash_stu.utils.stu_utils import convolve, nearest_power_of_two
+    xp, filt, _, _ = _stu_setup(dtype, B, T, d, L, 8, 6)
+    n = nearest_power_of_two(2 * L - 1, round_up=True)
+    assert n == O.nearest_power_of_two(2 * L - 1, True)
+    rp, rm = O.convolve(xp, filt, n, use_approx=True)
+    gp, gm = convolve(dev(xp), dev(filt), n, use_approx=True)
+    check(gp, rp, dtype, frac=0.05)
+    check(gm, rm, dtype, frac=0.05)
+    only, none = convolve(dev(xp), dev(filt), n, use_approx=True, return_both=False)
+    assert none is None and torch.equal(only, gp)
+    phi = torch.tensor(O.get_spectral_filters_f64(L, 6)).to(dtype)
+    ep, em = O.convolve(xp, phi, n, use_approx=False)
+    bp, bm = convolve(dev(xp), dev(phi), n, use_approx=False)
+    check(bp, ep, dtype, frac=0.05)
+    check(bm, em, dtype, frac=0.05)
+    with pytest.raises(ValueError):
+        convolve(dev(xp), dev(filt), T, use_approx=True)          # n shorter than the linear convolution
+
+
+@pytest.mark.parametrize("B,T,d,L,both", [(2, 70, 24, 70, True), (3, 40, 16, 64, True), (2, 20, 8, 32, False), (2, 50, 12, 30, True)])
+def test_convolve_operator_gradients(hip, B, T, d, L, both):
+    """Backward of the approx-mode convolution (every piece is the forward kernel on time-reversed operands) against
+    autograd through the oracle's FFT convolution, fp32; filters longer and shorter than the input."""
+    from flash_stu.utils.stu_utils import convolve
+    g = gen(31)
+    u = torch.randn(B, T, d, generator=g)
+    v = torch.randn(L, d, generator=g) / math.sqrt(L)
+    wp, wm = torch.randn(B, T, d, generator=g), torch.randn(B, T, d, generator=g)
+    n = O.nearest_power_of_two(2 * max(L, T) - 1, True)
+    uo, vo = u.clone().requires_grad_(True), v.clone().requires_grad_(True)
+    rp, rm = O.convolve(uo, vo, n, use_approx=True)
+    loss = (rp * wp).sum() + ((rm * wm).sum() if both else 0.0)
+    loss.backward()
+    ud, vd = dev(u).requires_grad_(True), dev(v).requires_grad_(True)
+    gp, gm = convolve(ud, vd, n, use_approx=True, return_both=both)
+    lossd = (gp * dev(wp)).sum() + ((gm * dev(wm)).sum() if both else 0.0)
+    lossd.backward()
+    su, sv = float(uo.grad.abs().max()), float(vo.grad.abs().max())
+    assert float((ud.grad.cpu() - uo.grad).abs().max()) <= 1e-4 * su
+    assert float((vd.grad.cpu() - vo.grad).abs().max()) <= 1e-4 * sv
+    with pytest.raises(NotImplementedError):
+        convolve(ud, dev(torch.randn(L, 4)), n, use_approx=False)
+
+
 def _fit_lds(filt_even, S):
     """ridge fit of the even-lag filter by S real poles (host-side helper of the product)."""
     from flash_stu.utils.lds_fit import fit_even_lag_lds
