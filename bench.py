@@ -217,7 +217,7 @@ def main():
     # HBM bytes per GLU launch from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; each scaled by what the same
     # counter reads for the library's plain 256 MiB copy kernel: x2.000 and x1.000).  Measured offline for the default
     # workload only; summary and commands in profiles/glu_c2_hbm_traffic_pmc.txt.
-    traffic = 28879872 if (cfg.n_embd, cfg.mlp_scale, B) == (768, 12, 8) else None
+    traffic = 28876800 if (cfg.n_embd, cfg.mlp_scale, B) == (768, 12, 8) else None
     out = {
         "metric": "decode tokens/sec at 1 GPU (768-d FlashSTU, bs=8) + achieved HBM GB/s",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
