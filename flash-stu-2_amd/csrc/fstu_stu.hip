@@ -319,7 +319,12 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   if (dyn) parity = dyn[0] & 1;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int tile = blockIdx.x, c0 = tile * 16;
+  // A tile's 16 channels are half a 128-byte line of every state and output-weight row.  Workgroups go round the 8
+  // XCDs, so consecutive tiles are dealt to one XCD (workgroups i, i+8, ...): both halves of a line then meet in the
+  // same L2 and the line comes from HBM once instead of twice.
+  int tile = blockIdx.x;
+  if ((gridDim.x & 15) == 0) tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const int c0 = tile * 16;
   // residual update + norm in the prologue
   typedef NormPrologue<256, 4, 4> Pro;
   typedef NormPrologue<256, 3, 4> Pro3;   // exact for rows * K / 8 <= 768: one straight line without idle chunks
