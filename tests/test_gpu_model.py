@@ -222,6 +222,31 @@ def test_c2_dims_bf16_teacher_forced(mode, init):
         assert float(agree) >= float(self_agree) - 0.03
 
 
+def test_c2_full_size_decode_against_full_sequence_recompute():
+    """BASELINE config 2 at its full size (batch 8, 512-token prompt, window 512, mlp_scale 12), where the CPU oracle is
+    out of reach: the stateful decode (ring past its wrap, recurrence state past the window) must give the logits of
+    a full-sequence forward over the same tokens (the prefill kernels, tied to the oracle at small sizes), and the
+    8-step graphs with the chained pick must reproduce the kernel-by-kernel loop token for token."""
+    from flash_stu import FlashSTU, FlashSTUConfig
+    torch.manual_seed(1)
+    cfg = FlashSTUConfig(n_embd=768, n_layers=12, n_heads=12, window_size=512, seq_len=2048, vocab_size=50257,
+                         num_eigh=24, mlp_scale=12, torch_dtype=torch.bfloat16)
+    with torch.device("cuda"):
+        model = FlashSTU(cfg)
+    model = model.cuda().eval()
+    B, P, N = 8, 512, 40
+    ids = prompt(B, P, cfg.vocab_size, 1).cuda()
+    eager, logits = model.generate(ids, max_length=P + N, do_sample=False, return_logits=True)      # step by step
+    graph = model.generate(ids, max_length=P + N, do_sample=False)                                  # 8-step graphs
+    assert torch.equal(graph, eager)
+    worst = 0.0
+    for s in (0, 1, 7, 20, N - 1):          # logits that picked token P+s come from positions < P+s
+        full = model(eager[:, :P + s].contiguous()).logits[:, -1, :].float()
+        got = logits[:, s, :].float()
+        worst = max(worst, float(((got - full).abs().amax(-1) / full.abs().amax(-1)).max()))
+    assert worst <= 2e-2, worst
+
+
 def test_window_wraps_the_ring_bf16():
     """Decode far past window+1 so every ring slot is overwritten several times."""
     ocfg, w, model = make_pair(seed=4, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=128, n_layers=4,
