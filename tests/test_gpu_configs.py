@@ -222,3 +222,37 @@ def test_c5_width_bf16_step_kernels(d, heads):
     ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
     err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
     assert float(err.max()) <= 2e-2
+
+
+def test_c5_full_architecture_decode_against_full_sequence_recompute():
+    """BASELINE config 5's full architecture (d=2048, 24 layers, 16 heads of 128, window 1024, L=8192, mlp_scale 12:
+    3.98 B parameters) at batch 32 (two row chunks of 16 on concurrent streams) with its sampler (top-k 40,
+    temperature 0.8, seeded stream); the CPU oracle is out of reach at this size, so the checks are size-independent:
+    graph replay equals the kernel-by-kernel loop token for token, a second run reproduces the ids, and the stateful
+    logits equal those of a full-sequence forward over the same tokens within the bf16 tolerance.  The prompt is
+    cut to 192 tokens to keep the test short (the window of 1024 is not reached; the ring wrap is covered at
+    config 2's full size and in test_window_wraps_the_ring_bf16)."""
+    from flash_stu import FlashSTU, FlashSTUConfig
+    from test_gpu_model import prompt
+    torch.manual_seed(2)
+    cfg = FlashSTUConfig(n_embd=2048, n_layers=24, n_heads=16, window_size=1024, seq_len=8192, vocab_size=50257,
+                         num_eigh=24, mlp_scale=12, torch_dtype=torch.bfloat16)
+    with torch.device("cuda"):
+        model = FlashSTU(cfg)
+    model = model.cuda().eval()
+    assert abs(model.get_num_params() - 3.98e9) < 0.05e9
+    B, P, N = 32, 192, 24
+    ids = prompt(B, P, cfg.vocab_size, 2).cuda()
+    kw = dict(max_length=P + N, do_sample=True, top_k=40, temperature=0.8, seed=2)
+    eager, logits = model.generate(ids, return_logits=True, **kw)
+    graph = model.generate(ids, **kw)
+    assert torch.equal(graph, eager)
+    assert torch.equal(model.generate(ids, **kw), graph)
+    worst = 0.0
+    for s in (0, 5, N - 1):
+        full = model(eager[:, :P + s].contiguous()).logits[:, -1, :].float()
+        got = logits[:, s, :].float()
+        worst = max(worst, float(((got - full).abs().amax(-1) / full.abs().amax(-1)).max()))
+    assert worst <= 2e-2, worst
+    del model
+    torch.cuda.empty_cache()
