@@ -247,6 +247,28 @@ def test_c2_full_size_decode_against_full_sequence_recompute():
     assert worst <= 2e-2, worst
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_single_token_prompt_and_ragged_batches(dtype):
+    """Edge cases of the token loop: a one-token prompt (the prefill is a single position), batches of 1 and of 17
+    rows (one full row chunk of 16 plus a chunk of one), a single new token, and max_length equal to the prompt."""
+    ocfg, w, model = make_pair(seed=9, init="healthy", dtype=dtype, mlp_scale=2, n_embd=128, n_layers=4, n_heads=2,
+                               window_size=8, num_eigh=8, seq_len=64, vocab_size=307)
+    for B in (1, 17):
+        ids = prompt(B, 1, ocfg.vocab_size, B)
+        if dtype == torch.float32:
+            ref = O.generate(w, ocfg, ids, max_length=20, do_sample=False, mode="recompute")
+            got = model.generate(ids.cuda(), max_length=20, do_sample=False)
+            assert torch.equal(got.cpu(), ref)
+        else:
+            got, gl = model.generate(ids.cuda(), max_length=20, do_sample=False, return_logits=True)
+            ref = _teacher_forced(w, ocfg, got.cpu(), 1).float()
+            assert float(((gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)).max()) <= 2e-2
+            assert torch.equal(model.generate(ids.cuda(), max_length=20, do_sample=False), got)      # graph path
+        one = model.generate(ids.cuda(), max_length=2, do_sample=False)
+        assert one.shape == (B, 2) and torch.equal(one[:, :2], got[:, :2])
+        assert torch.equal(model.generate(ids.cuda(), max_length=1), ids.cuda())
+
+
 def test_window_wraps_the_ring_bf16():
     """Decode far past window+1 so every ring slot is overwritten several times."""
     ocfg, w, model = make_pair(seed=4, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=128, n_layers=4,
