@@ -52,12 +52,13 @@ swa_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int qs = (blockIdx.x * 4 + w) * 16;          // first query of this wave
-  if (qs >= Tn) return;
+  const bool wave_on = qs < Tn;                      // an idle wave still loads tiles and meets the barriers
   const int d = H * HD;
   const size_t rs = (size_t)3 * d;                   // row stride of qkv
   const bf16_t* base = qkv + (size_t)b * Tn * rs + h * HD;
   const int myq = qs + c;                            // the query whose statistics this lane keeps
   const float scale = rsqrtf((float)HD), slope = slopes[h];
+  const float inv_cap2l = softcap > 0.f ? 2.8853900817779268f / softcap : 0.f;   // 2 log2(e) / softcap
 
   // Q^T fragments (B operand): lane holds Q[query c][dims ks*32 + 8g ..]
   uint4 qf[KS];
@@ -74,32 +75,59 @@ swa_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict
   const int klo = max(0, qs - window);
   const int khi = min(Tn - 1, qs + 15);              // last key any query of the tile may see
   // row i = c of key tile t is key kb + 8*(c>>2) + 4*t + (c&3)
-  const int koff = 8 * (c >> 2) + (c & 3);
-  const bf16_t* vtb = vt + ((size_t)b * d + h * HD + c) * Tp + g * 8;   // + nt*16*Tp + kb
-
-  for (int kb = (klo >> 5) << 5; kb <= khi; kb += 32) {
+  // The four waves of a workgroup (64 consecutive queries) see nearly the same keys: a block of 32 keys is brought
+  // into LDS once for all of them (K rows in the order the MFMA fragments read them, V^T rows; both padded by one
+  // 16-byte slot per row so that the 16 rows a quarter wave reads fall on distinct banks), the next block's
+  // pieces travel in registers meanwhile.
+  constexpr int KCH = HD / 8;                        // 16-byte pieces per key row
+  constexpr int KPT = 32 * KCH / 256;                // pieces of the K tile per thread
+  constexpr int VPT = HD * 4 / 256;                  // pieces of the V^T tile per thread
+  __shared__ uint4 k_lds[32 * (KCH + 1)];
+  __shared__ uint4 v_lds[HD * 5];
+  const int qs_wg = blockIdx.x * 64;
+  const int kb_first = (max(0, qs_wg - window) >> 5) << 5;
+  const int kb_last = min(Tn - 1, qs_wg + 63);
+  uint4 kreg[KPT], vreg[VPT];
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int e = threadIdx.x + i * 256, kk = e / KCH, ch = e % KCH;
+      kreg[i] = *(const uint4*)(base + (size_t)min(kb + kk, Tn - 1) * rs + d + ch * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = threadIdx.x + i * 256, dim = e >> 2, ch = e & 3;
+      vreg[i] = *(const uint4*)(vt + ((size_t)b * d + h * HD + dim) * Tp + kb + ch * 8);
+    }
+  };
+  fetch(kb_first);
+  for (int kb = kb_first; kb <= kb_last; kb += 32) {
+    __syncthreads();                                 // the previous block's fragments have been read
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int e = threadIdx.x + i * 256, kk = e / KCH, ch = e % KCH;
+      // key kk of the block is row c = 4*(kk>>3) + (kk&3) of key tile t = (kk>>2)&1
+      k_lds[(((kk >> 2) & 1) * 16 + 4 * (kk >> 3) + (kk & 3)) * (KCH + 1) + ch] = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = threadIdx.x + i * 256;
+      v_lds[(e >> 2) * 5 + (e & 3)] = vreg[i];
+    }
+    __syncthreads();
+    if (kb + 32 <= kb_last) fetch(kb + 32);
+    if (!wave_on || kb > khi || kb + 31 < klo) continue;   // wave-uniform: no key of this block is visible to the wave
     // ---- scores of the block: two key tiles
     floatx4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    {
-      const int k0 = min(kb + koff, Tn - 1), k1 = min(kb + koff + 4, Tn - 1);
-      const bf16_t* kr0 = base + (size_t)k0 * rs + d + g * 8;
-      const bf16_t* kr1 = base + (size_t)k1 * rs + d + g * 8;
-      uint4 ka[KS], kc[KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        ka[ks] = *(const uint4*)(kr0 + ks * 32);
-        kc[ks] = *(const uint4*)(kr1 + ks * 32);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ka[ks]), as_bf16x8(qf[ks]), s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kc[ks]), as_bf16x8(qf[ks]), s1, 0, 0, 0);
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint4 ka = k_lds[c * (KCH + 1) + ks * 4 + g], kc = k_lds[(16 + c) * (KCH + 1) + ks * 4 + g];
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ka), as_bf16x8(qf[ks]), s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kc), as_bf16x8(qf[ks]), s1, 0, 0, 0);
     }
-    // V^T fragments of the block go in flight while the softmax runs
     uint4 vf[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) vf[nt] = *(const uint4*)(vtb + (size_t)nt * 16 * Tp + kb);
+    for (int nt = 0; nt < NT; ++nt) vf[nt] = v_lds[(nt * 16 + c) * 5 + g];
 
     // lane (g, c): D rows 4g+r of tile t are keys kb + 8g + 4t + r, column c is query myq
     float sc[8];
@@ -108,13 +136,16 @@ swa_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict
     for (int e = 0; e < 8; ++e) {
       const int j = kb + 8 * g + e;
       float s = (e < 4 ? s0[e] : s1[e - 4]) * scale;
-      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      // soft-cap on the hardware exp2 / reciprocal: tanh(x) = 1 - 2 / (exp(2x) + 1), absolute error about 1e-7 in
+      // front of a probability that is rounded to bf16 (the library tanhf costs about 60 instructions per score
+      // and was most of this kernel's time)
+      if (softcap > 0.f) s = softcap - (2.0f * softcap) * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * inv_cap2l) + 1.0f);
       s -= slope * (float)(myq - j);
       const bool valid = j <= myq && j >= myq - window && j < Tn;
       sc[e] = valid ? s : -INFINITY;
       bm = fmaxf(bm, sc[e]);
     }
-    bm = fmaxf(bm, __shfl_xor(bm, 16, FSTU_WAVE));
+    bm = fmaxf(bm, fstu_swz16(bm));                       // lane ^ 16
     bm = fmaxf(bm, __shfl_xor(bm, 32, FSTU_WAVE));
     const float mn = fmaxf(m, bm);
     float corr = 1.f;
@@ -134,10 +165,8 @@ swa_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict
       l = l * corr + ps;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bf16_t h0 = f32_to_bf16(p[2 * e]), h1 = f32_to_bf16(p[2 * e + 1]);
-        const bf16_t l0 = f32_to_bf16(p[2 * e] - bf16_to_f32(h0)), l1 = f32_to_bf16(p[2 * e + 1] - bf16_to_f32(h1));
-        ph[e] = (unsigned)h0 | ((unsigned)h1 << 16);
-        pl[e] = (unsigned)l0 | ((unsigned)l1 << 16);
+        ph[e] = pack2_bf16(p[2 * e], p[2 * e + 1]);
+        pl[e] = pack2_bf16(p[2 * e] - __uint_as_float(ph[e] << 16), p[2 * e + 1] - __uint_as_float(ph[e] & 0xffff0000u));
       }
       m = mn;
     }
@@ -153,14 +182,14 @@ swa_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict
   // the four lane groups hold disjoint keys: total sum over g
   l += __shfl_xor(l, 16, FSTU_WAVE);
   l += __shfl_xor(l, 32, FSTU_WAVE);
-  if (myq < Tn) {
+  if (wave_on && myq < Tn) {
     const float inv = 1.0f / l;
     bf16_t* orow = out + ((size_t)b * Tn + myq) * d + h * HD + 4 * g;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       uint2 pk;
-      pk.x = (unsigned)f32_to_bf16(o[nt][0] * inv) | ((unsigned)f32_to_bf16(o[nt][1] * inv) << 16);
-      pk.y = (unsigned)f32_to_bf16(o[nt][2] * inv) | ((unsigned)f32_to_bf16(o[nt][3] * inv) << 16);
+      pk.x = pack2_bf16(o[nt][0] * inv, o[nt][1] * inv);
+      pk.y = pack2_bf16(o[nt][2] * inv, o[nt][3] * inv);
       *(uint2*)(orow + nt * 16) = pk;
     }
   }
