@@ -211,9 +211,69 @@ add_rmsnorm_kernel(T* __restrict__ x, const void* __restrict__ delta, int delta_
   }
 }
 
+// Many rows (a prompt): one wave per row, four rows per workgroup, a lane owns chunks lane, lane+64, ... of 8 channels;
+// no LDS and no barrier, every load of a row in flight at once.  Same arithmetic as add_rmsnorm_kernel with a
+// model-dtype delta: x' = T(x + delta) written back, y = T((x' * rstd) * w).
+__global__ void __launch_bounds__(256)
+add_rmsnorm_rows_bf16_kernel(bf16_t* __restrict__ x, const bf16_t* __restrict__ delta, const bf16_t* __restrict__ w,
+                             bf16_t* __restrict__ y, int rows, int d, float eps) {
+  constexpr int NCH = 4;   // d <= 2048
+  const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int nchunk = d >> 3;
+  const fstu_rsrc_t rx = fstu_make_rsrc(x + (size_t)r * d, (size_t)d * 2);
+  const fstu_rsrc_t rd = fstu_make_rsrc(delta ? delta + (size_t)r * d : nullptr, (size_t)d * 2);
+  const fstu_rsrc_t rw = fstu_make_rsrc(y ? w : nullptr, (size_t)d * 2);
+  uint4 xv[NCH], dv[NCH], wv[NCH];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const unsigned off = (unsigned)(lane + 64 * j) * 16u;   // beyond the row (or without the operand): zeros
+    xv[j] = fstu_buf_load16(rx, off);
+    dv[j] = fstu_buf_load16(rd, off);
+    wv[j] = fstu_buf_load16(rw, off);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    unsigned xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
+    const unsigned dw[4] = {dv[j].x, dv[j].y, dv[j].z, dv[j].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (delta)
+        xw[i] = pack2_bf16(__uint_as_float(xw[i] << 16) + __uint_as_float(dw[i] << 16),
+                           __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dw[i] & 0xffff0000u));
+      const float lo = __uint_as_float(xw[i] << 16), hi = __uint_as_float(xw[i] & 0xffff0000u);
+      ss = fmaf(lo, lo, ss);
+      ss = fmaf(hi, hi, ss);
+    }
+    xv[j] = make_uint4(xw[0], xw[1], xw[2], xw[3]);
+    if (delta && lane + 64 * j < nchunk) *(uint4*)(x + (size_t)r * d + (size_t)(lane + 64 * j) * 8) = xv[j];
+  }
+  if (y == nullptr) return;
+  const float rstd = rsqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    if (lane + 64 * j < nchunk) {
+      const unsigned xw[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w}, ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+      unsigned o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o[i] = pack2_bf16((__uint_as_float(xw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
+                          (__uint_as_float(xw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
+      *(uint4*)(y + (size_t)r * d + (size_t)(lane + 64 * j) * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 template <typename T>
 static int launch_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch, const void* w,
                               void* y, int rows, int d, float eps, hipStream_t s) {
+  if (sizeof(T) == 2 && rows >= 64 && (delta == nullptr || delta_mode == 0) && d % 8 == 0 && d <= 2048 &&
+      fstu_aligned(x, 16) && fstu_aligned(delta, 16) && fstu_aligned(w, 16) && fstu_aligned(y, 16)) {
+    hipLaunchKernelGGL(add_rmsnorm_rows_bf16_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)delta,
+                       (const bf16_t*)w, (bf16_t*)y, rows, d, eps);
+    return 0;
+  }
   const bool vec = (d % 4 == 0) && fstu_aligned(x, 16) && fstu_aligned(delta, 16) && fstu_aligned(w, 16) && fstu_aligned(y, 16);
   const int groups = vec ? d / 4 : d;
   const int ng = (groups + FSTU_NORM_THREADS - 1) / FSTU_NORM_THREADS;

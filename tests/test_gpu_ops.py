@@ -56,7 +56,7 @@ def test_embed(hip, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,d", [(8, 768), (3, 100), (64, 2048), (1, 256)])
+@pytest.mark.parametrize("rows,d", [(8, 768), (3, 100), (64, 2048), (1, 256), (4096, 768), (67, 200), (130, 1000)])
 def test_rmsnorm_plain_and_residual(hip, dtype, rows, d):
     g = gen(1)
     x = torch.randn(rows, d, generator=g).to(dtype)
