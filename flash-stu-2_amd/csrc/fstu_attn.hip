@@ -167,6 +167,25 @@ __global__ void kv_fill_kernel(const T* __restrict__ qkv, T* __restrict__ kring,
   }
 }
 
+// the same copy in 16-byte pieces (head dim a multiple of the piece, aligned pointers): one thread per piece
+template <typename T>
+__global__ void __launch_bounds__(256)
+kv_fill_vec_kernel(const T* __restrict__ qkv, T* __restrict__ kring, T* __restrict__ vring, int B, int Tn, int H, int hd,
+                   int cap, int pos0, int tstart) {
+  constexpr int EPP = 16 / (int)sizeof(T);
+  const int ppr = hd / EPP, d = H * hd, nt = Tn - tstart;
+  const unsigned n = (unsigned)B * nt * H * ppr;
+  for (unsigned idx = blockIdx.x * 256u + threadIdx.x; idx < n; idx += gridDim.x * 256u) {
+    const unsigned pc = idx % ppr, r1 = idx / ppr, h = r1 % H, r2 = r1 / H;
+    const int tt = tstart + (int)(r2 % nt), b = (int)(r2 / nt);
+    const T* src = qkv + ((size_t)b * Tn + tt) * 3 * d + h * hd + pc * EPP;
+    const int slot = (pos0 + tt) % cap;
+    const size_t dst = (((size_t)b * H + h) * cap + slot) * hd + pc * EPP;
+    *(uint4*)(kring + dst) = *(const uint4*)(src + d);
+    *(uint4*)(vring + dst) = *(const uint4*)(src + 2 * d);
+  }
+}
+
 static int check_kv(const char* name, const void* a, const void* b, const void* c, int B, int H, int hd, int cap) {
   FSTU_REQUIRE(a && b && c, FSTU_ENULL, "%s: null pointer", name);
   FSTU_REQUIRE(B >= 1 && H >= 1 && hd >= 1 && cap >= 1, FSTU_ESHAPE, "%s: bad shape B=%d H=%d hd=%d cap=%d", name, B, H, hd, cap);
@@ -181,6 +200,16 @@ extern "C" int fstu_kv_fill(const void* qkv, void* kring, void* vring, int B, in
   int tstart = T_ > cap ? T_ - cap : 0;
   size_t n = (size_t)B * (T_ - tstart) * H * hd;
   unsigned blocks = (unsigned)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
+  const int epp = dtype == FSTU_BF16 ? 8 : 4;
+  if (hd % epp == 0 && n / epp < 0xffffffffull && fstu_aligned(qkv, 16) && fstu_aligned(kring, 16) && fstu_aligned(vring, 16)) {
+    const size_t np = n / epp;
+    const unsigned vb = (unsigned)((np + 255) / 256 > 65535 ? 65535 : (np + 255) / 256);
+    FSTU_DISPATCH_DTYPE(dtype, "fstu_kv_fill",
+                        hipLaunchKernelGGL(kv_fill_vec_kernel<T>, dim3(vb), dim3(256), 0, (hipStream_t)stream,
+                                           (const T*)qkv, (T*)kring, (T*)vring, B, T_, H, hd, cap, pos0, tstart));
+    FSTU_CHECK_LAUNCH("fstu_kv_fill");
+    return FSTU_OK;
+  }
   FSTU_DISPATCH_DTYPE(dtype, "fstu_kv_fill",
                       hipLaunchKernelGGL(kv_fill_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                                          (const T*)qkv, (T*)kring, (T*)vring, B, T_, H, hd, cap, pos0, tstart));
