@@ -606,6 +606,44 @@ __device__ __forceinline__ double block_excl_scan_d(double v, double* red, doubl
   return base + inc - v;
 }
 
+// Bin selection of a radix-select pass by wave 0 (every lane of that wave calls it): the highest bin b with
+// base + (sum of the bins above b) + h[b] >= need (STRICT: > need), bin 0 if there is none; *above_out receives
+// base + the sum of the bins above the selected one.  Lane l owns bins 4l .. 4l+3; the sums over higher lanes come
+// from a suffix scan across the wave instead of one thread walking 256 LDS words.
+template <typename C, bool STRICT>
+__device__ __forceinline__ int select_bin_wave0(const C* h, C base, C need, C* above_out) {
+  const int lane = threadIdx.x & 63;
+  C v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = h[lane * 4 + j];
+  const C mine = v[0] + v[1] + v[2] + v[3];
+  C suf = mine;                                   // inclusive suffix sum over lanes >= lane
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const C t = __shfl_down(suf, o, FSTU_WAVE);
+    if (lane + o < 64) suf += t;
+  }
+  C ab = base + (suf - mine);                     // bins above this lane's highest bin
+  int found = -1;
+  C found_above = 0;
+#pragma unroll
+  for (int j = 3; j >= 0; --j) {
+    const bool hit = STRICT ? (ab + v[j] > need) : (ab + v[j] >= need);
+    if (found < 0 && hit) { found = lane * 4 + j; found_above = ab; }
+    ab += v[j];
+  }
+  const unsigned long long any = __ballot(found >= 0);
+  if (any == 0ull) {                              // no bin reaches it: bin 0, everything above bin 0
+    const C tot = __shfl(suf, 0, FSTU_WAVE);      // lane 0's inclusive suffix = all bins
+    const C h0 = __shfl(v[0], 0, FSTU_WAVE);
+    *above_out = base + tot - h0;
+    return 0;
+  }
+  const int top = 63 - __clzll((long long)any);   // the highest lane with a hit holds the highest bin
+  *above_out = __shfl(found_above, top, FSTU_WAVE);
+  return __shfl(found, top, FSTU_WAVE);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
 sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
@@ -669,20 +707,23 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.hist[i] = 0;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
-      for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
-        unsigned k = f32_key(sample_transform(row, i, t1, temperature));
-        if ((k & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k >> shift) & 255u], 1u);
+      // 8 strided loads in flight per thread (one load per trip would make every trip a round trip to the L2)
+      for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+        unsigned k[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) k[u] = f32_key(sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature));
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (i0 + u * FSTU_SAMPLE_THREADS < V && (k[u] & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k[u] >> shift) & 255u], 1u);
       }
       __syncthreads();
-      if (tid == 0) {
-        unsigned acc = 0;
-        int bin = 255;
-        for (; bin > 0; --bin) {
-          if (acc + sh.hist[bin] >= kk) break;
-          acc += sh.hist[bin];
+      if (w == 0) {
+        unsigned acc;
+        const int bin = select_bin_wave0<unsigned, false>(sh.hist, 0u, kk, &acc);
+        if (tid == 0) {
+          sh.sel_prefix = prefix | ((unsigned)bin << shift);
+          sh.sel_k = kk - acc;
         }
-        sh.sel_prefix = prefix | ((unsigned)bin << shift);
-        sh.sel_k = kk - acc;
       }
       __syncthreads();
       prefix = sh.sel_prefix;
@@ -698,9 +739,14 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   long long tie_keep = -1;  // -1: keep every tied token
   if (top_p > 0.f && top_p < 1.f) {
     double e = 0.0;
-    for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
-      float l = sample_transform(row, i, t1, temperature);
-      if (f32_key(l) >= thr_key) e += (double)expf(l - m);
+    // (sums stay in index order per thread: the batches only put 8 loads in flight together)
+    for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+      float l[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) l[u] = sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (i0 + u * FSTU_SAMPLE_THREADS < V && f32_key(l[u]) >= thr_key) e += (double)expf(l[u] - m);
     }
     double Z1;
     block_excl_scan_d(e, sh.redd, &Z1);
@@ -712,23 +758,26 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.mass[i] = 0ull;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
-      for (int i = tid; i < V; i += FSTU_SAMPLE_THREADS) {
-        float l = sample_transform(row, i, t1, temperature);
-        unsigned k = f32_key(l);
-        if (k >= thr_key && (k & himask) == (prefix & himask))
-          atomicAdd(&sh.mass[(k >> shift) & 255u], (unsigned long long)((double)expf(l - m) * scale));
+      for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+        float l[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) l[u] = sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const unsigned k = f32_key(l[u]);
+          if (i0 + u * FSTU_SAMPLE_THREADS < V && k >= thr_key && (k & himask) == (prefix & himask))
+            atomicAdd(&sh.mass[(k >> shift) & 255u], (unsigned long long)((double)expf(l[u] - m) * scale));
+        }
       }
       __syncthreads();
-      if (tid == 0) {
-        // lowest bin whose strictly-above mass is still <= target
-        unsigned long long acc = above;
-        int bin = 255;
-        for (; bin > 0; --bin) {
-          if (acc + sh.mass[bin] > target) break;  // bins below `bin` have mass-above > target
-          acc += sh.mass[bin];
+      if (w == 0) {
+        // lowest bin whose strictly-above mass is still <= target (bins below it have mass-above > target)
+        unsigned long long acc;
+        const int bin = select_bin_wave0<unsigned long long, true>(sh.mass, above, target, &acc);
+        if (tid == 0) {
+          sh.sel_prefix = prefix | ((unsigned)bin << shift);
+          sh.sel_mass = acc;
         }
-        sh.sel_prefix = prefix | ((unsigned)bin << shift);
-        sh.sel_mass = acc;
       }
       __syncthreads();
       prefix = sh.sel_prefix;
