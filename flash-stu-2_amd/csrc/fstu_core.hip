@@ -699,11 +699,18 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     return;
   }
 
+  // A 16-bit model dtype leaves the low 16 bits of every key the same for a given leading half (zeros for positive
+  // values, ones for negative ones, whose keys are complemented): the two low radix passes would find all their
+  // candidates in one bin, so they are skipped and the low half is filled in.
+  constexpr int LOW_SHIFT = sizeof(T) == 2 ? 16 : 0;
+  auto low_bits = [](unsigned prefix) -> unsigned {
+    return sizeof(T) == 2 ? ((prefix & 0x80000000u) ? 0u : 0xffffu) : 0u;
+  };
   // ---- top-k threshold by radix select on the monotone key
   unsigned thr_key = 0;  // keep keys >= thr_key
   if (top_k > 0 && top_k < V) {
     unsigned prefix = 0, kk = (unsigned)top_k;
-    for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int shift = 24; shift >= LOW_SHIFT; shift -= 8) {
       for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.hist[i] = 0;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
@@ -730,7 +737,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       kk = sh.sel_k;
       __syncthreads();
     }
-    thr_key = prefix;
+    thr_key = prefix | low_bits(prefix);
   }
 
   // ---- top-p over the survivors
@@ -754,7 +761,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     const unsigned long long target = (unsigned long long)((double)top_p * 17592186044416.0);
     unsigned prefix = 0;
     unsigned long long above = 0;  // mass of keys strictly above the current prefix range
-    for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int shift = 24; shift >= LOW_SHIFT; shift -= 8) {
       for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.mass[i] = 0ull;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
@@ -784,6 +791,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       above = sh.sel_mass;
       __syncthreads();
     }
+    prefix |= low_bits(prefix);
     // prefix = boundary key vb: mass strictly above it is `above` (<= target);
     // tokens tied at vb are kept while above + rank*p_b <= target.
     if (prefix >= thr_key) {
