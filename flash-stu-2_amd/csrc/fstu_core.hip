@@ -644,7 +644,10 @@ __device__ __forceinline__ int select_bin_wave0(const C* h, C base, C need, C* a
   return __shfl(found, top, FSTU_WAVE);
 }
 
-template <typename T>
+// CACHE (16-bit dtypes, rows of up to 64 K logits): the first pass leaves the transformed logits (temperature, clamp,
+// rounding: themselves 16-bit values) in LDS and every later pass reads them there instead of repeating the
+// division per element from L2.
+template <typename T, bool CACHE>
 __global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
 sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
               int top_k, float top_p, int do_sample, uint64_t seed, int step, int row0, const int* __restrict__ dyn) {
@@ -654,6 +657,10 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   const T* row = logits + (size_t)b * V;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const bool t1 = (temperature == 1.0f);
+  extern __shared__ unsigned short tl[];   // CACHE: transformed logits of the row
+  auto tv = [&](int i) -> float {
+    return CACHE ? __uint_as_float((unsigned)tl[i] << 16) : sample_transform(row, i, t1, temperature);
+  };
 
   // ---- pass A: maximum (lowest index on ties) over a strided walk
   float best = -INFINITY;
@@ -664,13 +671,17 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     for (; i + 7 * FSTU_SAMPLE_THREADS < V; i += 8 * FSTU_SAMPLE_THREADS) {
       float l[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) l[k] = sample_transform(row, i + k * FSTU_SAMPLE_THREADS, t1, temperature);
+      for (int k = 0; k < 8; ++k) {
+        l[k] = sample_transform(row, i + k * FSTU_SAMPLE_THREADS, t1, temperature);
+        if (CACHE) tl[i + k * FSTU_SAMPLE_THREADS] = (unsigned short)(__float_as_uint(l[k]) >> 16);
+      }
 #pragma unroll
       for (int k = 0; k < 8; ++k)
         if (besti == 0x7fffffff || l[k] > best) { best = l[k]; besti = i + k * FSTU_SAMPLE_THREADS; }
     }
     for (; i < V; i += FSTU_SAMPLE_THREADS) {
       float l = sample_transform(row, i, t1, temperature);
+      if (CACHE) tl[i] = (unsigned short)(__float_as_uint(l) >> 16);
       if (besti == 0x7fffffff || l > best) { best = l; besti = i; }
     }
   }
@@ -718,7 +729,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
         unsigned k[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) k[u] = f32_key(sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature));
+        for (int u = 0; u < 8; ++u) k[u] = f32_key(tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1)));
 #pragma unroll
         for (int u = 0; u < 8; ++u)
           if (i0 + u * FSTU_SAMPLE_THREADS < V && (k[u] & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k[u] >> shift) & 255u], 1u);
@@ -750,7 +761,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
       float l[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) l[u] = sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature);
+      for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1));
 #pragma unroll
       for (int u = 0; u < 8; ++u)
         if (i0 + u * FSTU_SAMPLE_THREADS < V && f32_key(l[u]) >= thr_key) e += (double)expf(l[u] - m);
@@ -768,7 +779,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
       for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
         float l[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) l[u] = sample_transform(row, min(i0 + u * FSTU_SAMPLE_THREADS, V - 1), t1, temperature);
+        for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const unsigned k = f32_key(l[u]);
@@ -810,14 +821,14 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   double tcount = 0.0;
   if (tie_keep >= 0)
     for (int i = i0; i < i1; ++i)
-      if (f32_key(sample_transform(row, i, t1, temperature)) == vb_key) tcount += 1.0;
+      if (f32_key(tv(i)) == vb_key) tcount += 1.0;
   double ttotal = 0.0;
   double tbase = (tie_keep >= 0) ? block_excl_scan_d(tcount, sh.redd, &ttotal) : 0.0;
   double mysum = 0.0;
   {
     long long rank = (long long)tbase;
     for (int i = i0; i < i1; ++i) {
-      float l = sample_transform(row, i, t1, temperature);
+      float l = tv(i);
       unsigned k = f32_key(l);
       bool keep = k > vb_key;
       if (k == vb_key) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
@@ -841,7 +852,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     long long rank = (long long)tbase;
     int pick = -1, lastkept = -1;
     for (int i = i0; i < i1; ++i) {
-      float l = sample_transform(row, i, t1, temperature);
+      float l = tv(i);
       unsigned k = f32_key(l);
       bool keep = k > vb_key;
       if (k == vb_key) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
@@ -886,8 +897,18 @@ int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B,
   FSTU_REQUIRE(temperature > 0.f, FSTU_EARG, "fstu_sample: temperature must be > 0");
   FSTU_REQUIRE(out_stride >= 1, FSTU_EARG, "fstu_sample: out_stride < 1");
   if (B == 0) return FSTU_OK;
+  if (dtype == FSTU_BF16 && do_sample && V <= 65536) {
+    const size_t shm = ((size_t)V * 2 + 15) & ~(size_t)15;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sample_kernel<bf16_t, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    FSTU_REQUIRE(e == hipSuccess, (int)e, "fstu_sample: %d bytes of dynamic LDS refused", 128 * 1024);
+    hipLaunchKernelGGL((sample_kernel<bf16_t, true>), dim3(B), dim3(FSTU_SAMPLE_THREADS), shm, (hipStream_t)stream,
+                       (const bf16_t*)logits, out, out_stride, V, temperature, top_k, top_p, do_sample, seed, step, row0, dyn);
+    FSTU_CHECK_LAUNCH("fstu_sample");
+    return FSTU_OK;
+  }
   FSTU_DISPATCH_DTYPE(dtype, "fstu_sample",
-                      hipLaunchKernelGGL(sample_kernel<T>, dim3(B), dim3(FSTU_SAMPLE_THREADS), 0, (hipStream_t)stream,
+                      hipLaunchKernelGGL((sample_kernel<T, false>), dim3(B), dim3(FSTU_SAMPLE_THREADS), 0, (hipStream_t)stream,
                                          (const T*)logits, out, out_stride, V, temperature, top_k, top_p, do_sample,
                                          seed, step, row0, dyn));
   FSTU_CHECK_LAUNCH("fstu_sample");
