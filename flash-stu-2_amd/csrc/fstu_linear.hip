@@ -14,6 +14,7 @@
 //
 // Other dtypes/shapes: a vector-ALU kernel, one wave per output feature.
 #include "fstu_common.h"
+#include <mutex>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
@@ -368,4 +369,53 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   rc = fstu_sample_dyn(logits, tok_out, tok_stride, rows, N, temperature, 0, 0.f, 0, 0, 0, 0, dyn, dtype, stream);
   if (rc == 0 && dyn && advance) rc = fstu_advance_dyn(dyn, stream);
   return rc;
+}
+
+// ---------------------------------------------------------------- head + greedy pick without any allocation
+// The packed per-row maxima of the head kernel live in a file-scope device array instead of a caller workspace, for
+// callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid hipMalloc).  Every GPU
+// holds its own copy of the array at its own address; the host only ever uses the address hipGetSymbolAddress returns
+// for the current device, never the array's name.
+#define FSTU_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned long long scratch[FSTU_MAX_DECODE_ROWS * 64];   // 8 KiB per GPU
+static unsigned long long* g_scratch_ptr[FSTU_STATIC_MAX_DEVICES];   // per device, filled on first use
+static std::mutex g_scratch_mu;
+
+__global__ void __launch_bounds__(1024) fill_zero_u64_kernel(unsigned long long* p, int n) {
+  const int i = blockIdx.x * 1024 + threadIdx.x;
+  if (i < n) p[i] = 0ull;
+}
+
+static int static_scratch(unsigned long long** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { fstu_set_error("fstu_head_argmax_static: hipGetDevice: %s", hipGetErrorString(e)); return (int)e; }
+  FSTU_REQUIRE(dev >= 0 && dev < FSTU_STATIC_MAX_DEVICES, FSTU_EARG, "fstu_head_argmax_static: device index %d outside 0..%d", dev,
+               FSTU_STATIC_MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fstu_set_error("fstu_head_argmax_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : FSTU_EARG;
+    }
+    g_scratch_ptr[dev] = (unsigned long long*)p;
+  }
+  *out = g_scratch_ptr[dev];
+  return FSTU_OK;
+}
+
+extern "C" int fstu_head_argmax_static(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                                       float temperature, int64_t* tok_out, int64_t tok_stride, int dtype, void* stream) {
+  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS, FSTU_ESHAPE,
+               "fstu_head_argmax_static: rows=%d beyond the static scratch (%d rows x 64 slots)", rows, FSTU_MAX_DECODE_ROWS);
+  unsigned long long* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc) return rc;
+  // the array keeps whatever the last call on this GPU left (an interrupted call may have left maxima behind)
+  hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ws, FSTU_MAX_DECODE_ROWS * 64);
+  FSTU_CHECK_LAUNCH("fstu_head_argmax_static");
+  return fstu_head_argmax_dyn(x, ldx, W, logits, ldy, rows, N, K, temperature, ws, tok_out, tok_stride, nullptr, 0, dtype,
+                              stream);
 }

@@ -57,6 +57,7 @@ SIGNATURES = {
     "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
+    "fstu_head_argmax_static": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i64, _i, _vp],
     "fstu_head_packed_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _vp],
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
     "fstu_packed_elems": [_i, _i],

@@ -301,6 +301,16 @@ int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ld
                      float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
                      void* stream);
 
+/* fstu_head_argmax for callers that cannot allocate or pass a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * fstu_head_argmax without best_ws: the packed per-row maxima live in a static device array of the library
+ * (FSTU_MAX_DECODE_ROWS * 64 64-bit words = 8 KiB, held on every GPU the library runs on until the process ends).
+ * rows > FSTU_MAX_DECODE_ROWS is rejected with FSTU_ESHAPE.  The call clears the array with a small fill kernel on
+ * `stream` first and allocates nothing (no hipMalloc / hipFree, no allocating library routine).  All calls on one GPU
+ * share that GPU's array: calls that overlap on one GPU (different streams or threads) race. */
+int fstu_head_argmax_static(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                            float temperature, int64_t* tok_out, int64_t tok_stride, int dtype, void* stream);
+
 /* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
  * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:
  *   h <- h*A + x_t @ Bm ;  y_t = T(h @ Cm)
