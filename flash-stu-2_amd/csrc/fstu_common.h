@@ -54,14 +54,17 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
-int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
-                             int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream);
+int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* y,
+                               int ldy, int B, int S, int d, int t, const int* dyn, int dtype, void* stream);
+int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
+                             const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn,
+                             void* stream);
 int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                                 const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
-                                 int d, int K, int t, const int* dyn, void* stream);
+                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
+                                 int B, int S, int d, int K, int t, const int* dyn, void* stream);
 int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
-                                  const float* ce, void* y, int ldy, int B, int S, int d, int K, int t, const int* dyn,
-                                  void* stream);
+                                  const float* ce, const float* co, void* y, int ldy, int B, int S, int d, int K, int t,
+                                  const int* dyn, void* stream);
 int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
                                 float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                                 void* stream);

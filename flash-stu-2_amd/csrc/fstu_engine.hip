@@ -151,6 +151,15 @@ static void warm_join_all(hipStream_t main) {
   for (int i = 0; i < w->n; ++i) (void)hipStreamWaitEvent(main, w->join[i], 0);
 }
 
+// recurrence step on m->xp: both sign branches rounded separately when the layer carries odd-lag weights
+static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, void* stream) {
+  if (L.lds_co)
+    return fstu_stu_step_lds_pair_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, L.lds_co, m->y, m->d, m->B, m->lds_S, m->d, pos,
+                                      dyn, m->dtype, stream);
+  return fstu_stu_step_lds_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, m->dtype,
+                               stream);
+}
+
 static int hist_nsplit(int nlags, int maxsplit) {
   int n = nlags / 64;
   if (n < 1) n = 1;
@@ -199,7 +208,7 @@ static int decode_step_fused(const fstu_model_desc* m, const int64_t* tok_in, in
       g.mode = 0; g.rows = B; g.N = d; g.K = d; g.Wp = L.wp_m_inputs; g.y = m->xp; g.ldy = d;
       pro(g, L.norm1_w);
       TIMED(PC_PROJ, fstu_gemv_packed_dyn(&g, dyn, 0, stream));
-      TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, pos, dyn, dt, stream));
+      TIMED(PC_STU, stu_step(L, m, pos, dyn, stream));
     } else {
       fstu_gemv_args g = {};
       g.mode = 0; g.rows = B; g.N = 3 * d; g.K = d; g.Wp = L.wp_qkv; g.y = m->qkv; g.ldy = 3 * d;
@@ -339,18 +348,18 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       } else {
         if (pending_slices) {
           TIMED(PC_STU, fstu_stu_res_inproj_step_dyn(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a,
-                                                     L.lds_ce, m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
+                                                     L.lds_ce, L.lds_co, m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
           void* t = xc; xc = xo; xo = t;
           pending_slices = false;
         } else if (res_chain) {
-          TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y,
+          TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, m->y,
                                                       d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
         } else if (dt == FSTU_BF16 && d % 256 == 0) {
-          TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, m->y, d, nullptr, B,
+          TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, m->y, d, nullptr, B,
                                                  m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
         } else {
           TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-          TIMED(PC_STU, fstu_stu_step_lds_dyn(L.lds_state, m->xp, d, L.lds_a, L.lds_ce, m->y, d, B, m->lds_S, d, stu_pos(pos), stu_dyn(dyn), dt, stream));
+          TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), stream));
         }
         pending_y = true;
       }

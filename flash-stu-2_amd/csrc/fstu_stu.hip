@@ -120,14 +120,16 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
                     const float* __restrict__ ce, const float* __restrict__ co /*optional: weights of the other bank*/,
-                    float scale, T* __restrict__ y, int ldy, int S, int d, int parity, const int* __restrict__ dyn) {
+                    float scale, T* __restrict__ y, int ldy, int S, int d, int parity, const int* __restrict__ dyn,
+                    int pair /* != 0 (needs co): y = T(T(E+O) + T(E-O)), the two sign branches rounded separately */) {
   __shared__ float sh[LDS_JG][32][4];
+  __shared__ float sho[LDS_JG][32][4];
   if (dyn) parity = dyn[0] & 1;
   const int b = blockIdx.y;
   const int q = threadIdx.x & 31, jg = threadIdx.x >> 5;
   const int c = (blockIdx.x * 32 + q) * 4;
   const bool ok = c < d;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acco[4] = {0.f, 0.f, 0.f, 0.f};
   if (ok) {
     float x[4];
 #pragma unroll
@@ -155,23 +157,24 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
       for (int j = jg; j < S; j += LDS_JG) {
         const float4 h = *(const float4*)(so + (size_t)j * d);
         const float4 oj = *(const float4*)(co + (size_t)j * d + c);
-        acc[0] = fmaf(oj.x, h.x, acc[0]);
-        acc[1] = fmaf(oj.y, h.y, acc[1]);
-        acc[2] = fmaf(oj.z, h.z, acc[2]);
-        acc[3] = fmaf(oj.w, h.w, acc[3]);
+        acco[0] = fmaf(oj.x, h.x, acco[0]);
+        acco[1] = fmaf(oj.y, h.y, acco[1]);
+        acco[2] = fmaf(oj.z, h.z, acco[2]);
+        acco[3] = fmaf(oj.w, h.w, acco[3]);
       }
     }
   }
 #pragma unroll
-  for (int v = 0; v < 4; ++v) sh[jg][q][v] = acc[v];
+  for (int v = 0; v < 4; ++v) { sh[jg][q][v] = acc[v]; sho[jg][q][v] = acco[v]; }
   __syncthreads();
   if (jg == 0 && ok) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      float s = 0.f;
+      float e = 0.f, o = 0.f;
 #pragma unroll
-      for (int g = 0; g < LDS_JG; ++g) s += sh[g][q][v];
-      DT<T>::st(y + (size_t)b * ldy + c + v, scale * s);
+      for (int g = 0; g < LDS_JG; ++g) { e += sh[g][q][v]; o += sho[g][q][v]; }
+      const float out = pair ? DT<T>::rnd(e + o) + DT<T>::rnd(e - o) : scale * (e + o);
+      DT<T>::st(y + (size_t)b * ldy + c + v, out);
     }
   }
 }
@@ -183,7 +186,7 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
 
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream);
+                               void* stream, int pair = 0);
 
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
@@ -198,9 +201,21 @@ extern "C" int fstu_stu_step_lds_single(float* state, const void* xp, int ldxp, 
   return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, nullptr, dtype, stream);
 }
 
+extern "C" int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce,
+                                      const float* co, void* y, int ldy, int B, int S, int d, int t, int dtype, void* stream) {
+  return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, y, ldy, B, S, d, t, nullptr, dtype, stream);
+}
+
+int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* y,
+                               int ldy, int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
+  FSTU_REQUIRE(co, FSTU_ENULL, "fstu_stu_step_lds_pair: null pointer");
+  FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_pair: co must be 16-byte aligned");
+  return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, dyn, dtype, stream, 1);
+}
+
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream) {
+                               void* stream, int pair) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
   FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
@@ -209,7 +224,7 @@ static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const flo
   dim3 grid((d / 4 + 31) / 32, B);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
                       hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
-                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn));
+                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair));
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }
@@ -311,7 +326,9 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
                        const bf16_t* __restrict__ x_res /*optional (B,K): normalise it instead of reading h*/,
                        const bf16_t* __restrict__ norm_w, float eps,
                        const float* __restrict__ slices /*optional, with x_res: up to 4 fp32 (B,K) slices added first*/,
-                       int nslices, bf16_t* __restrict__ x_out /*receives x_res + T(sum of slices); not x_res itself*/) {
+                       int nslices, bf16_t* __restrict__ x_out /*receives x_res + T(sum of slices); not x_res itself*/,
+                       const float* __restrict__ co /*optional (S,d): odd-lag weights on the other bank; then
+                       y = T(T(E+O) + T(E-O)) instead of T(2E)*/) {
   __shared__ float red[4][64][4];
   __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
   extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
@@ -510,6 +527,20 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
         sum.w = fmaf(cj.w, hv.w, sum.w);
       }
     }
+    // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (read only)
+    float4 sumo = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (co && c < d) {
+      const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
+#pragma unroll 8
+      for (int j = jsub; j < S; j += 8) {
+        const float4 hv = *(const float4*)(so + (size_t)j * d);
+        const float4 oj = *(const float4*)(co + (size_t)j * d + c);
+        sumo.x = fmaf(oj.x, hv.x, sumo.x);
+        sumo.y = fmaf(oj.y, hv.y, sumo.y);
+        sumo.z = fmaf(oj.z, hv.z, sumo.z);
+        sumo.w = fmaf(oj.w, hv.w, sumo.w);
+      }
+    }
     // reduce over the 8 mode groups (lanes differing in bits 2..4): two rotations inside the row of 16 lanes, one
     // swizzle across the two rows
     auto grp_sum = [](float v) {
@@ -521,78 +552,92 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     sum.y = grp_sum(sum.y);
     sum.z = grp_sum(sum.z);
     sum.w = grp_sum(sum.w);
+    float4 out = make_float4(2.f * sum.x, 2.f * sum.y, 2.f * sum.z, 2.f * sum.w);
+    if (co) {
+      sumo.x = grp_sum(sumo.x);
+      sumo.y = grp_sum(sumo.y);
+      sumo.z = grp_sum(sumo.z);
+      sumo.w = grp_sum(sumo.w);
+      out.x = DT<bf16_t>::rnd(sum.x + sumo.x) + DT<bf16_t>::rnd(sum.x - sumo.x);
+      out.y = DT<bf16_t>::rnd(sum.y + sumo.y) + DT<bf16_t>::rnd(sum.y - sumo.y);
+      out.z = DT<bf16_t>::rnd(sum.z + sumo.z) + DT<bf16_t>::rnd(sum.z - sumo.z);
+      out.w = DT<bf16_t>::rnd(sum.w + sumo.w) + DT<bf16_t>::rnd(sum.w - sumo.w);
+    }
     if (jsub == 0 && c < d) {
       bf16_t* yp = y + (size_t)b * ldy + c;
       if ((ldy & 3) == 0) {
-        *(uint2*)yp = make_uint2(pack2_bf16(2.f * sum.x, 2.f * sum.y), pack2_bf16(2.f * sum.z, 2.f * sum.w));
+        *(uint2*)yp = make_uint2(pack2_bf16(out.x, out.y), pack2_bf16(out.z, out.w));
       } else {
-        yp[0] = f32_to_bf16(2.f * sum.x);
-        yp[1] = f32_to_bf16(2.f * sum.y);
-        yp[2] = f32_to_bf16(2.f * sum.z);
-        yp[3] = f32_to_bf16(2.f * sum.w);
+        yp[0] = f32_to_bf16(out.x);
+        yp[1] = f32_to_bf16(out.y);
+        yp[2] = f32_to_bf16(out.z);
+        yp[3] = f32_to_bf16(out.w);
       }
     }
   }
   STU_STAMP(5);
 }
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
-                              float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
-                              int K, int t, const int* dyn, void* stream, const float* slices = nullptr, int nslices = 0,
-                              void* x_out = nullptr);
+                              float* state, const float* a, const float* ce, const float* co, void* y, int ldy, void* xp_out,
+                              int B, int S, int d, int K, int t, const int* dyn, void* stream, const float* slices = nullptr,
+                              int nslices = 0, void* x_out = nullptr);
 
-int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce, void* y,
-                             int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn, void* stream) {
-  return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, y, ldy, xp_out, B, S, d, K, t, dyn, stream);
+int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
+                             const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn,
+                             void* stream) {
+  return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, dyn, stream);
 }
 
 int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
-                                  const float* ce, void* y, int ldy, int B, int S, int d, int K, int t, const int* dyn,
-                                  void* stream) {
+                                  const float* ce, const float* co, void* y, int ldy, int B, int S, int d, int K, int t,
+                                  const int* dyn, void* stream) {
   FSTU_REQUIRE(x_res && norm_w, FSTU_ENULL, "fstu_stu_norm_inproj_step: null pointer");
-  return inproj_step_launch(x_res, K, x_res, norm_w, eps, Mt, state, a, ce, y, ldy, nullptr, B, S, d, K, t, dyn, stream);
+  return inproj_step_launch(x_res, K, x_res, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream);
 }
 
 // x' = x_in + T(sum of nslices <= 4 fp32 slices) goes to x_out, h = rmsnorm(x') * norm_w feeds the projection: the
 // add+norm launch between the previous layer's down projection and this layer, folded into this kernel
 int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                                 const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
-                                 int d, int K, int t, const int* dyn, void* stream) {
+                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
+                                 int B, int S, int d, int K, int t, const int* dyn, void* stream) {
   FSTU_REQUIRE(x_in && slices && x_out && norm_w, FSTU_ENULL, "fstu_stu_res_inproj_step: null pointer");
   FSTU_REQUIRE(nslices >= 1 && nslices <= 4, FSTU_EARG, "fstu_stu_res_inproj_step: nslices=%d outside 1..4", nslices);
   FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_stu_res_inproj_step: x_out must not alias x_in");
   FSTU_REQUIRE((NormPrologue<256, 4, 4>::supported(B, K)), FSTU_ESHAPE, "fstu_stu_res_inproj_step: B=%d K=%d not supported", B, K);
   FSTU_REQUIRE(fstu_aligned(slices, 16) && fstu_aligned(x_out, 16), FSTU_EALIGN, "fstu_stu_res_inproj_step: pointers must be 16-byte aligned");
-  return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, y, ldy, nullptr, B, S, d, K, t, dyn, stream, slices,
+  return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream, slices,
                             nslices, x_out);
 }
 
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
-                              float* state, const float* a, const float* ce, void* y, int ldy, void* xp_out, int B, int S, int d,
-                              int K, int t, const int* dyn, void* stream, const float* slices, int nslices, void* x_out) {
+                              float* state, const float* a, const float* ce, const float* co, void* y, int ldy, void* xp_out,
+                              int B, int S, int d, int K, int t, const int* dyn, void* stream, const float* slices, int nslices,
+                              void* x_out) {
   FSTU_REQUIRE(h && Mt && state && a && ce && y, FSTU_ENULL, "fstu_stu_inproj_step: null pointer");
   FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
   FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(Mt, 16) && fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_inproj_step: pointers must be 16-byte aligned");
   const size_t shm = x_res ? (size_t)B * (K + 8) * 2 : 0;
   FSTU_REQUIRE(shm <= 56 * 1024, FSTU_ESHAPE, "fstu_stu_inproj_step: B*K too large for the norm prologue");
-  FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w must be 16-byte aligned");
+  FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w/co must be 16-byte aligned");
   hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,
                      (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,
-                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out);
+                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out, co);
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
 }
 
 extern "C" int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w,
-                                        float eps, const void* Mt, float* state, const float* a, const float* ce, void* y,
-                                        int ldy, int B, int S, int d, int K, int t, void* stream) {
-  return fstu_stu_res_inproj_step_dyn(x_in, slices, nslices, x_out, norm_w, eps, Mt, state, a, ce, y, ldy, B, S, d, K, t, nullptr,
-                                      stream);
+                                        float eps, const void* Mt, float* state, const float* a, const float* ce,
+                                        const float* co, void* y, int ldy, int B, int S, int d, int K, int t, void* stream) {
+  return fstu_stu_res_inproj_step_dyn(x_in, slices, nslices, x_out, norm_w, eps, Mt, state, a, ce, co, y, ldy, B, S, d, K, t,
+                                      nullptr, stream);
 }
 
 extern "C" int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                                    void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream) {
-  return fstu_stu_inproj_step_dyn(h, ldh, Mt, state, a, ce, y, ldy, xp_out, B, S, d, K, t, nullptr, stream);
+                                    const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t,
+                                    void* stream) {
+  return fstu_stu_inproj_step_dyn(h, ldh, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, nullptr, stream);
 }
 
 // ---------------------------------------------------------------- state from history

@@ -34,10 +34,11 @@ SIGNATURES = {
     "fstu_bias_act": [_vp, _vp, _i64, _i, _i, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_pair": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_single": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
-    "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_scan_lds": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -284,9 +285,10 @@ def stu_step_hist(hist: torch.Tensor, filt: torch.Tensor, t: int, nsplit: int, e
 
 
 def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
-                 out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d).  With co (S,d), the single-branch form:
-    y = ce . bank(t) + co . other bank (use_hankel_L), without the factor 2 of the two sign branches."""
+                 out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None, pair: bool = False) -> torch.Tensor:
+    """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d) = T(2E), E = ce . bank(t).  With co (S,d) and
+    O = co . other bank: the single-branch form y = T(E+O) (use_hankel_L), or with pair=True the two sign branches
+    rounded separately, y = T(T(E+O) + T(E-O))."""
     _dev(state, a, ce, co)
     B, two, S, d = state.shape
     assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
@@ -299,6 +301,10 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
     assert orow == B and out.dtype == xp.dtype
     if co is not None:
         assert co.dtype == torch.float32 and co.shape == (S, d)
+        if pair:
+            _check(load().fstu_stu_step_lds_pair(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), _p(out), ldy, B, S, d, t,
+                                                 _dt(xp), _stream()), "fstu_stu_step_lds_pair")
+            return out
         _check(load().fstu_stu_step_lds_single(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), _p(out), ldy, B, S, d, t,
                                                _dt(xp), _stream()), "fstu_stu_step_lds_single")
         return out
@@ -331,24 +337,26 @@ def stu_scan_lds(xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, state: Opt
 
 
 def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
-                    out: Optional[torch.Tensor] = None, xp_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """h (B,K) bf16, Mt = M_inputs^T (d,K): projection + recurrence step in one launch -> y (B,d)."""
-    _dev(h, Mt, state, a, ce, out, xp_out)
+                    out: Optional[torch.Tensor] = None, xp_out: Optional[torch.Tensor] = None,
+                    co: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h (B,K) bf16, Mt = M_inputs^T (d,K): projection + recurrence step in one launch -> y (B,d); with co the step
+    of stu_step_lds(pair=True)."""
+    _dev(h, Mt, state, a, ce, out, xp_out, co)
     B, K = h.shape
     d = Mt.shape[0]
     S = a.numel()
     assert h.dtype == Mt.dtype == torch.bfloat16 and Mt.shape[1] == K and state.shape == (B, 2, S, d)
     if out is None:
         out = torch.empty(B, d, dtype=h.dtype, device=h.device)
-    _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(out), d, _p(xp_out), B, S, d, K, t,
-                                       _stream()), "fstu_stu_inproj_step")
+    _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(co), _p(out), d, _p(xp_out), B, S, d,
+                                       K, t, _stream()), "fstu_stu_inproj_step")
     return out
 
 
 def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tensor, eps: float, Mt: torch.Tensor,
-                        state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int):
+                        state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int, co: Optional[torch.Tensor] = None):
     """(x', y): x' = x + bf16(sum of the fp32 slices); y = projection + recurrence step of rmsnorm(x') * norm_w."""
-    _dev(x, partial, norm_w, Mt, state, a, ce)
+    _dev(x, partial, norm_w, Mt, state, a, ce, co)
     B, K = x.shape
     d = Mt.shape[0]
     S = a.numel()
@@ -356,7 +364,7 @@ def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Te
     x_out = torch.empty_like(x)
     y = torch.empty(B, d, dtype=x.dtype, device=x.device)
     _check(load().fstu_stu_res_inproj_step(_p(x), _p(partial), partial.shape[0], _p(x_out), _p(norm_w), float(eps), _p(Mt),
-                                           _p(state), _p(a), _p(ce), _p(y), d, B, S, d, K, t, _stream()),
+                                           _p(state), _p(a), _p(ce), _p(co), _p(y), d, B, S, d, K, t, _stream()),
            "fstu_stu_res_inproj_step")
     return x_out, y
 

@@ -28,7 +28,7 @@ _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
 class LayerDesc(ctypes.Structure):
     _fields_ = [("kind", _i), ("norm1_w", _vp), ("mlp_norm_w", _vp), ("w_gate", _vp), ("w_up", _vp), ("w_down", _vp),
-                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_state", _vp),
+                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_co", _vp), ("lds_state", _vp),
                 ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp),
                 ("wp_gate", _vp), ("wp_up", _vp), ("wp_down", _vp), ("wp_m_inputs", _vp), ("wp_qkv", _vp),
                 ("wp_proj", _vp)]
@@ -175,10 +175,10 @@ class DecodeEngine:
                 ld.m_inputs_t = mit.data_ptr()
                 hist, state, pos = caches[i]
                 if mode == "lds":
-                    a, ce = stu.lds_params()
+                    a, ce, co = stu.lds_params()
                     st = state[b0:b1]
-                    keep(a), keep(ce), keep(st)
-                    ld.lds_a, ld.lds_ce, ld.lds_state = a.data_ptr(), ce.data_ptr(), st.data_ptr()
+                    keep(a), keep(ce), keep(co), keep(st)
+                    ld.lds_a, ld.lds_ce, ld.lds_co, ld.lds_state = a.data_ptr(), ce.data_ptr(), co.data_ptr(), st.data_ptr()
                 else:
                     hs = hist[b0:b1]
                     if hist_cap and hs.shape[1] != hist_cap:
@@ -402,8 +402,10 @@ class DecodeEngine:
             raise _hip.FlashSTUHipError("input_ids must be on the GPU: this model has no CPU path")
         B, P = input_ids.shape
         total = P + n_new
-        if self.cfg.resolved_stu_decode_mode() == "history" and total > self.cfg.seq_len:
-            raise ValueError(f"history-mode decode needs prompt+new tokens ({total}) <= seq_len ({self.cfg.seq_len})")
+        if total > self.cfg.seq_len:
+            # the history ends there, and the recurrence state would carry a tail the filters (zero from lag seq_len
+            # on) do not have; FlashSTU.generate routes such calls to the recompute loop
+            raise ValueError(f"stateful decode needs prompt+new tokens ({total}) <= seq_len ({self.cfg.seq_len})")
         tokens = torch.zeros(B, total, dtype=torch.int64, device=input_ids.device)
         tokens[:, :P] = input_ids
         logits = self.prefill(input_ids, total)

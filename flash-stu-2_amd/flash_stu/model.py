@@ -73,7 +73,7 @@ class FlashSTU(nn.Module):
             else:
                 self.layers.append(AttentionLayer(config))
         self.norm = RMSNorm(config.n_embd, config.rms_norm_eps, dtype=config.torch_dtype)
-        self.lm_head = nn.Linear(config.n_embd, config.vocab_size, bias=False, dtype=config.torch_dtype)
+        self.lm_head = nn.Linear(config.n_embd, config.vocab_size, bias=config.bias, dtype=config.torch_dtype)   # model.py:100-102
         self.tok_emb.weight = self.lm_head.weight
         self.std = config.n_embd ** -0.5
         self.apply(self._init_weights)
@@ -107,7 +107,7 @@ class FlashSTU(nn.Module):
                     torch.nn.init.zeros_(lin.bias)
 
     @torch.no_grad()
-    def load_oracle_weights(self, w: Dict[str, torch.Tensor]) -> None:
+    def load_named_tensors(self, w: Dict[str, torch.Tensor]) -> None:
         """Copies a {reference state-dict name: tensor} mapping into the model."""
         sd = self.state_dict()
         for k, v in w.items():
@@ -125,10 +125,7 @@ class FlashSTU(nn.Module):
         return _hip.embed(input_ids, self.tok_emb.weight)
 
     def _head(self, x: torch.Tensor) -> torch.Tensor:
-        B, T, d = x.shape
-        if B * T <= _hip.MAX_DECODE_ROWS:
-            return _hip.linear_decode(x.reshape(B * T, d), self.lm_head.weight).reshape(B, T, -1)
-        return torch.matmul(x, self.lm_head.weight.t())
+        return _hip.linear(x, self.lm_head.weight, self.lm_head.bias)
 
     @torch.no_grad()
     def _run_layers(self, x, past_key_values, use_cache, hidden):
@@ -212,7 +209,9 @@ class FlashSTU(nn.Module):
         if n_new <= 0:
             return input_ids
         from .engine import DecodeEngine
-        if use_cache and P <= self.config.seq_len and DecodeEngine.supports(self.config):
+        # Sequences that outgrow seq_len leave the stateful paths: the filters end at lag seq_len, so the reference
+        # re-runs the last seq_len tokens without a cache from there on (model.py:250-255), and so does the loop below.
+        if use_cache and max_length <= self.config.seq_len and DecodeEngine.supports(self.config):
             return self.decode_engine().generate(input_ids, n_new, temperature, top_k, top_p, do_sample, seed,
                                                  return_logits=return_logits, use_graph=kwargs.get("use_graph", True))
         tokens = torch.empty(B, max_length, dtype=torch.int64, device=input_ids.device)
@@ -275,10 +274,13 @@ class FlashSTU(nn.Module):
         if new_num_tokens == old:
             return self.tok_emb
         dev, dt = self.lm_head.weight.device, self.config.torch_dtype
-        head = nn.Linear(self.config.n_embd, new_num_tokens, bias=False, dtype=dt).to(dev)
+        head = nn.Linear(self.config.n_embd, new_num_tokens, bias=self.lm_head.bias is not None, dtype=dt).to(dev)
         torch.nn.init.normal_(head.weight, mean=0.0, std=self.std)
         keep = min(old, new_num_tokens)
         head.weight.data[:keep] = self.lm_head.weight.data[:keep]
+        if head.bias is not None:
+            torch.nn.init.zeros_(head.bias)
+            head.bias.data[:keep] = self.lm_head.bias.data[:keep]
         emb = nn.Embedding(new_num_tokens, self.config.n_embd, dtype=dt).to(dev)
         self.lm_head, self.tok_emb = head, emb
         self.tok_emb.weight = self.lm_head.weight

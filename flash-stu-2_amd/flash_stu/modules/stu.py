@@ -21,7 +21,7 @@ import torch
 import torch.nn as nn
 
 from .. import _hip
-from ..utils.lds_fit import fit_even_lag_lds
+from ..utils.lds_fit import check_lds_fit, fit_even_lag_lds
 
 
 FFT_MIN_T = 32     # shorter inputs take the time-domain kernel (a 64-point transform would be mostly padding)
@@ -101,12 +101,25 @@ class STU(nn.Module):
     def m_inputs_t(self) -> torch.Tensor:
         return self._cached("mit", (self.M_inputs,), lambda: self.m_inputs_eff().t().contiguous())
 
-    def lds_params(self) -> Tuple[torch.Tensor, torch.Tensor]:
+    def lds_params(self) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Poles a (S) and per-channel output weights ce, co (S,d) fitted to the even / odd lags of phi_proj.  The two
+        sign branches are plus = E + O and minus = E - O (E, O the even- / odd-lag parts of the convolution): the
+        decode step forms E on the bank of the token's parity and O on the other bank, and rounds the branches
+        separately as the reference does (stu_utils.py:226-228, stu.py:120)."""
         def build():
-            a, ce, err = fit_even_lag_lds(self.effective_filter()[0::2], self.config.stu_lds_state_dim)
-            self.lds_fit_error = err
+            S = self.config.stu_lds_state_dim
+            f = self.effective_filter()
+            if f.shape[0] % 2 != 0:
+                f = torch.cat([f, torch.zeros_like(f[:1])], 0)      # equally long even- and odd-lag halves
+            a, ce, e1 = fit_even_lag_lds(f[0::2], S, per_channel=True)
+            a2, co, e2 = fit_even_lag_lds(f[1::2], S, per_channel=True)
+            if not torch.equal(a, a2):
+                raise RuntimeError("pole grids of the even and odd lags differ")
+            self.lds_fit_error = float(max(e1.max(), e2.max()))
+            check_lds_fit(e1, f[0::2])
+            check_lds_fit(e2, f[0::2])          # the odd lags against the scale of the channel's leading (even) taps
             dev = self.M_filters.device
-            return a.to(dev), ce.to(dev).contiguous()
+            return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
         return self._cached("lds", (self.phi, self.M_filters), build)
 
     def lds_single_params(self):
@@ -115,11 +128,13 @@ class STU(nn.Module):
         def build():
             S = self.config.stu_lds_state_dim
             f = self.effective_filter()
-            a, ce, e1 = fit_even_lag_lds(f[0::2], S)
-            a2, co, e2 = fit_even_lag_lds(f[1::2], S)
+            a, ce, e1 = fit_even_lag_lds(f[0::2], S, per_channel=True)
+            a2, co, e2 = fit_even_lag_lds(f[1::2], S, per_channel=True)
             if not torch.equal(a, a2):
                 raise RuntimeError("pole grids of the even and odd lags differ")
-            self.lds_fit_error = max(e1, e2)
+            self.lds_fit_error = float(max(e1.max(), e2.max()))
+            check_lds_fit(e1, f[0::2])
+            check_lds_fit(e2, f[0::2])          # the odd lags against the scale of the channel's leading (even) taps
             dev = self.M_filters.device
             return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
         return self._cached("ldssingle", (self.phi, self.M_filters), build)
@@ -137,6 +152,8 @@ class STU(nn.Module):
             if phi.shape[0] % 2 == 0 and not torch.equal(a, a2):
                 raise RuntimeError("pole grids of the even and odd lags differ")
             self.lds_fit_error = max(e1, e2)
+            # the K filters are contracted together (M_phi): the error counts against the largest tap of the bank
+            check_lds_fit(self.lds_fit_error, phi.detach().float().abs().max().reshape(1, 1))
             dev = phi.device
             return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
         return self._cached("banklds", (self.phi,), build)
@@ -236,7 +253,7 @@ class STU(nn.Module):
             if self.use_approx and self._scan_prefill():
                 # the distilled recurrence over the whole prompt: outputs and the decode state in one launch
                 xp = self._project(x)
-                a, ce = self.lds_params()
+                a, ce, _ = self.lds_params()
                 y, state = _hip.stu_scan_lds(xp, a, ce)
                 if not use_cache:
                     return y
@@ -283,8 +300,8 @@ class STU(nn.Module):
                 a, ce, co = self.lds_single_params()
                 y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co)
             else:
-                a, ce = self.lds_params()
-                y = _hip.stu_step_lds(state, xp, a, ce, pos)
+                a, ce, co = self.lds_params()
+                y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co, pair=True)
             return y, (hist, state, pos_t + 1)
         if not self.use_approx and state.numel() > 0:
             # exact mode on the recurrence state: U+- for all K filters, then the two contractions as skinny GEMVs

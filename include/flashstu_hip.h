@@ -127,6 +127,15 @@ int fstu_stu_step_hist(const void* hist, const void* filt, float* eo, int B, int
 int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                       int B, int S, int d, int t, int dtype, void* stream);
 
+/* The two-branch step with the reference's rounding points: besides E = sum_j ce[j,c]*h_j over the bank of parity t&1
+ * (after its advance; even lags), O = sum_j co[j,c]*h_j over the other bank (odd lags: lag 2m+1 reaches position
+ * t-1-2m), co (S,d) fitted to phi_proj's odd lags, and
+ *   y[b,c] = T( T(E + O) + T(E - O) )
+ * i.e. the plus and the minus branch rounded to the model dtype separately before their sum
+ * (flash_stu/utils/stu_utils.py:226-228, flash_stu/modules/stu.py:120); fstu_stu_step_lds returns T(2E). */
+int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                           void* y, int ldy, int B, int S, int d, int t, int dtype, void* stream);
+
 /* The same step for the single-branch filters of use_hankel_L=True (flash_stu/utils/stu_utils.py:22-25,229-246:
  * one convolution over ALL lags, no sign branch): ce (S,d) is fitted to the even lags and weighs the bank of parity
  * t&1 after its advance, co (S,d) is fitted to the odd lags and weighs the other bank (lag 2m+1 reaches position
@@ -144,18 +153,18 @@ int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, const float* a,
 
 /* Input projection and recurrence step in one launch (bf16, K % 256 == 0):
  *   xp[b,c] = T( h[b,:] . Mt[c,:] )  with Mt = M_inputs^T (d,K) row-major, then the step of
- * fstu_stu_step_lds on xp.  xp_out (B,d) receives xp when not NULL.
+ * fstu_stu_step_lds_pair on xp (co != NULL) or of fstu_stu_step_lds (co == NULL).  xp_out (B,d) receives xp when not NULL.
  * Replaces `x @ M_inputs` + the convolution at flash_stu/modules/stu.py:87-98,120 for one token. */
 int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                         void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream);
+                         const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream);
 
 /* The same launch with the residual update and the RMSNorm of its input as the prologue
  * (flash_stu/layers/stu_layer.py:78-82 after the previous layer's :93-97): x' = T(x_in + T(sum of nslices <= 4 fp32
  * (B,K) slices)) goes to x_out (not x_in itself), h = rmsnorm(x') * norm_w feeds the projection.  K % 256 == 0,
  * B*K/8 <= 1024. */
 int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                             const void* Mt, float* state, const float* a, const float* ce, void* y, int ldy, int B, int S,
-                             int d, int K, int t, void* stream);
+                             const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
+                             int B, int S, int d, int K, int t, void* stream);
 
 /* The step of fstu_stu_step_lds applied to T consecutive positions t_start .. t_start+T-1 in one launch (scan form
  * of the prefill: no FFT, no history buffer): y[b,t,c] for every position and the state after the last one.
@@ -464,7 +473,8 @@ typedef struct {
   const void* filt;         /* (L,d) phi_proj, model dtype       (history mode) */
   void* hist;               /* (B,hist_cap,d) x_proj history      (history mode) */
   const float* lds_a;       /* (S)                                (lds mode) */
-  const float* lds_ce;      /* (S,d)                              (lds mode) */
+  const float* lds_ce;      /* (S,d) even-lag output weights      (lds mode) */
+  const float* lds_co;      /* (S,d) odd-lag output weights on the other bank, or NULL: y = T(2E) (lds mode) */
   float* lds_state;         /* (B,2,S,d)                          (lds mode) */
   /* attention */
   const void* w_qkv;        /* (3d,d) */

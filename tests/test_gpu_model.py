@@ -26,7 +26,7 @@ def make_pair(seed=0, init="healthy", **kw):
                          use_attn=ocfg.use_attn, softcap=ocfg.softcap, torch_dtype=dt, **extra)
     torch.manual_seed(1234)
     model = FlashSTU(cfg)
-    model.load_oracle_weights(w)
+    model.load_named_tensors(w)
     return ocfg, w, model.cuda().eval()
 
 
@@ -185,41 +185,55 @@ class _wide_accumulation:
         O.F.linear = self.saved
 
 
-@pytest.mark.parametrize("mode", ["history", "lds"])
-@pytest.mark.parametrize("init", ["healthy", "reference"])
-def test_c2_dims_bf16_teacher_forced(mode, init):
-    """BASELINE config 2's architecture (768-d, 12 layers, 12 heads, window 512,
-    L=2048) at a prompt/batch the CPU oracle finishes in seconds."""
-    ocfg, w, model = make_pair(seed=1, init=init, dtype=torch.bfloat16, mlp_scale=4, n_embd=768, n_layers=12,
-                               n_heads=12, window_size=512, num_eigh=24, seq_len=2048, vocab_size=50257,
-                               stu_decode_mode=mode)
-    B, P, N = 4, 40, 88          # 352 scored tokens
-    ids = prompt(B, P, ocfg.vocab_size, 3)
+def _bf16_parity(ocfg, w, model, ids, N, label):
+    """Greedy decode on the device, the oracle teacher-forced on the device's tokens.  Returns (worst relative
+    logit error, strict agreement of the greedy ids, the comparison's own noise floor, scored picks).  The floor
+    is the oracle against itself with float64 accumulation inside every linear (same rounding points, another
+    summation order): two faithful evaluations of one bf16 specification do not pick the same token every time."""
+    B, P = ids.shape
     got, got_logits = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
     got, got_logits = got.cpu(), got_logits.float().cpu()
     ref_logits = _teacher_forced(w, ocfg, got, P).float()
     assert ref_logits.shape == got_logits.shape
-    err = (got_logits - ref_logits).abs().amax(-1) / ref_logits.abs().amax(-1)
-    assert float(err.max()) <= 2e-2, float(err.max())
-    agree = (ref_logits.argmax(-1) == got[:, P:]).float().mean()
-    # random-init logits are near-ties in bf16: count a device pick as agreeing when the
-    # oracle scores it within one bf16 ulp of its own maximum
-    picked = ref_logits.gather(-1, got[:, P:, None])[..., 0]
-    near = (picked >= ref_logits.amax(-1) * (1 - 2.0 ** -7) - 1e-30).float().mean()
-    print(f"mode={mode} init={init}: max rel logit err {float(err.max()):.2e}, strict agreement {float(agree):.3f}, "
-          f"within-one-ulp agreement {float(near):.3f}")
-    assert float(near) >= 0.99
-    assert float(agree) >= 0.9
-    if mode == "history" and init == "healthy":
-        # noise floor of the comparison: the oracle against itself with float64 accumulation in every linear.
-        # Two faithful evaluations of the same bf16 specification do not pick the same token every time either.
-        with _wide_accumulation():
-            ref2 = _teacher_forced(w, ocfg, got, P).float()
-        self_agree = (ref2.argmax(-1) == ref_logits.argmax(-1)).float().mean()
-        self_err = ((ref2 - ref_logits).abs().amax(-1) / ref_logits.abs().amax(-1)).max()
-        print(f"oracle vs oracle(float64 accumulation): strict agreement {float(self_agree):.3f}, "
-              f"max rel logit difference {float(self_err):.2e}")
-        assert float(agree) >= float(self_agree) - 0.03
+    err = float(((got_logits - ref_logits).abs().amax(-1) / ref_logits.abs().amax(-1)).max())
+    agree = float((ref_logits.argmax(-1) == got[:, P:]).float().mean())
+    with _wide_accumulation():
+        ref2 = _teacher_forced(w, ocfg, got, P).float()
+    floor = float((ref2.argmax(-1) == ref_logits.argmax(-1)).float().mean())
+    floor_err = float(((ref2 - ref_logits).abs().amax(-1) / ref_logits.abs().amax(-1)).max())
+    print(f"{label}: {B * N} picks, max rel logit err {err:.2e} (oracle vs oracle(float64 accumulation) {floor_err:.2e}), "
+          f"strict greedy agreement {agree:.4f}, floor {floor:.4f}")
+    return err, agree, floor, B * N
+
+
+@pytest.mark.parametrize("mode", ["history", "lds"])
+@pytest.mark.parametrize("init", ["healthy", "reference"])
+def test_c2_dims_bf16_teacher_forced(mode, init):
+    """BASELINE config 2's architecture (768-d, 12 layers, 12 heads, window 512, L=2048) at a prompt/batch the CPU
+    oracle finishes in seconds, 2000 scored picks per cell.  Tolerances from BASELINE.json: logits within 2e-2
+    relative; greedy ids agree on >= 99 % of the tokens wherever the specification agrees with itself that often, and
+    never fall more than one point below the comparison's own noise floor."""
+    ocfg, w, model = make_pair(seed=1, init=init, dtype=torch.bfloat16, mlp_scale=4, n_embd=768, n_layers=12,
+                               n_heads=12, window_size=512, num_eigh=24, seq_len=2048, vocab_size=50257,
+                               stu_decode_mode=mode)
+    B, P, N = 8, 40, 250
+    err, agree, floor, picks = _bf16_parity(ocfg, w, model, prompt(B, P, ocfg.vocab_size, 3), N, f"mode={mode} init={init}")
+    assert picks >= 2000
+    assert err <= 2e-2, err
+    assert agree >= min(0.99, floor - 0.01), (agree, floor)
+
+
+def test_c2_benched_config_bf16_against_the_oracle_past_the_ring_wrap():
+    """The configuration bench.py runs (mlp_scale 12, recurrence STU state, window 512) with a prompt longer than the
+    ring (513 slots): the decode steps read a wrapped ring and a recurrence state older than the window, and their
+    logits are compared with the oracle's full-sequence forward (teacher-forced on the device's tokens)."""
+    ocfg, w, model = make_pair(seed=1, init="reference", dtype=torch.bfloat16, mlp_scale=12, n_embd=768, n_layers=12,
+                               n_heads=12, window_size=512, num_eigh=24, seq_len=2048, vocab_size=50257,
+                               stu_decode_mode="lds")
+    B, P, N = 2, 530, 32
+    err, agree, floor, picks = _bf16_parity(ocfg, w, model, prompt(B, P, ocfg.vocab_size, 5), N, "benched config, lds")
+    assert err <= 2e-2, err
+    assert agree >= min(0.99, floor - 0.01) - 1.0 / picks, (agree, floor)      # 64 picks: one token is 1.6 points
 
 
 def test_c2_full_size_decode_against_full_sequence_recompute():

@@ -419,6 +419,7 @@ def test_stu_inproj_step_equals_projection_then_step(hip):
     Mt = dev((torch.randn(d, d, generator=g) / math.sqrt(d)).bfloat16())
     st1 = dev(torch.randn(B, 2, S, d, generator=g))
     st2 = st1.clone()
+    co = dev((torch.randn(S, d, generator=g) / S).float())
     for t in range(5):
         h = dev(torch.randn(B, d, generator=g).bfloat16())
         xp = hip.linear_decode(h, Mt)
@@ -428,6 +429,10 @@ def test_stu_inproj_step_equals_projection_then_step(hip):
         assert torch.equal(xp2, xp)
         check(y, y_ref, torch.bfloat16, frac=0.02)
         assert float((st1 - st2).abs().max()) == 0.0
+        # with odd-lag weights: the step of stu_step_lds(pair=True)
+        y_pair_ref = hip.stu_step_lds(st1.clone(), xp, a, ce, t, co=co, pair=True)
+        y_pair = hip.stu_inproj_step(h, Mt, st2.clone(), a, ce, t, co=co)
+        check(y_pair, y_pair_ref, torch.bfloat16, frac=0.03, atol=2.0 ** -8 * float(y_pair_ref.float().abs().max()))
 
 
 @pytest.mark.parametrize("B,ns", [(8, 4), (3, 2), (1, 1)])
@@ -470,6 +475,44 @@ def test_stu_step_lds_tracks_the_convolution(hip, L):
         y = hip.stu_step_lds(state, dev(xp[:, t].contiguous()), ad, ced, t)
         worst = max(worst, float((y.cpu() - ref[:, t]).abs().max()))
     assert worst < 1e-3 * float(ref.abs().max()), (worst, float(ref.abs().max()), err)
+
+
+def test_stu_step_lds_pair_keeps_the_reference_rounding_points(hip):
+    """bf16, two sign branches: the reference rounds plus = E+O and minus = E-O separately before adding them
+    (stu_utils.py:226-228, stu.py:120).  The pair step forms E on the bank of the token's parity and O on the other
+    bank and rounds the same way: the kernel equals a float64 evaluation of that recurrence with those roundings, and
+    its outputs differ from the oracle's convolution on far fewer elements than T(2E), which drops O."""
+    dtype = torch.bfloat16
+    B, d, L, K, S = 2, 128, 1024, 24, 64
+    T = 600
+    xp, filt, ref, _ = _stu_setup(dtype, B, T, d, L, K, 9)
+    a, ce, _ = _fit_lds(filt[0::2], S)
+    a2, co, _ = _fit_lds(filt[1::2], S)
+    assert torch.equal(a, a2)
+    st_pair = torch.zeros(B, 2, S, d, device="cuda")
+    st_2e = torch.zeros(B, 2, S, d, device="cuda")
+    h64 = torch.zeros(B, 2, S, d, dtype=torch.float64)
+    ad, ced, cod = dev(a), dev(ce), dev(co)
+    bad_pair = bad_2e = bad_model = total = 0
+    rb = lambda v: v.float().to(dtype).double()
+    for t in range(T):
+        xt = dev(xp[:, t].contiguous())
+        y = hip.stu_step_lds(st_pair, xt, ad, ced, t, co=cod, pair=True).cpu()
+        y2 = hip.stu_step_lds(st_2e, xt, ad, ced, t).cpu()
+        p = t & 1
+        h64[:, p] = a.double()[None, :, None] * h64[:, p] + xp[:, t].double()[:, None, :]
+        E = (ce.double()[None] * h64[:, p]).sum(1)
+        Od = (co.double()[None] * h64[:, p ^ 1]).sum(1)
+        model = rb(rb(E + Od) + rb(E - Od))
+        bad_model += int((y.double() != model).sum())
+        if t >= 64:
+            bad_pair += int((y != ref[:, t]).sum())
+            bad_2e += int((y2 != ref[:, t]).sum())
+            total += y.numel()
+    assert torch.equal(st_pair, st_2e)
+    assert bad_model <= 0.03 * T * B * d, bad_model           # fp32 vs float64 accumulation flips a rounding now and then
+    print(f"elements differing from the oracle: pair {bad_pair / total:.3f}, T(2E) {bad_2e / total:.3f}")
+    assert bad_pair <= 0.22 * total and bad_pair < 0.6 * bad_2e, (bad_pair / total, bad_2e / total)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

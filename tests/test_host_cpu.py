@@ -146,4 +146,61 @@ def test_product_never_imports_the_oracle():
         for f in files:
             if f.endswith((".py", ".hip", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
-                assert "oracle" not in src.replace("load_oracle_weights", ""), f"{f} mentions the oracle"
+                assert "oracle" not in src.replace("load_named_tensors", ""), f"{f} mentions the oracle"
+
+
+@pytest.mark.parametrize("L,K", [(128, 8), (2048, 24), (8192, 24)])
+def test_lds_fit_reproduces_hankel_filters_and_rejects_what_it_cannot_fit(L, K):
+    """The recurrence that replaces the STU filter in bf16 decode must reproduce it: fit error of the even- and the
+    odd-lag halves below one bf16 step of the filters' largest taps, for random and for structured (all-ones,
+    single-filter) M_filters; a filter that is no sum of decaying exponentials is refused."""
+    from flash_stu.utils.lds_fit import check_lds_fit, fit_even_lag_lds
+    phi = torch.tensor(O.get_spectral_filters_f64(L, K)).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(L)
+    d = 16
+    cases = {"random": torch.randn(K, d, generator=g) / K ** 0.5, "ones": torch.ones(K, d) / K,
+             "one filter": torch.eye(K)[:, :d] if K >= d else torch.eye(K).repeat(1, 2)[:, :d]}
+    for name, Mf in cases.items():
+        f = torch.matmul(phi, Mf.to(torch.bfloat16))
+        refused = False
+        for half in (f[0::2], f[1::2]):
+            a, c, err = fit_even_lag_lds(half, 64, per_channel=True)
+            assert a.shape == (64,) and c.shape == (64, d) and err.shape == (d,)
+            try:
+                check_lds_fit(err, f[0::2])
+            except ValueError as e:
+                assert "history" in str(e)
+                refused = True
+        # mixtures led by the large eigenvectors fit; the 16 smallest, oscillating eigenvectors on channels of their
+        # own ("one filter": the first columns of phi) do not once the filters are long
+        assert refused == (name == "one filter" and L >= 2048), (name, L, refused)
+    noise = torch.randn(L // 2, d, generator=g)
+    _, _, err = fit_even_lag_lds(noise, 64, per_channel=True)
+    with pytest.raises(ValueError, match="history"):
+        check_lds_fit(err, noise)
+
+
+def test_generate_beyond_seq_len_leaves_the_stateful_paths():
+    """prompt + new tokens > seq_len: the decode engine refuses (its state has no counterpart in the reference's
+    truncated re-run, model.py:250-255) and FlashSTU.generate takes the recompute loop instead of the engine."""
+    from flash_stu import FlashSTU, FlashSTUConfig
+    from flash_stu.engine import DecodeEngine
+    cfg = FlashSTUConfig(n_embd=64, n_heads=2, n_layers=2, seq_len=32, window_size=8, vocab_size=50, num_eigh=4,
+                         torch_dtype=torch.bfloat16)
+    model = FlashSTU(cfg)
+    eng = DecodeEngine(model)
+    with pytest.raises(Exception, match="seq_len|GPU"):
+        eng.generate(torch.zeros(1, 30, dtype=torch.int64), 8)
+    import inspect
+    src = inspect.getsource(FlashSTU.generate)
+    assert "max_length <= self.config.seq_len and DecodeEngine.supports" in src
+
+
+def test_lm_head_follows_config_bias():
+    """model.py:100-102: lm_head is built with bias=config.bias, so a bias=True checkpoint carries lm_head.bias."""
+    from flash_stu import FlashSTU, FlashSTUConfig
+    kw = dict(n_embd=64, n_heads=2, n_layers=2, seq_len=32, window_size=8, vocab_size=50, num_eigh=4)
+    assert FlashSTU(FlashSTUConfig(bias=False, **kw)).lm_head.bias is None
+    m = FlashSTU(FlashSTUConfig(bias=True, **kw))
+    assert m.lm_head.bias is not None and "lm_head.bias" in m.state_dict()
+    assert float(m.lm_head.bias.abs().max()) == 0.0
