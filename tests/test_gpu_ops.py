@@ -7,6 +7,8 @@ rounded values except where a different fp32 summation order flips a rounding:
 at most one bf16 ulp (2^-7 relative) on a small fraction of elements."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -615,27 +617,90 @@ def test_head_with_fused_greedy_pick(hip, dtype, temperature):
     assert bool((ws == 0).all()) and bool((toks[:, [0, 2]] == -7).all())
 
 
+def _nucleus_fp32(logits_bf16, temperature, top_k, top_p):
+    """The kernel's own top-p rule restated in numpy (fstu_sample): transformed logits rounded to bf16; survivors
+    of top-k; fp32 exponentials relative to the row maximum, summed in float64; descending value order with ties by
+    lower index; a token is kept iff the probability mass ranked before it is <= top_p.  Returns the filtered
+    logits (fp32, -inf outside the nucleus) and the set of boundary tokens whose mass-before is within 1e-6 of top_p
+    (their membership may depend on the last bit of an exponential)."""
+    l = (logits_bf16.float() / temperature).to(torch.bfloat16).float().clamp(-1e4, 1e4).to(torch.bfloat16).float()
+    B, V = l.shape
+    out = torch.full_like(l, float("-inf"))
+    slack = []
+    for b in range(B):
+        row = l[b].numpy()
+        alive = np.ones(V, bool)
+        if top_k:
+            kth = np.sort(row)[::-1][top_k - 1]
+            alive = row >= kth
+        e = np.exp((row - row.max()).astype(np.float32)).astype(np.float64) * alive
+        order = np.lexsort((np.arange(V), -row))            # value descending, index ascending inside ties
+        order = order[alive[order]]
+        before = (np.cumsum(e[order]) - e[order]) / e.sum()
+        keep = before <= top_p
+        kept = order[keep]
+        out[b, kept] = torch.from_numpy(row[kept])
+        slack.append(set(order[np.abs(before - top_p) < 1e-6].tolist()))
+    return out, slack
+
+
+@pytest.mark.parametrize("V", [3001, 50257])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, None, 0.7), (0.8, None, 0.9), (1.0, 40, 0.7), (1.3, 200, 0.9)])
+def test_sample_top_p_bf16_nucleus(hip, V, temperature, top_k, top_p):
+    """bf16 rows through the two-pass radix selects and the LDS logits cache of the sampler: every draw lies in the
+    nucleus of the kernel's rule (fp32 exponentials, float64 sums over the bf16 transformed logits) and equals the
+    oracle's inverse-CDF pick from the counter stream over that nucleus.  Row 0 carries a plateau of tied bf16 values
+    that the boundary cuts through (tie ranks in index order)."""
+    g = gen(31 + V)
+    B = 4
+    logits = (2.5 * torch.randn(B, V, generator=g)).to(torch.bfloat16)
+    big = logits[0].float().topk(3)[0][-1]
+    tied = torch.randperm(V, generator=g)[:300]
+    logits[0, tied] = big.to(torch.bfloat16)                 # 300 tokens tied near the top of row 0
+    ld = dev(logits)
+    filt, slack = _nucleus_fp32(logits, temperature, top_k, top_p)
+    sizes = torch.isfinite(filt).sum(-1)
+    assert int(sizes.min()) >= 1 and int(sizes.max()) < V
+    if not top_k:
+        assert 3 < int(sizes[0]) < 303 + 40, int(sizes[0])   # the boundary lies inside the plateau of row 0
+    agree = total = 0
+    for step in range(40):
+        out = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample(ld, out, temperature, top_k, top_p, True, seed=91, step=step)
+        got = out.cpu()
+        ref = O.sample_from_logits(filt, 91, step)[:, 0]
+        for b in range(B):
+            inside = bool(torch.isfinite(filt[b, got[b]])) or int(got[b]) in slack[b]
+            assert inside, f"row {b} step {step}: drew token {int(got[b])} outside the nucleus"
+        agree += int((got == ref).sum())
+        total += B
+    assert agree >= total - 1, (agree, total)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 40, None), (1.0, None, None), (1.0, 5, 0.7),
                                                       (1.3, None, 0.9), (0.7, 1, None)])
 def test_sample_draws_match_oracle(hip, dtype, temperature, top_k, top_p):
-    """Same counter-based stream, same filters: ids equal the oracle's draw.
-    (fp32 only for top-p: the oracle restates the reference's model-dtype
-    softmax/cumsum, which the kernel evaluates in fp32.)"""
-    if top_p is not None and dtype == torch.bfloat16:
-        pytest.skip("top-p cumulative sums in bf16 are not reproduced bit-wise; covered in fp32")
+    """Same counter-based stream, same filters: ids equal the oracle's draw.  With top-p in bf16 the reference takes
+    softmax and cumsum in the model dtype while the kernel evaluates its nucleus in fp32/float64 (documented in the
+    header): there the expected pick is the oracle's draw over the kernel's own nucleus rule (_nucleus_fp32)."""
     g = gen(12)
     B, V = 4, 3001
     logits = (2.5 * torch.randn(B, V, generator=g)).to(dtype)
     ld = dev(logits)
+    own_rule = top_p is not None and dtype == torch.bfloat16
+    if own_rule:
+        filt = _nucleus_fp32(logits, temperature, top_k, top_p)[0]
+    else:
+        filt = O.filter_logits(logits.float() if dtype == torch.float32 else logits, temperature, top_k, top_p)
     agree = total = 0
     for step in range(40):
         out = torch.empty(B, dtype=torch.int64, device="cuda")
         hip.sample(ld, out, temperature, top_k, top_p, True, seed=77, step=step)
-        ref = O.next_token(logits, temperature, top_k, top_p, True, seed=77, step=step)[:, 0]
+        ref = (O.sample_from_logits(filt, 77, step) if own_rule else
+               O.next_token(logits, temperature, top_k, top_p, True, seed=77, step=step))[:, 0]
         agree += int((out.cpu() == ref).sum())
         total += B
-        filt = O.filter_logits(logits.float() if dtype == torch.float32 else logits, temperature, top_k, top_p)
         assert bool(torch.isfinite(filt.float().gather(1, out.cpu()[:, None])).all()), "drew a filtered token"
     assert agree >= total - 1, (agree, total)
 
