@@ -69,6 +69,11 @@ int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* lo
                                 float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                                 void* stream);
 int fstu_gemv_packed_dyn(const fstu_gemv_args* a, int* dyn, int advance, void* stream);
+// the whole step as one persistent launch: tokens / tok_out are the column-0 bases of the input and output views, the
+// step reads column `pos` (dyn[0] when dyn is given) of the first and writes the same column of the second
+bool fstu_step_mega_ok(const fstu_model_desc* m);
+int fstu_step_mega_launch(const fstu_model_desc* m, int64_t* tokens, int64_t* tok_out, int64_t tok_stride, int pos,
+                          float temperature, int greedy, int* dyn, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -294,6 +294,19 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                    "fstu_decode_step: layer %d has no attention state", l);
     }
   }
+  if (fstu_step_mega_ok(m)) {
+    // the whole step as one persistent launch; sampling (when asked for) reads the logits it leaves
+    const int greedy = do_sample ? 0 : 1;
+    int64_t* in0 = const_cast<int64_t*>(tok_in) - (dyn ? 0 : pos);
+    int64_t* out0 = tok_out - (dyn ? 0 : pos);
+    TIMED(PC_GLU, fstu_step_mega_launch(m, in0, out0, tok_stride, pos, temperature, greedy, dyn, stream));
+    if (!greedy) {
+      TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, m->B, m->V, temperature, top_k, top_p, do_sample, seed, step,
+                                       m->row0, dyn, m->dtype, stream));
+      if (dyn) STEP(fstu_advance_dyn(dyn, stream));
+    }
+    return FSTU_OK;
+  }
   if (fused_available(m))
     return decode_step_fused(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
   // x = embedding rows, h = norm(x) with the first layer's norm weight

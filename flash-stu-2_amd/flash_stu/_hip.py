@@ -75,6 +75,9 @@ SIGNATURES = {
     "fstu_mlp_block_trace": [_vp],
     "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
     "fstu_mlp_block": [_vp] * 12 + [_i, _i, _i, _f, _vp],
+    "fstu_step_mega_ws_bytes": [_vp],
+    "fstu_step_mega_prepare": [_vp, _vp, _vp],
+    "fstu_step_mega_status": [_vp, _vp],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _i, _i, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
@@ -112,6 +115,7 @@ def load(path: Optional[str] = None):
     lib.fstu_packed_elems.restype = ctypes.c_int64
     lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
     lib.fstu_mlp_block_sync_bytes.restype = ctypes.c_size_t
+    lib.fstu_step_mega_ws_bytes.restype = ctypes.c_size_t
     if path is None:
         _lib = lib
     return lib

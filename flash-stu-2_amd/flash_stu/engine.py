@@ -43,7 +43,8 @@ class ModelDesc(ctypes.Structure):
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
                 ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
-                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i), ("merge_norm", _i), ("swa_fused", _i)]
+                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i), ("merge_norm", _i), ("swa_fused", _i),
+                ("mega_ws", _vp)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -313,6 +314,30 @@ class DecodeEngine:
             m.partial_fix = buf(m.ksplit_down * ((d + 15) // 16) * 256, dtype=torch.float32).data_ptr()
             m.counters = buf((d + 15) // 16, dtype=torch.int32).data_ptr()
         ch.arr, ch.desc = arr, m
+        ch.mega = None
+        if (dt == torch.bfloat16 and mode == "lds" and m.glu_packed and m.down_packed and not cfg.use_hankel_L
+                and os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") == "1"):
+            # opt-in: the whole step as one persistent launch (packed copies of every weight, one workspace for the
+            # tagged hand-over between the phases).  Correct and tested, but measured slower than the chain of launches
+            # (0.52 against 0.32 ms per step at 768-d, batch 8): a hand-over through memory costs a phase 3-5 us once
+            # the arrival skew of 256 polling workgroups is counted, as much as a kernel boundary
+            for i, layer in enumerate(model.layers):
+                if isinstance(layer, STULayer):
+                    arr[i].wp_m_inputs = self._pack(layer.stu.m_inputs_t()).data_ptr()
+                else:
+                    arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                    arr[i].wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
+            m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
+            nbytes = int(self.lib.fstu_step_mega_ws_bytes(ctypes.byref(m)))
+            if nbytes > 0:
+                ws = torch.zeros(nbytes // 8 + 32, dtype=torch.int64, device=dev)
+                keep(ws)
+                _hip._check(self.lib.fstu_step_mega_prepare(ctypes.byref(m), ws.data_ptr(), torch.cuda.current_stream().cuda_stream),
+                            "fstu_step_mega_prepare")
+                m.mega_ws = ws.data_ptr()
+                ch.mega = ws
+            else:
+                m.wp_emb = None
 
     # ------------------------------------------------------------------ eager step
     def step(self, tokens: torch.Tensor, pos: int, temperature, top_k, top_p, do_sample, seed, step_idx):
@@ -341,7 +366,9 @@ class DecodeEngine:
         advances pos on the device."""
         self.graph_end()
         self.graph_steps = int(steps_per_graph)
-        concurrent = os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1" and os.environ.get("FSTU_FUSED_MLP", "0") != "1"
+        # a persistent one-launch step needs every compute unit: row chunks then replay one after the other
+        concurrent = (os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1" and os.environ.get("FSTU_FUSED_MLP", "0") != "1"
+                      and not any(getattr(ch, "mega", None) is not None for ch in self.chunks))
         n_streams = len(self.chunks) if concurrent else 1
         self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
         stride = tokens.stride(0)
@@ -365,6 +392,16 @@ class DecodeEngine:
     def graph_step(self):
         for ch in self.chunks:
             _hip._check(self.lib.fstu_decode_graph_launch(ch.graph, ch.stream.cuda_stream), "fstu_decode_graph_launch")
+
+    def check_status(self):
+        """Raises when a wait inside the one-launch step timed out (synchronises the device)."""
+        for ch in self.chunks:
+            if getattr(ch, "mega", None) is not None:
+                err = ctypes.c_int(0)
+                _hip._check(self.lib.fstu_step_mega_status(ch.mega.data_ptr(), ctypes.byref(err)), "fstu_step_mega_status")
+                if err.value:
+                    raise _hip.FlashSTUHipError(f"one-launch decode step: a wait timed out in phase {err.value - 0x100} "
+                                                "(is another process using the GPU?)")
 
     def graph_sync(self):
         """Blocks until every chunk's replay stream has drained."""
