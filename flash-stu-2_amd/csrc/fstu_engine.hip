@@ -488,6 +488,7 @@ struct fstu_graph {
   WarmCtx* warm;
   long long next_pos;        // position the next launch will process first
   int nsteps;                // decode steps per launch
+  bool baked;                // the STU launches carry the parity of their position as an argument
 };
 
 static void warm_destroy(WarmCtx* w) {
@@ -524,10 +525,11 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
       }
     }
   }
-  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0, nsteps};
   // One graph per parity of the first position: the STU launches carry their parity as an argument.  A graph of an
-  // even number of steps always starts on the parity of pos0, so the other one is not captured.
-  const bool baked = m->stu_mode == 1 && warm == nullptr;
+  // even number of steps always starts on the parity of pos0, so the other one is not captured.  (The one-launch step
+  // reads the position on the device: one graph serves both parities.)
+  const bool baked = m->stu_mode == 1 && warm == nullptr && !fstu_step_mega_ok(m);
+  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0, nsteps, baked};
   for (int par = 0; par < 2; ++par) {
     if (!baked && par == 1) break;
     if (baked && (nsteps & 1) == 0 && par != (pos0 & 1)) continue;
@@ -562,6 +564,17 @@ extern "C" int fstu_decode_graph_launch(void* graph, void* stream) {
   hipError_t e = hipGraphLaunch(h->exec[par], (hipStream_t)stream);
   if (e != hipSuccess) { fstu_set_error("fstu_decode_graph_launch: %s", hipGetErrorString(e)); return (int)e; }
   h->next_pos += h->nsteps;
+  return FSTU_OK;
+}
+
+extern "C" int fstu_decode_graph_seek(void* graph, long long next_pos) {
+  FSTU_REQUIRE(graph && next_pos >= 0, FSTU_EARG, "fstu_decode_graph_seek: null graph or negative position");
+  fstu_graph* h = (fstu_graph*)graph;
+  // with the parity of the position baked into the STU launches, a graph of an even number of steps exists for one
+  // parity of its first position only
+  FSTU_REQUIRE(!h->baked || h->exec[next_pos & 1], FSTU_EARG,
+               "fstu_decode_graph_seek: this %d-step graph was captured for positions of the other parity", h->nsteps);
+  h->next_pos = next_pos;
   return FSTU_OK;
 }
 

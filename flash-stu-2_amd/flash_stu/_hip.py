@@ -81,12 +81,15 @@ SIGNATURES = {
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _i, _i, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
+    "fstu_decode_graph_seek": [_vp, ctypes.c_longlong],
     "fstu_decode_graph_destroy": [_vp],
     "fstu_set_warm_workgroups": [_i],
     "fstu_prof_begin": [_i, _i],
     "fstu_prof_end": [_vp, _vp],
     "fstu_prof_copy": [_vp, _vp, ctypes.c_size_t, _vp],
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
+    "fstu_lds_sequence_ws_floats": [_i, _i, _i],
+    "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -116,6 +119,7 @@ def load(path: Optional[str] = None):
     lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
     lib.fstu_mlp_block_sync_bytes.restype = ctypes.c_size_t
     lib.fstu_step_mega_ws_bytes.restype = ctypes.c_size_t
+    lib.fstu_lds_sequence_ws_floats.restype = ctypes.c_size_t
     if path is None:
         _lib = lib
     return lib
@@ -768,9 +772,12 @@ def gemv_packed(mode: int, Wp: torch.Tensor, N: int, K: int, out: torch.Tensor, 
 
 
 def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Dense LDS: h fp32 (Bt,S) carried in place over x (T,Bt,d_in) -> y (T,Bt,d_out)."""
-    _dev(h, x, A, Bm, Cm, out)
+              out: Optional[torch.Tensor] = None, transposed=None, ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Dense LDS: h fp32 (Bt,S) carried in place over x (T,Bt,d_in) -> y (T,Bt,d_out).  bf16 with MFMA-friendly shapes
+    runs on the matrix cores (fstu_lds_sequence); `transposed` = (Bm^T, Cm^T) contiguous copies and `ws` (fp32,
+    lds_sequence_ws_floats elements) may be passed by callers that step position by position, to keep the two
+    transposes and the allocation out of every call."""
+    _dev(h, x, A, Bm, Cm, out, ws)
     T, Bt, d_in = x.shape
     S = A.numel()
     d_out = Cm.shape[1]
@@ -778,6 +785,19 @@ def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tenso
     assert Bm.shape == (d_in, S) and Cm.shape == (S, d_out) and Bm.dtype == Cm.dtype == x.dtype
     if out is None:
         out = torch.empty(T, Bt, d_out, dtype=x.dtype, device=x.device)
+    if (x.dtype == torch.bfloat16 and T >= 1 and d_in % 32 == 0 and S % 32 == 0 and S <= 256 and d_out % 16 == 0
+            and x.is_contiguous() and out.is_contiguous()):
+        # blocks of 128 positions in parallel on the matrix cores (weights passed transposed)
+        lib = load()
+        need = int(lib.fstu_lds_sequence_ws_floats(T, Bt, S))
+        if ws is None:
+            ws = torch.empty(need, dtype=torch.float32, device=x.device)
+        assert ws.dtype == torch.float32 and ws.numel() >= need and ws.is_contiguous()
+        bmt, cmt = transposed if transposed is not None else (Bm.t().contiguous(), Cm.t().contiguous())
+        assert bmt.shape == (S, d_in) and cmt.shape == (d_out, S) and bmt.is_contiguous() and cmt.is_contiguous()
+        _check(lib.fstu_lds_sequence(_p(h), _p(x), _p(A), _p(bmt), _p(cmt), _p(out), _p(ws), T, Bt, d_in, S, d_out, _stream()),
+               "fstu_lds_sequence")
+        return out
     _check(load().fstu_lds_steps(_p(h), _p(x), _p(A), _p(Bm), _p(Cm), _p(out), T, Bt, d_in, S, d_out, _dt(x), _stream()),
            "fstu_lds_steps")
     return out

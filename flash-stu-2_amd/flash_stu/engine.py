@@ -71,7 +71,7 @@ class _Chunk:
         self.arr = None
         self.desc: Optional[ModelDesc] = None
         self.logits: Optional[torch.Tensor] = None
-        self.graph = None
+        self.graphs = {}            # steps per graph -> handle
         self.dyn: Optional[torch.Tensor] = None
         self.stream = None
 
@@ -358,40 +358,53 @@ class DecodeEngine:
     GRAPH_STEPS = 8     # decode steps per graph launch in generate() (the launch of a graph costs several microseconds)
 
     def graph_begin(self, tokens: torch.Tensor, pos: int, step_idx: int, temperature, top_k, top_p, do_sample, seed,
-                    steps_per_graph: int = 1):
-        """Captures one decode step per row chunk as a HIP graph, each chunk on a side stream of its own: the chunks
-        are independent (own workspaces, state rows and device-side position), so their graphs run concurrently and
-        the second chunk finds the layer's weights, which the first has just streamed, in the Infinity Cache.  Each
+                    steps_per_graph: int = 1, keep: bool = False):
+        """Captures steps_per_graph decode steps per row chunk as a HIP graph, each chunk on a side stream of its own: the
+        chunks are independent (own workspaces, state rows and device-side position), so their graphs run concurrently
+        and the second chunk finds the layer's weights, which the first has just streamed, in the Infinity Cache.  Each
         graph_step() then runs steps_per_graph decode steps: each feeds tokens[:, pos], writes tokens[:, pos+1] and
-        advances pos on the device."""
-        self.graph_end()
-        self.graph_steps = int(steps_per_graph)
+        advances pos on the device.  `pos` is the position the first launch of THIS graph will process.  keep=True adds
+        the graph to those already captured (same tokens, sampling arguments and device-side counters) instead of
+        replacing them: a run can then mix long graphs with single-step ones (graph_step(n), graph_seek)."""
+        if not keep:
+            self.graph_end()
+        n = int(steps_per_graph)
+        self.graph_steps = n
         # a persistent one-launch step needs every compute unit: row chunks then replay one after the other
-        concurrent = (os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1" and os.environ.get("FSTU_FUSED_MLP", "0") != "1"
+        concurrent = (os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1"
                       and not any(getattr(ch, "mega", None) is not None for ch in self.chunks))
         n_streams = len(self.chunks) if concurrent else 1
-        self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
+        if not self._gstreams:
+            self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
         stride = tokens.stride(0)
         for ch in self.chunks:
-            ch.dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
+            if ch.dyn is None:
+                ch.dyn = torch.tensor([pos, step_idx], dtype=torch.int32, device=tokens.device)
         for st in self._gstreams:
             st.wait_stream(torch.cuda.current_stream())
         for i, ch in enumerate(self.chunks):
             handle = _vp()
-            ch.stream = self._gstreams[i % n_streams]
+            ch.stream = self._gstreams[i % len(self._gstreams)]
             rc = self.lib.fstu_decode_graph_create(ctypes.byref(ch.desc), tokens.data_ptr() + 8 * ch.b0 * stride, stride,
-                                                   ch.dyn.data_ptr(), int(pos), self.graph_steps, float(temperature),
+                                                   ch.dyn.data_ptr(), int(pos), n, float(temperature),
                                                    int(top_k) if top_k else 0,
                                                    float(top_p) if top_p else 0.0, int(bool(do_sample)),
                                                    int(seed) & ((1 << 64) - 1), ch.stream.cuda_stream,
                                                    ctypes.byref(handle))
             _hip._check(rc, "fstu_decode_graph_create")
-            ch.graph = handle
+            ch.graphs[n] = handle
         self._graph_tokens = tokens
 
-    def graph_step(self):
+    def graph_step(self, steps_per_graph: Optional[int] = None):
+        n = self.graph_steps if steps_per_graph is None else int(steps_per_graph)
         for ch in self.chunks:
-            _hip._check(self.lib.fstu_decode_graph_launch(ch.graph, ch.stream.cuda_stream), "fstu_decode_graph_launch")
+            _hip._check(self.lib.fstu_decode_graph_launch(ch.graphs[n], ch.stream.cuda_stream), "fstu_decode_graph_launch")
+
+    def graph_seek(self, steps_per_graph: int, pos: int):
+        """Tells the graph of that length which position its next launch will process (needed after graphs of another
+        length have advanced the device-side position in between)."""
+        for ch in self.chunks:
+            _hip._check(self.lib.fstu_decode_graph_seek(ch.graphs[int(steps_per_graph)], int(pos)), "fstu_decode_graph_seek")
 
     def check_status(self):
         """Raises when a wait inside the one-launch step timed out (synchronises the device)."""
@@ -409,14 +422,18 @@ class DecodeEngine:
             st.synchronize()
 
     def graph_end(self):
-        live = [ch for ch in self.chunks if ch.graph is not None]
+        live = [ch for ch in self.chunks if ch.graphs]
         if live:
             for st in self._gstreams:
                 torch.cuda.current_stream().wait_stream(st)
                 st.synchronize()
             for ch in live:
-                self.lib.fstu_decode_graph_destroy(ch.graph)
-                ch.graph = None
+                for handle in ch.graphs.values():
+                    self.lib.fstu_decode_graph_destroy(handle)
+                ch.graphs = {}
+        for ch in self.chunks:
+            ch.dyn = None
+        self._gstreams = []
 
     # ------------------------------------------------------------------
     @torch.no_grad()

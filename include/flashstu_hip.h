@@ -328,6 +328,15 @@ int fstu_head_argmax_static(const void* x, int ldx, const void* W, void* logits,
 int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, const void* Cm, void* y,
                    int T_steps, int Bt, int d_in, int S, int d_out, int dtype, void* stream);
 
+/* The same loop over a whole sequence on the matrix cores (bf16): blocks of 128 positions run in parallel (x_t @ Bm
+ * does not depend on the state), a short chain hands the state from block to block.  Weights are given TRANSPOSED:
+ * BmT (S,d_in), CmT (d_out,S).  ws: fstu_lds_sequence_ws_floats(T,Bt,S) floats, owned by the caller.  d_in % 32 == 0,
+ * S % 32 == 0, S <= 256, d_out % 16 == 0.  Same values as fstu_lds_steps up to the fp32 summation order; a sequence
+ * split at a multiple of 128 positions into two calls gives bit-identical outputs and states. */
+size_t fstu_lds_sequence_ws_floats(int T, int Bt, int S);
+int fstu_lds_sequence(float* h, const void* x, const float* A, const void* BmT, const void* CmT, void* y, float* ws,
+                      int T, int Bt, int d_in, int S, int d_out, void* stream);
+
 /* ---- decode GEMVs over packed weights ---------------------------------------
  * Packed layout of an (N,K) bf16 row-major weight, K % 32 == 0 (fstu_pack_rows):
  *   Wp[tile][kstep][lane][8],  tile = n/16, kstep = k/32, lane = 16*g + r,
@@ -585,6 +594,10 @@ int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t 
                              int nsteps, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
                              void* stream, void** graph_out);
 int fstu_decode_graph_launch(void* graph, void* stream);
+/* Tells the graph which position its next launch will process: needed when other graphs (of another length) over the
+ * same tokens and `dyn` have advanced the device-side position since this graph's last launch.  A graph of an even
+ * number of steps is captured for one parity of its first position only; seeking it to the other parity is rejected. */
+int fstu_decode_graph_seek(void* graph, long long next_pos);
 /* The captured graph carries a parallel branch whose kernels only read the MLP / head weights a layer is about
  * to need (cache warm-up; `n` workgroups per kernel; default 0 = no such branch, which measured faster).  Applies to graphs created
  * afterwards. */
