@@ -10,11 +10,8 @@ FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-u
          # packed fp32 instructions are kept out of the generated code
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # The first 16 kernel-argument dwords are preloaded into SGPRs by the command processor instead of being fetched by
-# the kernel's first instructions (one dependent fetch less at the start of every launch: 0.445 -> 0.442 ms per decode
-# step).  FSTU_KERNARG_PRELOAD=0 switches it off, another number changes the count.
-_preload = os.environ.get("FSTU_KERNARG_PRELOAD", "16")
-if _preload != "0":
-    FLAGS += ["-mllvm", "-amdgpu-kernarg-preload-count=" + _preload]
+# the kernel's first instructions (one dependent fetch less at the start of every launch).
+FLAGS += ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 def build(verbose: bool = True) -> str:

@@ -230,15 +230,6 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 // k,v (read from the qkv row) into ring slot pos % cap and attends to that key
 // straight from the qkv row, so the ring sweep covers the older keys only.
 #define SWA_U 4
-#ifdef FSTU_GLU_TRACE
-__device__ long long swa_trace_buf[96 * 8];
-#define SWA_STAMP(k) do { if (threadIdx.x == 0) swa_trace_buf[(blockIdx.y * gridDim.x + blockIdx.x) % 96 * 8 + (k)] = wall_clock64(); } while (0)
-extern "C" int fstu_swa_trace(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(swa_trace_buf), sizeof(long long) * 96 * 8);
-}
-#else
-#define SWA_STAMP(k) do { } while (0)
-#endif
 template <typename T, int HD, int NWAVES>
 __global__ void __launch_bounds__(NWAVES * 64)
 swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__ out, const float* __restrict__ slopes,
@@ -246,7 +237,6 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
                   int pos, int window, float softcap, int append) {
   constexpr int DPL = HD / 8;
   constexpr int NGRP = NWAVES * 8;
-  SWA_STAMP(0);
   if (dyn) pos = dyn[0];
   const int h = blockIdx.x, b = blockIdx.y;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -323,7 +313,6 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
     }
     M = Mn;
   }
-  SWA_STAMP(1);
   if (append && w == NWAVES - 1) {     // the new token's own key, taken by the last group of the last wave
     const float v = score(kself, pos);
     const float ss = self_grp ? v : -INFINITY;
@@ -352,7 +341,6 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
     if (lane == 0) { wm[w] = M; wl[w] = l; }
   }
   __syncthreads();
-  SWA_STAMP(3);
   if (threadIdx.x < HD) {
     float M = -INFINITY;
 #pragma unroll
@@ -371,7 +359,6 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
     kring[dst] = app_k;
     vring[dst] = app_v;
   }
-  SWA_STAMP(4);
 }
 
 static int check_swa(const char* name, int H, int hd, int window, const void* slopes) {
@@ -426,246 +413,6 @@ extern "C" int fstu_swa_append_decode(const void* qkv, void* kring, void* vring,
                                       int H, int hd, int cap, int pos, int window, float softcap, int dtype,
                                       void* stream) {
   return fstu_swa_decode_impl(qkv, kring, vring, out, slopes, B, H, hd, cap, pos, window, softcap, 1, nullptr, dtype, stream);
-}
-
-// ---------------------------------------------------------------- QKV projection + decode in one launch
-// One workgroup (16 waves) per (batch row, head), head dim 64, bf16.  The workgroup forms its own 192 rows of
-// qkv = h W_qkv^T (q, k, v of its head: 12 tiles of the packed weight, 4 K quarters -> 3 units per wave, every
-// weight fragment requested at the first instruction), so no qkv launch precedes it and nothing but the ring is
-// read from another workgroup's output.  h is either given (h_in) or formed here from the residual stream:
-// x' = T(x_in[b] + T(sum of <= 4 fp32 split-K slices)), h = T((x' * rstd) * norm_w) for the one row the workgroup
-// needs (reference: attention_layer.py:53-57 in front of attention.py:66-70); the head-0 workgroup of a row stores x'.
-// Measured at 768-d / 12 heads / batch 8: 10.8 us against 6.1 + 7.9 us for the two launches it replaces when timed
-// alone, but no gain inside the full step (0.362 vs 0.361 ms): the 8 workgroups of a head each pull the head's
-// 295 KB of weights through their own CU's 64 B/clk vector-memory path (2 us) where the stand-alone projection
-// spreads 3.5 MB over 192 workgroups.  The step uses it only when asked to (swa_fused in the model descriptor).
-typedef __bf16 swa_bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float swa_floatx4_t __attribute__((ext_vector_type(4)));
-#define SWAQ_KPU 6   // k steps (of 32) per unit: d / 32 / 4 <= 6, i.e. d <= 768
-
-__global__ void __launch_bounds__(1024)
-swa_qkv_decode_kernel(const bf16_t* __restrict__ x_in, const float* __restrict__ slices, bf16_t* __restrict__ x_out,
-                      const bf16_t* __restrict__ norm_w, const uint4* __restrict__ wp_qkv, const float* __restrict__ slopes,
-                      const int* __restrict__ dyn, const bf16_t* __restrict__ h_in, bf16_t* kring, bf16_t* vring,
-                      bf16_t* __restrict__ out, int nslices, int B, int H, int cap, int pos, int window, float softcap,
-                      float eps) {
-  constexpr int HD = 64, NWAVES = 16, DPL = 8, NGRP = NWAVES * 8;
-  typedef bf16_t T;
-  if (dyn) pos = dyn[0];
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int d = H * HD, nchunk = d >> 3, ksteps = d >> 5, kpu = ksteps >> 2;
-  __shared__ __align__(16) bf16_t hrow[1024];
-  __shared__ float sp[32];
-  __shared__ __align__(16) float redq[192][4];
-  __shared__ __align__(16) float qkv_s[192];   // this head's q, k, v of the new token, bf16-rounded values
-  __shared__ float sm[NGRP], sl[NGRP];
-  __shared__ float sacc[NGRP][HD];
-  __shared__ float wm[NWAVES], wl[NWAVES];
-  __shared__ float wacc[NWAVES][HD];
-
-  // ---- the row's operands, then every weight fragment of the workgroup.  Thread t < 4*nchunk takes slice t&3 of
-  // chunk t>>2 (whole waves: nchunk is a multiple of 32), so a thread holds 32 bytes of slices instead of 128
-  const int q = threadIdx.x >> 2, sl4 = threadIdx.x & 3;
-  uint4 xv = make_uint4(0, 0, 0, 0), nv = xv, sv0 = xv, sv1 = xv;
-  const bool prow = x_in ? (threadIdx.x < 4 * nchunk) : (threadIdx.x < nchunk);   // uniform per wave
-  if (prow) {
-    const size_t rowoff = (size_t)b * d;
-    if (x_in) {
-      xv = *(const uint4*)(x_in + rowoff + (size_t)q * 8);
-      nv = *(const uint4*)(norm_w + (size_t)q * 8);
-      if (sl4 < nslices) {
-        const float* sp4 = slices + ((size_t)sl4 * B + b) * d + (size_t)q * 8;
-        sv0 = *(const uint4*)sp4;
-        sv1 = *(const uint4*)(sp4 + 4);
-      }
-    } else {
-      xv = *(const uint4*)(h_in + rowoff + (size_t)threadIdx.x * 8);
-    }
-  }
-  const int kq = w & 3, tsub = w >> 2;
-  uint4 wq[3][SWAQ_KPU];
-  {
-    const fstu_rsrc_t rw = fstu_make_rsrc(wp_qkv, (size_t)(3 * d / 16) * ksteps * 1024);
-#pragma unroll
-    for (int u = 0; u < 3; ++u) {
-      const unsigned tile = (unsigned)((u * d + h * HD) >> 4) + (unsigned)tsub;
-#pragma unroll
-      for (int s = 0; s < SWAQ_KPU; ++s)
-        wq[u][s] = fstu_buf_load16(rw, s < kpu ? ((tile * (unsigned)ksteps + (unsigned)(kq * kpu + s)) * 64u + (unsigned)lane) * 16u
-                                               : FSTU_BUF_OOB);
-    }
-  }
-  // ---- x' and the row statistics
-  if (prow) {
-    if (x_in) {
-      // the four slices of a chunk sit in the four lanes of a quad: fetch the other three and add in slice order
-      auto quad = [](unsigned v, float& a0) {
-        const float f = __uint_as_float(v);
-        a0 = ((fstu_dpp<0x00>(f) + fstu_dpp<0x55>(f)) + fstu_dpp<0xAA>(f)) + fstu_dpp<0xFF>(f);
-      };
-      float dsum[8];
-      quad(sv0.x, dsum[0]); quad(sv0.y, dsum[1]); quad(sv0.z, dsum[2]); quad(sv0.w, dsum[3]);
-      quad(sv1.x, dsum[4]); quad(sv1.y, dsum[5]); quad(sv1.z, dsum[6]); quad(sv1.w, dsum[7]);
-      unsigned xw[4] = {xv.x, xv.y, xv.z, xv.w};
-      float ss = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const unsigned dp = pack2_bf16(dsum[2 * i], dsum[2 * i + 1]);
-        xw[i] = pack2_bf16(__uint_as_float(xw[i] << 16) + __uint_as_float(dp << 16),
-                           __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dp & 0xffff0000u));
-        const float lo = __uint_as_float(xw[i] << 16), hi = __uint_as_float(xw[i] & 0xffff0000u);
-        ss = fmaf(lo, lo, ss);
-        ss = fmaf(hi, hi, ss);
-      }
-      xv = make_uint4(xw[0], xw[1], xw[2], xw[3]);
-      ss = fstu_half_wave_sum(sl4 == 0 ? ss : 0.f);      // 8 chunks per 32 lanes
-      if ((lane & 31) == 0) sp[threadIdx.x >> 5] = ss;
-      if (h == 0 && x_out && sl4 == 0) *(uint4*)(x_out + (size_t)b * d + (size_t)q * 8) = xv;
-    } else {
-      *(uint4*)(hrow + threadIdx.x * 8) = xv;
-    }
-  }
-  __syncthreads();
-  if (x_in && prow && sl4 == 0) {
-    float ss = 0.f;
-    for (int i = 0; i < (nchunk >> 3); ++i) ss += sp[i];
-    const float rstd = rsqrtf(ss / (float)d + eps);
-    unsigned vw[4] = {xv.x, xv.y, xv.z, xv.w}, ww[4] = {nv.x, nv.y, nv.z, nv.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      vw[i] = pack2_bf16((__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
-                         (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
-    *(uint4*)(hrow + q * 8) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-  }
-  if (x_in) __syncthreads();
-  // ---- this wave's three units: A = weight fragment, B = the row in column 0 (lanes 0, 16, 32, 48)
-  {
-    const bool col0 = (lane & 15) == 0;
-    swa_floatx4_t acc[3];
-#pragma unroll
-    for (int u = 0; u < 3; ++u) acc[u] = swa_floatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < SWAQ_KPU; ++s) {
-      if (s < kpu) {
-        uint4 xb = make_uint4(0, 0, 0, 0);
-        if (col0) xb = *(const uint4*)(hrow + (kq * kpu + s) * 32 + (lane >> 4) * 8);
-#pragma unroll
-        for (int u = 0; u < 3; ++u)
-          acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(swa_bf16x8_t, wq[u][s]),
-                                                           __builtin_bit_cast(swa_bf16x8_t, xb), acc[u], 0, 0, 0);
-      }
-    }
-    if (col0) {
-#pragma unroll
-      for (int u = 0; u < 3; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) redq[u * 64 + tsub * 16 + (lane >> 4) * 4 + i][kq] = acc[u][i];
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x < 192) {
-    const float4 p = *(const float4*)redq[threadIdx.x];
-    qkv_s[threadIdx.x] = DT<T>::rnd(((p.x + p.y) + p.z) + p.w);
-  }
-  __syncthreads();
-  // ---- ring append and the sweep, as swa_decode_kernel with the new token's q, k, v taken from LDS
-  const int grp = lane >> 3, gl = lane & 7;
-  const int G = w * 8 + grp;
-  const size_t hbase = ((size_t)b * H + h) * cap * HD;
-  if (threadIdx.x < HD) {
-    const size_t dst = hbase + (size_t)(pos % cap) * HD + threadIdx.x;
-    kring[dst] = f32_to_bf16(qkv_s[HD + threadIdx.x]);
-    vring[dst] = f32_to_bf16(qkv_s[2 * HD + threadIdx.x]);
-  }
-  float qv[DPL];
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) qv[i] = qkv_s[gl * DPL + i];
-  const bool self_grp = (G == NGRP - 1);
-  Partial<DPL> P;
-  P.m = -INFINITY;
-  P.l = 0.f;
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) P.acc[i] = 0.f;
-  const int lo = max(0, pos - window);
-  const float scale = rsqrtf((float)HD), slope = slopes[h];
-  attend_keys<T, DPL, SWA_U, true>(P, kring + hbase + gl * DPL, vring + hbase + gl * DPL, HD, cap, lo, lo % cap, qv,
-                                   lo + G * SWA_U, pos, NGRP * SWA_U, pos, scale, softcap, slope);
-  if (self_grp) {
-    float kself[DPL], vself[DPL];
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) { kself[i] = qkv_s[HD + gl * DPL + i]; vself[i] = qkv_s[2 * HD + gl * DPL + i]; }
-    attend_one<DPL, true>(P, qv, kself, vself, pos, pos, scale, softcap, slope);
-  }
-  if (gl == 0) { sm[G] = P.m; sl[G] = P.l; }
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) sacc[G][gl * DPL + i] = P.acc[i];
-  __syncthreads();
-  {
-    const int i = lane;
-    float M = -INFINITY;
-#pragma unroll
-    for (int g = 0; g < 8; ++g) M = fmaxf(M, sm[w * 8 + g]);
-    float Lsum = 0.f, o = 0.f;
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      const float e = (sm[w * 8 + g] == -INFINITY) ? 0.f : __expf(sm[w * 8 + g] - M);
-      Lsum = fmaf(sl[w * 8 + g], e, Lsum);
-      o = fmaf(sacc[w * 8 + g][i], e, o);
-    }
-    wacc[w][i] = o;
-    if (i == 0) { wm[w] = M; wl[w] = Lsum; }
-  }
-  __syncthreads();
-  if (threadIdx.x < HD) {
-    float M = -INFINITY;
-#pragma unroll
-    for (int g = 0; g < NWAVES; ++g) M = fmaxf(M, wm[g]);
-    float Lsum = 0.f, o = 0.f;
-#pragma unroll
-    for (int g = 0; g < NWAVES; ++g) {
-      const float e = (wm[g] == -INFINITY) ? 0.f : __expf(wm[g] - M);
-      Lsum = fmaf(wl[g], e, Lsum);
-      o = fmaf(wacc[g][threadIdx.x], e, o);
-    }
-    DT<T>::st(out + (size_t)b * d + h * HD + threadIdx.x, o / Lsum);
-  }
-}
-
-// h_in (B,d) normalised rows, or (x_in, slices, nslices <= 4, x_out, norm_w, eps) to form them here; x_out must not
-// alias x_in.  Head dim 64, d % 256 == 0, d <= 768, bf16.
-int fstu_swa_qkv_decode_dyn(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
-                            const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
-                            const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
-                            const int* dyn, void* stream) {
-  int rc = check_kv("fstu_swa_qkv_decode", wp_qkv, kring, vring, B, H, hd, cap);
-  if (rc) return rc;
-  FSTU_REQUIRE(slopes && out, FSTU_ENULL, "fstu_swa_qkv_decode: null pointer");
-  FSTU_REQUIRE((h_in != nullptr) != (x_in != nullptr), FSTU_EARG, "fstu_swa_qkv_decode: give h_in or x_in, not both");
-  FSTU_REQUIRE(x_in == nullptr || (norm_w && x_out && x_out != x_in), FSTU_EARG,
-               "fstu_swa_qkv_decode: the norm prologue needs norm_w and an x_out that is not x_in");
-  FSTU_REQUIRE(nslices >= 0 && nslices <= 4 && (nslices == 0 || slices), FSTU_EARG, "fstu_swa_qkv_decode: nslices=%d", nslices);
-  const int d = H * hd;
-  FSTU_REQUIRE(hd == 64 && d % 256 == 0 && d <= 32 * 4 * SWAQ_KPU && B <= 65535, FSTU_ESHAPE,
-               "fstu_swa_qkv_decode: head dim %d / width %d not supported (head dim 64, width a multiple of 256 up to %d)", hd,
-               d, 32 * 4 * SWAQ_KPU);
-  FSTU_REQUIRE(pos >= 0 && window >= 0 && cap >= window + 1, FSTU_EARG, "fstu_swa_qkv_decode: pos=%d, ring capacity %d < window+1=%d", pos, cap, window + 1);
-  FSTU_REQUIRE(fstu_aligned(h_in, 16) && fstu_aligned(x_in, 16) && fstu_aligned(slices, 16) && fstu_aligned(x_out, 16) &&
-                   fstu_aligned(norm_w, 16) && fstu_aligned(wp_qkv, 16) && fstu_aligned(kring, 16) && fstu_aligned(vring, 16),
-               FSTU_EALIGN, "fstu_swa_qkv_decode: pointers must be 16-byte aligned");
-  hipLaunchKernelGGL(swa_qkv_decode_kernel, dim3(H, B), dim3(1024), 0, (hipStream_t)stream, (const bf16_t*)x_in, slices,
-                     (bf16_t*)x_out, (const bf16_t*)norm_w, (const uint4*)wp_qkv, slopes, dyn, (const bf16_t*)h_in,
-                     (bf16_t*)kring, (bf16_t*)vring, (bf16_t*)out, nslices, B, H, cap, pos, window, softcap, eps);
-  FSTU_CHECK_LAUNCH("fstu_swa_qkv_decode");
-  return FSTU_OK;
-}
-
-extern "C" int fstu_swa_qkv_decode(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
-                                   const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
-                                   const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
-                                   void* stream) {
-  return fstu_swa_qkv_decode_dyn(h_in, x_in, slices, nslices, x_out, norm_w, eps, wp_qkv, kring, vring, out, slopes, B, H, hd,
-                                 cap, pos, window, softcap, nullptr, stream);
 }
 
 // ---------------------------------------------------------------- prefill

@@ -38,10 +38,6 @@ int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream);
 int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, const float* slopes, int B, int H, int hd,
                          int cap, int pos, int window, float softcap, int append, const int* dyn, int dtype, void* stream);
-int fstu_swa_qkv_decode_dyn(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
-                            const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
-                            const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
-                            const int* dyn, void* stream);
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                          float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream);
@@ -62,13 +58,6 @@ int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* stat
 int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
                                  const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
                                  int B, int S, int d, int K, int t, const int* dyn, void* stream);
-int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
-                                  const float* ce, const float* co, void* y, int ldy, int B, int S, int d, int K, int t,
-                                  const int* dyn, void* stream);
-int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
-                                float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
-                                void* stream);
-int fstu_gemv_packed_dyn(const fstu_gemv_args* a, int* dyn, int advance, void* stream);
 // the whole step as one persistent launch: tokens / tok_out are the column-0 bases of the input and output views, the
 // step reads column `pos` (dyn[0] when dyn is given) of the first and writes the same column of the second
 bool fstu_step_mega_ok(const fstu_model_desc* m);

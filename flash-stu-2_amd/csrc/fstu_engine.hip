@@ -104,53 +104,6 @@ extern "C" int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* st
     if (rc__ != 0) return rc__;                                                                 \
   } while (0)
 
-// ---------------------------------------------------------------- cache warm-up branch (graph capture only)
-// While the latency-bound kernels of a sub-layer run, a few workgroups on a forked capture stream read the MLP
-// weights the layer needs next, so that the big GEMV kernels find them in the memory-side cache instead of
-// starting cold from HBM.  Pure reads; results are discarded.
-__global__ void __launch_bounds__(256)
-warm_ranges_kernel(const uint4* p0, size_t n0, const uint4* p1, size_t n1, const uint4* p2, size_t n2, unsigned* sink) {
-  unsigned acc = 0;
-  const size_t stride = (size_t)gridDim.x * 256, first = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const uint4* ps[3] = {p0, p1, p2};
-  const size_t ns[3] = {n0, n1, n2};
-#pragma unroll
-  for (int k = 0; k < 3; ++k) {
-    const uint4* p = ps[k];
-    size_t i = first;
-    for (; i + 3 * stride < ns[k]; i += 4 * stride) {
-      uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], e = p[i + 3 * stride];
-      acc ^= a.x ^ b.y ^ c.z ^ e.w;
-    }
-    for (; i < ns[k]; i += stride) acc ^= p[i].x;
-  }
-  if (acc == 0x9e3779b9u && sink) sink[0] = acc;   // keeps the loads alive; practically never taken
-}
-
-struct WarmCtx {
-  hipStream_t side = nullptr;
-  hipEvent_t fork[64], join[64];
-  int n = 0, cap = 0, wgs = 48;
-};
-static thread_local WarmCtx* g_warm = nullptr;
-
-static void warm_fork(hipStream_t main, const void* a, size_t abytes, const void* b, size_t bbytes, const void* c, size_t cbytes) {
-  WarmCtx* w = g_warm;
-  if (!w || w->n >= w->cap) return;
-  const int i = w->n++;
-  (void)hipEventRecord(w->fork[i], main);
-  (void)hipStreamWaitEvent(w->side, w->fork[i], 0);
-  hipLaunchKernelGGL(warm_ranges_kernel, dim3(w->wgs), dim3(256), 0, w->side, (const uint4*)a, abytes / 16, (const uint4*)b,
-                     bbytes / 16, (const uint4*)c, cbytes / 16, (unsigned*)nullptr);
-  (void)hipEventRecord(w->join[i], w->side);
-}
-
-static void warm_join_all(hipStream_t main) {
-  WarmCtx* w = g_warm;
-  if (!w) return;
-  for (int i = 0; i < w->n; ++i) (void)hipStreamWaitEvent(main, w->join[i], 0);
-}
-
 // recurrence step on m->xp: both sign branches rounded separately when the layer carries odd-lag weights
 static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, void* stream) {
   if (L.lds_co)
@@ -168,85 +121,6 @@ static int hist_nsplit(int nlags, int maxsplit) {
   return n;
 }
 
-// ---------------------------------------------------------------- fused bf16 step over packed weights
-// 58 launches: every residual add + RMSNorm runs as the prologue of the GEMV that consumes it, the down
-// projection reduces its K split in-kernel, the head picks the greedy token itself.
-static bool fused_available(const fstu_model_desc* m) {
-  if (m->dtype != FSTU_BF16 || m->stu_mode != 1 || !m->wp_emb || !m->x2 || !m->yd || !m->partial_fix || !m->counters || !m->best)
-    return false;
-  if (m->d % 128 != 0 || m->I % (128 * m->ksplit_down) != 0) return false;
-  if ((size_t)m->B * (m->d + 8) * 2 + 8192 > 64 * 1024) return false;
-  for (int l = 0; l < m->n_layers; ++l) {
-    const fstu_layer_desc& L = m->layers[l];
-    if (!L.wp_gate || !L.wp_up || !L.wp_down) return false;
-    if (L.kind == 0 ? !L.wp_m_inputs : (!L.wp_qkv || !L.wp_proj)) return false;
-  }
-  return true;
-}
-
-static int decode_step_fused(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
-                             int pos, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
-                             int step, int* dyn, void* stream) {
-  const int B = m->B, d = m->d, I = m->I, dt = m->dtype;
-  void* xb[2] = {m->x, m->x2};
-  int cur = 0;
-  TIMED(PC_NORM, fstu_embed_strided(tok_in, tok_stride, m->emb, xb[0], B, d, m->V, dt, stream, dyn));
-  const void* pending = nullptr;   // output of the previous sub-layer, not yet added to the residual stream
-  auto pro = [&](fstu_gemv_args& g, const void* norm_w) {
-    g.res_in = xb[cur];
-    g.delta = pending;
-    g.res_out = pending ? xb[cur ^ 1] : nullptr;
-    g.norm_w = norm_w;
-    g.eps = m->eps;
-    if (pending) cur ^= 1;
-    pending = nullptr;
-  };
-  for (int l = 0; l < m->n_layers; ++l) {
-    const fstu_layer_desc& L = m->layers[l];
-    if (L.kind == 0) {
-      fstu_gemv_args g = {};
-      g.mode = 0; g.rows = B; g.N = d; g.K = d; g.Wp = L.wp_m_inputs; g.y = m->xp; g.ldy = d;
-      pro(g, L.norm1_w);
-      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&g, dyn, 0, stream));
-      TIMED(PC_STU, stu_step(L, m, pos, dyn, stream));
-    } else {
-      fstu_gemv_args g = {};
-      g.mode = 0; g.rows = B; g.N = 3 * d; g.K = d; g.Wp = L.wp_qkv; g.y = m->qkv; g.ldy = 3 * d;
-      pro(g, L.norm1_w);
-      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&g, dyn, 0, stream));
-      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
-                                         m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
-      fstu_gemv_args p = {};
-      p.mode = 0; p.rows = B; p.N = d; p.K = d; p.Wp = L.wp_proj; p.x = m->attn; p.ldx = d; p.y = m->y; p.ldy = d;
-      TIMED(PC_PROJ, fstu_gemv_packed_dyn(&p, dyn, 0, stream));
-    }
-    pending = m->y;
-    fstu_gemv_args u = {};
-    u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
-    pro(u, L.mlp_norm_w);
-    TIMED(PC_GLU, fstu_gemv_packed_dyn(&u, dyn, 0, stream));
-    fstu_gemv_args dn = {};
-    dn.mode = 2; dn.rows = B; dn.N = d; dn.K = I; dn.Wp = L.wp_down; dn.x = m->act; dn.ldx = I; dn.y = m->yd; dn.ldy = d;
-    dn.ksplit = m->ksplit_down; dn.partial_ws = m->partial_fix; dn.counters = m->counters;
-    TIMED(PC_DOWN, fstu_gemv_packed_dyn(&dn, dyn, 0, stream));
-    pending = m->yd;
-  }
-  fstu_gemv_args hd = {};
-  hd.rows = B; hd.N = m->V; hd.K = d; hd.Wp = m->wp_emb; hd.y = m->logits; hd.ldy = m->V;
-  if (!do_sample) {
-    hd.mode = 3; hd.temperature = temperature; hd.best_ws = m->best; hd.tok_out = tok_out; hd.tok_stride = tok_stride;
-    pro(hd, m->final_norm_w);
-    TIMED(PC_HEAD, fstu_gemv_packed_dyn(&hd, dyn, 1, stream));
-  } else {
-    hd.mode = 0;
-    pro(hd, m->final_norm_w);
-    TIMED(PC_HEAD, fstu_gemv_packed_dyn(&hd, dyn, 0, stream));
-    TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));
-    if (dyn) STEP(fstu_advance_dyn(dyn, stream));
-  }
-  return FSTU_OK;
-}
-
 // While a graph is captured for one parity of the position, the STU launches get that parity as a plain argument
 // instead of reading the device-side position first: their state addresses then depend on nothing, which takes one
 // dependent trip to memory (about 1 us) off each of them.  -1: no override.
@@ -259,8 +133,7 @@ static inline int stu_pos(int pos) { return g_stu_parity >= 0 ? g_stu_parity : p
 // this step's head leaves its maxima for the next step.
 static thread_local bool g_chain_prev = false, g_chain_next = false;
 static bool chain_ok(const fstu_model_desc* m, int do_sample, const int* dyn) {
-  return dyn && !do_sample && m->best && m->dtype == FSTU_BF16 && !m->head_packed && !fused_available(m) &&
-         fstu_head_argmax_fused_pick(m->h, m->d, m->emb, m->d, m->dtype) &&
+  return dyn && !do_sample && m->best && m->dtype == FSTU_BF16 && fstu_head_argmax_fused_pick(m->h, m->d, m->emb, m->d, m->dtype) &&
          fstu_finish_embed_supported(m->B, m->d, m->emb, m->x, m->layers[0].norm1_w, m->h);
 }
 
@@ -307,8 +180,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     }
     return FSTU_OK;
   }
-  if (fused_available(m))
-    return decode_step_fused(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
   // x = embedding rows, h = norm(x) with the first layer's norm weight
   const bool chain = chain_ok(m, do_sample, dyn);
   if (chain && g_chain_prev)
@@ -318,28 +189,15 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt,
                                       stream, dyn));
   // The residual stream starts in m->x.  Where a layer has packed gate/up weights, its MLP norm runs as the
-  // prologue of the GLU GEMV, which writes the updated residual to the other buffer (xc <-> xo swap).
+  // prologue of the gate/up launch, which writes the updated residual to the other buffer (xc <-> xo swap).
   void* xc = m->x;
   void* xo = m->x2;
-  const bool glu_pro = dt == FSTU_BF16 && xo != nullptr && d % 128 == 0 && (size_t)B * (d + 8) * 2 + 16384 <= 64 * 1024;
-  const size_t wsz = (dt == FSTU_BF16) ? 2 : 4;
   const bool glu_bal = dt == FSTU_BF16 && m->glu_packed && fstu_glu_packed_supported(B, d, I);
-  const bool mlp_fused = dt == FSTU_BF16 && m->mlp_sync && m->mlp_partial &&
-                         fstu_mlp_block_plan(B, d, I, nullptr, nullptr, nullptr) == FSTU_OK;
-  // Residual chain: the down projection adds straight into the residual stream (no split across workgroups) and the
-  // next sub-layer normalises it in its own prologue, so no stand-alone add+norm launch remains inside the layers.
-  bool res_chain = m->res_chain && glu_bal && m->x2 && m->stu_mode == 1 && d % 256 == 0 && !mlp_fused &&
-                   (size_t)B * (d + 8) * 2 <= 56 * 1024;
-  for (int l = 0; l < m->n_layers && res_chain; ++l) {
-    const fstu_layer_desc& L = m->layers[l];
-    res_chain = L.wp_gate && L.wp_up && L.wp_down && (L.kind == 0 || L.wp_qkv);
-  }
-  const int down_fpw = (m->down_fpw == 4 || m->down_fpw == 8 || m->down_fpw == 16) ? m->down_fpw : 8;
   // Merged norms: the down projection leaves 4 split-K slices and the first projection of the NEXT layer adds them
   // to the residual stream and normalises it in its own prologue, so the add+norm launch between two layers is gone
   // (the one in front of the head stays).
-  bool merge_norm = m->merge_norm && glu_bal && m->down_packed && m->x2 && m->stu_mode == 1 && d % 256 == 0 && !mlp_fused &&
-                    !res_chain && (size_t)B * (d / 8) <= 1024 && I % 128 == 0 && I / 128 <= 96;
+  bool merge_norm = m->merge_norm && glu_bal && m->down_packed && m->x2 && m->stu_mode == 1 && d % 256 == 0 &&
+                    (size_t)B * (d / 8) <= 1024 && I % 128 == 0 && I / 128 <= 96;
   for (int l = 0; l < m->n_layers && merge_norm; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     merge_norm = L.wp_gate && L.wp_up && L.wp_down && (L.kind == 0 || L.wp_qkv);
@@ -348,9 +206,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     bool pending_y = false;   // m->y holds a sub-layer output not yet added to the residual stream
-    // warm this layer's MLP weights while its (latency-bound) STU / attention sub-layer runs
-    warm_fork((hipStream_t)stream, L.w_gate, (size_t)I * d * wsz, L.w_up, (size_t)I * d * wsz, L.w_down, (size_t)I * d * wsz);
-    if (l == m->n_layers - 1) warm_fork((hipStream_t)stream, m->emb, (size_t)m->V * d * wsz, nullptr, 0, nullptr, 0);
     if (L.kind == 0) {
       if (m->stu_mode == 0) {
         char* row = (char*)L.hist + (size_t)pos * d * esz;  // hist[:, pos, :] with row stride hist_cap*d
@@ -364,9 +219,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                                                      L.lds_ce, L.lds_co, m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
           void* t = xc; xc = xo; xo = t;
           pending_slices = false;
-        } else if (res_chain) {
-          TIMED(PC_STU, fstu_stu_norm_inproj_step_dyn(xc, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, m->y,
-                                                      d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
         } else if (dt == FSTU_BF16 && d % 256 == 0) {
           TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, m->y, d, nullptr, B,
                                                  m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
@@ -377,56 +229,24 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         pending_y = true;
       }
     } else {
-      // QKV projection inside the attention launch: every (row, head) workgroup forms its own q, k, v
-      const bool swa_fused = m->swa_fused && dt == FSTU_BF16 && L.wp_qkv && m->head_dim == 64 && d % 256 == 0 && d <= 768 &&
-                             !res_chain;
-      if (swa_fused) {
-        if (pending_slices) {
-          TIMED(PC_SWA, fstu_swa_qkv_decode_dyn(nullptr, xc, m->partial, 4, xo, L.norm1_w, m->eps, L.wp_qkv, L.kring, L.vring,
-                                                m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos, m->window,
-                                                m->softcap, dyn, stream));
-          void* t = xc; xc = xo; xo = t;
-          pending_slices = false;
-        } else {
-          TIMED(PC_SWA, fstu_swa_qkv_decode_dyn(m->h, nullptr, nullptr, 0, nullptr, nullptr, 0.f, L.wp_qkv, L.kring, L.vring,
-                                                m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos, m->window,
-                                                m->softcap, dyn, stream));
-        }
-      } else if (pending_slices) {
+      if (pending_slices) {
         TIMED(PC_PROJ, fstu_linear_packed_res(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d,
                                               stream));
         void* t = xc; xc = xo; xo = t;
         pending_slices = false;
-      } else if (res_chain)
-        TIMED(PC_PROJ, fstu_linear_packed(xc, d, L.norm1_w, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
-      else if (glu_bal && L.wp_qkv)
+      } else if (glu_bal && L.wp_qkv)
         TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else
         TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.w_qkv, m->qkv, 3 * d, B, 3 * d, d, dt, stream));
-      if (!swa_fused)
-        TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
-                                           m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
-      if (glu_bal && L.wp_proj)
-        TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
-      else
-        TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
+      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim,
+                                         m->kv_cap, pos, m->window, m->softcap, 1, dyn, dt, stream));
+      TIMED(PC_PROJ, fstu_linear_decode(m->attn, d, L.w_proj, m->y, d, B, d, d, dt, stream));
       pending_y = true;
     }
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
-    if (mlp_fused && L.wp_gate && L.wp_up && L.wp_down) {
-      TIMED(PC_GLU, fstu_mlp_block(xc, pending_y ? m->y : nullptr, xc, L.mlp_norm_w, L.wp_gate, L.wp_up, L.wp_down, next_w,
-                                   m->h, m->act, m->mlp_partial, m->mlp_sync, B, d, I, m->eps, stream));
-      continue;
-    }
     if (pending_y && glu_bal && m->x2 && L.wp_gate && L.wp_up) {
       // residual add + mlp_norm as the prologue of the balanced gate/up launch; the stream moves to the other buffer
       TIMED(PC_GLU, fstu_glu_packed_norm(xc, m->y, xo, L.mlp_norm_w, m->eps, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
-      void* t = xc; xc = xo; xo = t;
-    } else if (pending_y && glu_pro && L.wp_gate && L.wp_up) {
-      fstu_gemv_args u = {};
-      u.mode = 1; u.rows = B; u.N = I; u.K = d; u.Wp = L.wp_gate; u.Wp2 = L.wp_up; u.y = m->act; u.ldy = I;
-      u.res_in = xc; u.delta = m->y; u.res_out = xo; u.norm_w = L.mlp_norm_w; u.eps = m->eps;
-      TIMED(PC_GLU, fstu_gemv_packed_dyn(&u, dyn, 0, stream));
       void* t = xc; xc = xo; xo = t;
     } else {
       if (pending_y) TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
@@ -434,12 +254,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
         TIMED(PC_GLU, fstu_glu_packed(m->h, d, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
       else
         TIMED(PC_GLU, fstu_glu_decode(m->h, d, L.w_gate, L.w_up, m->act, I, B, I, d, dt, stream));
-    }
-    if (res_chain) {
-      TIMED(PC_DOWN, fstu_down_packed_res(m->act, I, L.wp_down, xc, xc, B, d, I, down_fpw, stream));
-      if (l + 1 == m->n_layers)   // the head reads normalised rows
-        TIMED(PC_NORM, fstu_add_rmsnorm(xc, nullptr, 0, 1, 0, next_w, m->h, B, d, m->eps, dt, stream));
-      continue;
     }
     if (merge_norm) {
       int nsl = 4;
@@ -459,10 +273,7 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     }
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
-  if (!do_sample && m->best && glu_bal && m->head_packed && m->wp_emb && fstu_glu_packed_supported(B, d, m->V)) {
-    TIMED(PC_HEAD, fstu_head_packed_argmax_dyn(m->h, d, m->wp_emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
-                                               tok_stride, dyn, 1, stream));
-  } else if (!do_sample && m->best) {
+  if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
                                         tok_stride, dyn, (chain && g_chain_next) ? -1 : 1, dt, stream));
   } else {
@@ -470,7 +281,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));
     if (dyn) STEP(fstu_advance_dyn(dyn, stream));
   }
-  warm_join_all((hipStream_t)stream);
   return FSTU_OK;
 }
 
@@ -485,26 +295,10 @@ extern "C" int fstu_decode_step(const fstu_model_desc* m, const int64_t* tok_in,
 struct fstu_graph {
   hipGraph_t graph[2];       // one per parity of the position (the second is null when the model has no STU state)
   hipGraphExec_t exec[2];
-  WarmCtx* warm;
   long long next_pos;        // position the next launch will process first
   int nsteps;                // decode steps per launch
   bool baked;                // the STU launches carry the parity of their position as an argument
 };
-
-static void warm_destroy(WarmCtx* w) {
-  if (!w) return;
-  for (int i = 0; i < w->cap; ++i) { (void)hipEventDestroy(w->fork[i]); (void)hipEventDestroy(w->join[i]); }
-  if (w->side) (void)hipStreamDestroy(w->side);
-  delete w;
-}
-
-static int g_warm_wgs = 0;   // workgroups of the cache warm-up branch; 0 (default) disables it: forked graph branches
-                             // cost more than the warm cache saves on this stack (0.68 ms vs 0.47 ms per step measured)
-extern "C" int fstu_set_warm_workgroups(int n) {
-  FSTU_REQUIRE(n >= 0 && n <= 1024, FSTU_EARG, "fstu_set_warm_workgroups: %d", n);
-  g_warm_wgs = n;
-  return FSTU_OK;
-}
 
 extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* tokens, int64_t tok_stride, int* dyn, int pos0,
                                         int nsteps, float temperature, int top_k, float top_p, int do_sample, uint64_t seed,
@@ -512,30 +306,16 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
   FSTU_REQUIRE(m && tokens && dyn && graph_out && stream, FSTU_ENULL, "fstu_decode_graph_create: null pointer (a non-default stream is required)");
   FSTU_REQUIRE(pos0 >= 0 && nsteps >= 1 && nsteps <= 64, FSTU_EARG, "fstu_decode_graph_create: pos0=%d nsteps=%d (1..64)", pos0, nsteps);
   hipStream_t s = (hipStream_t)stream;
-  WarmCtx* warm = nullptr;
-  if (g_warm_wgs > 0 && m->n_layers + 1 <= 64) {
-    warm = new WarmCtx();
-    warm->wgs = g_warm_wgs;
-    if (hipStreamCreateWithFlags(&warm->side, hipStreamNonBlocking) != hipSuccess) { delete warm; warm = nullptr; }
-    else {
-      warm->cap = m->n_layers + 1;
-      for (int i = 0; i < warm->cap; ++i) {
-        (void)hipEventCreateWithFlags(&warm->fork[i], hipEventDisableTiming);
-        (void)hipEventCreateWithFlags(&warm->join[i], hipEventDisableTiming);
-      }
-    }
-  }
   // One graph per parity of the first position: the STU launches carry their parity as an argument.  A graph of an
   // even number of steps always starts on the parity of pos0, so the other one is not captured.  (The one-launch step
   // reads the position on the device: one graph serves both parities.)
-  const bool baked = m->stu_mode == 1 && warm == nullptr && !fstu_step_mega_ok(m);
-  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, warm, pos0, nsteps, baked};
+  const bool baked = m->stu_mode == 1 && !fstu_step_mega_ok(m);
+  fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, pos0, nsteps, baked};
   for (int par = 0; par < 2; ++par) {
     if (!baked && par == 1) break;
     if (baked && (nsteps & 1) == 0 && par != (pos0 & 1)) continue;
     hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
     if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: begin capture: %s", hipGetErrorString(e)); return (int)e; }
-    g_warm = warm;
     int rc = 0;
     for (int st = 0; st < nsteps && rc == 0; ++st) {
       g_stu_parity = baked ? ((par + st) & 1) : -1;
@@ -545,7 +325,6 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
     }
     g_stu_parity = -1;
     g_chain_prev = g_chain_next = false;
-    g_warm = nullptr;
     e = hipStreamEndCapture(s, &h->graph[par]);
     if (rc != 0) { fstu_decode_graph_destroy(h); return rc; }
     if (e != hipSuccess) { fstu_decode_graph_destroy(h); fstu_set_error("fstu_decode_graph_create: end capture: %s", hipGetErrorString(e)); return (int)e; }
@@ -585,7 +364,6 @@ extern "C" int fstu_decode_graph_destroy(void* graph) {
     if (h->exec[par]) (void)hipGraphExecDestroy(h->exec[par]);
     if (h->graph[par]) (void)hipGraphDestroy(h->graph[par]);
   }
-  warm_destroy(h->warm);
   delete h;
   return FSTU_OK;
 }

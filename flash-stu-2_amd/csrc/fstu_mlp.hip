@@ -1,22 +1,7 @@
-// The whole MLP sub-layer of one decode step in ONE launch (bf16):
-//   x' = T(x + delta);  h = rmsnorm(x') * w_mlp                 (flash_stu/layers/stu_layer.py:93-96,
-//   act = T(gelu_tanh(T(h Wg^T))) * T(h Wu^T)                    flash_stu/layers/attention_layer.py:59-62,
-//   x'' = T(x' + T(act Wd^T));  h_next = rmsnorm(x'') * w_next   flash_stu/modules/swiglu.py:22-29)
-// replacing four dependent launches (add+norm, gate/up GEMV, down GEMV, add+norm).
-//
-// A persistent grid of G workgroups (one per CU, all resident) walks two GEMV phases over packed weights
-// (layout of fstu_pack_rows):
-//   phase A  every workgroup recomputes x' and h into LDS (12-25 KB of input), then owns I/G gate/up features
-//            (4-feature granularity, so the bytes per CU are equal); the 8 waves split K and are reduced
-//            through LDS in fixed order; act goes out through agent-scope stores.
-//   barrier  one light hierarchical grid barrier (relaxed agent-scope atomics, no cache flushes: everything
-//            exchanged between workgroups moves through agent-scope 64-bit loads/stores, which are coherent
-//            across the XCDs); the first down-projection weights are already in flight while it spins.
-//   phase B  workgroup (tile group, K chunk) streams its slab of W_down; the KS partial tiles are published
-//            and the LAST workgroup to arrive for a tile group (ticket) adds them in chunk order
-//            (deterministic), forms x'' and stores it; the last workgroup of all normalises x'' into h_next
-//            and returns every counter to zero, so the launch can be replayed from a graph.
-// Every spin is bounded; a timeout raises a flag in the sync block and the kernel still exits.
+// Decode-step projections of the MLP sub-layer over packed bf16 weights (layout of fstu_pack_rows), one workgroup per
+// CU with equal bytes each: the gate/up projection with the GLU epilogue (and the QKV / plain projections on the same
+// launch), optionally with the sub-layer's residual add + RMSNorm as its prologue, and the split-K down projection
+// (flash_stu/modules/swiglu.py:22-29, flash_stu/layers/stu_layer.py:93-96, flash_stu/layers/attention_layer.py:59-62).
 #include <type_traits>
 #include "fstu_common.h"
 #include "fstu_prologue.h"
@@ -27,35 +12,8 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
-struct MlpArgs {
-  const bf16_t* x_in;
-  const bf16_t* delta;
-  bf16_t* x_out;
-  const bf16_t* norm_w;
-  const bf16_t* next_norm_w;
-  bf16_t* h_out;
-  const uint4* wp_gate;
-  const uint4* wp_up;
-  const uint4* wp_down;
-  bf16_t* act;          // rows x I
-  float* partial;       // KS x tiles_out x 256
-  unsigned* sync;       // counters, all zero between launches
-  int rows, d, I;
-  int fpw;              // gate/up features per workgroup (multiple of 4)
-  int KS, tpw, tiles_out, kch;   // phase B: K chunks, tiles per group, output tiles, k steps per chunk
-  float eps;
-  long long* trace;     // optional: 8 timestamps per workgroup (wall clock ticks), NULL = off
-};
-
-// sync block layout (32-bit words; every counter on its own 128-byte line)
-enum { SY_GRP = 0, SY_TOP = 8 * 32, SY_ALL = 9 * 32, SY_ERR = 10 * 32, SY_TG = 11 * 32, SY_WORDS = (11 + 64) * 32 };
-#define MLP_NG 8
-#define MLP_SPIN_LIMIT (1L << 22)
-
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
 
-__device__ __forceinline__ u64 ld_agent(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void st_agent(u64* p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Raw buffer loads: a lane whose byte offset lies beyond the descriptor's range reads zeros without a branch, so
 // every load of the kernel sits in straight-line code and the compiler's vmcnt bookkeeping stays exact (the
@@ -155,303 +113,9 @@ __device__ __forceinline__ void load_norm_w(uint4 (&nwv)[4], const bf16_t* __res
   }
 }
 
-#define MLP_RED_FLOATS 16384   // reduction staging: up to 4 tiles x 8 waves x 512 floats
-
-template <int KSA, int KSB>
-__global__ void __launch_bounds__(512)
-mlp_block_kernel(MlpArgs a) {
-  constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);   // gate/up tiles whose weights are in flight together
-  constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : 2);   // down tiles in flight together
-  constexpr int NXC = 4;                                  // 16-byte chunks of x / delta a thread holds in registers
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int wgi = blockIdx.x, G = gridDim.x;
-  const int ld = a.d + 8;
-  bf16_t* xs = (bf16_t*)smem;                          // x' (rows x ld)
-  bf16_t* hs = xs + (size_t)a.rows * ld;               // h  (rows x ld)
-  float* red = (float*)(hs + (size_t)a.rows * ld);     // MLP_RED_FLOATS
-  __shared__ int flag;
-  const bool xrow = r < a.rows;
-#define MLP_STAMP(k)                                                                     \
-  do {                                                                                   \
-    if (a.trace && threadIdx.x == 0) a.trace[(size_t)wgi * 8 + (k)] = wall_clock64();    \
-  } while (0)
-  MLP_STAMP(0);
-
-  // ------------------------------------------------------------ loads in issue order: x, delta, norm weights, W
-  const int nchunk = a.d >> 3, total = a.rows * nchunk;
-  uint4 xv[NXC], dv[NXC];
-  {
-    const rsrc_t rx = make_rsrc(a.x_in, (size_t)total * 16), rd = make_rsrc(a.delta, (size_t)total * 16);
-#pragma unroll
-    for (int j = 0; j < NXC; ++j) {
-      const unsigned q = threadIdx.x + j * 512;
-      xv[j] = buf_load16(rx, q * 16u);          // beyond total: zeros
-      dv[j] = buf_load16(rd, q * 16u);          // no delta: zeros
-    }
-  }
-  uint4 nwv[4];
-  load_norm_w(nwv, a.norm_w, a.d, lane);
-
-  const int f0 = wgi * a.fpw, f1 = min(a.I, f0 + a.fpw);
-  const int ta0 = f0 >> 4, ta1 = (f1 > f0) ? ((f1 + 15) >> 4) : ta0;
-  const size_t tsa = (size_t)(a.d >> 5) * 64;          // uint4 per tile of the gate/up packing
-  const size_t wa_bytes = (size_t)((a.I + 15) >> 4) * tsa * 16;
-  const rsrc_t rg = make_rsrc(a.wp_gate, wa_bytes), ru = make_rsrc(a.wp_up, wa_bytes);
-  const unsigned abase = ((unsigned)(w * KSA) * 64 + lane) * 16u;
-  uint4 wa[DA][KSA], wb[DA][KSA];
-  auto load_a = [&](int j, int tile) {
-    const int f = tile * 16 + r;
-    const bool ok = tile < ta1 && f >= f0 && f < f1;
-#pragma unroll
-    for (int u = 0; u < KSA; ++u) {
-      const unsigned off = ok ? abase + ((unsigned)tile * (unsigned)tsa + (unsigned)u * 64u) * 16u : MLP_OOB;
-      wa[j][u] = buf_load16(rg, off);
-      wb[j][u] = buf_load16(ru, off);
-    }
-  };
-
-  // ------------------------------------------------------------ prologue: x' and h into LDS
-  // (the weight loads are issued only once x has arrived: issued together with x they fill the memory queues of
-  // the whole chip and x, which every workgroup reads from the same few lines, comes back microseconds later)
-  auto add_chunk = [&](uint4 x4, uint4 d4) {
-    unsigned xw[4] = {x4.x, x4.y, x4.z, x4.w}, dw[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float lo = __uint_as_float(xw[i] << 16) + __uint_as_float(dw[i] << 16);
-      float hi = __uint_as_float(xw[i] & 0xffff0000u) + __uint_as_float(dw[i] & 0xffff0000u);
-      xw[i] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
-    }
-    return make_uint4(xw[0], xw[1], xw[2], xw[3]);
-  };
-#pragma unroll
-  for (int j = 0; j < NXC; ++j) {
-    const int q = threadIdx.x + j * 512;
-    if (q < total) {
-      const int row = q / nchunk, c = (q - row * nchunk) << 3;
-      *(uint4*)(xs + (size_t)row * ld + c) = add_chunk(xv[j], dv[j]);
-    }
-  }
-  for (int q = threadIdx.x + NXC * 512; q < total; q += 512) {
-    const int row = q / nchunk, c = (q - row * nchunk) << 3;
-    uint4 x4 = *(const uint4*)(a.x_in + (size_t)q * 8);
-    if (a.delta) x4 = add_chunk(x4, *(const uint4*)(a.delta + (size_t)q * 8));
-    *(uint4*)(xs + (size_t)row * ld + c) = x4;
-  }
-#pragma unroll
-  for (int j = 0; j < DA; ++j) load_a(j, ta0 + j);
-  MLP_STAMP(1);
-  __syncthreads();
-  norm_rows(xs, ld, hs, ld, a.norm_w, nwv, a.rows, a.d, a.eps, w, lane);
-  __syncthreads();
-  MLP_STAMP(2);
-
-  // ------------------------------------------------------------ phase A: gate/up tiles, DA at a time
-  {
-    const bf16_t* hl = hs + (size_t)(xrow ? r : 0) * ld + (w * KSA) * 32 + g * 8;
-    uint4 xa[KSA];
-#pragma unroll
-    for (int u = 0; u < KSA; ++u) xa[u] = xrow ? *(const uint4*)(hl + u * 32) : make_uint4(0, 0, 0, 0);
-    for (int t0 = ta0; t0 < ta1; t0 += DA) {
-#pragma unroll
-      for (int j = 0; j < DA; ++j) {
-        floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int u = 0; u < KSA; ++u) {
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc, 0, 0, 0);
-          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
-        }
-        load_a(j, t0 + DA + j);     // the next group's tile takes over these registers
-        float* mine = red + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          mine[i] = acc[i];
-          mine[256 + i] = acc2[i];
-        }
-      }
-      __syncthreads();
-      if (w < DA && t0 + w < ta1) {      // wave j finishes tile t0 + j: the 8 K shares in wave order
-        const int tile = t0 + w;
-        float sg[4] = {0.f, 0.f, 0.f, 0.f}, su[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const float* o = red + (size_t)((w * 8 + s) * 2 * 64 + lane) * 4;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            sg[i] += o[i];
-            su[i] += o[256 + i];
-          }
-        }
-        const int fb = tile * 16 + g * 4;     // this lane's 4 features of batch row r
-        if (xrow && fb >= f0 && fb < f1) {
-          float o[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(sg[i])));
-            o[i] = ge * DT<bf16_t>::rnd(su[i]);
-          }
-          st_agent((u64*)(a.act + (size_t)r * a.I + fb), pack4_bf16(o));
-        }
-      }
-      if (t0 + DA < ta1) __syncthreads();
-    }
-  }
-  MLP_STAMP(3);
-  __builtin_amdgcn_s_waitcnt(0);   // this wave's act stores have reached the coherence point
-
-  // ------------------------------------------------------------ phase B set-up: W_down fragments in flight
-  const int chunk = wgi % a.KS, tgrp = wgi / a.KS;
-  const int tb0 = tgrp * a.tpw, tb1 = min(a.tiles_out, tb0 + a.tpw);
-  const int ksb0 = w * KSB;                                   // first k step of this wave inside the chunk
-  const int nks = max(0, min(KSB, a.kch - ksb0));             // k steps this wave owns
-  const size_t tsb = (size_t)(a.I >> 5) * 64;
-  const rsrc_t rdn = make_rsrc(a.wp_down, (size_t)a.tiles_out * tsb * 16);
-  const unsigned bbase = ((unsigned)(chunk * a.kch + ksb0) * 64 + lane) * 16u;
-  uint4 wd[DB][KSB];
-  auto load_b = [&](int j, int tile) {
-#pragma unroll
-    for (int u = 0; u < KSB; ++u)
-      wd[j][u] = buf_load16(rdn, (u < nks && tile < tb1) ? bbase + ((unsigned)tile * (unsigned)tsb + (unsigned)u * 64u) * 16u : MLP_OOB);
-  };
-#pragma unroll
-  for (int j = 0; j < DB; ++j) load_b(j, tb0 + j);
-
-  // ------------------------------------------------------------ grid barrier (wave 7 arrives and spins)
-  __syncthreads();
-  if (threadIdx.x == 448) {
-    const unsigned grp = wgi % MLP_NG;
-    const unsigned gsize = (G + MLP_NG - 1 - grp) / MLP_NG;
-    unsigned old = __hip_atomic_fetch_add(a.sync + SY_GRP + grp * 32, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (old + 1 == gsize) __hip_atomic_fetch_add(a.sync + SY_TOP, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    long spins = 0;
-    while (__hip_atomic_load(a.sync + SY_TOP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)min(G, MLP_NG)) {
-      if (++spins > MLP_SPIN_LIMIT) {
-        __hip_atomic_store(a.sync + SY_ERR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-    }
-  }
-  __syncthreads();
-  MLP_STAMP(4);
-
-  // ------------------------------------------------------------ phase B: partial tiles of (tile group, chunk)
-  {
-    const bf16_t* al = a.act + (size_t)(xrow ? r : 0) * a.I + (size_t)(chunk * a.kch + ksb0) * 32 + g * 8;
-    uint4 xb[KSB];
-#pragma unroll
-    for (int u = 0; u < KSB; ++u) {
-      xb[u] = make_uint4(0, 0, 0, 0);
-      if (xrow && u < nks) {
-        const u64 lo = ld_agent((const u64*)(al + u * 32)), hi = ld_agent((const u64*)(al + u * 32) + 1);
-        xb[u] = make_uint4((unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32));
-      }
-    }
-    for (int t0 = tb0; t0 < tb1; t0 += DB) {
-#pragma unroll
-      for (int j = 0; j < DB; ++j) {
-        floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int u = 0; u < KSB; ++u)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc, 0, 0, 0);
-        load_b(j, t0 + DB + j);
-        float* mine = red + (size_t)((j * 8 + w) * 64 + lane) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) mine[i] = acc[i];
-      }
-      __syncthreads();
-      if (w < DB && t0 + w < tb1) {
-        const int tile = t0 + w;
-        float sd[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const float* o = red + (size_t)((w * 8 + s) * 64 + lane) * 4;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) sd[i] += o[i];
-        }
-        u64* slot = (u64*)(a.partial + (((size_t)chunk * a.tiles_out + tile) * 64 + lane) * 4);
-        st_agent(slot, (u64)__float_as_uint(sd[0]) | ((u64)__float_as_uint(sd[1]) << 32));
-        st_agent(slot + 1, (u64)__float_as_uint(sd[2]) | ((u64)__float_as_uint(sd[3]) << 32));
-      }
-      if (t0 + DB < tb1) __syncthreads();
-    }
-  }
-
-  // ------------------------------------------------------------ ticket 1: last workgroup of the tile group
-  load_norm_w(nwv, a.h_out ? a.next_norm_w : nullptr, a.d, lane);
-  __builtin_amdgcn_s_waitcnt(0);     // the partial tiles have reached the coherence point
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned old = __hip_atomic_fetch_add(a.sync + SY_TG + tgrp * 32, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    flag = (old == (unsigned)(a.KS - 1)) ? 1 : 0;
-  }
-  __syncthreads();
-  MLP_STAMP(5);
-  if (!flag) return;
-  __syncthreads();
-  for (int tile = tb0 + w; tile < tb1; tile += 8) {
-    // wave w sums the KS partial tiles of its output tile in chunk order, 16 chunks in flight at a time
-    float tot[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < a.KS; s0 += 16) {
-      u64 v[16][2];
-#pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const u64* p = (const u64*)(a.partial + (((size_t)(s0 + k) * a.tiles_out + tile) * 64 + lane) * 4);
-        v[k][0] = (s0 + k < a.KS) ? ld_agent(p) : 0ull;
-        v[k][1] = (s0 + k < a.KS) ? ld_agent(p + 1) : 0ull;
-      }
-#pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        tot[0] += __uint_as_float((unsigned)v[k][0]);
-        tot[1] += __uint_as_float((unsigned)(v[k][0] >> 32));
-        tot[2] += __uint_as_float((unsigned)v[k][1]);
-        tot[3] += __uint_as_float((unsigned)(v[k][1] >> 32));
-      }
-    }
-    const int fb = tile * 16 + g * 4;
-    if (xrow && fb < a.d) {
-      const bf16_t* xr = xs + (size_t)r * ld + fb;
-      float o[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = bf16_to_f32(xr[i]) + DT<bf16_t>::rnd(tot[i]);
-      st_agent((u64*)(a.x_out + (size_t)r * a.d + fb), pack4_bf16(o));
-    }
-  }
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-
-  // ------------------------------------------------------------ ticket 2: last workgroup of all
-  if (threadIdx.x == 0) {
-    __hip_atomic_store(a.sync + SY_TG + tgrp * 32, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned ngroups = (unsigned)(G / a.KS);
-    unsigned old = __hip_atomic_fetch_add(a.sync + SY_ALL, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    flag = (old == ngroups - 1) ? 1 : 0;
-  }
-  __syncthreads();
-  MLP_STAMP(6);
-  if (!flag) return;
-  {
-    const int nq = a.d >> 2, totq = a.rows * nq;       // 4 bf16 per 64-bit load
-    for (int q = threadIdx.x; q < totq; q += 512) {
-      const int row = q / nq, c = (q - row * nq) << 2;
-      *(u64*)(xs + (size_t)row * ld + c) = ld_agent((const u64*)(a.x_out + (size_t)row * a.d + c));
-    }
-    __syncthreads();
-    if (a.h_out) norm_rows(xs, ld, a.h_out, a.d, a.next_norm_w, nwv, a.rows, a.d, a.eps, w, lane);
-    if (threadIdx.x < MLP_NG) __hip_atomic_store(a.sync + SY_GRP + threadIdx.x * 32, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (threadIdx.x == 0) {
-      __hip_atomic_store(a.sync + SY_TOP, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(a.sync + SY_ALL, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  __syncthreads();
-  MLP_STAMP(7);
-}
-
 // ---------------------------------------------------------------- balanced gate/up GEMV (stand-alone launch)
-// The gate/up phase of mlp_block_kernel as a kernel of its own: one workgroup per CU, I/G features each at
-// 4-feature granularity (equal bytes per CU), every weight fragment of a workgroup in flight from the first
-// instruction, the 8 waves split K.  Input h is already normalised.
+// One workgroup per CU, I/G features each in groups of 8 (equal bytes per CU), every weight fragment of a workgroup in
+// flight from the first instruction, the 8 waves split K.
 struct GluArgs {
   const bf16_t* h;        // normalised input (rows x ldh); unused with the prologue
   const uint4* wp_gate;
@@ -466,36 +130,21 @@ struct GluArgs {
   const bf16_t* norm_w;
   float eps;
   int nslices;
-  // EPI 2: greedy pick fused into the epilogue (packed (value key << 32 | ~index) maxima into 64 slots per row)
-  unsigned long long* best_ws;
-  float temperature;
 };
 
-// EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus the greedy-pick maxima
+// EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T
 // (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
-#ifdef FSTU_GLU_TRACE
-__device__ long long glu_trace_buf[256 * 8];
-#define GLU_STAMP(k) do { if (threadIdx.x == 0 && blockIdx.x < 256) glu_trace_buf[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
-#else
-#define GLU_STAMP(k) do { } while (0)
-#endif
-
 template <int KSA, int PRO, int EPI>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
                     const void* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
-                    int fpw, float eps, float temperature, unsigned long long* best_ws, int nslices) {
+                    int fpw, float eps, int nslices) {
   GluArgs a;
   a.h = h; a.wp_gate = wp_gate; a.wp_up = wp_up; a.act = act; a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
-  a.fpw = fpw; a.x_in = x_in; a.delta = delta; a.x_out = x_out; a.norm_w = norm_w; a.eps = eps; a.best_ws = best_ws;
-  a.temperature = temperature; a.nslices = nslices;
+  a.fpw = fpw; a.x_in = x_in; a.delta = delta; a.x_out = x_out; a.norm_w = norm_w; a.eps = eps; a.nslices = nslices;
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
-  GLU_STAMP(0);
-#ifdef FSTU_GLU_TRACE
-  if (threadIdx.x == 0 && blockIdx.x == 0) glu_trace_buf[255 * 8 + 7] = (long long)__builtin_amdgcn_s_getpc();
-#endif
   __shared__ float red[DA * 8 * 512];
   extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -589,7 +238,6 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       for (int j = 1; j < DA; ++j)
         if (j < DA - 1 || ta0 + j < ta1) load_a(j, ta0 + j);
       __syncthreads();
-      GLU_STAMP(1);
       pro.scale(ss_part, hs, ld, a.rows, a.d, a.eps);
     };
     constexpr int NXMAX = PRO == 2 ? 2 : NXC;
@@ -617,7 +265,6 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       norm_rows(hs, ld, hs, ld, a.norm_w, nwv, a.rows, a.d, a.eps, w, lane);
     }
     __syncthreads();
-    GLU_STAMP(2);
     const bf16_t* hl = hs + (size_t)(xrow ? r : 0) * ld + (w * KSA) * 32 + g * 8;
 #pragma unroll
     for (int u = 0; u < KSA; ++u) xa[u] = xrow ? *(const uint4*)(hl + u * 32) : make_uint4(0, 0, 0, 0);
@@ -642,7 +289,6 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       }
     }
     __syncthreads();
-    GLU_STAMP(3);
     // reduction over the 8 K slices and the epilogue: wave w takes half a tile (two of a lane's four features)
     if ((w >> 1) < DA && t0 + (w >> 1) < ta1) {
       const int jt = w >> 1, hf = (w & 1) * 2;
@@ -683,140 +329,14 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
             if (fb + i < f1) yr[i] = f32_to_bf16(o[i]);
         }
       }
-      if (EPI == 2) {
-        unsigned long long key = 0ull;
-        if (grp_ok) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            const int f = fb + i;
-            if (f < f1) {
-              float l = DT<bf16_t>::rnd(o[i]);
-              if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
-              l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
-              unsigned u = __float_as_uint(l);
-              u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-              unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
-              key = k > key ? k : key;
-            }
-          }
-        }
-        unsigned long long ok2 = __shfl_xor(key, 16, FSTU_WAVE);
-        key = ok2 > key ? ok2 : key;
-        ok2 = __shfl_xor(key, 32, FSTU_WAVE);
-        key = ok2 > key ? ok2 : key;
-        if (g == 0 && xrow && key != 0ull) atomicMax(a.best_ws + (size_t)r * 64 + (tile & 63), key);
-      }
     }
     if (t0 + DA < ta1) __syncthreads();
-  }
-  GLU_STAMP(4);
-}
-
-#ifdef FSTU_GLU_TRACE
-__global__ void __launch_bounds__(256) touch_kernel(const uint4* p, unsigned n16, unsigned* sink) {
-  unsigned acc = 0;
-  for (unsigned i = threadIdx.x; i < n16; i += 256) {
-    uint4 v = p[i];
-    acc ^= v.x ^ v.y ^ v.z ^ v.w;
-  }
-  if (acc == 0x12345679u) sink[0] = acc;
-}
-}  // namespace
-extern "C" int fstu_glu_trace(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(glu_trace_buf), sizeof(long long) * 256 * 8);
-}
-extern "C" int fstu_touch(unsigned long long addr, unsigned bytes, void* sink, hipStream_t s) {
-  hipLaunchKernelGGL(touch_kernel, dim3(256), dim3(256), 0, s, (const uint4*)addr, bytes / 16, (unsigned*)sink);
-  return (int)hipGetLastError();
-}
-namespace {
-#endif
-
-// ---------------------------------------------------------------- down projection + residual, no split across workgroups
-// x_out[r, f] = T( x_res[r, f] + T( act[r, :] . Wd[f, :] ) ): a workgroup owns `fpw` (4, 8 or 16) output features over
-// the WHOLE K range, its 8 waves split K and are reduced through LDS in wave order (deterministic), so the result is
-// complete in one launch and the next kernel can normalise it in its own prologue.  Weight and activation
-// fragments are double-buffered in registers (two chunks of CH k steps in flight per wave).
-struct DownArgs {
-  const bf16_t* act;
-  const uint4* wp_down;
-  const bf16_t* x_res;
-  bf16_t* x_out;
-  int rows, d, I, ldact, fpw;
-};
-
-template <int CH>
-__global__ void __launch_bounds__(512)
-down_res_kernel(DownArgs a) {
-  __shared__ float red[8 * 256];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const bool xrow = r < a.rows;
-  const int f0 = blockIdx.x * a.fpw, f1 = min(a.d, f0 + a.fpw);
-  const int tile = f0 >> 4;
-  const int fr = tile * 16 + r;                           // feature of this lane's A-operand row
-  const bool fok = fr >= f0 && fr < f1;
-  const int ksteps = a.I >> 5;
-  const int kpw = (ksteps + 7) >> 3;
-  const int ks_beg = w * kpw, ks_end = min(ksteps, ks_beg + kpw);
-  const size_t tsb = (size_t)ksteps * 64;
-  const rsrc_t rw = make_rsrc(a.wp_down, (size_t)((a.d + 15) >> 4) * tsb * 16);
-  const rsrc_t rx = make_rsrc(a.act, ((size_t)(a.rows - 1) * a.ldact + a.I) * 2);
-  const unsigned wbase = (unsigned)tile * (unsigned)tsb * 16u;   // byte offset of the tile (tsb 16-byte fragments per tile)
-  const unsigned wlane = (unsigned)lane * 16u;
-  const unsigned xbase = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldact + (unsigned)g * 8u) * 2u;
-  // residual of this lane's 4 output features (D layout: features tile*16 + 4g + i of row r), fetched up front
-  const int fb = tile * 16 + 4 * g;
-  const bool ook = xrow && fb >= f0 && fb < f1;
-  u64 resv = 0;
-  if (w == 0 && ook) resv = *(const u64*)(a.x_res + (size_t)r * a.d + fb);
-  uint4 wA[CH], xA[CH], wB[CH], xB[CH];
-  auto ld = [&](uint4 (&wv)[CH], uint4 (&xv)[CH], int ks0) {
-#pragma unroll
-    for (int u = 0; u < CH; ++u) {
-      const int ks = ks0 + u;
-      const bool ok = ks < ks_end;
-      wv[u] = buf_load16(rw, (ok && fok) ? wbase + (unsigned)ks * 1024u + wlane : MLP_OOB);
-      xv[u] = buf_load16(rx, (ok && xrow) ? xbase + (unsigned)ks * 64u : MLP_OOB);
-    }
-  };
-  floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
-  auto mm = [&](uint4 (&wv)[CH], uint4 (&xv)[CH]) {
-#pragma unroll
-    for (int u = 0; u < CH; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wv[u]), as_bf16x8(xv[u]), acc, 0, 0, 0);
-  };
-  ld(wA, xA, ks_beg);
-  for (int ks0 = ks_beg; ks0 < ks_end; ks0 += 2 * CH) {
-    ld(wB, xB, ks0 + CH);
-    mm(wA, xA);
-    ld(wA, xA, ks0 + 2 * CH);
-    mm(wB, xB);
-  }
-  float* mine = red + (size_t)(w * 64 + lane) * 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) mine[i] = acc[i];
-  __syncthreads();
-  if (w == 0 && ook) {
-    float sd[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const float* o = red + (size_t)(s * 64 + lane) * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) sd[i] += o[i];
-    }
-    const unsigned lo = (unsigned)resv, hi = (unsigned)(resv >> 32);
-    const float xr[4] = {__uint_as_float(lo << 16), __uint_as_float(lo & 0xffff0000u), __uint_as_float(hi << 16),
-                         __uint_as_float(hi & 0xffff0000u)};
-    float o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = xr[i] + DT<bf16_t>::rnd(sd[i]);
-    *(u64*)(a.x_out + (size_t)r * a.d + fb) = pack4_bf16(o);
   }
 }
 
 // ---------------------------------------------------------------- balanced split-K down projection (stand-alone launch)
-// partial[chunk][row][feature] (fp32 slices, the layout fstu_add_rmsnorm sums): workgroup (tile group, K chunk) as in
-// phase B of mlp_block_kernel, every weight fragment and the activations of the chunk in flight from the first
+// partial[chunk][row][feature] (fp32 slices, the layout fstu_add_rmsnorm sums): workgroup (tile group, K chunk), every
+// weight fragment and the activations of the chunk in flight from the first
 // instruction, the 8 waves split the chunk's k steps and are reduced through LDS in wave order.
 struct DownSkArgs {
   const bf16_t* act;
@@ -898,91 +418,7 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
 }
 
 int g_cus = 0;
-long long* g_trace = nullptr;
-
 }  // namespace
-
-extern "C" int fstu_mlp_block_trace(long long* buf) {
-  g_trace = buf;
-  return FSTU_OK;
-}
-
-extern "C" size_t fstu_mlp_block_sync_bytes(void) { return (size_t)SY_WORDS * sizeof(unsigned); }
-
-extern "C" int fstu_mlp_block_plan(int rows, int d, int I, int* G_out, int* KS_out, size_t* partial_floats) {
-  // G = 16 K chunks x (number of tile groups): the largest grid of at most one workgroup per CU
-  if (g_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return FSTU_EARG;
-    g_cus = p.multiProcessorCount;
-  }
-  if (rows < 1 || rows > FSTU_MAX_DECODE_ROWS || d < 256 || d % 256 != 0 || I < 512 || I % 512 != 0) return FSTU_ESHAPE;
-  if ((size_t)I * d * 2 >= 0xfff00000ull) return FSTU_ESHAPE;   // 32-bit buffer offsets
-  const int ksa = d / 256;
-  if (!(ksa == 1 || ksa == 2 || ksa == 3 || ksa == 4 || ksa == 8)) return FSTU_ESHAPE;
-  const int KS = 16;
-  const int tiles_out = d / 16;
-  int ngroups = g_cus / KS;
-  if (ngroups < 1) return FSTU_ESHAPE;
-  if (ngroups > tiles_out) ngroups = tiles_out;
-  if (ngroups > 64) ngroups = 64;
-  const int kch = I / 32 / KS;                     // k steps per chunk
-  if (kch < 1 || (kch + 7) / 8 > 8) return FSTU_ESHAPE;
-  const size_t lds = (size_t)2 * rows * (d + 8) * 2 + MLP_RED_FLOATS * 4;
-  if (lds > 150 * 1024) return FSTU_ESHAPE;
-  if (G_out) *G_out = ngroups * KS;
-  if (KS_out) *KS_out = KS;
-  if (partial_floats) *partial_floats = (size_t)KS * tiles_out * 256;
-  return FSTU_OK;
-}
-
-extern "C" int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, const void* norm_w, const void* wp_gate,
-                              const void* wp_up, const void* wp_down, const void* next_norm_w, void* h_out, void* act_ws,
-                              float* partial_ws, unsigned* sync_ws, int rows, int d, int I, float eps, void* stream) {
-  FSTU_REQUIRE(x_in && x_out && norm_w && wp_gate && wp_up && wp_down && act_ws && partial_ws && sync_ws, FSTU_ENULL,
-               "fstu_mlp_block: null pointer");
-  FSTU_REQUIRE(h_out == nullptr || next_norm_w != nullptr, FSTU_ENULL, "fstu_mlp_block: h_out given without next_norm_w");
-  int G = 0, KS = 0;
-  size_t pf = 0;
-  int rc = fstu_mlp_block_plan(rows, d, I, &G, &KS, &pf);
-  FSTU_REQUIRE(rc == FSTU_OK, rc, "fstu_mlp_block: unsupported shape rows=%d d=%d I=%d (d %% 256, I %% 512, d <= 2048)", rows, d, I);
-  FSTU_REQUIRE(fstu_aligned(x_in, 16) && fstu_aligned(delta, 16) && fstu_aligned(x_out, 16) && fstu_aligned(norm_w, 16) &&
-                   fstu_aligned(next_norm_w, 16) && fstu_aligned(h_out, 16) && fstu_aligned(wp_gate, 16) &&
-                   fstu_aligned(wp_up, 16) && fstu_aligned(wp_down, 16) && fstu_aligned(act_ws, 16) &&
-                   fstu_aligned(partial_ws, 16) && fstu_aligned(sync_ws, 128),
-               FSTU_EALIGN, "fstu_mlp_block: pointers must be 16-byte aligned (sync_ws 128)");
-  MlpArgs a;
-  a.x_in = (const bf16_t*)x_in; a.delta = (const bf16_t*)delta; a.x_out = (bf16_t*)x_out;
-  a.norm_w = (const bf16_t*)norm_w; a.next_norm_w = (const bf16_t*)next_norm_w; a.h_out = (bf16_t*)h_out;
-  a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.wp_down = (const uint4*)wp_down;
-  a.act = (bf16_t*)act_ws; a.partial = partial_ws; a.sync = sync_ws;
-  a.rows = rows; a.d = d; a.I = I; a.eps = eps; a.trace = g_trace;
-  a.fpw = (((I + G - 1) / G) + 3) & ~3;
-  a.KS = KS; a.tiles_out = d / 16; a.tpw = (a.tiles_out + G / KS - 1) / (G / KS); a.kch = I / 32 / KS;
-  const int ksa = d / 256, ksb = (a.kch + 7) / 8;
-  const int ksb_r = ksb <= 4 ? ksb : (ksb <= 6 ? 6 : 8);   // phase-B unroll rounded up to an instantiated value
-  const size_t shm = (size_t)2 * rows * (d + 8) * 2 + MLP_RED_FLOATS * 4;
-  hipStream_t s = (hipStream_t)stream;
-  bool launched = false;
-#define MLP_CASE(A, Bv)                                                                                         \
-  if (!launched && ksa == A && ksb_r == Bv) {                                                                   \
-    if (shm > 48 * 1024) {                                                                                      \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_block_kernel<A, Bv>),                \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);                 \
-      FSTU_REQUIRE(e == hipSuccess, (int)e, "fstu_mlp_block: %zu bytes of LDS refused", shm);                   \
-    }                                                                                                           \
-    hipLaunchKernelGGL((mlp_block_kernel<A, Bv>), dim3(G), dim3(512), shm, s, a);                               \
-    launched = true;                                                                                            \
-  }
-#define MLP_ROW(A) MLP_CASE(A, 1) MLP_CASE(A, 2) MLP_CASE(A, 3) MLP_CASE(A, 4) MLP_CASE(A, 6) MLP_CASE(A, 8)
-  MLP_ROW(1) MLP_ROW(2) MLP_ROW(3) MLP_ROW(4) MLP_ROW(8)
-#undef MLP_ROW
-#undef MLP_CASE
-  FSTU_REQUIRE(launched, FSTU_ESHAPE, "fstu_mlp_block: no kernel for d=%d I=%d", d, I);
-  FSTU_CHECK_LAUNCH("fstu_mlp_block");
-  return FSTU_OK;
-}
 
 static int query_cus() {
   if (g_cus == 0) {
@@ -1010,15 +446,13 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
       FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                  \
     }                                                                                                            \
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,    \
-                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.temperature, a.best_ws, a.nslices); \
-                    \
+                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);                    \
   } while (0)
   if (pro == 2) GLU_GO(2, 1);
   else if (pro && epi == 0) GLU_GO(1, 0);
   else if (pro) GLU_GO(1, 1);
   else if (epi == 0) GLU_GO(0, 0);
-  else if (epi == 1) GLU_GO(0, 1);
-  else GLU_GO(0, 2);
+  else GLU_GO(0, 1);
 #undef GLU_GO
   return FSTU_OK;
 }
@@ -1028,22 +462,13 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
   FSTU_REQUIRE(G > 0, FSTU_EARG, "%s: no device", name);
   // Features are dealt out in groups of 8: no 128-byte line is shared between two workgroups (HBM traffic of the
   // gate/up launch 1.00x the algorithmic bytes instead of 1.125x with groups of 4), at the price of workgroups of 32
-  // and 40 features instead of 36 each.  Measured 0.3305 vs 0.3326 ms per decode step; FSTU_GLU_BY4=1 brings the
-  // groups of 4 back.
-  const char* by4_env = getenv("FSTU_GLU_BY4");   // read at every launch: a graph keeps what it was captured with
-  const bool by4 = by4_env && by4_env[0] == '1';
-  if (by4) {
-    if (G > (a.I + 3) / 4) G = (a.I + 3) / 4;
-    a.fpw = (((a.I + G - 1) / G) + 3) & ~3;
-    G = (a.I + a.fpw - 1) / a.fpw;
-  } else {
-    if (G > (a.I + 7) / 8) G = (a.I + 7) / 8;
-    // a plain projection narrower than 16 features per CU (QKV at d = 768: 2304 features) gets one whole tile per
-    // workgroup rather than half tiles on every CU: every workgroup repeats the norm prologue, and its operands come
-    // out of one L2 per XCD (0.3113 -> 0.3105 ms per decode step)
-    if (epi != 0 && G > (a.I + 15) / 16) G = (a.I + 15) / 16;
-    a.fpw = 0;
-  }
+  // and 40 features instead of 36 each.
+  if (G > (a.I + 7) / 8) G = (a.I + 7) / 8;
+  // a plain projection narrower than 16 features per CU (QKV at d = 768: 2304 features) gets one whole tile per
+  // workgroup rather than half tiles on every CU: every workgroup repeats the norm prologue, and its operands come
+  // out of one L2 per XCD
+  if (epi != 0 && G > (a.I + 15) / 16) G = (a.I + 15) / 16;
+  a.fpw = 0;
   const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
   int rc;
   switch (a.d / 256) {
@@ -1134,24 +559,6 @@ extern "C" int fstu_linear_packed_res(const void* x_in, const float* partial, in
   return glu_launch(a, 2, 1, "fstu_linear_packed_res", (hipStream_t)stream);
 }
 
-extern "C" int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
-                                    int d, int I, int fpw, void* stream) {
-  FSTU_REQUIRE(act && wp_down && x_res && x_out, FSTU_ENULL, "fstu_down_packed_res: null pointer");
-  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d >= 4 && d % 4 == 0 && I >= 32 && I % 32 == 0 &&
-                   (size_t)I * d * 2 < 0xfff00000ull,
-               FSTU_ESHAPE, "fstu_down_packed_res: unsupported shape rows=%d d=%d I=%d", rows, d, I);
-  FSTU_REQUIRE(fpw == 4 || fpw == 8 || fpw == 16, FSTU_EARG, "fstu_down_packed_res: fpw=%d not in {4,8,16}", fpw);
-  FSTU_REQUIRE(ldact >= I && ldact % 8 == 0, FSTU_ESHAPE, "fstu_down_packed_res: ldact=%d", ldact);
-  FSTU_REQUIRE(fstu_aligned(act, 16) && fstu_aligned(wp_down, 16) && fstu_aligned(x_res, 8) && fstu_aligned(x_out, 8),
-               FSTU_EALIGN, "fstu_down_packed_res: pointers must be 16-byte aligned");
-  DownArgs a;
-  a.act = (const bf16_t*)act; a.wp_down = (const uint4*)wp_down; a.x_res = (const bf16_t*)x_res; a.x_out = (bf16_t*)x_out;
-  a.rows = rows; a.d = d; a.I = I; a.ldact = ldact; a.fpw = fpw;
-  hipLaunchKernelGGL(down_res_kernel<9>, dim3((d + fpw - 1) / fpw), dim3(512), 0, (hipStream_t)stream, a);
-  FSTU_CHECK_LAUNCH("fstu_down_packed_res");
-  return FSTU_OK;
-}
-
 // Balanced split-K down projection: partial (ksplit, rows, d) fp32 slices, summed by fstu_add_rmsnorm(delta_mode 1).
 // Returns the number of slices through *ksplit_out (16, the K chunks of the launch).
 extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
@@ -1191,32 +598,4 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
   if (ksplit_io) *ksplit_io = KS;
   return FSTU_OK;
-}
-
-// Tied head with the greedy pick over packed weights: logits (rows, ldy) and, through best_ws (rows*64 64-bit words,
-// zero between calls) and the finish launch, the index of the largest logit per row (lowest index on ties).
-int fstu_argmax_finish_launch(void* best_ws, int64_t* tok_out, int64_t tok_stride, int rows, int* dyn, int advance, void* stream);
-
-int fstu_head_packed_argmax_dyn(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
-                                float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
-                                void* stream) {
-  FSTU_REQUIRE(x && wp && logits && best_ws && tok_out, FSTU_ENULL, "fstu_head_packed_argmax: null pointer");
-  FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N), FSTU_ESHAPE, "fstu_head_packed_argmax: unsupported shape rows=%d K=%d N=%d", rows, K, N);
-  FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && tok_stride >= 1 && temperature > 0.f, FSTU_EARG,
-               "fstu_head_packed_argmax: bad ldx / ldy / stride / temperature");
-  FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(wp, 16) && fstu_aligned(logits, 2) && fstu_aligned(best_ws, 8), FSTU_EALIGN,
-               "fstu_head_packed_argmax: pointers must be 16-byte aligned");
-  GluArgs a = {};
-  a.h = (const bf16_t*)x; a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)logits;
-  a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy;
-  a.best_ws = (unsigned long long*)best_ws; a.temperature = temperature;
-  int rc = glu_launch(a, false, 2, "fstu_head_packed_argmax", (hipStream_t)stream);
-  if (rc) return rc;
-  return fstu_argmax_finish_launch(best_ws, tok_out, tok_stride, rows, dyn, advance, stream);
-}
-
-extern "C" int fstu_head_packed_argmax(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
-                                       float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, void* stream) {
-  return fstu_head_packed_argmax_dyn(x, ldx, wp, logits, ldy, rows, N, K, temperature, best_ws, tok_out, tok_stride, nullptr, 0,
-                                     stream);
 }

@@ -308,15 +308,6 @@ extern "C" int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, cons
 typedef __bf16 stu_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float stu_floatx4_t __attribute__((ext_vector_type(4)));
 
-#ifdef FSTU_GLU_TRACE
-__device__ long long stu_trace_buf[48 * 8];
-#define STU_STAMP(k) do { if (threadIdx.x == 0 && blockIdx.x < 48) stu_trace_buf[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
-extern "C" int fstu_stu_trace(long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(stu_trace_buf), sizeof(long long) * 48 * 8);
-}
-#else
-#define STU_STAMP(k) do { } while (0)
-#endif
 __global__ void __launch_bounds__(256)
 stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
                        float* __restrict__ state, const float* __restrict__ a, const float* __restrict__ ce,
@@ -332,7 +323,6 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   __shared__ float red[4][64][4];
   __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
   extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
-  STU_STAMP(0);
   if (dyn) parity = dyn[0] & 1;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -398,10 +388,8 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     if (exact3) pro3.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
     else pro.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
     __syncthreads();
-    STU_STAMP(1);
     if (exact3) pro3.scale(ss_part, hs, ldn, B, K, eps); else pro.scale(ss_part, hs, ldn, B, K, eps);
     __syncthreads();
-    STU_STAMP(2);
     hp = hs + (size_t)(xrow ? r : 0) * ldn + w * kw + g * 16;
   } else if (x_res) {
     // h = rmsnorm(x_res) * norm_w for all rows into LDS (every workgroup recomputes it: B*K*2 bytes of input)
@@ -473,7 +461,6 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[w][lane][i] = acc[i];
   __syncthreads();
-  STU_STAMP(3);
   if (w == 0) {
     // D layout: lane holds channels 4*g+i of batch row r
 #pragma unroll
@@ -484,7 +471,6 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     }
   }
   __syncthreads();
-  STU_STAMP(4);
   // ---- recurrence step of the tile's channels
   for (int b = bsub; b < B; b += 8) {
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -575,7 +561,6 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
       }
     }
   }
-  STU_STAMP(5);
 }
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
                               float* state, const float* a, const float* ce, const float* co, void* y, int ldy, void* xp_out,
@@ -586,13 +571,6 @@ int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* stat
                              const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn,
                              void* stream) {
   return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, dyn, stream);
-}
-
-int fstu_stu_norm_inproj_step_dyn(const void* x_res, const void* norm_w, float eps, const void* Mt, float* state, const float* a,
-                                  const float* ce, const float* co, void* y, int ldy, int B, int S, int d, int K, int t,
-                                  const int* dyn, void* stream) {
-  FSTU_REQUIRE(x_res && norm_w, FSTU_ENULL, "fstu_stu_norm_inproj_step: null pointer");
-  return inproj_step_launch(x_res, K, x_res, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream);
 }
 
 // x' = x_in + T(sum of nslices <= 4 fp32 slices) goes to x_out, h = rmsnorm(x') * norm_w feeds the projection: the

@@ -52,29 +52,20 @@ SIGNATURES = {
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_swa_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_append_decode": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
-    "fstu_swa_qkv_decode": [_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_swa_prefill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp],
     "fstu_swa_prefill_ws_elems": [_i, _i, _i, _i],
     "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
     "fstu_head_argmax_static": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i64, _i, _vp],
-    "fstu_head_packed_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _vp],
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
     "fstu_packed_elems": [_i, _i],
-    "fstu_gemv_packed": [_vp, _vp],
-    "fstu_set_gemv_target_workgroups": [_i],
     "fstu_glu_packed_supported": [_i, _i, _i],
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed_res": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
-    "fstu_down_packed_res": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
-    "fstu_mlp_block_sync_bytes": [],
-    "fstu_mlp_block_trace": [_vp],
-    "fstu_mlp_block_plan": [_i, _i, _i, _vp, _vp, _vp],
-    "fstu_mlp_block": [_vp] * 12 + [_i, _i, _i, _f, _vp],
     "fstu_step_mega_ws_bytes": [_vp],
     "fstu_step_mega_prepare": [_vp, _vp, _vp],
     "fstu_step_mega_status": [_vp, _vp],
@@ -83,7 +74,6 @@ SIGNATURES = {
     "fstu_decode_graph_launch": [_vp, _vp],
     "fstu_decode_graph_seek": [_vp, ctypes.c_longlong],
     "fstu_decode_graph_destroy": [_vp],
-    "fstu_set_warm_workgroups": [_i],
     "fstu_prof_begin": [_i, _i],
     "fstu_prof_end": [_vp, _vp],
     "fstu_prof_copy": [_vp, _vp, ctypes.c_size_t, _vp],
@@ -117,7 +107,6 @@ def load(path: Optional[str] = None):
         fn.restype = ctypes.c_int
     lib.fstu_packed_elems.restype = ctypes.c_int64
     lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
-    lib.fstu_mlp_block_sync_bytes.restype = ctypes.c_size_t
     lib.fstu_step_mega_ws_bytes.restype = ctypes.c_size_t
     lib.fstu_lds_sequence_ws_floats.restype = ctypes.c_size_t
     if path is None:
@@ -530,24 +519,6 @@ def swa_decode(qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slop
     return out
 
 
-def swa_qkv_decode(wp_qkv: torch.Tensor, kring: torch.Tensor, vring: torch.Tensor, slopes: torch.Tensor, pos: int,
-                   window: int, softcap: float, h: Optional[torch.Tensor] = None, x: Optional[torch.Tensor] = None,
-                   partial: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0):
-    """QKV projection + ring append + one-token attention in one launch.  Give h (B,d) normalised rows, or x (B,d)
-    with norm_w (and optionally partial (ns,B,d) fp32 slices to add first).  Returns out (B,d), or (x', out)."""
-    _dev(wp_qkv, kring, vring, slopes, h, x, partial, norm_w)
-    src = h if h is not None else x
-    B, d = src.shape
-    _, H, cap, hd = kring.shape
-    out = torch.empty(B, d, dtype=src.dtype, device=src.device)
-    x_out = torch.empty_like(x) if x is not None else None
-    ns = 0 if partial is None else partial.shape[0]
-    _check(load().fstu_swa_qkv_decode(_p(h), _p(x), _p(partial), ns, _p(x_out), _p(norm_w), float(eps), _p(wp_qkv), _p(kring),
-                                      _p(vring), _p(out), _p(slopes), B, H, hd, cap, pos, window, float(softcap), _stream()),
-           "fstu_swa_qkv_decode")
-    return out if x is None else (x_out, out)
-
-
 def swa_prefill(qkv: torch.Tensor, slopes: torch.Tensor, n_heads: int, window: int, softcap: float,
                 out: Optional[torch.Tensor] = None, force_valu: bool = False) -> torch.Tensor:
     """Prefill attention: the MFMA kernel for bf16 with head dim 64/128, the wave-per-query kernel otherwise."""
@@ -597,13 +568,6 @@ def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best
                                    _p(best_ws), out_tokens.data_ptr(), out_tokens.stride(0), _dt(x), _stream()),
            "fstu_head_argmax")
     return logits
-
-
-class GemvArgs(ctypes.Structure):
-    _fields_ = [("mode", _i), ("rows", _i), ("N", _i), ("K", _i), ("Wp", _vp), ("Wp2", _vp), ("x", _vp), ("ldx", _i),
-                ("res_in", _vp), ("delta", _vp), ("res_out", _vp), ("norm_w", _vp), ("eps", _f), ("y", _vp), ("ldy", _i),
-                ("ksplit", _i), ("partial_ws", _vp), ("counters", _vp), ("temperature", _f), ("best_ws", _vp),
-                ("tok_out", _vp), ("tok_stride", _i64)]
 
 
 def pack_rows(W: torch.Tensor) -> torch.Tensor:
@@ -658,19 +622,6 @@ def linear_packed(x: torch.Tensor, wp: torch.Tensor, N: int, norm_w: Optional[to
     return out
 
 
-def down_packed_res(act: torch.Tensor, wp_down: torch.Tensor, x_res: torch.Tensor, fpw: int = 8,
-                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x_res + act @ Wd^T over packed Wd (d,I), complete in one launch; `out` may be x_res itself."""
-    _dev(act, wp_down, x_res, out)
-    rows, I = act.shape
-    d = x_res.shape[1]
-    if out is None:
-        out = torch.empty_like(x_res)
-    _check(load().fstu_down_packed_res(_p(act), I, _p(wp_down), _p(x_res), _p(out), rows, d, I, fpw, _stream()),
-           "fstu_down_packed_res")
-    return out
-
-
 def down_packed_splitk(act: torch.Tensor, wp_down: torch.Tensor, d: int, ksplit: int = 16) -> torch.Tensor:
     """Balanced split-K down projection: returns the fp32 slices (ksplit, rows, d); their sum in slice order is the
     result.  ksplit: 4, 8 or 16."""
@@ -694,81 +645,6 @@ def linear_packed_res(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tens
     _check(load().fstu_linear_packed_res(_p(x), _p(partial), ns, _p(x_out), _p(norm_w), float(eps), _p(wp), _p(y), N, rows,
                                          N, K, _stream()), "fstu_linear_packed_res")
     return x_out, y
-
-
-def head_packed_argmax(x: torch.Tensor, wp: torch.Tensor, N: int, temperature: float, best_ws: torch.Tensor,
-                       tok_out: torch.Tensor):
-    """Tied head over packed weights + greedy pick: returns logits (rows,N); tok_out (rows,) int64 receives the ids."""
-    _dev(wp, best_ws)
-    rows, ldx = _rows_view(x)
-    K = x.shape[1]
-    logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
-    assert tok_out.dtype == torch.int64 and tok_out.is_cuda and tok_out.dim() == 1 and tok_out.shape[0] == rows
-    _check(load().fstu_head_packed_argmax(_p(x), ldx, _p(wp), _p(logits), N, rows, N, K, float(temperature), _p(best_ws),
-                                          tok_out.data_ptr(), tok_out.stride(0), _stream()), "fstu_head_packed_argmax")
-    return logits
-
-
-def mlp_block_sync_bytes() -> int:
-    return int(load().fstu_mlp_block_sync_bytes())
-
-
-def mlp_block_plan(rows: int, d: int, I: int):
-    """(grid, K split, floats of partial workspace) of the one-launch MLP sub-layer, or None if unsupported."""
-    g, ks, pf = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
-    rc = load().fstu_mlp_block_plan(rows, d, I, ctypes.byref(g), ctypes.byref(ks), ctypes.byref(pf))
-    return None if rc != 0 else (g.value, ks.value, pf.value)
-
-
-def mlp_block(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torch.Tensor, wp_gate: torch.Tensor,
-              wp_up: torch.Tensor, wp_down: torch.Tensor, next_norm_w: Optional[torch.Tensor], I: int, eps: float,
-              ws: Optional[dict] = None):
-    """One launch: x <- x + delta + MLP(rmsnorm(x + delta)); returns (x, rmsnorm(x) * next_norm_w or None).
-    x is updated in place.  `ws` caches the workspaces between calls."""
-    _dev(x, delta, norm_w, wp_gate, wp_up, wp_down, next_norm_w)
-    rows, d = x.shape
-    plan = mlp_block_plan(rows, d, I)
-    if plan is None or x.dtype != torch.bfloat16:
-        raise FlashSTUHipError(f"fstu_mlp_block does not support rows={rows} d={d} I={I} dtype={x.dtype}")
-    ws = {} if ws is None else ws
-    if "sync" not in ws:
-        ws["sync"] = torch.zeros(mlp_block_sync_bytes() // 4, dtype=torch.int32, device=x.device)
-        ws["partial"] = torch.empty(plan[2], dtype=torch.float32, device=x.device)
-        ws["act"] = torch.empty(rows, I, dtype=x.dtype, device=x.device)
-    h = torch.empty_like(x) if next_norm_w is not None else None
-    _check(load().fstu_mlp_block(_p(x), _p(delta), _p(x), _p(norm_w), _p(wp_gate), _p(wp_up), _p(wp_down),
-                                 _p(next_norm_w), _p(h), _p(ws["act"]), _p(ws["partial"]), _p(ws["sync"]), rows, d, I,
-                                 float(eps), _stream()), "fstu_mlp_block")
-    return x, h
-
-
-def gemv_packed(mode: int, Wp: torch.Tensor, N: int, K: int, out: torch.Tensor, x: Optional[torch.Tensor] = None,
-                Wp2: Optional[torch.Tensor] = None, res_in: Optional[torch.Tensor] = None,
-                delta: Optional[torch.Tensor] = None, res_out: Optional[torch.Tensor] = None,
-                norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ksplit: int = 1,
-                partial_ws: Optional[torch.Tensor] = None, counters: Optional[torch.Tensor] = None,
-                temperature: float = 1.0, best_ws: Optional[torch.Tensor] = None,
-                tok_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Thin wrapper over fstu_gemv_packed (see include/flashstu_hip.h for the modes)."""
-    _dev(Wp, Wp2, res_in, delta, res_out, norm_w, partial_ws, counters, best_ws)
-    a = GemvArgs()
-    rows = out.shape[0]
-    a.mode, a.rows, a.N, a.K = mode, rows, N, K
-    a.Wp, a.Wp2 = _p(Wp), _p(Wp2)
-    if x is not None:
-        xr, ldx = _rows_view(x)
-        assert xr == rows and x.shape[1] == K
-        a.x, a.ldx = x.data_ptr(), ldx
-    a.res_in, a.delta, a.res_out, a.norm_w, a.eps = _p(res_in), _p(delta), _p(res_out), _p(norm_w), float(eps)
-    orow, ldy = _rows_view(out)
-    a.y, a.ldy = out.data_ptr(), ldy
-    a.ksplit, a.partial_ws, a.counters = ksplit, _p(partial_ws), _p(counters)
-    a.temperature, a.best_ws = float(temperature), _p(best_ws)
-    if tok_out is not None:
-        assert tok_out.dtype == torch.int64 and tok_out.dim() == 1 and tok_out.shape[0] == rows
-        a.tok_out, a.tok_stride = tok_out.data_ptr(), tok_out.stride(0)
-    _check(load().fstu_gemv_packed(ctypes.byref(a), _stream()), "fstu_gemv_packed")
-    return out
 
 
 def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,

@@ -41,18 +41,13 @@ class ModelDesc(ctypes.Structure):
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
-                ("wp_emb", _vp), ("x2", _vp), ("yd", _vp), ("partial_fix", _vp), ("counters", _vp),
-                ("mlp_partial", _vp), ("mlp_sync", _vp), ("glu_packed", _i), ("res_chain", _i),
-                ("down_fpw", _i), ("down_packed", _i), ("head_packed", _i), ("merge_norm", _i), ("swa_fused", _i),
+                ("wp_emb", _vp), ("x2", _vp), ("glu_packed", _i), ("down_packed", _i), ("merge_norm", _i),
                 ("mega_ws", _vp)]
 
 
 def pick_ksplit_down(I: int) -> int:
     """K split of the down projection: enough waves to fill 256 CUs while every
     slice still divides into the 64-wide k steps of the MFMA kernel."""
-    forced = int(os.environ.get("FSTU_KSPLIT_DOWN", "0"))
-    if forced > 0 and I % (forced * 64) == 0:
-        return forced
     for ks in (12, 16, 8, 6, 4, 3, 2):
         if I % (ks * 256) == 0:
             return ks
@@ -109,14 +104,6 @@ class DecodeEngine:
             hit = (w._version, _hip.pack_rows(w))
             self._packed[key] = hit
         return hit[1]
-
-    def _use_packed(self, B: int) -> bool:
-        if os.environ.get("FSTU_PACKED_STEP", "0") != "1":
-            return False
-        cfg = self.cfg
-        d, I = cfg.n_embd, cfg.n_embd * cfg.mlp_scale
-        return (cfg.torch_dtype == torch.bfloat16 and cfg.resolved_stu_decode_mode() == "lds" and d % 128 == 0
-                and I % (128 * pick_ksplit_down(I)) == 0 and B * (d + 8) * 2 + 8192 <= 64 * 1024)
 
     @property
     def desc(self) -> ModelDesc:
@@ -230,89 +217,25 @@ class DecodeEngine:
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = ch.logits.data_ptr()
         m.best = buf(16 * 64, dtype=torch.int64).data_ptr()
-        if (dt == torch.bfloat16 and d % 128 == 0 and B * (d + 8) * 2 + 16384 <= 64 * 1024
-                and os.environ.get("FSTU_GLU_PROLOGUE", "0") == "1"):
-            # experimental: MLP norm fused into the GLU GEMV (packed gate/up copies + a second residual buffer);
-            # measured slower than the separate norm kernel (0.494 vs 0.475 ms per step), hence off by default
-            for i, layer in enumerate(model.layers):
-                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
-                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
-            m.x2 = buf(B, d).data_ptr()
-        if (dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(B, d, I)
-                and os.environ.get("FSTU_GLU_PACKED", "1") == "1"):
+        if dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(B, d, I):
             # gate/up projection over packed weights, one workgroup per CU with equal bytes each
             for i, layer in enumerate(model.layers):
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
             m.glu_packed = 1
-            if os.environ.get("FSTU_DOWN_PACKED", "1") == "1" and I % 512 == 0 and d % 16 == 0:
+            if I % 512 == 0 and d % 16 == 0:
                 for i, layer in enumerate(model.layers):
                     arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
                 m.down_packed = 1
-            if os.environ.get("FSTU_HEAD_PACKED", "0") == "1":     # measured 3 us slower than the row-major head kernel
-                m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
-                m.head_packed = 1
-            if os.environ.get("FSTU_PACKED_QKV", "0") == "1":
-                for i, layer in enumerate(model.layers):
-                    if isinstance(layer, AttentionLayer):
-                        arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
-                        arr[i].wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
-            if os.environ.get("FSTU_GLU_NORM", "1") == "1" and B * (d + 8) * 2 <= 96 * 1024:
+            if B * (d + 8) * 2 <= 96 * 1024:
                 m.x2 = buf(B, d).data_ptr()     # second residual buffer: the MLP norm runs as the gate/up prologue
-                if mode == "lds" and d % 256 == 0 and os.environ.get("FSTU_RES_CHAIN", "0") == "1":
-                    # opt-in: down projection adds into the residual stream, the next sub-layer normalises in its
-                    # prologue (12 launches fewer).  Measured slower, 0.503 vs 0.454 ms per step: the down projection
-                    # without a split across workgroups takes 5 us longer than the split-K kernel and the norm
-                    # prologues add 2.8 us to each consumer, more than the removed add+norm launches cost
-                    for i, layer in enumerate(model.layers):
-                        arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
-                        if isinstance(layer, AttentionLayer):
-                            arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
-                    m.res_chain = 1
-                    m.down_fpw = int(os.environ.get("FSTU_DOWN_FPW", "8"))
-                elif (mode == "lds" and d % 256 == 0 and m.down_packed and B * (d // 8) <= 1024 and I % 128 == 0
-                      and os.environ.get("FSTU_MERGE_NORM", "1") == "1"):
+                if mode == "lds" and d % 256 == 0 and m.down_packed and B * (d // 8) <= 1024 and I % 128 == 0:
                     # the add+norm between two layers runs as the prologue of the next layer's first projection
                     # (the down projection leaves 4 split-K slices for it): one launch less per layer
                     for i, layer in enumerate(model.layers):
                         if isinstance(layer, AttentionLayer):
                             arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
                     m.merge_norm = 1
-            if (d // cfg.n_heads == 64 and d % 256 == 0 and d <= 768 and not m.res_chain
-                    and os.environ.get("FSTU_SWA_FUSED", "0") == "1"):
-                # opt-in: QKV projection inside the attention launch (one launch less per attention layer).  Measured
-                # equal to the separate launches inside the step (0.362 vs 0.361 ms): each (row, head) workgroup
-                # re-reads the head's 295 KB of weights through its own CU
-                for i, layer in enumerate(model.layers):
-                    if isinstance(layer, AttentionLayer) and not arr[i].wp_qkv:
-                        arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
-                m.swa_fused = 1
-        plan = _hip.mlp_block_plan(B, d, I) if dt == torch.bfloat16 else None
-        if plan is not None and os.environ.get("FSTU_FUSED_MLP", "0") == "1":
-            # opt-in: the MLP sub-layer as one persistent launch per layer (packed gate/up/down copies + its
-            # workspaces).  Correct and tested, but measured slower inside the full step (0.485 vs 0.472 ms): its
-            # ~14 dependent device-scope round trips of 1.3-1.5 us each cost as much as the launches they replace
-            for i, layer in enumerate(model.layers):
-                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
-                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
-                arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
-            m.mlp_partial = buf(plan[2], dtype=torch.float32).data_ptr()
-            m.mlp_sync = buf(_hip.mlp_block_sync_bytes() // 4, dtype=torch.int32).data_ptr()
-        if self._use_packed(B):
-            for i, layer in enumerate(model.layers):
-                ld = arr[i]
-                ld.wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
-                ld.wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
-                ld.wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
-                if isinstance(layer, STULayer):
-                    ld.wp_m_inputs = self._pack(layer.stu.m_inputs_t()).data_ptr()
-                else:
-                    ld.wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
-                    ld.wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
-            m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
-            m.x2, m.yd = buf(B, d).data_ptr(), buf(B, d).data_ptr()
-            m.partial_fix = buf(m.ksplit_down * ((d + 15) // 16) * 256, dtype=torch.float32).data_ptr()
-            m.counters = buf((d + 15) // 16, dtype=torch.int32).data_ptr()
         ch.arr, ch.desc = arr, m
         ch.mega = None
         if (dt == torch.bfloat16 and mode == "lds" and m.glu_packed and m.down_packed and not cfg.use_hankel_L
@@ -371,8 +294,7 @@ class DecodeEngine:
         n = int(steps_per_graph)
         self.graph_steps = n
         # a persistent one-launch step needs every compute unit: row chunks then replay one after the other
-        concurrent = (os.environ.get("FSTU_CHUNK_STREAMS", "1") == "1"
-                      and not any(getattr(ch, "mega", None) is not None for ch in self.chunks))
+        concurrent = not any(getattr(ch, "mega", None) is not None for ch in self.chunks)
         n_streams = len(self.chunks) if concurrent else 1
         if not self._gstreams:
             self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]

@@ -264,16 +264,6 @@ int fstu_swa_append_decode(const void* qkv, void* kring, void* vring, void* out,
                            int B, int H, int hd, int cap, int pos, int window, float softcap, int dtype,
                            void* stream);
 
-/* QKV projection + ring append + decode in one launch (reference: flash_stu/modules/attention.py:66-105 for one new
- * token): every (batch row, head) workgroup forms its own q, k, v = h W_qkv^T from the packed weight (fstu_pack_rows of
- * c_attn.weight (3d,d)).  h is given (h_in, (B,d) normalised rows; x_in NULL) or formed here from the residual stream
- * (h_in NULL): x' = T(x_in + T(sum of nslices <= 4 fp32 (B,d) slices)), h = rmsnorm(x') * norm_w
- * (attention_layer.py:53-57); x' goes to x_out (not x_in itself).  Head dim 64, d % 256 == 0, d <= 768, bf16. */
-int fstu_swa_qkv_decode(const void* h_in, const void* x_in, const float* slices, int nslices, void* x_out,
-                        const void* norm_w, float eps, const void* wp_qkv, void* kring, void* vring, void* out,
-                        const float* slopes, int B, int H, int hd, int cap, int pos, int window, float softcap,
-                        void* stream);
-
 /* Prefill form: qkv (B,T,3*H*hd), positions 0..T-1, out (B,T,H*hd). */
 int fstu_swa_prefill(const void* qkv, void* out, const float* slopes, int B, int T, int H, int hd,
                      int window, float softcap, int dtype, void* stream);
@@ -337,82 +327,14 @@ size_t fstu_lds_sequence_ws_floats(int T, int Bt, int S);
 int fstu_lds_sequence(float* h, const void* x, const float* A, const void* BmT, const void* CmT, void* y, float* ws,
                       int T, int Bt, int d_in, int S, int d_out, void* stream);
 
-/* ---- decode GEMVs over packed weights ---------------------------------------
+/* ---- packed weights -------------------------------------------------------------
  * Packed layout of an (N,K) bf16 row-major weight, K % 32 == 0 (fstu_pack_rows):
  *   Wp[tile][kstep][lane][8],  tile = n/16, kstep = k/32, lane = 16*g + r,
- *   element e of lane (r,g) = W[16*tile + r][32*kstep + 8*g + e]; rows >= N are zero.
- * fstu_packed_elems(N,K) is the number of bf16 elements of the packed copy.
- * fstu_gemv_packed computes, for rows <= 16 activation rows,
- *   mode 0: y[m,n] = T(h[m,:] . W[n,:])
- *   mode 1: y[m,i] = T( T(gelu_tanh(T(h.Wg[i]))) * T(h.Wu[i]) )        (Wp = gate, Wp2 = up)
- *   mode 2: mode 0 with K split over `ksplit` workgroups per feature tile; the last
- *           workgroup of a tile to finish adds the fp32 partials in slice order
- *           (deterministic).  partial_ws: ksplit*ceil(N/16)*256 floats; counters:
- *           ceil(N/16) uint32, zero before the first call (left zero).
- *   mode 3: mode 0 plus the greedy pick of fstu_head_argmax; best_ws: rows*64 uint64,
- *           zero before the first call (left zero).
- * Activations h: if norm_w == NULL, h = x (rows,K) with row stride ldx.  Otherwise the
- * fused prologue h = RMSNorm(T(res_in + delta)) * norm_w with res_in/delta (rows,K)
- * dense; delta may be NULL (no add); when delta != NULL and res_out != NULL the
- * updated residual T(res_in + delta) is written to res_out (must not alias res_in).
- * bf16 only; K % 128 == 0 (K % (128*ksplit) == 0 in mode 2).
- * Replaces the same reference call sites as fstu_linear_decode / fstu_glu_decode /
- * fstu_add_rmsnorm / fstu_head_argmax. */
-typedef struct {
-  int mode;
-  int rows, N, K;
-  const void* Wp;
-  const void* Wp2;
-  const void* x;
-  int ldx;
-  const void* res_in;
-  const void* delta;
-  void* res_out;
-  const void* norm_w;
-  float eps;
-  void* y;
-  int ldy;
-  int ksplit;
-  float* partial_ws;
-  unsigned* counters;
-  float temperature;
-  void* best_ws;
-  int64_t* tok_out;
-  int64_t tok_stride;
-} fstu_gemv_args;
-
+ *   element e of lane (r,g) = W[16*tile + r][32*kstep + 8*g + e]; rows >= N are zero
+ * i.e. the A-operand fragment of v_mfma_f32_16x16x32_bf16: one wave load reads 1 KB of contiguous memory.
+ * fstu_packed_elems(N,K) is the number of bf16 elements of the packed copy. */
 int64_t fstu_packed_elems(int N, int K);
 int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
-int fstu_gemv_packed(const fstu_gemv_args* a, void* stream);
-/* Tuning knob: number of workgroups a packed GEMV launch aims for (default 256 = one per CU);
- * each workgroup then walks ceil(tiles/n) consecutive tiles. */
-int fstu_set_gemv_target_workgroups(int n);
-
-/* ---- MLP sub-layer of one decode step in one launch (bf16) -------------------
- *   x' = T(x_in + delta)                       (delta may be NULL)
- *   h = rmsnorm(x') * norm_w;  act = T(gelu_tanh(T(h Wg^T))) * T(h Wu^T)
- *   x_out = T(x' + T(act Wd^T));  h_out = rmsnorm(x_out) * next_norm_w   (h_out may be NULL)
- * Replaces mlp_norm + MLP + residual add + the next sub-layer's norm of
- * flash_stu/layers/stu_layer.py:93-96, flash_stu/layers/attention_layer.py:59-62
- * and flash_stu/modules/swiglu.py:22-29 for <= 16 rows.  wp_* are fstu_pack_rows
- * copies of gate_proj (I,d), up_proj (I,d), down_proj (d,I).  x_out may alias x_in.
- * A persistent grid (one workgroup per CU, grid barrier in the middle): nothing
- * else may run on the GPU at the same time.  Workspaces, owned by the caller:
- * act_ws rows*I bf16; partial_ws and the grid size from fstu_mlp_block_plan
- * (returns FSTU_ESHAPE when the shape is not supported: d in {256,512,768,1024,2048},
- * I % 512 == 0); sync_ws fstu_mlp_block_sync_bytes() bytes, 128-byte aligned,
- * zeroed once (every launch returns it to zero; word 320 is raised if a bounded
- * spin ever timed out).
- * fstu_mlp_block_trace: profiling hook; with a device buffer of grid*8 int64 every later launch stamps the wall
- * clock (100 MHz ticks) of each workgroup at start, with x in LDS, after the norm prologue, after the gate/up
- * phase, after the barrier, at the first ticket, at the second ticket and at exit (0 where a workgroup left
- * earlier); NULL switches it off. */
-size_t fstu_mlp_block_sync_bytes(void);
-int fstu_mlp_block_trace(long long* buf);
-int fstu_mlp_block_plan(int rows, int d, int I, int* grid, int* ksplit, size_t* partial_floats);
-int fstu_mlp_block(const void* x_in, const void* delta, void* x_out, const void* norm_w, const void* wp_gate,
-                   const void* wp_up, const void* wp_down, const void* next_norm_w, void* h_out, void* act_ws,
-                   float* partial_ws, unsigned* sync_ws, int rows, int d, int I, float eps, void* stream);
 
 /* Gate/up projection with the GLU epilogue over packed weights, one workgroup per CU with equal bytes each
  * (4-feature granularity) and every weight fragment in flight from the first instruction:
@@ -434,13 +356,6 @@ int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const
  * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, rows <= 16, bf16. */
 int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                        int rows, int N, int K, void* stream);
-/* Down projection with the residual add, complete in one launch (no split across workgroups):
- *   x_out[r,f] = T( x_res[r,f] + T( act[r,:] . Wd[f,:] ) )      (swiglu.py:27 + the x.add_ of stu_layer.py:96)
- * wp_down = fstu_pack_rows of down_proj (d,I); a workgroup owns fpw (4, 8 or 16) output features over the whole K range.
- * x_out may alias x_res. */
-int fstu_down_packed_res(const void* act, int ldact, const void* wp_down, const void* x_res, void* x_out, int rows,
-                         int d, int I, int fpw, void* stream);
-
 /* Split-K form of the down projection over packed weights (reference: flash_stu/modules/swiglu.py:22-29, down_proj):
  * partial receives *ksplit_io fp32 slices (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1) or the norm prologue of
  * the next projection sums in slice order.  *ksplit_io on entry: slices wanted (4, 8 or 16; anything else: 16); on
@@ -455,13 +370,6 @@ int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, flo
  * x_out (must not alias x_in).  K % 256 == 0, rows*K/8 <= 1024, rows <= 16, bf16. */
 int fstu_linear_packed_res(const void* x_in, const float* partial, int nslices, void* x_out, const void* norm_w, float eps,
                            const void* wp, void* y, int ldy, int rows, int N, int K, void* stream);
-
-/* Tied head + greedy pick over packed weights (fstu_pack_rows of the (V,d) embedding), one workgroup per CU:
- * logits (rows,ldy) and tok_out[b*tok_stride] = argmax_v logits[b,v] (lowest index on ties) after dividing by
- * temperature and clamping to +-1e4 in the model dtype, as fstu_head_argmax (model.py:176,267-271,299).
- * best_ws: rows*64 64-bit words, zero before the first call (left zero by every call). */
-int fstu_head_packed_argmax(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
-                            float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, void* stream);
 
 /* ---- whole decode step -----------------------------------------------------
  * One call launches every kernel of one token step for all layers: embedding of
@@ -527,30 +435,16 @@ typedef struct {
   float* eo;                /* fp32 */
   void* logits;             /* (B,V) */
   void* best;               /* max(B,16)*64 64-bit words, zero-initialised once by the caller */
-  /* fused bf16 step (used when wp_emb and every layer's packed copies are set) */
-  const void* wp_emb;       /* packed tied head */
-  void* x2;                 /* (B,d) second residual buffer (the stream ping-pongs x <-> x2) */
-  void* yd;                 /* (B,d) down-projection output */
-  float* partial_fix;       /* ksplit_down * ceil(d/16) * 256 floats */
-  unsigned* counters;       /* ceil(d/16) uint32, zero-initialised once */
-  /* one-launch MLP sub-layer (fstu_mlp_block), used for every layer that has wp_gate, wp_up and wp_down when both
-   * are set and the shape is supported */
-  float* mlp_partial;       /* fstu_mlp_block_plan's partial_floats */
-  unsigned* mlp_sync;       /* fstu_mlp_block_sync_bytes(), zero-initialised once */
+  const void* wp_emb;       /* packed tied head (one-launch step) */
+  void* x2;                 /* (B,d) second residual buffer (the stream ping-pongs x <-> x2); NULL: the add + norm
+                               between sub-layers runs as launches of its own */
   int glu_packed;           /* != 0: layers with wp_gate and wp_up run their gate/up projection through fstu_glu_packed */
-  int res_chain;            /* != 0 (needs glu_packed, x2, lds mode, wp_down everywhere and wp_qkv on attention layers): the
-                               down projection adds into the residual stream (fstu_down_packed_res) and the next
-                               sub-layer normalises it in its prologue; no stand-alone add+norm launch inside the layers */
-  int down_fpw;             /* output features per workgroup of that down projection: 4, 8 (default) or 16 */
   int down_packed;          /* != 0: layers with wp_down use fstu_down_packed_splitk (16 slices: partial must hold
                                max(ksplit_down,16)*B*d floats) */
-  int head_packed;          /* != 0 and wp_emb set: the greedy path runs the tied head through fstu_head_packed_argmax */
   int merge_norm;           /* != 0 (needs glu_packed, down_packed, x2, lds mode, wp_gate/up/down everywhere and wp_qkv on
                                attention layers, B*d <= 8192): the down projection leaves 4 split-K slices and the next
                                layer's first projection adds and normalises them in its prologue
                                (fstu_stu_res_inproj_step / fstu_linear_packed_res); one add+norm launch less per layer */
-  int swa_fused;            /* != 0 (bf16, head dim 64, width <= 768, wp_qkv set): the QKV projection runs inside the
-                               attention launch (fstu_swa_qkv_decode), together with the merged add+norm when merge_norm */
   void* mega_ws;            /* != NULL: workspace of the one-launch step (fstu_step_mega_ws_bytes, fstu_step_mega_prepare);
                                fstu_decode_step and the graphs then run the whole step as ONE persistent kernel when
                                the model is covered (bf16, recurrence STU state with lds_co, packed copies of every
@@ -598,10 +492,6 @@ int fstu_decode_graph_launch(void* graph, void* stream);
  * same tokens and `dyn` have advanced the device-side position since this graph's last launch.  A graph of an even
  * number of steps is captured for one parity of its first position only; seeking it to the other parity is rejected. */
 int fstu_decode_graph_seek(void* graph, long long next_pos);
-/* The captured graph carries a parallel branch whose kernels only read the MLP / head weights a layer is about
- * to need (cache warm-up; `n` workgroups per kernel; default 0 = no such branch, which measured faster).  Applies to graphs created
- * afterwards. */
-int fstu_set_warm_workgroups(int n);
 int fstu_decode_graph_destroy(void* graph);
 
 /* ---- live kernel timing (measurement aid; no counterpart in the reference) ----

@@ -121,61 +121,6 @@ def test_mlp_decode_chain(hip, dtype, rows, d, I):
         check(rd, ref, dtype, frac=0.05, atol=(2.0 ** -7 * float(down.float().abs().max())) if dtype == torch.bfloat16 else 0.0)
 
 
-def test_packed_gemv_modes_match_the_unfused_ops(hip):
-    """Packed-weight GEMVs with fused residual+RMSNorm prologue, GLU epilogue, in-kernel split-K fix-up and
-    greedy pick against the row-major ops (which are checked against the oracle above)."""
-    g = gen(20)
-    dt = torch.bfloat16
-    B, d, I, V = 8, 768, 3072, 5003
-    x = dev(torch.randn(B, d, generator=g).to(dt))
-    delta = dev(torch.randn(B, d, generator=g).to(dt))
-    nw = dev((1 + 0.2 * torch.randn(d, generator=g)).to(dt))
-    Wg, Wu = (dev((torch.randn(I, d, generator=g) / math.sqrt(d)).to(dt)) for _ in range(2))
-    Wd = dev((torch.randn(d, I, generator=g) / math.sqrt(I)).to(dt))
-    Wh = dev((torch.randn(V, d, generator=g) / math.sqrt(d)).to(dt))
-    pg, pu, pd, ph = (hip.pack_rows(w) for w in (Wg, Wu, Wd, Wh))
-    # reference chain with the unfused kernels
-    xr = x.clone()
-    h = hip.add_rmsnorm(xr, delta, nw, O.RMS_EPS_DEFAULT)
-    act_ref = hip.glu_decode(h, Wg, Wu)
-    down_ref = hip.linear_decode(act_ref, Wd)
-    logits_ref = hip.linear_decode(h, Wh)
-    # mode 1 with prologue
-    res_out = torch.zeros_like(x)
-    act = torch.empty(B, I, dtype=dt, device="cuda")
-    hip.gemv_packed(1, pg, I, d, act, Wp2=pu, res_in=x, delta=delta, res_out=res_out, norm_w=nw, eps=O.RMS_EPS_DEFAULT)
-    assert torch.equal(res_out, xr)
-    check(act, act_ref, dt, frac=0.01)
-    # prologue without delta leaves res_out untouched and equals plain norm
-    res2 = torch.full_like(x, 7.0)
-    act2 = torch.empty_like(act)
-    hip.gemv_packed(1, pg, I, d, act2, Wp2=pu, res_in=xr, res_out=res2, norm_w=nw, eps=O.RMS_EPS_DEFAULT)
-    assert torch.equal(act2, act) and bool((res2 == 7.0).all())
-    # mode 2: split-K with fix-up, twice (counters must return to zero), and unsplit
-    ws = torch.zeros(12 * 48 * 256, device="cuda")
-    cnt = torch.zeros(48, dtype=torch.int32, device="cuda")
-    for _ in range(2):
-        y = torch.empty(B, d, dtype=dt, device="cuda")
-        hip.gemv_packed(2, pd, d, I, y, x=act_ref, ksplit=12, partial_ws=ws, counters=cnt)
-        check(y, down_ref, dt, frac=0.01)
-        assert int(cnt.abs().sum()) == 0
-    y1 = torch.empty(B, d, dtype=dt, device="cuda")
-    hip.gemv_packed(2, pd, d, I, y1, x=act_ref, ksplit=1)
-    check(y1, down_ref, dt, frac=0.01)
-    # mode 0 plain (N not a multiple of 16) and mode 3 greedy pick
-    lg = torch.empty(B, V, dtype=dt, device="cuda")
-    hip.gemv_packed(0, ph, V, d, lg, x=h)
-    check(lg, logits_ref, dt, frac=0.01)
-    best = torch.zeros(16 * 64, dtype=torch.int64, device="cuda")
-    toks = torch.full((B, 2), -1, dtype=torch.int64, device="cuda")
-    lg3 = torch.empty(B, V, dtype=dt, device="cuda")
-    hip.gemv_packed(3, ph, V, d, lg3, res_in=x, delta=delta, res_out=res_out, norm_w=nw, eps=O.RMS_EPS_DEFAULT,
-                    temperature=0.9, best_ws=best, tok_out=toks[:, 1])
-    assert torch.equal(lg3, lg)
-    ref_tok = O.next_token(lg3.cpu(), temperature=0.9, do_sample=False)[:, 0]
-    assert torch.equal(toks[:, 1].cpu(), ref_tok) and int(best.abs().sum()) == 0 and bool((toks[:, 0] == -1).all())
-
-
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gelu_mul(hip, dtype):
     g = gen(5)
@@ -734,80 +679,6 @@ def test_argument_errors_do_not_launch(hip):
                        torch.zeros(2, device="cuda"), 3, 8, 50.0)
 
 
-@pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 512, 2048), (8, 1024, 4096), (4, 2048, 8192)])
-def test_mlp_block_one_launch(hip, rows, d, I):
-    """The one-launch MLP sub-layer against the oracle's residual add + RMSNorm + MLP + residual add + RMSNorm,
-    launched three times on the same workspaces (its counters must return to zero)."""
-    dtype = torch.bfloat16
-    g = gen(31)
-    x = torch.randn(rows, d, generator=g).to(dtype)
-    delta = (0.5 * torch.randn(rows, d, generator=g)).to(dtype)
-    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
-    nw2 = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
-    wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
-    wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
-    wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
-    x1 = x + delta
-    h = O.rms_norm(x1, nw, O.RMS_EPS_DEFAULT)
-    y = O.mlp_forward(h, {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd})
-    x2 = x1 + y
-    h2 = O.rms_norm(x2, nw2, O.RMS_EPS_DEFAULT)
-    pg, pu, pd = hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu)), hip.pack_rows(dev(wd))
-    ws = {}
-    for it in range(3):
-        xd = dev(x).clone()
-        xo, ho = hip.mlp_block(xd, dev(delta), dev(nw), pg, pu, pd, dev(nw2), I, O.RMS_EPS_DEFAULT, ws)
-        torch.cuda.synchronize()
-        assert int(ws["sync"].abs().sum()) == 0, "counters not returned to zero / spin timeout flag raised"
-        sc = float(x2.float().abs().max())
-        check(xo, x2, dtype, frac=0.10, scale=sc, atol=2.0 ** -7 * float(y.float().abs().max()))
-        err = (ho.float().cpu() - h2.float()).abs().max() / h2.float().abs().max()
-        assert float(err) <= 2e-2
-    # no delta, no trailing norm
-    xd = dev(x).clone()
-    xo, ho = hip.mlp_block(xd, None, dev(nw), pg, pu, pd, None, I, O.RMS_EPS_DEFAULT, ws)
-    h0 = O.rms_norm(x, nw, O.RMS_EPS_DEFAULT)
-    y0 = O.mlp_forward(h0, {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd})
-    assert ho is None
-    check(xo, x + y0, dtype, frac=0.10, scale=float((x + y0).float().abs().max()), atol=2.0 ** -7 * float(y0.float().abs().max()))
-
-
-@pytest.mark.parametrize("B,H,W,ns", [(8, 12, 512, 4), (3, 4, 16, 2), (2, 8, 40, 0)])
-def test_swa_qkv_decode_equals_projection_then_decode(hip, B, H, W, ns):
-    """QKV projection (+ split-K slices, residual and RMSNorm in front of it) inside the attention launch == the
-    separate launches: add+norm, packed QKV projection, append+decode.  Ring and residual bit for bit; the output up
-    to the K split of the projection.  Several positions, the ring wrapping in the small cases."""
-    dtype = torch.bfloat16
-    g = gen(71)
-    hd, d, cap = 64, H * 64, W + 1
-    Wqkv = (torch.randn(3 * d, d, generator=g) / math.sqrt(d)).to(dtype)
-    wp = hip.pack_rows(dev(Wqkv))
-    nw = dev((1 + 0.1 * torch.randn(d, generator=g)).to(dtype))
-    slopes = dev(torch.tensor([0.25 * 2.0 ** (-(h + 1) * 8.0 / H) for h in range(H)], dtype=torch.float32))
-    kr1 = dev((0.5 * torch.randn(B, H, cap, hd, generator=g)).to(dtype))
-    vr1 = dev(torch.randn(B, H, cap, hd, generator=g).to(dtype))
-    kr2, vr2, kr3, vr3 = kr1.clone(), vr1.clone(), kr1.clone(), vr1.clone()
-    for pos in (W + 7, W + 8, 3 * W + 1):
-        x = dev(torch.randn(B, d, generator=g).to(dtype))
-        part = dev(0.3 * torch.randn(ns, B, d, generator=g)) if ns else None
-        x_ref = x.clone()
-        h = (hip.add_rmsnorm(x_ref, part, nw, O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ns) if ns
-             else hip.add_rmsnorm(x_ref, None, nw, O.RMS_EPS_DEFAULT))
-        qkv = hip.linear_packed(h, wp, 3 * d)
-        ref = hip.swa_decode(qkv, kr1, vr1, slopes, pos, W, 50.0, append=True)
-        x_out, out = hip.swa_qkv_decode(wp, kr2, vr2, slopes, pos, W, 50.0, x=x, partial=part, norm_w=nw,
-                                        eps=O.RMS_EPS_DEFAULT)
-        assert torch.equal(x_out, x_ref)
-        out_h = hip.swa_qkv_decode(wp, kr3, vr3, slopes, pos, W, 50.0, h=h)
-        for o in (out, out_h):
-            check(o, ref, dtype, frac=0.10, atol=2.0 ** -8 * float(ref.float().abs().max()))
-        # the appended keys / values: equal up to a rounding flip of the projection
-        for a, b_ in ((kr2, kr1), (vr2, vr1), (kr3, kr1), (vr3, vr1)):
-            dk = (a.float() - b_.float()).abs()
-            assert float(dk.max()) <= 2.0 ** -7 * float(b_.float().abs().max())
-            assert float((dk > 0).float().mean()) <= 1e-3
-
-
 @pytest.mark.parametrize("B,H,hd,W,T", [(2, 4, 64, 16, 50), (2, 12, 64, 512, 700), (1, 4, 128, 32, 100),
                                          (1, 2, 64, 1000, 333), (1, 2, 128, 64, 17)])
 def test_swa_prefill_mfma(hip, B, H, hd, W, T):
@@ -893,14 +764,11 @@ def test_glu_packed_balanced(hip, rows, d, I):
     close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
 
 
-@pytest.mark.parametrize("by4", ["0", "1"])
 @pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192),
                                       (16, 2048, 4096)])     # the last: more chunks than threads x 4, wave-per-row norm
-def test_glu_packed_norm_prologue(hip, rows, d, I, monkeypatch, by4):
+def test_glu_packed_norm_prologue(hip, rows, d, I):
     """Residual add + RMSNorm as the prologue of the balanced gate/up launch == the separate add+norm kernel followed
-    by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored.  Features dealt to the
-    workgroups in groups of 8 (default) and of 4."""
-    monkeypatch.setenv("FSTU_GLU_BY4", by4)
+    by the plain balanced launch (same arithmetic, bit for bit), and the sum is stored."""
     dtype = torch.bfloat16
     g = gen(61)
     x = torch.randn(rows, d, generator=g).to(dtype)
@@ -920,24 +788,6 @@ def test_glu_packed_norm_prologue(hip, rows, d, I, monkeypatch, by4):
     assert float((diff > 0).float().mean()) <= 0.10
     x_out2, act2 = hip.glu_packed_norm(dev(x), None, dev(nw), O.RMS_EPS_DEFAULT, pg, pu, I)
     assert torch.equal(x_out2.cpu(), x)
-
-
-@pytest.mark.parametrize("rows,d,I,fpw", [(8, 768, 9216, 8), (8, 768, 9216, 4), (3, 256, 512, 16), (16, 1024, 4096, 8),
-                                          (5, 100, 800, 4)])
-def test_down_packed_res(hip, rows, d, I, fpw):
-    """Down projection + residual add in one launch against the float64-accumulated specification."""
-    dtype = torch.bfloat16
-    g = gen(62)
-    act = torch.randn(rows, I, generator=g).to(dtype)
-    x = torch.randn(rows, d, generator=g).to(dtype)
-    wd = (torch.randn(d, I, generator=g) / math.sqrt(I)).to(dtype)
-    y = (act.double() @ wd.double().t()).to(dtype)
-    ref = x + y
-    out = hip.down_packed_res(dev(act), hip.pack_rows(dev(wd)), dev(x), fpw)
-    check(out, ref, dtype, frac=0.05, atol=2.0 ** -8 * float(y.float().abs().max()))
-    xin = dev(x).clone()
-    hip.down_packed_res(dev(act), hip.pack_rows(dev(wd)), xin, fpw, out=xin)          # in place
-    assert torch.equal(xin, out)
 
 
 @pytest.mark.parametrize("rows,K,N,ns", [(8, 768, 2304, 4), (4, 256, 96, 3), (2, 1024, 3072, 1)])
@@ -1018,30 +868,6 @@ def test_down_packed_splitk(hip, rows, d, I, ks):
     assert part.shape[0] == ks
     got = part.double().sum(0).cpu()
     assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
-
-
-@pytest.mark.parametrize("rows,K,N,temp", [(8, 768, 50257, 1.0), (3, 256, 1001, 0.7), (16, 1024, 4099, 1.0)])
-def test_head_packed_argmax(hip, rows, K, N, temp):
-    """Packed tied head + greedy pick: logits equal to the row-major head kernel's within a bf16 ulp, ids equal to the
-    argmax (lowest index on ties) of its own logits after temperature and clamp; ragged vocabulary sizes."""
-    dtype = torch.bfloat16
-    g = gen(65)
-    x = torch.randn(rows, K, generator=g).to(dtype)
-    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
-    best = torch.zeros(16 * 64, dtype=torch.int64, device="cuda")
-    tok = torch.zeros(rows, dtype=torch.int64, device="cuda")
-    logits = hip.head_packed_argmax(dev(x), hip.pack_rows(dev(W)), N, temp, best, tok)
-    ref = (x.double() @ W.double().t()).to(dtype)
-    check(logits, ref, dtype, frac=0.05)
-    l = logits.cpu()
-    if temp != 1.0:
-        l = (l / temp)
-    l = torch.clamp(l, -1e4, 1e4)
-    assert torch.equal(tok.cpu(), l.float().argmax(-1))
-    assert int(best.abs().sum()) == 0
-    tok2 = torch.zeros_like(tok)
-    hip.head_packed_argmax(dev(x), hip.pack_rows(dev(W)), N, temp, best, tok2)      # slots were left clean
-    assert torch.equal(tok2, tok)
 
 
 def test_kernels_against_committed_known_answers(hip):
