@@ -1,0 +1,319 @@
+// Prefill GEMMs on the matrix cores (bf16, fp32 accumulation):  C[m, n] = sum_k A[m, k] W[n, k]
+// for activations A (M rows, K contiguous) and nn.Linear weights W (N, K) — the dense contractions of the prompt pass
+// (c_attn / c_proj flash_stu/modules/attention.py:74,101; gate / up / down flash_stu/modules/swiglu.py:22-29;
+// x @ M_inputs flash_stu/modules/stu.py:87), with the element-wise work that follows them as epilogues:
+//   mode 0  C = T(acc)
+//   mode 1  GLU: C[m, i] = T( T(gelu_tanh(T(acc_gate))) * T(acc_up) ) from two weight matrices (swiglu.py:23-26),
+//           so the gate and up activations never travel through HBM
+//   mode 2  C = T( R + T(acc) ): the residual add behind c_proj / down_proj (attention_layer.py:57,62, stu_layer.py:96)
+//
+// A workgroup is WFN x WTN waves; a wave owns FI x TJ MFMA tiles of 32 features x 32 rows
+// (v_mfma_f32_32x32x16_bf16), the workgroup 32*FI*WFN features x 32*TJ*WTN rows.  K runs in tiles of BK through NS
+// LDS stages that are filled straight from global memory (global_load_lds_dwordx4, no stop in registers) one or more
+// tiles ahead of the multiplication.  LDS rows are BK*2 bytes with the 16-byte chunk index XOR-ed with bits of the
+// row, so neither the fills nor the fragment reads meet bank conflicts.  The weights are the MFMA A operand and the
+// activations the B operand, so a lane ends up with 4 consecutive features of one row: 8-byte stores.  In mode 1 a
+// wave's feature tiles are half gate, half up rows of the same features.  Workgroup ids are dealt round-robin to the
+// 8 XCDs; each XCD works through its own contiguous share of the tiles in panels of 8 feature tiles, so the workgroups
+// resident on an XCD share a few weight and activation tiles in its L2.
+#include "fstu_common.h"
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+#define GM_PANEL 8     // feature tiles per panel of the tile order
+
+__device__ __forceinline__ float rnd_bf16(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  const float e = __builtin_amdgcn_exp2f(2.8853900817779268f * inner);   // exp(2 inner)
+  const float th = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return 0.5f * x * (1.0f + th);
+}
+
+// 16 bytes per lane from global memory into LDS: the 64 lanes fill 64 consecutive 16-byte slots from `l` (wave-uniform) on
+__device__ __forceinline__ void load16_to_lds(const void* g, void* l) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+}
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+  return (unsigned)(size_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// Fragment reads are written as asm: the compiler orders every LDS read it knows of behind all outstanding
+// global->LDS loads (s_waitcnt vmcnt(0)), which would serialise the next tile's fetch with this tile's reads.
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read16(unsigned addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int N, int STEP, int I = 0>
+__device__ __forceinline__ void lds_read_rows(u32x4_t* f, unsigned addr) {   // N reads, 32 rows (STEP bytes) apart
+  if constexpr (I < N) {
+    f[I] = lds_read16<I * STEP>(addr);
+    lds_read_rows<N, STEP, I + 1>(f, addr);
+  }
+}
+// Waits until at most LEFT of the reads issued so far are outstanding; the fragments pass through the statement so
+// that nothing that uses them is placed ahead of the wait.
+template <int LEFT, int N>
+__device__ __forceinline__ void lds_wait(u32x4_t (&f)[N]) {
+  static_assert(N == 4 || N == 6 || N == 8, "fragment group");
+  if constexpr (N == 4)
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]) : "n"(LEFT));
+  else if constexpr (N == 6)
+    asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]) : "n"(LEFT));
+  else
+    asm volatile("s_waitcnt lgkmcnt(%8)"
+                 : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7])
+                 : "n"(LEFT));
+}
+
+template <int WFN_, int WTN_, int FI_, int TJ_, int BK_, int NS_>
+struct GemmTile {
+  static constexpr int WFN = WFN_, WTN = WTN_, FI = FI_, TJ = TJ_, BK = BK_, NS = NS_;
+  static constexpr int NW = WFN * WTN, THREADS = 64 * NW;
+  static constexpr int BF = 32 * FI * WFN, BT = 32 * TJ * WTN;   // LDS rows of the weight / activation tile
+  static constexpr int RB = BK * 2, CPR = RB / 16;               // bytes and 16-byte chunks per LDS row
+  static constexpr int KK = BK / 16;                             // MFMA k steps per tile
+  static constexpr int WL = BF * CPR / (64 * NW), AL = BT * CPR / (64 * NW);   // fill instructions per wave and tile
+  static constexpr unsigned STAGE = (unsigned)(BF + BT) * RB;
+  static constexpr unsigned LDS = STAGE * NS;
+  static constexpr int NFR = FI + TJ;                            // fragments per k step
+  static_assert(BK == 32 || BK == 64, "k tile");
+  static_assert((BF * CPR) % (64 * NW) == 0 && (BT * CPR) % (64 * NW) == 0, "fill split");
+  // byte offset of 16-byte chunk c of a row inside a tile
+  __device__ static __forceinline__ unsigned swz(int row, int c) {
+    return (unsigned)row * RB + (unsigned)((c ^ (BK == 64 ? (row & 7) : ((row >> 1) & 3))) << 4);
+  }
+};
+
+template <class G, int MODE>
+__global__ void __launch_bounds__(G::THREADS)
+gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
+                 const bf16_t* __restrict__ R, long long ldr, bf16_t* __restrict__ C, long long ldc, int M, int N, int K,
+                 int mt, int nt, int share) {
+  constexpr int FI = G::FI, TJ = G::TJ, BF = G::BF, BT = G::BT, WL = G::WL, AL = G::AL, NS = G::NS, KK = G::KK, NFR = G::NFR;
+  constexpr int NF = MODE == 1 ? BF / 2 : BF;         // output features per workgroup
+  constexpr unsigned STAGE = G::STAGE;
+  extern __shared__ __align__(16) unsigned char gm_smem[];   // NS stages of (weights BF rows, activations BT rows)
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int wf = w % G::WFN, wt = w / G::WFN;
+  // ---- tile of this workgroup
+  const int o = (int)(blockIdx.x & 7) * share + (int)(blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= share || o >= mt * nt) return;
+  const int per_panel = mt * GM_PANEL;
+  const int panel = o / per_panel, in_panel = o - panel * per_panel;
+  const int pw = min(GM_PANEL, nt - panel * GM_PANEL);        // the last panel may be narrower
+  const int bt = in_panel / pw, bf = panel * GM_PANEL + in_panel % pw;
+  const int m0 = bt * BT, n0 = bf * NF;
+  // ---- fills: the XOR of the layout is applied on the global side: the lane that owns slot s (row s / CPR, physical
+  // chunk s % CPR) fetches the logical chunk that belongs there
+  const bf16_t* wsrc[WL];
+  const bf16_t* asrc[AL];
+#pragma unroll
+  for (int j = 0; j < WL; ++j) {
+    const int slot = (w * WL + j) * 64 + lane, row = slot / G::CPR;
+    const int ch = (int)((G::swz(row, slot % G::CPR) - (unsigned)row * G::RB) >> 4);   // XOR is its own inverse
+    int n;
+    const bf16_t* wb = W;
+    if (MODE == 1) {
+      // LDS rows of wave column wf': gate rows first, then the up rows of the same features
+      constexpr int HALF = 16 * FI;                   // gate (or up) rows per wave column
+      const int q = row / (2 * HALF), rr = row % (2 * HALF);
+      n = n0 + q * HALF + (rr % HALF);
+      if (rr >= HALF) wb = W2;
+    } else {
+      n = n0 + row;
+    }
+    n = min(n, N - 1);
+    wsrc[j] = wb + (size_t)n * K + ch * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < AL; ++j) {
+    const int slot = (w * AL + j) * 64 + lane, row = slot / G::CPR;
+    const int ch = (int)((G::swz(row, slot % G::CPR) - (unsigned)row * G::RB) >> 4);
+    asrc[j] = A + (size_t)min(m0 + row, M - 1) * lda + ch * 8;
+  }
+  const unsigned wslot = (unsigned)(w * WL) * 1024u, aslot = (unsigned)BF * G::RB + (unsigned)(w * AL) * 1024u;   // wave-uniform
+#define GM_FETCH(stage_, k0)                                                                                 \
+  {                                                                                                          \
+    unsigned char* st_ = gm_smem + (unsigned)(stage_) * STAGE;                                               \
+    _Pragma("unroll") for (int j = 0; j < WL; ++j) load16_to_lds(wsrc[j] + (k0), st_ + wslot + j * 1024);    \
+    _Pragma("unroll") for (int j = 0; j < AL; ++j) load16_to_lds(asrc[j] + (k0), st_ + aslot + j * 1024);    \
+  }
+#define GM_MFMAS(f_)                                                                                         \
+  _Pragma("unroll") for (int i = 0; i < FI; ++i)                                                             \
+    _Pragma("unroll") for (int j = 0; j < TJ; ++j)                                                           \
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f_[i]),               \
+                                                          __builtin_bit_cast(bf16x8_t, f_[FI + j]), acc[i][j], 0, 0, 0);
+  const int l32 = lane & 31, lh = lane >> 5;
+  // fragment addresses inside a stage for the k steps of a tile (rows 32 apart share the XOR term)
+  unsigned fw_off[KK], fa_off[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    fw_off[kk] = G::swz(wf * (32 * FI) + l32, kk * 2 + lh);
+    fa_off[kk] = (unsigned)BF * G::RB + G::swz(wt * (32 * TJ) + l32, kk * 2 + lh);
+  }
+  floatx16_t acc[FI][TJ];
+#pragma unroll
+  for (int i = 0; i < FI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  const int nkt = K / G::BK;
+  // Tiles kt+1 .. kt+NS-2 stay in flight while tile kt is multiplied.  Per k tile: wait for this wave's share of
+  // tile kt, barrier (every wave's share has landed and every wave has left the stage of tile kt-1), refill that
+  // stage with tile kt+NS-1, then the k steps: the fragments of step kk+1 are read while step kk is multiplied.  The
+  // compiler's own schedule would wait for each fragment read in turn; the fences keep the order written here.
+  constexpr int LPT = WL + AL;                        // fills per wave and tile
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t)
+    if (t < nkt) GM_FETCH(t, t * G::BK)
+  const unsigned smem0 = lds_addr(gm_smem);
+  int cur = 0, refill = NS - 1;                       // stage of tile kt, stage of tile kt+NS-1
+  for (int kt = 0; kt < nkt; ++kt) {
+    if (kt + NS - 2 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();   // bare: the fence of __syncthreads would wait for the tiles still in flight
+    if (kt + NS - 1 < nkt) GM_FETCH(refill, (kt + NS - 1) * G::BK)
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned cb = smem0 + (unsigned)cur * STAGE;
+    u32x4_t fa_[NFR], fb_[NFR];                       // the two fragment sets, used by alternate k steps
+    lds_read_rows<FI, 32 * G::RB>(fa_, cb + fw_off[0]);
+    lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, cb + fa_off[0]);
+    lds_read_rows<FI, 32 * G::RB>(fb_, cb + fw_off[1]);
+    lds_read_rows<TJ, 32 * G::RB>(fb_ + FI, cb + fa_off[1]);
+    lds_wait<NFR>(fa_);
+    GM_MFMAS(fa_)
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (KK == 2) {
+      lds_wait<0>(fb_);
+      GM_MFMAS(fb_)
+    } else {
+      lds_read_rows<FI, 32 * G::RB>(fa_, cb + fw_off[KK - 2]);
+      lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, cb + fa_off[KK - 2]);
+      lds_wait<NFR>(fb_);
+      GM_MFMAS(fb_)
+      __builtin_amdgcn_sched_barrier(0);
+      lds_read_rows<FI, 32 * G::RB>(fb_, cb + fw_off[KK - 1]);
+      lds_read_rows<TJ, 32 * G::RB>(fb_ + FI, cb + fa_off[KK - 1]);
+      lds_wait<NFR>(fa_);
+      GM_MFMAS(fa_)
+      __builtin_amdgcn_sched_barrier(0);
+      lds_wait<0>(fb_);
+      GM_MFMAS(fb_)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    cur = cur + 1 == NS ? 0 : cur + 1;
+    refill = refill + 1 == NS ? 0 : refill + 1;
+  }
+#undef GM_FETCH
+#undef GM_MFMAS
+  // ---- epilogue.  D of a 32x32 tile: lane l holds row (token) l % 32 and features 8*(e/4) + 4*(l/32) + e%4
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) {
+    const int m = m0 + wt * (32 * TJ) + j * 32 + l32;
+    if (m >= M) continue;
+    if (MODE == 1) {
+#pragma unroll
+      for (int i = 0; i < FI / 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int f = n0 + wf * (16 * FI) + i * 32 + q * 8 + lh * 4;
+          if (f >= N) continue;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[e] = rnd_bf16(gelu_tanh_fast(rnd_bf16(acc[i][j][q * 4 + e]))) * rnd_bf16(acc[i + FI / 2][j][q * 4 + e]);
+          *(uint2*)(C + (size_t)m * ldc + f) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < FI; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int f = n0 + wf * (32 * FI) + i * 32 + q * 8 + lh * 4;
+          if (f >= N) continue;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+          if (MODE == 2) {
+            const uint2 rv = *(const uint2*)(R + (size_t)m * ldr + f);
+            v[0] = __uint_as_float(rv.x << 16) + rnd_bf16(v[0]);
+            v[1] = __uint_as_float(rv.x & 0xffff0000u) + rnd_bf16(v[1]);
+            v[2] = __uint_as_float(rv.y << 16) + rnd_bf16(v[2]);
+            v[3] = __uint_as_float(rv.y & 0xffff0000u) + rnd_bf16(v[3]);
+          }
+          *(uint2*)(C + (size_t)m * ldc + f) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+        }
+    }
+  }
+}
+
+template <class G, int MODE>
+int gemm_launch_tile(const void* A, long long lda, const void* W, const void* W2, const void* R, long long ldr, void* C,
+                     long long ldc, int M, int N, int K, hipStream_t s) {
+  constexpr int NF = MODE == 1 ? G::BF / 2 : G::BF;
+  static hipError_t attr_err = hipFuncSetAttribute((const void*)gemm_bf16_kernel<G, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS);
+  if (attr_err != hipSuccess) { fstu_set_error("fstu_gemm_bf16: hipFuncSetAttribute: %s", hipGetErrorString(attr_err)); return (int)attr_err; }
+  const int mt = (M + G::BT - 1) / G::BT, nt = (N + NF - 1) / NF;
+  const long long tiles = (long long)mt * nt;
+  const int share = (int)((tiles + 7) / 8);
+  hipLaunchKernelGGL((gemm_bf16_kernel<G, MODE>), dim3((unsigned)share * 8u), dim3(G::THREADS), G::LDS, s, (const bf16_t*)A, lda,
+                     (const bf16_t*)W, (const bf16_t*)W2, (const bf16_t*)R, ldr, (bf16_t*)C, ldc, M, N, K, mt, nt, share);
+  return 0;
+}
+
+int gemm_cus() {
+  static int cus = [] {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
+    return p.multiProcessorCount;
+  }();
+  return cus;
+}
+
+//                     waves  tiles  BK  stages
+using TileBig = GemmTile<4, 2, 2, 4, 64, 2>;     // 256 x 256, 8 waves, 128 KB of LDS
+using TileSmall = GemmTile<2, 2, 2, 2, 64, 2>;   // 128 x 128, 4 waves, 64 KB: two workgroups per compute unit
+using TileK32 = GemmTile<2, 2, 4, 2, 32, 3>;     // 256 x 128, 4 waves, 72 KB, k tiles of 32 for K % 64 != 0
+
+template <int MODE>
+int gemm_launch(const void* A, long long lda, const void* W, const void* W2, const void* R, long long ldr, void* C, long long ldc,
+                int M, int N, int K, hipStream_t s) {
+  if (K % 64 != 0) return gemm_launch_tile<TileK32, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  // The large tile halves the fill traffic per flop; it pays once K is long enough to amortise its start-up and the
+  // grid still covers the chip twice (measured: 1.04-1.16 PFLOP/s against 0.90-0.98 at M=131072 with K >= 2048, but
+  // 97 us against 85 us at M=4096, N=9216, K=768).
+  const long long big = (long long)((M + 255) / 256) * ((N + (MODE == 1 ? 127 : 255)) / (MODE == 1 ? 128 : 256));
+  if (K >= 1024 && big >= 2 * gemm_cus()) return gemm_launch_tile<TileBig, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  return gemm_launch_tile<TileSmall, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+}
+
+}  // namespace
+
+extern "C" int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, const void* R, int64_t ldr, void* C,
+                              int64_t ldc, int M, int N, int K, int mode, void* stream) {
+  FSTU_REQUIRE(A && W && C, FSTU_ENULL, "fstu_gemm_bf16: null pointer");
+  FSTU_REQUIRE(mode >= 0 && mode <= 2, FSTU_EARG, "fstu_gemm_bf16: mode %d", mode);
+  FSTU_REQUIRE((mode != 1 || W2) && (mode != 2 || R), FSTU_ENULL, "fstu_gemm_bf16: mode %d needs its second operand", mode);
+  FSTU_REQUIRE(M >= 1 && N >= 4 && N % 4 == 0 && K >= 32 && K % 32 == 0, FSTU_ESHAPE,
+               "fstu_gemm_bf16: need K %% 32 == 0 and N %% 4 == 0 (M=%d N=%d K=%d)", M, N, K);
+  FSTU_REQUIRE(lda >= K && lda % 8 == 0 && ldc >= N && ldc % 4 == 0 && (mode != 2 || (ldr >= N && ldr % 4 == 0)), FSTU_ESHAPE,
+               "fstu_gemm_bf16: row strides (lda=%lld ldc=%lld ldr=%lld)", (long long)lda, (long long)ldc, (long long)ldr);
+  FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(W2, 16) && fstu_aligned(C, 8) && fstu_aligned(R, 8),
+               FSTU_EALIGN, "fstu_gemm_bf16: pointers must be 16-byte aligned (C, R: 8)");
+  int rc;
+  if (mode == 0) rc = gemm_launch<0>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
+  else if (mode == 1) rc = gemm_launch<1>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
+  else rc = gemm_launch<2>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
+  if (rc) return rc;
+  FSTU_CHECK_LAUNCH("fstu_gemm_bf16");
+  return FSTU_OK;
+}

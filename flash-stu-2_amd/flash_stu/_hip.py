@@ -78,6 +78,7 @@ SIGNATURES = {
     "fstu_prof_end": [_vp, _vp],
     "fstu_prof_copy": [_vp, _vp, ctypes.c_size_t, _vp],
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
+    "fstu_gemm_bf16": [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
     "fstu_lds_sequence_ws_floats": [_i, _i, _i],
     "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -252,12 +253,58 @@ def bias_act(y: torch.Tensor, bias: Optional[torch.Tensor], silu: bool = False) 
     return y
 
 
+def gemm_supported(x2: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Shapes the matrix-core prompt GEMM takes: bf16, K a multiple of 32, N a multiple of 4, rows 16-byte aligned."""
+    K = x2.shape[-1]
+    return (x2.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x2.dim() == 2 and K % 32 == 0 and
+            weight.shape[0] % 4 == 0 and weight.is_contiguous() and x2.stride(1) == 1 and x2.stride(0) % 8 == 0 and
+            x2.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def gemm(x2: torch.Tensor, weight: torch.Tensor, up_weight: Optional[torch.Tensor] = None,
+         residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x2 (M,K) @ weight (N,K)^T on the matrix cores (bf16).  up_weight: the gated pair
+    T(T(gelu_tanh(T(x2 @ weight^T))) * T(x2 @ up_weight^T)); residual (M,N): T(residual + T(x2 @ weight^T))."""
+    _dev(weight, up_weight)
+    for t in (x2, residual, out):          # rows may be strided
+        if t is not None and not t.is_cuda:
+            raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    if not gemm_supported(x2, weight):
+        raise FlashSTUHipError(f"gemm: unsupported operands {tuple(x2.shape)} {x2.dtype} x {tuple(weight.shape)} {weight.dtype}")
+    if up_weight is not None and residual is not None:
+        raise FlashSTUHipError("gemm: the gated pair and the residual epilogue do not combine")
+    M, K = x2.shape
+    N = weight.shape[0]
+    if weight.shape[1] != K or (up_weight is not None and (up_weight.shape != weight.shape or not up_weight.is_contiguous()
+                                                            or up_weight.dtype != weight.dtype)):
+        raise FlashSTUHipError("gemm: weight shapes")
+    if out is None:
+        out = torch.empty(M, N, dtype=x2.dtype, device=x2.device)
+    if out.shape != (M, N) or out.stride(1) != 1 or out.dtype != x2.dtype:
+        raise FlashSTUHipError("gemm: out must be (M,N) with contiguous rows")
+    mode, ldr = 0, 0
+    if up_weight is not None:
+        mode = 1
+    elif residual is not None:
+        if residual.shape != (M, N) or residual.stride(1) != 1 or residual.dtype != x2.dtype:
+            raise FlashSTUHipError("gemm: residual must be (M,N) with contiguous rows")
+        mode, ldr = 2, residual.stride(0)
+    _check(load().fstu_gemm_bf16(_p(x2), x2.stride(0), _p(weight), _p(up_weight), _p(residual), ldr, _p(out), out.stride(0),
+                                 M, N, K, mode, _stream()), "fstu_gemm_bf16")
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x (..., K) @ weight (N,K)^T (+ bias): the skinny GEMV kernel for up to 16 rows, a library GEMM beyond."""
+    """x (..., K) @ weight (N,K)^T (+ bias): the skinny GEMV kernel for up to 16 rows, the matrix-core GEMM kernel for
+    more rows in bf16; other dtypes and shapes the kernel does not take go to a library GEMM."""
     shape = x.shape
     x2 = x.reshape(-1, shape[-1])
     if x2.shape[0] <= MAX_DECODE_ROWS:
         y = linear_decode(x2.contiguous(), weight)
+        if bias is not None:
+            bias_act(y, bias)
+    elif gemm_supported(x2, weight):
+        y = gemm(x2, weight)
         if bias is not None:
             bias_act(y, bias)
     elif bias is not None:

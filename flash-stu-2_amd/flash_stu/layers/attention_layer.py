@@ -26,6 +26,7 @@ class AttentionLayer(nn.Module):
         else:
             y, present = self.attn(a, past_key_value=None, use_cache=False), None
         h2 = self.mlp_norm.add_then_norm(x, y)
-        m = self.mlp(h2)
-        _hip.add_rmsnorm(x, m.contiguous(), None, 0.0, want_norm=False)
+        m = self.mlp(h2, residual=x)
+        if m is not None:
+            _hip.add_rmsnorm(x, m.contiguous(), None, 0.0, want_norm=False)
         return (x, present) if use_cache else x

@@ -47,6 +47,7 @@ class STULayer(nn.Module):
         if self.stu_mlp_enabled:
             y = _hip.linear(y.contiguous(), self.stu_mlp_out_proj.weight, self.stu_mlp_out_proj.bias).contiguous()
         h2 = self.mlp_norm.add_then_norm(x, y)
-        m = self.mlp(h2)
-        _hip.add_rmsnorm(x, m.contiguous(), None, 0.0, want_norm=False)
+        m = self.mlp(h2, residual=x)
+        if m is not None:
+            _hip.add_rmsnorm(x, m.contiguous(), None, 0.0, want_norm=False)
         return (x, state) if use_cache else x

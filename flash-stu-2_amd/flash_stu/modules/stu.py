@@ -187,6 +187,9 @@ class STU(nn.Module):
         B, T, d = x.shape
         if B * T <= _hip.MAX_DECODE_ROWS:
             return _hip.linear_decode(x.reshape(B * T, d), self.m_inputs_t()).reshape(B, T, self.d_out)
+        x2 = x.reshape(B * T, d)
+        if _hip.gemm_supported(x2, self.m_inputs_t()):
+            return _hip.gemm(x2, self.m_inputs_t()).reshape(B, T, self.d_out)
         return torch.matmul(x, self.m_inputs_eff())
 
     def _convolve(self, xp: torch.Tensor) -> torch.Tensor:

@@ -18,9 +18,11 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=config.bias, dtype=dtype)
 
     @torch.no_grad()
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x (..., d).  Up to 16 rows take the skinny MFMA kernels with the gate
-        fused; more rows use library GEMMs plus the fused gelu*up kernel."""
+    def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
+        """x (..., d).  Up to 16 rows take the skinny MFMA kernels with the gate fused; more rows in bf16 take the
+        matrix-core GEMM kernel with the gate as the epilogue of the gate/up pair.  With `residual` (same shape as x,
+        contiguous rows) the sum residual + mlp(x) is written into `residual` where the down projection can carry the add
+        as its epilogue, and None is returned; otherwise the MLP output is returned and the caller adds it."""
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         rows = x2.shape[0]
@@ -32,6 +34,15 @@ class MLP(nn.Module):
         elif rows <= _hip.MAX_DECODE_ROWS:
             act = _hip.glu_decode(x2, self.gate_proj.weight, self.up_proj.weight)
             out = _hip.linear_decode(act, self.down_proj.weight)
+        elif (_hip.gemm_supported(x2, self.gate_proj.weight) and self.up_proj.weight.is_contiguous()
+              and self.intermediate_size % 32 == 0 and self.down_proj.weight.is_contiguous()
+              and self.down_proj.weight.data_ptr() % 16 == 0):
+            act = _hip.gemm(x2, self.gate_proj.weight, up_weight=self.up_proj.weight)
+            if residual is not None and residual.is_contiguous():
+                r2 = residual.view(-1, shape[-1])
+                _hip.gemm(act, self.down_proj.weight, residual=r2, out=r2)
+                return None
+            out = _hip.gemm(act, self.down_proj.weight)
         else:
             g = torch.matmul(x2, self.gate_proj.weight.t())
             u = torch.matmul(x2, self.up_proj.weight.t())

@@ -310,6 +310,19 @@ int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ld
 int fstu_head_argmax_static(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                             float temperature, int64_t* tok_out, int64_t tok_stride, int dtype, void* stream);
 
+/* ---- prompt-pass GEMMs on the matrix cores (bf16) ---------------------------
+ * C[m,n] = sum_k A[m,k] W[n,k] over M > 16 rows, fp32 accumulation, with the element-wise step that follows the
+ * projection in the reference as the epilogue:
+ *   mode 0  C = T(acc)                                   c_attn (flash_stu/modules/attention.py:74), x @ M_inputs
+ *                                                        (flash_stu/modules/stu.py:87 with W = M_inputs^T)
+ *   mode 1  C = T(T(gelu_tanh(T(acc_W))) * T(acc_W2))    gate_proj, up_proj and the gate (flash_stu/modules/swiglu.py:23-26)
+ *   mode 2  C = T(R + T(acc))                            c_proj / down_proj and the residual add
+ *                                                        (flash_stu/layers/attention_layer.py:57,62)
+ * A (M,K) with row stride lda, W and W2 (N,K) contiguous, R / C (M,N) with row strides ldr / ldc (elements).
+ * K % 64 == 0, N % 4 == 0, lda % 8 == 0; A, W, W2 16-byte aligned.  C may alias R. */
+int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, const void* R, int64_t ldr, void* C,
+                   int64_t ldc, int M, int N, int K, int mode, void* stream);
+
 /* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
  * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:
  *   h <- h*A + x_t @ Bm ;  y_t = T(h @ Cm)

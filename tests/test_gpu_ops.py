@@ -121,6 +121,67 @@ def test_mlp_decode_chain(hip, dtype, rows, d, I):
         check(rd, ref, dtype, frac=0.05, atol=(2.0 ** -7 * float(down.float().abs().max())) if dtype == torch.bfloat16 else 0.0)
 
 
+# Prompt-pass GEMM kernel: the three tile shapes (128 x 128; 256 x 256 for K >= 1024 on grids that cover the chip
+# twice; k tiles of 32 for K % 64 != 0), ragged M and N, one- and many-tile grids.
+GEMM_SHAPES = [(4096, 2304, 768), (512, 768, 768), (1000, 772, 96), (17, 4, 32), (300, 200, 1056), (2048, 16384, 1024),
+               (257, 132, 64)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_bf16_plain_and_residual(hip, M, N, K):
+    """fstu_gemm_bf16 modes 0 and 2 against F.linear in fp32 rounded once (c_attn / c_proj / down_proj / M_inputs of
+    the prompt pass): bf16 results within one ulp, few rounding flips."""
+    g = gen(61)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    res = torch.randn(M, N, generator=g).bfloat16()
+    ref = F.linear(x.float(), W.float()).bfloat16()
+    xd, Wd = dev(x), dev(W)
+    check(hip.gemm(xd, Wd), ref, torch.bfloat16)
+    rd = dev(res.clone())
+    out = hip.gemm(xd, Wd, residual=rd, out=rd)          # in place, as the MLP's down projection uses it
+    assert out.data_ptr() == rd.data_ptr()
+    check(rd, (res.float() + ref.float()).bfloat16(), torch.bfloat16, frac=0.05, atol=2.0 ** -7 * float(ref.float().abs().max()))
+
+
+@pytest.mark.parametrize("M,d,I", [(4096, 768, 3072), (300, 256, 1000), (2048, 1024, 8192), (100, 96, 132)])
+def test_gemm_bf16_gated_pair(hip, M, d, I):
+    """Mode 1: T(T(gelu_tanh(T(x Wg^T))) * T(x Wu^T)) in one kernel equals the three-step bf16 chain of the reference
+    MLP (flash_stu/modules/swiglu.py:23-26)."""
+    g = gen(62)
+    x = torch.randn(M, d, generator=g).bfloat16()
+    Wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).bfloat16()
+    Wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).bfloat16()
+    act = hip.gemm(dev(x), dev(Wg), up_weight=dev(Wu))
+    gate = F.linear(x.float(), Wg.float()).bfloat16()
+    up = F.linear(x.float(), Wu.float()).bfloat16()
+    ref = F.gelu(gate, approximate="tanh") * up
+    # a different fp32 summation order may flip the rounding of either projection by one ulp: a flip of `up` and the
+    # roundings of gelu and of the product stay within two ulps of the product; a flip of `gate` passes through gelu's
+    # slope (<= 1.13), which for negative gates is large against gelu(gate) itself: 1.2 ulp(gate) * |up|
+    got, r = act.float().cpu(), ref.float()
+    tol = r.abs() * 2.0 ** -6 + 1.2 * 2.0 ** -7 * (gate.float() * up.float()).abs() + 1e-3 * 2.0 ** -7 * float(r.abs().max())
+    assert bool(((got - r).abs() <= tol).all()), float(((got - r).abs() - tol).max())
+    assert float(((got - r).abs() > 0).float().mean()) <= 0.05
+
+
+def test_gemm_bf16_strided_operands_and_errors(hip):
+    g = gen(63)
+    big = torch.randn(200, 3, 128, generator=g).bfloat16()
+    W = (torch.randn(64, 128, generator=g) / 11).bfloat16()
+    bd = dev(big)
+    out = torch.zeros(200, 2, 64, dtype=torch.bfloat16, device="cuda")
+    hip.gemm(bd[:, 1, :], dev(W), out=out[:, 1, :])
+    check(out[:, 1].cpu(), F.linear(big[:, 1].float(), W.float()).bfloat16(), torch.bfloat16)
+    assert float(out[:, 0].abs().max()) == 0
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.gemm(dev(torch.zeros(32, 40).bfloat16()), dev(torch.zeros(8, 40).bfloat16()))       # K % 32
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.gemm(dev(torch.zeros(32, 64)), dev(torch.zeros(8, 64)))                               # fp32
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.gemm(bd[:, 1, :], dev(W), up_weight=dev(W), residual=out[:, 1, :])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gelu_mul(hip, dtype):
     g = gen(5)
