@@ -270,21 +270,33 @@ def run_lm(args, torch, _hip, which):
         torch.cuda.synchronize()
         del a_, b_
     if which == "c2":
-        # MFMA rate of the prefill's largest GEMM (the gate projection of the whole prompt), timed with events
-        gm, gn, gk = B * P, cfg.n_embd * cfg.mlp_scale, cfg.n_embd
-        ga = torch.randn(gm, gk, device="cuda", dtype=torch.bfloat16)
-        gw = model.layers[0].mlp.gate_proj.weight
-        for _ in range(3):
-            _hip.linear(ga, gw)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(20):
-            _hip.linear(ga, gw)
-        e1.record()
-        torch.cuda.synchronize()
-        tf = 2.0 * gm * gn * gk * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12
-        out["prefill_gemm"] = {"what": "gate projection of the prompt (M, N, K)", "shape": [gm, gn, gk], "achieved": tf,
-                               "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS}
+        # MFMA rates of the prompt pass's two largest contractions as the MLP runs them (hand-written kernel
+        # fstu_gemm_bf16): gate+up with the gelu*up epilogue, and the down projection with the residual add
+        gm, gi, gd = B * P, cfg.n_embd * cfg.mlp_scale, cfg.n_embd
+        ga = torch.randn(gm, gd, device="cuda", dtype=torch.bfloat16)
+        mlp0 = model.layers[0].mlp
+        gres = torch.zeros(gm, gd, device="cuda", dtype=torch.bfloat16)
+
+        def _rate(fn, flops):
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 20
+            tf = flops / (us * 1e-6) / 1e12
+            return {"us": us, "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS}
+        gact = _hip.gemm(ga, mlp0.gate_proj.weight, up_weight=mlp0.up_proj.weight)
+        out["prefill_gemm"] = dict(_rate(lambda: _hip.gemm(ga, mlp0.gate_proj.weight, up_weight=mlp0.up_proj.weight, out=gact),
+                                         4.0 * gm * gi * gd),
+                                   what="gate+up projection of the prompt with the gelu*up epilogue (M, 2N, K)", shape=[gm, 2 * gi, gd])
+        out["prefill_gemm_down"] = dict(_rate(lambda: _hip.gemm(gact, mlp0.down_proj.weight, residual=gres, out=gres),
+                                              2.0 * gm * gi * gd),
+                                        what="down projection of the prompt with the residual add (M, N, K)", shape=[gm, gd, gi])
+        del gact, gres
         del ga
     if args.breakdown:
         names = {1: "glu", 2: "down", 3: "head", 4: "attention", 5: "stu_step", 6: "proj_qkv", 7: "embed_add_norm", 8: "sample"}

@@ -166,51 +166,59 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   const int nkt = K / G::BK;
-  // Tiles kt+1 .. kt+NS-2 stay in flight while tile kt is multiplied.  Per k tile: wait for this wave's share of
-  // tile kt, barrier (every wave's share has landed and every wave has left the stage of tile kt-1), refill that
-  // stage with tile kt+NS-1, then the k steps: the fragments of step kk+1 are read while step kk is multiplied.  The
-  // compiler's own schedule would wait for each fragment read in turn; the fences keep the order written here.
+  // Software pipeline over the k tiles.  NS-1 tiles are in flight ahead of the one being multiplied.  Within a tile the
+  // fragments of k step kk+1 are read while step kk is multiplied; before the last step of tile kt the wave makes sure
+  // its reads of the tile are complete, waits for its share of tile kt+1, meets the barrier (every wave's share has
+  // landed, every wave has left the stage of tile kt), refills that stage with tile kt+NS and reads the first
+  // fragments of tile kt+1 — so the MFMAs of the last step cover the barrier and those reads.  The compiler's own
+  // schedule would wait for each fragment read in turn; the fences keep the order written here.
   constexpr int LPT = WL + AL;                        // fills per wave and tile
 #pragma unroll
   for (int t = 0; t < NS - 1; ++t)
     if (t < nkt) GM_FETCH(t, t * G::BK)
   const unsigned smem0 = lds_addr(gm_smem);
-  int cur = 0, refill = NS - 1;                       // stage of tile kt, stage of tile kt+NS-1
+  if (NS - 2 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();   // bare: the fence of __syncthreads would wait for the tiles still in flight
+  if (NS - 1 < nkt) GM_FETCH(NS - 1, (NS - 1) * G::BK)
+  u32x4_t fa_[NFR], fb_[NFR];                         // the two fragment sets, used by alternate k steps
+  lds_read_rows<FI, 32 * G::RB>(fa_, smem0 + fw_off[0]);
+  lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, smem0 + fa_off[0]);
+  int cur = 0;                                        // stage of tile kt
   for (int kt = 0; kt < nkt; ++kt) {
-    if (kt + NS - 2 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();   // bare: the fence of __syncthreads would wait for the tiles still in flight
-    if (kt + NS - 1 < nkt) GM_FETCH(refill, (kt + NS - 1) * G::BK)
-    __builtin_amdgcn_sched_barrier(0);
     const unsigned cb = smem0 + (unsigned)cur * STAGE;
-    u32x4_t fa_[NFR], fb_[NFR];                       // the two fragment sets, used by alternate k steps
-    lds_read_rows<FI, 32 * G::RB>(fa_, cb + fw_off[0]);
-    lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, cb + fa_off[0]);
+    const int nxt = cur + 1 == NS ? 0 : cur + 1;
+    __builtin_amdgcn_sched_barrier(0);
     lds_read_rows<FI, 32 * G::RB>(fb_, cb + fw_off[1]);
     lds_read_rows<TJ, 32 * G::RB>(fb_ + FI, cb + fa_off[1]);
     lds_wait<NFR>(fa_);
     GM_MFMAS(fa_)
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (KK == 2) {
-      lds_wait<0>(fb_);
-      GM_MFMAS(fb_)
-    } else {
-      lds_read_rows<FI, 32 * G::RB>(fa_, cb + fw_off[KK - 2]);
-      lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, cb + fa_off[KK - 2]);
+    if constexpr (KK == 4) {
+      lds_read_rows<FI, 32 * G::RB>(fa_, cb + fw_off[2]);
+      lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, cb + fa_off[2]);
       lds_wait<NFR>(fb_);
       GM_MFMAS(fb_)
       __builtin_amdgcn_sched_barrier(0);
-      lds_read_rows<FI, 32 * G::RB>(fb_, cb + fw_off[KK - 1]);
-      lds_read_rows<TJ, 32 * G::RB>(fb_ + FI, cb + fa_off[KK - 1]);
+      lds_read_rows<FI, 32 * G::RB>(fb_, cb + fw_off[3]);
+      lds_read_rows<TJ, 32 * G::RB>(fb_ + FI, cb + fa_off[3]);
       lds_wait<NFR>(fa_);
       GM_MFMAS(fa_)
       __builtin_amdgcn_sched_barrier(0);
-      lds_wait<0>(fb_);
-      GM_MFMAS(fb_)
+    }
+    lds_wait<0>(fb_);                                 // this wave has left the stage of tile kt
+    if (kt + 1 < nkt) {
+      if (kt + NS - 1 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      if (kt + NS < nkt) GM_FETCH(cur, (kt + NS) * G::BK)
+      const unsigned nb = smem0 + (unsigned)nxt * STAGE;
+      lds_read_rows<FI, 32 * G::RB>(fa_, nb + fw_off[0]);
+      lds_read_rows<TJ, 32 * G::RB>(fa_ + FI, nb + fa_off[0]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    cur = cur + 1 == NS ? 0 : cur + 1;
-    refill = refill + 1 == NS ? 0 : refill + 1;
+    GM_MFMAS(fb_)
+    cur = nxt;
   }
 #undef GM_FETCH
 #undef GM_MFMAS
@@ -282,17 +290,22 @@ int gemm_cus() {
 //                     waves  tiles  BK  stages
 using TileBig = GemmTile<4, 2, 2, 4, 64, 2>;     // 256 x 256, 8 waves, 128 KB of LDS
 using TileSmall = GemmTile<2, 2, 2, 2, 64, 2>;   // 128 x 128, 4 waves, 64 KB: two workgroups per compute unit
+using TileDeep = GemmTile<2, 2, 2, 2, 64, 4>;    // 128 x 128, 4 waves, 3 tiles in flight: one workgroup per compute unit
 using TileK32 = GemmTile<2, 2, 4, 2, 32, 3>;     // 256 x 128, 4 waves, 72 KB, k tiles of 32 for K % 64 != 0
 
 template <int MODE>
 int gemm_launch(const void* A, long long lda, const void* W, const void* W2, const void* R, long long ldr, void* C, long long ldc,
                 int M, int N, int K, hipStream_t s) {
   if (K % 64 != 0) return gemm_launch_tile<TileK32, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
-  // The large tile halves the fill traffic per flop; it pays once K is long enough to amortise its start-up and the
-  // grid still covers the chip twice (measured: 1.04-1.16 PFLOP/s against 0.90-0.98 at M=131072 with K >= 2048, but
-  // 97 us against 85 us at M=4096, N=9216, K=768).
-  const long long big = (long long)((M + 255) / 256) * ((N + (MODE == 1 ? 127 : 255)) / (MODE == 1 ? 128 : 256));
+  // Measured choices (MI355X, bf16): the large tile halves the fill traffic per flop and pays once K amortises its
+  // start-up and the grid still covers the chip twice (M=32768, K >= 2048: 1.01-1.18 PFLOP/s against 0.89-0.99;
+  // M=4096, N=9216, K=768: 92 us against 80 us).  A grid that leaves one workgroup per compute unit anyway gains from
+  // the deeper pipeline when K is long (M=4096, N=768, K=9216: 83 us against 93 us).
+  const int nf = MODE == 1 ? 2 : 1;
+  const long long big = (long long)((M + 255) / 256) * ((N * nf + 255) / 256);
+  const long long small = (long long)((M + 127) / 128) * ((N * nf + 127) / 128);
   if (K >= 1024 && big >= 2 * gemm_cus()) return gemm_launch_tile<TileBig, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  if (K >= 2048 && small <= gemm_cus()) return gemm_launch_tile<TileDeep, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
   return gemm_launch_tile<TileSmall, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
 }
 
