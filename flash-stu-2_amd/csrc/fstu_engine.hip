@@ -137,6 +137,56 @@ static bool chain_ok(const fstu_model_desc* m, int do_sample, const int* dyn) {
          fstu_finish_embed_supported(m->B, m->d, m->emb, m->x, m->layers[0].norm1_w, m->h);
 }
 
+// 17..32 rows: the MLP, where nearly all the weight bytes are, runs once over all rows on the tiled matrix-core kernel
+// (gate/up with the GLU epilogue, split-K down projection), so every MLP weight is read once per step; the
+// STU recurrence and the window attention, per-row operators, run over all rows in one launch each, and the small
+// projections and the head keep their 16-row kernels and run on the two halves of the rows in turn.  bf16 and the recurrence (lds) STU state only.
+static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride, int pos,
+                            float temperature, int top_k, float top_p, int do_sample, uint64_t seed, int step, int* dyn,
+                            void* stream) {
+  const int B = m->B, d = m->d, I = m->I, dt = m->dtype, R = FSTU_MAX_DECODE_ROWS;
+  FSTU_REQUIRE(dt == FSTU_BF16 && m->stu_mode == 1 && d % 256 == 0 && I % 64 == 0, FSTU_ESHAPE,
+               "fstu_decode_step: more than %d rows need bf16, the recurrence STU state, d %% 256 == 0 and I %% 64 == 0", R);
+  FSTU_REQUIRE(m->qkv && m->attn && m->y && m->xp && m->partial, FSTU_ENULL, "fstu_decode_step: incomplete model descriptor");
+  // K slices of the down projection: its d/128 output tiles times the slices should cover the chip; the partial-sum
+  // buffer holds at least 16 slices
+  int ks = 16;
+  while (ks > 1 && (I % (64 * ks) != 0 || (d / 128) * ks > 512)) ks >>= 1;
+  const size_t esz = 2;
+  auto rows_of = [&](int c) { return c == 0 ? R : B - R; };
+  auto at = [&](void* p, int c, size_t per_row) { return (void*)((char*)p + (size_t)c * R * per_row * esz); };
+  TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt, stream, dyn));
+  for (int l = 0; l < m->n_layers; ++l) {
+    const fstu_layer_desc& L = m->layers[l];
+    if (L.kind == 0) {
+      // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
+      for (int c = 0; c < 2; ++c)
+        TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.m_inputs_t, at(m->xp, c, d), d, rows_of(c), d, d, dt, stream));
+      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), stream));
+    } else {
+      for (int c = 0; c < 2; ++c)
+        TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.w_qkv, at(m->qkv, c, 3 * (size_t)d), 3 * d, rows_of(c), 3 * d, d, dt, stream));
+      TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
+                                         m->window, m->softcap, 1, dyn, dt, stream));
+      for (int c = 0; c < 2; ++c)
+        TIMED(PC_PROJ, fstu_linear_decode(at(m->attn, c, d), d, L.w_proj, at(m->y, c, d), d, rows_of(c), d, d, dt, stream));
+    }
+    const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
+    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+    TIMED(PC_GLU, fstu_gemm_bf16(m->h, d, L.w_gate, L.w_up, nullptr, 0, m->act, I, B, I, d, 1, stream));
+    TIMED(PC_DOWN, fstu_gemm_bf16_splitk(m->act, I, L.w_down, m->partial, B, d, I, ks, stream));
+    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, ks, 0, next_w, m->h, B, d, m->eps, dt, stream));
+  }
+  for (int c = 0; c < 2; ++c) {
+    const int rc = rows_of(c);
+    TIMED(PC_HEAD, fstu_linear_decode(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rc, m->V, d, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_dyn(at(m->logits, c, (size_t)m->V), tok_out + (size_t)c * R * tok_stride, tok_stride, rc, m->V, temperature,
+                                     top_k, top_p, do_sample, seed, step, m->row0 + c * R, dyn, dt, stream));
+  }
+  if (dyn) STEP(fstu_advance_dyn(dyn, stream));
+  return FSTU_OK;
+}
+
 // dyn == nullptr: pos/step come from the host arguments.  dyn != nullptr (graph capture): every position-dependent
 // kernel reads {pos, step} from that device int[2]; tok_in/tok_out are then the bases of token columns 0 and 1.
 static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int64_t* tok_out, int64_t tok_stride,
@@ -146,8 +196,8 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   FSTU_REQUIRE(dyn == nullptr || m->stu_mode == 1, FSTU_EARG, "fstu_decode_step: graph replay needs the recurrence (lds) STU state");
   FSTU_REQUIRE(m->layers && m->emb && m->final_norm_w && m->x && m->h && m->act && m->partial && m->logits,
                FSTU_ENULL, "fstu_decode_step: incomplete model descriptor");
-  FSTU_REQUIRE(m->B >= 1 && m->B <= FSTU_MAX_DECODE_ROWS, FSTU_ESHAPE, "fstu_decode_step: batch %d outside 1..%d", m->B,
-               FSTU_MAX_DECODE_ROWS);
+  FSTU_REQUIRE(m->B >= 1 && m->B <= 2 * FSTU_MAX_DECODE_ROWS, FSTU_ESHAPE, "fstu_decode_step: batch %d outside 1..%d", m->B,
+               2 * FSTU_MAX_DECODE_ROWS);
   FSTU_REQUIRE(m->n_layers >= 1 && m->ksplit_down >= 1 && pos >= 0, FSTU_EARG, "fstu_decode_step: bad layer count / split / pos");
   FSTU_REQUIRE(tok_stride >= 1, FSTU_EARG, "fstu_decode_step: tok_stride < 1");
   const int B = m->B, d = m->d, I = m->I, dt = m->dtype;
@@ -167,6 +217,8 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
                    "fstu_decode_step: layer %d has no attention state", l);
     }
   }
+  if (m->B > FSTU_MAX_DECODE_ROWS)
+    return decode_step_wide(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
   if (fstu_step_mega_ok(m)) {
     // the whole step as one persistent launch; sampling (when asked for) reads the logits it leaves
     const int greedy = do_sample ? 0 : 1;

@@ -6,6 +6,8 @@
 //   mode 1  GLU: C[m, i] = T( T(gelu_tanh(T(acc_gate))) * T(acc_up) ) from two weight matrices (swiglu.py:23-26),
 //           so the gate and up activations never travel through HBM
 //   mode 2  C = T( R + T(acc) ): the residual add behind c_proj / down_proj (attention_layer.py:57,62, stu_layer.py:96)
+//   split-K C = fp32 partial sums per K slice (fstu_add_rmsnorm adds the slices): the down projection of a decode
+//           step over 17..32 rows, whose 16 output tiles would leave most of the chip without weights to stream
 //
 // A workgroup is WFN x WTN waves; a wave owns FI x TJ MFMA tiles of 32 features x 32 rows
 // (v_mfma_f32_32x32x16_bf16), the workgroup 32*FI*WFN features x 32*TJ*WTN rows.  K runs in tiles of BK through NS
@@ -61,8 +63,10 @@ __device__ __forceinline__ void lds_read_rows(u32x4_t* f, unsigned addr) {   // 
 // that nothing that uses them is placed ahead of the wait.
 template <int LEFT, int N>
 __device__ __forceinline__ void lds_wait(u32x4_t (&f)[N]) {
-  static_assert(N == 4 || N == 6 || N == 8, "fragment group");
-  if constexpr (N == 4)
+  static_assert(N == 3 || N == 4 || N == 6 || N == 8, "fragment group");
+  if constexpr (N == 3)
+    asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]) : "n"(LEFT));
+  else if constexpr (N == 4)
     asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]) : "n"(LEFT));
   else if constexpr (N == 6)
     asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]) : "n"(LEFT));
@@ -95,7 +99,7 @@ template <class G, int MODE>
 __global__ void __launch_bounds__(G::THREADS)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                  const bf16_t* __restrict__ R, long long ldr, bf16_t* __restrict__ C, long long ldc, int M, int N, int K,
-                 int mt, int nt, int share) {
+                 int mt, int nt, int share, int ksplit) {
   constexpr int FI = G::FI, TJ = G::TJ, BF = G::BF, BT = G::BT, WL = G::WL, AL = G::AL, NS = G::NS, KK = G::KK, NFR = G::NFR;
   constexpr int NF = MODE == 1 ? BF / 2 : BF;         // output features per workgroup
   constexpr unsigned STAGE = G::STAGE;
@@ -103,8 +107,11 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wf = w % G::WFN, wt = w / G::WFN;
   // ---- tile of this workgroup
-  const int o = (int)(blockIdx.x & 7) * share + (int)(blockIdx.x >> 3);
-  if ((int)(blockIdx.x >> 3) >= share || o >= mt * nt) return;
+  int o = (int)(blockIdx.x & 7) * share + (int)(blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= share || o >= mt * nt * ksplit) return;
+  const int slice = o / (mt * nt);                    // MODE 3: K slice of this workgroup (slices outermost)
+  o -= slice * (mt * nt);
+  const int kbeg = slice * (K / ksplit);
   const int per_panel = mt * GM_PANEL;
   const int panel = o / per_panel, in_panel = o - panel * per_panel;
   const int pw = min(GM_PANEL, nt - panel * GM_PANEL);        // the last panel may be narrower
@@ -130,13 +137,13 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
       n = n0 + row;
     }
     n = min(n, N - 1);
-    wsrc[j] = wb + (size_t)n * K + ch * 8;
+    wsrc[j] = wb + (size_t)n * K + kbeg + ch * 8;
   }
 #pragma unroll
   for (int j = 0; j < AL; ++j) {
     const int slot = (w * AL + j) * 64 + lane, row = slot / G::CPR;
     const int ch = (int)((G::swz(row, slot % G::CPR) - (unsigned)row * G::RB) >> 4);
-    asrc[j] = A + (size_t)min(m0 + row, M - 1) * lda + ch * 8;
+    asrc[j] = A + (size_t)min(m0 + row, M - 1) * lda + kbeg + ch * 8;
   }
   const unsigned wslot = (unsigned)(w * WL) * 1024u, aslot = (unsigned)BF * G::RB + (unsigned)(w * AL) * 1024u;   // wave-uniform
 #define GM_FETCH(stage_, k0)                                                                                 \
@@ -165,7 +172,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
     for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  const int nkt = K / G::BK;
+  const int nkt = K / ksplit / G::BK;
   // Software pipeline over the k tiles.  NS-1 tiles are in flight ahead of the one being multiplied.  Within a tile the
   // fragments of k step kk+1 are read while step kk is multiplied; before the last step of tile kt the wave makes sure
   // its reads of the tile are complete, waits for its share of tile kt+1, meets the barrier (every wave's share has
@@ -250,6 +257,10 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+          if (MODE == 3) {
+            *(float4*)((float*)C + ((size_t)slice * M + m) * ldc + f) = make_float4(v[0], v[1], v[2], v[3]);
+            continue;
+          }
           if (MODE == 2) {
             const uint2 rv = *(const uint2*)(R + (size_t)m * ldr + f);
             v[0] = __uint_as_float(rv.x << 16) + rnd_bf16(v[0]);
@@ -265,15 +276,15 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long long lda, const bf16_t* __re
 
 template <class G, int MODE>
 int gemm_launch_tile(const void* A, long long lda, const void* W, const void* W2, const void* R, long long ldr, void* C,
-                     long long ldc, int M, int N, int K, hipStream_t s) {
+                     long long ldc, int M, int N, int K, hipStream_t s, int ksplit = 1) {
   constexpr int NF = MODE == 1 ? G::BF / 2 : G::BF;
   static hipError_t attr_err = hipFuncSetAttribute((const void*)gemm_bf16_kernel<G, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS);
   if (attr_err != hipSuccess) { fstu_set_error("fstu_gemm_bf16: hipFuncSetAttribute: %s", hipGetErrorString(attr_err)); return (int)attr_err; }
   const int mt = (M + G::BT - 1) / G::BT, nt = (N + NF - 1) / NF;
-  const long long tiles = (long long)mt * nt;
+  const long long tiles = (long long)mt * nt * ksplit;
   const int share = (int)((tiles + 7) / 8);
   hipLaunchKernelGGL((gemm_bf16_kernel<G, MODE>), dim3((unsigned)share * 8u), dim3(G::THREADS), G::LDS, s, (const bf16_t*)A, lda,
-                     (const bf16_t*)W, (const bf16_t*)W2, (const bf16_t*)R, ldr, (bf16_t*)C, ldc, M, N, K, mt, nt, share);
+                     (const bf16_t*)W, (const bf16_t*)W2, (const bf16_t*)R, ldr, (bf16_t*)C, ldc, M, N, K, mt, nt, share, ksplit);
   return 0;
 }
 
@@ -291,12 +302,14 @@ int gemm_cus() {
 using TileBig = GemmTile<4, 2, 2, 4, 64, 2>;     // 256 x 256, 8 waves, 128 KB of LDS
 using TileSmall = GemmTile<2, 2, 2, 2, 64, 2>;   // 128 x 128, 4 waves, 64 KB: two workgroups per compute unit
 using TileDeep = GemmTile<2, 2, 2, 2, 64, 4>;    // 128 x 128, 4 waves, 3 tiles in flight: one workgroup per compute unit
+using TileRows32 = GemmTile<2, 1, 2, 1, 64, 4>;  // 128 features x 32 rows, 2 waves, 80 KB: weight streaming, two workgroups per compute unit
 using TileK32 = GemmTile<2, 2, 4, 2, 32, 3>;     // 256 x 128, 4 waves, 72 KB, k tiles of 32 for K % 64 != 0
 
 template <int MODE>
 int gemm_launch(const void* A, long long lda, const void* W, const void* W2, const void* R, long long ldr, void* C, long long ldc,
                 int M, int N, int K, hipStream_t s) {
   if (K % 64 != 0) return gemm_launch_tile<TileK32, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  if (M <= 32) return gemm_launch_tile<TileRows32, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
   // Measured choices (MI355X, bf16): the large tile halves the fill traffic per flop and pays once K amortises its
   // start-up and the grid still covers the chip twice (M=32768, K >= 2048: 1.01-1.18 PFLOP/s against 0.89-0.99;
   // M=4096, N=9216, K=768: 92 us against 80 us).  A grid that leaves one workgroup per compute unit anyway gains from
@@ -310,6 +323,23 @@ int gemm_launch(const void* A, long long lda, const void* W, const void* W2, con
 }
 
 }  // namespace
+
+extern "C" int fstu_gemm_bf16_splitk(const void* A, int64_t lda, const void* W, float* partial, int M, int N, int K, int ksplit,
+                                     void* stream) {
+  FSTU_REQUIRE(A && W && partial, FSTU_ENULL, "fstu_gemm_bf16_splitk: null pointer");
+  FSTU_REQUIRE(ksplit >= 1 && ksplit <= 64 && K % (64 * ksplit) == 0, FSTU_ESHAPE,
+               "fstu_gemm_bf16_splitk: K=%d must be a multiple of 64*ksplit (ksplit=%d, 1..64)", K, ksplit);
+  FSTU_REQUIRE(M >= 1 && N >= 4 && N % 4 == 0 && lda >= K && lda % 8 == 0, FSTU_ESHAPE,
+               "fstu_gemm_bf16_splitk: M=%d N=%d (N %% 4 == 0) lda=%lld", M, N, (long long)lda);
+  FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(partial, 16), FSTU_EALIGN,
+               "fstu_gemm_bf16_splitk: pointers must be 16-byte aligned");
+  int rc;
+  if (M <= 32) rc = gemm_launch_tile<TileRows32, 3>(A, lda, W, nullptr, nullptr, 0, partial, N, M, N, K, (hipStream_t)stream, ksplit);
+  else rc = gemm_launch_tile<TileSmall, 3>(A, lda, W, nullptr, nullptr, 0, partial, N, M, N, K, (hipStream_t)stream, ksplit);
+  if (rc) return rc;
+  FSTU_CHECK_LAUNCH("fstu_gemm_bf16_splitk");
+  return FSTU_OK;
+}
 
 extern "C" int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, const void* R, int64_t ldr, void* C,
                               int64_t ldc, int M, int N, int K, int mode, void* stream) {

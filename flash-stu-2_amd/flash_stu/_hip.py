@@ -79,6 +79,7 @@ SIGNATURES = {
     "fstu_prof_copy": [_vp, _vp, ctypes.c_size_t, _vp],
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
     "fstu_gemm_bf16": [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
+    "fstu_gemm_bf16_splitk": [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_lds_sequence_ws_floats": [_i, _i, _i],
     "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -292,6 +293,23 @@ def gemm(x2: torch.Tensor, weight: torch.Tensor, up_weight: Optional[torch.Tenso
     _check(load().fstu_gemm_bf16(_p(x2), x2.stride(0), _p(weight), _p(up_weight), _p(residual), ldr, _p(out), out.stride(0),
                                  M, N, K, mode, _stream()), "fstu_gemm_bf16")
     return out
+
+
+def gemm_splitk(x2: torch.Tensor, weight: torch.Tensor, ksplit: int, partial: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 partial sums (ksplit, M, N) of x2 (M,K) @ weight (N,K)^T over ksplit slices of K; add_rmsnorm with
+    delta_mode=1, nslices=ksplit folds them into the residual stream."""
+    _dev(weight, partial)
+    if not gemm_supported(x2, weight) or not x2.is_cuda or x2.shape[1] % (64 * ksplit) != 0:
+        raise FlashSTUHipError(f"gemm_splitk: unsupported operands {tuple(x2.shape)} x {tuple(weight.shape)} / {ksplit}")
+    M, K = x2.shape
+    N = weight.shape[0]
+    if partial is None:
+        partial = torch.empty(ksplit, M, N, dtype=torch.float32, device=x2.device)
+    if partial.shape != (ksplit, M, N) or partial.dtype != torch.float32:
+        raise FlashSTUHipError("gemm_splitk: partial must be (ksplit, M, N) fp32")
+    _check(load().fstu_gemm_bf16_splitk(_p(x2), x2.stride(0), _p(weight), _p(partial), M, N, K, ksplit, _stream()),
+           "fstu_gemm_bf16_splitk")
+    return partial
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -130,10 +130,18 @@ class DecodeEngine:
                         caches[i] = (bigger, state, pos)
         self.graph_end()
         self.chunks = []
-        for b0 in range(0, B, _hip.MAX_DECODE_ROWS):
-            ch = _Chunk(b0, min(B, b0 + _hip.MAX_DECODE_ROWS))
+        R = _hip.MAX_DECODE_ROWS
+        # Rows are stepped in chunks of up to 16 (the width of the skinny decode kernels), each chunk re-reading the
+        # weights.  A chunk of 17..32 rows instead runs its MLP, nearly all of the weight bytes, once over all rows on the
+        # tiled GEMM kernel (bf16, recurrence STU state).
+        wide = (cfg.torch_dtype == torch.bfloat16 and mode == "lds" and d % 256 == 0 and (d * cfg.mlp_scale) % 64 == 0)
+        b0 = 0
+        while b0 < B:
+            rows = min(B - b0, 2 * R if (wide and B - b0 > R) else R)
+            ch = _Chunk(b0, b0 + rows)
             self._build_chunk(ch, caches)
             self.chunks.append(ch)
+            b0 += rows
         return tuple(caches)
 
     def _build_chunk(self, ch: _Chunk, caches):
@@ -238,6 +246,12 @@ class DecodeEngine:
                     m.merge_norm = 1
         ch.arr, ch.desc = arr, m
         ch.mega = None
+        if B > _hip.MAX_DECODE_ROWS:
+            # first use of the tiled kernels outside any graph capture (their launch set-up raises an LDS limit once)
+            wx = torch.zeros(B, 64, dtype=dt, device=dev)
+            ww = torch.zeros(8, 64, dtype=dt, device=dev)
+            _hip.gemm(wx, ww, up_weight=ww)
+            _hip.gemm_splitk(wx, ww, 1)
         if (dt == torch.bfloat16 and mode == "lds" and m.glu_packed and m.down_packed and not cfg.use_hankel_L
                 and os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") == "1"):
             # opt-in: the whole step as one persistent launch (packed copies of every weight, one workspace for the

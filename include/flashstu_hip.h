@@ -322,6 +322,12 @@ int fstu_head_argmax_static(const void* x, int ldx, const void* W, void* logits,
  * K % 64 == 0, N % 4 == 0, lda % 8 == 0; A, W, W2 16-byte aligned.  C may alias R. */
 int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, const void* R, int64_t ldr, void* C,
                    int64_t ldc, int M, int N, int K, int mode, void* stream);
+/* The same contraction cut into ksplit slices of K, for a long K with few output tiles (down_proj of a decode step over
+ * 17..32 rows, flash_stu/modules/swiglu.py:28): partial (ksplit,M,N) fp32 receives the unrounded slice sums, which
+ * fstu_add_rmsnorm (delta_mode 1, nslices = ksplit) adds into the residual stream as T(x + T(sum)).
+ * K % (64*ksplit) == 0, ksplit 1..64. */
+int fstu_gemm_bf16_splitk(const void* A, int64_t lda, const void* W, float* partial, int M, int N, int K, int ksplit,
+                          void* stream);
 
 /* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
  * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:

@@ -190,16 +190,18 @@ def test_c5_shape_sampling_parity_reduced():
     assert torch.equal(got.cpu(), ref)
 
 
-def test_c5_shape_bf16_lds_teacher_forced():
-    """Same structure in bf16 with the recurrence state, logits within the bf16 tolerance."""
+@pytest.mark.parametrize("rows", [17, 20, 32])
+def test_c5_shape_bf16_lds_teacher_forced(rows):
+    """Same structure in bf16 with the recurrence state, logits within the bf16 tolerance.  17..32 rows step as one
+    chunk: the MLP once over all rows on the tiled GEMM kernel, the state operators on the two halves of the rows."""
     from test_gpu_model import make_pair, prompt, _teacher_forced
     ocfg, w, model = make_pair(seed=2, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=256, n_layers=4,
                                n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
                                stu_decode_mode="lds")
     P, N = 20, 60
-    ids = prompt(20, P, ocfg.vocab_size, 4)           # 16 + 4 rows
+    ids = prompt(rows, P, ocfg.vocab_size, 4)
     got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
-    again = model.generate(ids.cuda(), max_length=P + N, do_sample=False)        # graph replay, chunked
+    again = model.generate(ids.cuda(), max_length=P + N, do_sample=False)        # graph replay
     assert torch.equal(again, got)
     ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
     err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
