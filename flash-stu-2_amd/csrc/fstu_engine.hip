@@ -177,12 +177,10 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
     TIMED(PC_DOWN, fstu_gemm_bf16_splitk(m->act, I, L.w_down, m->partial, B, d, I, ks, stream));
     TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, ks, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
-  for (int c = 0; c < 2; ++c) {
-    const int rc = rows_of(c);
-    TIMED(PC_HEAD, fstu_linear_decode(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rc, m->V, d, dt, stream));
-    TIMED(PC_SAMPLE, fstu_sample_dyn(at(m->logits, c, (size_t)m->V), tok_out + (size_t)c * R * tok_stride, tok_stride, rc, m->V, temperature,
-                                     top_k, top_p, do_sample, seed, step, m->row0 + c * R, dyn, dt, stream));
-  }
+  for (int c = 0; c < 2; ++c)
+    TIMED(PC_HEAD, fstu_linear_decode(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, dt, stream));
+  TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0,
+                                   dyn, dt, stream));
   if (dyn) STEP(fstu_advance_dyn(dyn, stream));
   return FSTU_OK;
 }
