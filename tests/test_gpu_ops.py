@@ -124,7 +124,7 @@ def test_mlp_decode_chain(hip, dtype, rows, d, I):
 # Prompt-pass GEMM kernel: the three tile shapes (128 x 128; 256 x 256 for K >= 1024 on grids that cover the chip
 # twice; k tiles of 32 for K % 64 != 0), ragged M and N, one- and many-tile grids.
 GEMM_SHAPES = [(4096, 2304, 768), (512, 768, 768), (1000, 772, 96), (17, 4, 32), (300, 200, 1056), (2048, 16384, 1024),
-               (257, 132, 64)]
+               (257, 132, 64), (32, 2048, 512), (20, 260, 128), (4096, 768, 3072)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -163,6 +163,26 @@ def test_gemm_bf16_gated_pair(hip, M, d, I):
     tol = r.abs() * 2.0 ** -6 + 1.2 * 2.0 ** -7 * (gate.float() * up.float()).abs() + 1e-3 * 2.0 ** -7 * float(r.abs().max())
     assert bool(((got - r).abs() <= tol).all()), float(((got - r).abs() - tol).max())
     assert float(((got - r).abs() > 0).float().mean()) <= 0.05
+
+
+@pytest.mark.parametrize("M,N,K,ks", [(32, 2048, 8192, 16), (17, 768, 3072, 4), (300, 132, 512, 2), (32, 256, 64, 1)])
+def test_gemm_bf16_splitk_feeds_the_residual_norm(hip, M, N, K, ks):
+    """fstu_gemm_bf16_splitk leaves fp32 slice sums; fstu_add_rmsnorm (delta_mode 1) folds them into the residual stream
+    as T(x + T(sum)) and normalises: the down projection of a decode step over 17..32 rows."""
+    g = gen(64)
+    act = torch.randn(M, K, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    x = torch.randn(M, N, generator=g).bfloat16()
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).bfloat16()
+    part = hip.gemm_splitk(dev(act), dev(W), ks)
+    assert part.shape == (ks, M, N) and part.dtype == torch.float32
+    full = F.linear(act.float(), W.float())
+    assert float((part.sum(0).cpu() - full).abs().max()) <= 2e-5 * float(full.abs().max()) * math.sqrt(K / 64)
+    xd = dev(x.clone())
+    h = hip.add_rmsnorm(xd, part, dev(nw), O.RMS_EPS_DEFAULT, delta_mode=1, nslices=ks)
+    xr = (x.float() + full.bfloat16().float()).bfloat16()
+    check(xd, xr, torch.bfloat16, frac=0.05, atol=2.0 ** -7 * float(full.abs().max()))
+    check(h, O.rms_norm(xd.cpu(), nw, O.RMS_EPS_DEFAULT), torch.bfloat16, frac=0.05)
 
 
 def test_gemm_bf16_strided_operands_and_errors(hip):
