@@ -89,9 +89,12 @@ struct GemmTile {
   static constexpr int NFR = FI + TJ;                            // fragments per k step
   static_assert(BK == 32 || BK == 64, "k tile");
   static_assert((BF * CPR) % (64 * NW) == 0 && (BT * CPR) % (64 * NW) == 0, "fill split");
-  // byte offset of 16-byte chunk c of a row inside a tile
+  // Byte offset of 16-byte chunk c of a row inside a tile.  A 16-byte fragment read is served 16 lanes (16 consecutive
+  // rows, one chunk each) at a time and is free of bank conflicts when those 16 pieces fall into 16 different 16-byte
+  // slots of a 256-byte window: the row's position inside the window supplies 1 (128-byte rows) or 2 (64-byte rows) of
+  // the 4 slot bits, the XOR with the next higher row bits the other 3 or 2.
   __device__ static __forceinline__ unsigned swz(int row, int c) {
-    return (unsigned)row * RB + (unsigned)((c ^ (BK == 64 ? (row & 7) : ((row >> 1) & 3))) << 4);
+    return (unsigned)row * RB + (unsigned)((c ^ (BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3))) << 4);
   }
 };
 
