@@ -48,6 +48,9 @@ def decode_step_bytes(cfg, B, t, mode, S):
     kv = n_att * B * 2 * d * w * (min(t, cfg.window_left + 1) + 1)
     if mode == "lds":
         stu = n_stu * (B * S * d * 4 * 3 + 2 * S * d * 4)      # both parity banks read, one written; ce and co
+        R = int(getattr(cfg, "stu_lds_fir_taps", 0) or 0)
+        if R and not cfg.use_hankel_L:
+            stu += n_stu * (B * R * d * w + B * d * w + R * d * 4)   # ring of the last R inputs read, one row written; taps
     else:
         stu = n_stu * (B * (t + 1) * d * w + (t + 1) * d * w)
     return weights + kv + stu + B * V * w
@@ -223,7 +226,8 @@ def run_lm(args, torch, _hip, which):
     K, W = args.steps, args.warmup
 
     def build(mlp_scale):
-        cfg = FlashSTUConfig(mlp_scale=mlp_scale, torch_dtype=dt, stu_decode_mode=stu_mode, stu_prefill_mode=args.stu_prefill, **kw)
+        fir = {} if args.fir_taps is None else {"stu_lds_fir_taps": args.fir_taps}
+        cfg = FlashSTUConfig(mlp_scale=mlp_scale, torch_dtype=dt, stu_decode_mode=stu_mode, stu_prefill_mode=args.stu_prefill, **fir, **kw)
         torch.manual_seed(seed)
         with torch.device("cuda"):
             model = FlashSTU(cfg)
@@ -276,6 +280,7 @@ def run_lm(args, torch, _hip, which):
         "config": {"workload": label, "mlp_scale": cfg.mlp_scale, "params": res["params"], "batch": B, "prompt": P,
                    "stu_decode_mode": stu_mode, "stu_prefill_mode": args.stu_prefill, "hip_graph": res["hip_graph"],
                    "graph_steps": args.graph_steps, "stu_state_dim": cfg.stu_lds_state_dim if stu_mode == "lds" else None,
+                   "stu_fir_taps": cfg.stu_lds_fir_taps if stu_mode == "lds" else None,
                    "one_launch_step": os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") == "1"},
         "step_roofline": res["step_roofline"],
         "prefill_tokens_per_s": res.get("prefill_tokens_per_s"), "prefill_ms": res.get("prefill_ms"),
@@ -444,6 +449,8 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"], help="BASELINE.json workload (default: config 2)")
     ap.add_argument("--mlp-scale", type=int, default=12, dest="mlp_scale")
     ap.add_argument("--stu-mode", default="lds", choices=["lds", "history"], dest="stu_mode")
+    ap.add_argument("--fir-taps", type=int, default=None, dest="fir_taps",
+                    help="exact head of the distilled STU filter: first lags taken from phi_proj itself (0: off; default: the config's)")
     ap.add_argument("--stu-prefill", default="fft", choices=["fft", "scan"], dest="stu_prefill",
                     help="prompt pass of the STU layers: the reference's FFT convolution, or the distilled recurrence as a scan")
     ap.add_argument("--batch", type=int, default=0, help="batch rows (default: the workload's own)")

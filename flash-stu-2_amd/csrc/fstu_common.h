@@ -50,14 +50,16 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
-int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* y,
-                               int ldy, int B, int S, int d, int t, const int* dyn, int dtype, void* stream);
+int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
+                               const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
+                               const int* pos_dyn, int dtype, void* stream);
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                             const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn,
-                             void* stream);
+                             const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, void* xp_out, int B,
+                             int S, int d, int K, int t, const int* dyn, const int* pos_dyn, void* stream);
 int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
-                                 int B, int S, int d, int K, int t, const int* dyn, void* stream);
+                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* ring,
+                                 const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int K, int t,
+                                 const int* dyn, const int* pos_dyn, void* stream);
 // the whole step as one persistent launch: tokens / tok_out are the column-0 bases of the input and output views, the
 // step reads column `pos` (dyn[0] when dyn is given) of the first and writes the same column of the second
 bool fstu_step_mega_ok(const fstu_model_desc* m);
@@ -65,6 +67,11 @@ int fstu_step_mega_launch(const fstu_model_desc* m, int64_t* tokens, int64_t* to
                           float temperature, int greedy, int* dyn, void* stream);
 
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+// the optional exact head of the distilled filter: ring, taps and their count go together; count a power of two in 8..1024
+static inline bool fstu_fir_ok(const void* ring, const float* fir, int taps) {
+  if (!ring && !fir && taps == 0) return true;
+  return ring && fir && taps >= 8 && taps <= 1024 && (taps & (taps - 1)) == 0 && fstu_aligned(ring, 16) && fstu_aligned(fir, 16);
+}
 
 // ---------------------------------------------------------------- dtypes
 typedef unsigned short bf16_t;  // raw bf16 bits

@@ -105,10 +105,11 @@ extern "C" int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* st
   } while (0)
 
 // recurrence step on m->xp: both sign branches rounded separately when the layer carries odd-lag weights
-static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, void* stream) {
+static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, const int* pos_dyn, void* stream) {
   if (L.lds_co)
-    return fstu_stu_step_lds_pair_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, L.lds_co, m->y, m->d, m->B, m->lds_S, m->d, pos,
-                                      dyn, m->dtype, stream);
+    return fstu_stu_step_lds_pair_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, L.lds_co, L.lds_ring, L.lds_fir,
+                                      L.lds_fir ? m->lds_fir_taps : 0, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, pos_dyn,
+                                      m->dtype, stream);
   return fstu_stu_step_lds_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, m->dtype,
                                stream);
 }
@@ -162,7 +163,7 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
       for (int c = 0; c < 2; ++c)
         TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.m_inputs_t, at(m->xp, c, d), d, rows_of(c), d, d, dt, stream));
-      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), stream));
+      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream));
     } else {
       for (int c = 0; c < 2; ++c)
         TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.w_qkv, at(m->qkv, c, 3 * (size_t)d), 3 * d, rows_of(c), 3 * d, d, dt, stream));
@@ -266,15 +267,17 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
       } else {
         if (pending_slices) {
           TIMED(PC_STU, fstu_stu_res_inproj_step_dyn(xc, m->partial, 4, xo, L.norm1_w, m->eps, L.m_inputs_t, L.lds_state, L.lds_a,
-                                                     L.lds_ce, L.lds_co, m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
+                                                     L.lds_ce, L.lds_co, L.lds_ring, L.lds_fir, L.lds_fir ? m->lds_fir_taps : 0,
+                                                     m->y, d, B, m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), dyn, stream));
           void* t = xc; xc = xo; xo = t;
           pending_slices = false;
         } else if (dt == FSTU_BF16 && d % 256 == 0) {
-          TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, m->y, d, nullptr, B,
-                                                 m->lds_S, d, d, stu_pos(pos), stu_dyn(dyn), stream));
+          TIMED(PC_STU, fstu_stu_inproj_step_dyn(m->h, d, L.m_inputs_t, L.lds_state, L.lds_a, L.lds_ce, L.lds_co, L.lds_ring, L.lds_fir,
+                                                 L.lds_fir ? m->lds_fir_taps : 0, m->y, d, nullptr, B, m->lds_S, d, d, stu_pos(pos),
+                                                 stu_dyn(dyn), dyn, stream));
         } else {
           TIMED(PC_PROJ, fstu_linear_decode(m->h, d, L.m_inputs_t, m->xp, d, B, d, d, dt, stream));
-          TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), stream));
+          TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream));
         }
         pending_y = true;
       }

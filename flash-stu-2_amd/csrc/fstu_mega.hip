@@ -973,7 +973,8 @@ bool mega_plan(const fstu_model_desc* m, MegaPlan* p) {
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     if (!L.wp_gate || !L.wp_up || !L.wp_down || !L.norm1_w || !L.mlp_norm_w) return false;
-    if (L.kind == 0) { if (!L.wp_m_inputs || !L.lds_state || !L.lds_a || !L.lds_ce || !L.lds_co) return false; }
+    // (the one-launch step does not carry the exact head of the filter)
+    if (L.kind == 0) { if (!L.wp_m_inputs || !L.lds_state || !L.lds_a || !L.lds_ce || !L.lds_co || L.lds_fir) return false; }
     else if (!L.wp_qkv || !L.wp_proj || !L.kring || !L.vring || !L.slopes) return false;
   }
   if (!m->wp_emb || !m->emb || !m->final_norm_w || !m->logits) return false;

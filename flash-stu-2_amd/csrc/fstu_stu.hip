@@ -111,6 +111,48 @@ extern "C" int fstu_stu_step_hist(const void* hist, const void* filt, float* eo,
   return FSTU_OK;
 }
 
+// ---------------------------------------------------------------- exact head of the distilled filter
+// The recurrence reproduces the effective filter phi_proj up to its lag-by-lag bf16 rounding, which is largest on the
+// first lags.  fir[s, c] = f[s, c] - f_fit[s, c] for the first R lags (R a power of two, a multiple of 8) corrects them
+// exactly from a ring of the last R projected inputs (ring[b, p % R, c] = x_proj of position p, zero before the first
+// position): even lags add to E, odd lags to O.  Mode group g of a (row, 4 channels) pair takes lags g, g+8, ...: their
+// parity is that of g, so the partial sum joins E (g even) or O (g odd) before the reduction over the mode groups.
+template <typename T> struct Ring4 {
+  static __device__ __forceinline__ void ld(const T* p, float (&v)[4]) {
+    const float4 q = *(const float4*)p;
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  }
+  static __device__ __forceinline__ void st(T* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Ring4<bf16_t> {
+  static __device__ __forceinline__ void ld(const bf16_t* p, float (&v)[4]) {
+    const uint2 q = *(const uint2*)p;
+    v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+    v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, const float (&v)[4]) {
+    *(uint2*)p = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+  }
+};
+template <typename T>
+__device__ __forceinline__ void fir_head(const T* __restrict__ ring, const float* __restrict__ fir, int R, int tt, int b, int c,
+                                         int d, int g, const float (&x)[4], float (&f)[4]) {
+  const T* rb = ring + (size_t)b * R * d + c;
+  // (all 16 lags of a thread in flight at once was measured slower than four at a time: 0.354 against 0.336 ms per
+  // step at 128 taps)
+#pragma unroll 4
+  for (int s = g; s < R; s += 8) {
+    float xv[4];
+    const int p = tt - s;
+    // a position before the sequence contributes nothing; its slot is read all the same (no branch around the load)
+    Ring4<T>::ld(rb + (size_t)(p & (R - 1)) * d, xv);
+    const float m = (s > 0 && p >= 0) ? 1.f : 0.f;
+    const float4 rv = *(const float4*)(fir + (size_t)s * d + c);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = fmaf(i == 0 ? rv.x : i == 1 ? rv.y : i == 2 ? rv.z : rv.w, s == 0 ? x[i] : m * xv[i], f[i]);
+  }
+}
+
 // ---------------------------------------------------------------- LDS-form step
 // Workgroup = 32 channel quads (128 channels) x 8 mode groups.  Each thread
 // advances S/8 modes of 4 channels (float4 state accesses, 512 contiguous
@@ -121,10 +163,13 @@ __global__ void __launch_bounds__(256)
 stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
                     const float* __restrict__ ce, const float* __restrict__ co /*optional: weights of the other bank*/,
                     float scale, T* __restrict__ y, int ldy, int S, int d, int parity, const int* __restrict__ dyn,
-                    int pair /* != 0 (needs co): y = T(T(E+O) + T(E-O)), the two sign branches rounded separately */) {
+                    int pair /* != 0 (needs co): y = T(T(E+O) + T(E-O)), the two sign branches rounded separately */,
+                    T* __restrict__ ring /*optional (B,R,d), with fir (R,d) and co: exact head of the filter*/,
+                    const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn) {
   __shared__ float sh[LDS_JG][32][4];
   __shared__ float sho[LDS_JG][32][4];
   if (dyn) parity = dyn[0] & 1;
+  if (pos_dyn) t = pos_dyn[0];
   const int b = blockIdx.y;
   const int q = threadIdx.x & 31, jg = threadIdx.x >> 5;
   const int c = (blockIdx.x * 32 + q) * 4;
@@ -162,6 +207,15 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
         acco[2] = fmaf(oj.z, h.z, acco[2]);
         acco[3] = fmaf(oj.w, h.w, acco[3]);
       }
+      if (fir) {
+        float f[4] = {0.f, 0.f, 0.f, 0.f};
+        fir_head<T>(ring, fir, R, t, b, c, d, jg, x, f);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          if (jg & 1) acco[v] += f[v]; else acc[v] += f[v];
+        }
+        if (jg == 0) Ring4<T>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, x);
+      }
     }
   }
 #pragma unroll
@@ -186,7 +240,8 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
 
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream, int pair = 0);
+                               void* stream, int pair = 0, void* ring = nullptr, const float* fir = nullptr, int R = 0,
+                               const int* pos_dyn = nullptr);
 
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
@@ -202,20 +257,28 @@ extern "C" int fstu_stu_step_lds_single(float* state, const void* xp, int ldxp, 
 }
 
 extern "C" int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce,
-                                      const float* co, void* y, int ldy, int B, int S, int d, int t, int dtype, void* stream) {
-  return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, y, ldy, B, S, d, t, nullptr, dtype, stream);
+                                      const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S,
+                                      int d, int t, int dtype, void* stream) {
+  return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
+                                    stream);
 }
 
-int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* y,
-                               int ldy, int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
+// ring / fir / fir_taps: optional exact head of the filter (all three or none).  dyn: device-side {position, step} that
+// supplies the parity; pos_dyn: the same words where only the ring slot is read from them (the parity then comes with t)
+int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
+                               const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
+                               const int* pos_dyn, int dtype, void* stream) {
   FSTU_REQUIRE(co, FSTU_ENULL, "fstu_stu_step_lds_pair: null pointer");
   FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_pair: co must be 16-byte aligned");
-  return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, dyn, dtype, stream, 1);
+  FSTU_REQUIRE(fstu_fir_ok(ring, fir, fir_taps), FSTU_EARG,
+               "fstu_stu_step_lds_pair: ring, fir and fir_taps (a power of two, 8..1024) go together, 16-byte aligned");
+  return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, dyn, dtype, stream, 1, ring, fir, fir_taps,
+                             dyn ? dyn : pos_dyn);
 }
 
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream, int pair) {
+                               void* stream, int pair, void* ring, const float* fir, int R, const int* pos_dyn) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
   FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
@@ -224,7 +287,8 @@ static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const flo
   dim3 grid((d / 4 + 31) / 32, B);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
                       hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
-                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair));
+                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair, (T*)ring, fir, R,
+                                         t, pos_dyn));
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }
@@ -319,11 +383,14 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
                        const float* __restrict__ slices /*optional, with x_res: up to 4 fp32 (B,K) slices added first*/,
                        int nslices, bf16_t* __restrict__ x_out /*receives x_res + T(sum of slices); not x_res itself*/,
                        const float* __restrict__ co /*optional (S,d): odd-lag weights on the other bank; then
-                       y = T(T(E+O) + T(E-O)) instead of T(2E)*/) {
+                       y = T(T(E+O) + T(E-O)) instead of T(2E)*/,
+                       bf16_t* __restrict__ ring /*optional (B,R,d), with fir (R,d) and co: exact head of the filter*/,
+                       const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn) {
   __shared__ float red[4][64][4];
   __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
   extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
   if (dyn) parity = dyn[0] & 1;
+  if (pos_dyn) t = pos_dyn[0];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   // A tile's 16 channels are half a 128-byte line of every state and output-weight row.  Workgroups go round the 8
@@ -526,6 +593,14 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
         sumo.z = fmaf(oj.z, hv.z, sumo.z);
         sumo.w = fmaf(oj.w, hv.w, sumo.w);
       }
+      if (fir) {
+        const float xv[4] = {xps[b][cq * 4], xps[b][cq * 4 + 1], xps[b][cq * 4 + 2], xps[b][cq * 4 + 3]};
+        float f[4] = {0.f, 0.f, 0.f, 0.f};
+        fir_head<bf16_t>(ring, fir, R, t, b, c, d, jsub, xv, f);
+        if (jsub & 1) { sumo.x += f[0]; sumo.y += f[1]; sumo.z += f[2]; sumo.w += f[3]; }
+        else { sum.x += f[0]; sum.y += f[1]; sum.z += f[2]; sum.w += f[3]; }
+        if (jsub == 0) Ring4<bf16_t>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, xv);
+      }
     }
     // reduce over the 8 mode groups (lanes differing in bits 2..4): two rotations inside the row of 16 lanes, one
     // swizzle across the two rows
@@ -562,36 +637,46 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
     }
   }
 }
+struct FirArgs {
+  void* ring;
+  const float* fir;
+  int taps;
+  const int* pos_dyn;
+};
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
                               float* state, const float* a, const float* ce, const float* co, void* y, int ldy, void* xp_out,
-                              int B, int S, int d, int K, int t, const int* dyn, void* stream, const float* slices = nullptr,
-                              int nslices = 0, void* x_out = nullptr);
+                              int B, int S, int d, int K, int t, const int* dyn, void* stream, FirArgs fa,
+                              const float* slices = nullptr, int nslices = 0, void* x_out = nullptr);
 
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                             const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, const int* dyn,
-                             void* stream) {
-  return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, dyn, stream);
+                             const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, void* xp_out, int B,
+                             int S, int d, int K, int t, const int* dyn, const int* pos_dyn, void* stream) {
+  return inproj_step_launch(h, ldh, nullptr, nullptr, 0.f, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, dyn, stream,
+                            FirArgs{ring, fir, fir_taps, dyn ? dyn : pos_dyn});
 }
 
 // x' = x_in + T(sum of nslices <= 4 fp32 slices) goes to x_out, h = rmsnorm(x') * norm_w feeds the projection: the
 // add+norm launch between the previous layer's down projection and this layer, folded into this kernel
 int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
-                                 int B, int S, int d, int K, int t, const int* dyn, void* stream) {
+                                 const void* Mt, float* state, const float* a, const float* ce, const float* co, void* ring,
+                                 const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int K, int t,
+                                 const int* dyn, const int* pos_dyn, void* stream) {
   FSTU_REQUIRE(x_in && slices && x_out && norm_w, FSTU_ENULL, "fstu_stu_res_inproj_step: null pointer");
   FSTU_REQUIRE(nslices >= 1 && nslices <= 4, FSTU_EARG, "fstu_stu_res_inproj_step: nslices=%d outside 1..4", nslices);
   FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_stu_res_inproj_step: x_out must not alias x_in");
   FSTU_REQUIRE((NormPrologue<256, 4, 4>::supported(B, K)), FSTU_ESHAPE, "fstu_stu_res_inproj_step: B=%d K=%d not supported", B, K);
   FSTU_REQUIRE(fstu_aligned(slices, 16) && fstu_aligned(x_out, 16), FSTU_EALIGN, "fstu_stu_res_inproj_step: pointers must be 16-byte aligned");
-  return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream, slices,
-                            nslices, x_out);
+  return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream,
+                            FirArgs{ring, fir, fir_taps, dyn ? dyn : pos_dyn}, slices, nslices, x_out);
 }
 
 static int inproj_step_launch(const void* h, int ldh, const void* x_res, const void* norm_w, float eps, const void* Mt,
                               float* state, const float* a, const float* ce, const float* co, void* y, int ldy, void* xp_out,
-                              int B, int S, int d, int K, int t, const int* dyn, void* stream, const float* slices, int nslices,
-                              void* x_out) {
+                              int B, int S, int d, int K, int t, const int* dyn, void* stream, FirArgs fa, const float* slices,
+                              int nslices, void* x_out) {
   FSTU_REQUIRE(h && Mt && state && a && ce && y, FSTU_ENULL, "fstu_stu_inproj_step: null pointer");
+  FSTU_REQUIRE(fstu_fir_ok(fa.ring, fa.fir, fa.taps) && (!fa.fir || co), FSTU_EARG,
+               "fstu_stu_inproj_step: ring, fir and fir_taps (a power of two, 8..1024) go together with co, 16-byte aligned");
   FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
   FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(Mt, 16) && fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_inproj_step: pointers must be 16-byte aligned");
@@ -600,22 +685,25 @@ static int inproj_step_launch(const void* h, int ldh, const void* x_res, const v
   FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w/co must be 16-byte aligned");
   hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,
                      (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,
-                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out, co);
+                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out, co, (bf16_t*)fa.ring,
+                     fa.fir, fa.taps, t, fa.pos_dyn);
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
 }
 
 extern "C" int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w,
                                         float eps, const void* Mt, float* state, const float* a, const float* ce,
-                                        const float* co, void* y, int ldy, int B, int S, int d, int K, int t, void* stream) {
-  return fstu_stu_res_inproj_step_dyn(x_in, slices, nslices, x_out, norm_w, eps, Mt, state, a, ce, co, y, ldy, B, S, d, K, t,
-                                      nullptr, stream);
+                                        const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, int B,
+                                        int S, int d, int K, int t, void* stream) {
+  return fstu_stu_res_inproj_step_dyn(x_in, slices, nslices, x_out, norm_w, eps, Mt, state, a, ce, co, ring, fir, fir_taps, y, ldy,
+                                      B, S, d, K, t, nullptr, nullptr, stream);
 }
 
 extern "C" int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                                    const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t,
-                                    void* stream) {
-  return fstu_stu_inproj_step_dyn(h, ldh, Mt, state, a, ce, co, y, ldy, xp_out, B, S, d, K, t, nullptr, stream);
+                                    const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, void* xp_out,
+                                    int B, int S, int d, int K, int t, void* stream) {
+  return fstu_stu_inproj_step_dyn(h, ldh, Mt, state, a, ce, co, ring, fir, fir_taps, y, ldy, xp_out, B, S, d, K, t, nullptr, nullptr,
+                                  stream);
 }
 
 // ---------------------------------------------------------------- state from history

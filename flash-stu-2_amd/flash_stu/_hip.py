@@ -34,11 +34,11 @@ SIGNATURES = {
     "fstu_bias_act": [_vp, _vp, _i64, _i, _i, _i, _vp],
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "fstu_stu_step_lds_pair": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_pair": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_single": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
-    "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_scan_lds": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -346,11 +346,26 @@ def stu_step_hist(hist: torch.Tensor, filt: torch.Tensor, t: int, nsplit: int, e
     return eo
 
 
+def _fir_args(ring, fir, B, d, dtype):
+    """(ring pointer, fir pointer, taps) of the optional exact head of the filter."""
+    if ring is None and fir is None:
+        return None, None, 0
+    if ring is None or fir is None:
+        raise FlashSTUHipError("ring and fir go together")
+    _dev(ring, fir)
+    R = fir.shape[0]
+    if ring.shape != (B, R, d) or fir.shape != (R, d) or fir.dtype != torch.float32 or ring.dtype != dtype:
+        raise FlashSTUHipError(f"ring must be (B,{R},d) in the model dtype and fir ({R},d) fp32")
+    return _p(ring), _p(fir), R
+
+
 def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
-                 out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None, pair: bool = False) -> torch.Tensor:
+                 out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None, pair: bool = False,
+                 ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None) -> torch.Tensor:
     """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d) = T(2E), E = ce . bank(t).  With co (S,d) and
     O = co . other bank: the single-branch form y = T(E+O) (use_hankel_L), or with pair=True the two sign branches
-    rounded separately, y = T(T(E+O) + T(E-O))."""
+    rounded separately, y = T(T(E+O) + T(E-O)).  pair=True with ring (B,R,d) and fir (R,d): the exact head of the
+    filter on the first R lags (the ring is updated in place)."""
     _dev(state, a, ce, co)
     B, two, S, d = state.shape
     assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
@@ -364,8 +379,9 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
     if co is not None:
         assert co.dtype == torch.float32 and co.shape == (S, d)
         if pair:
-            _check(load().fstu_stu_step_lds_pair(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), _p(out), ldy, B, S, d, t,
-                                                 _dt(xp), _stream()), "fstu_stu_step_lds_pair")
+            rp, fp, R = _fir_args(ring, fir, B, d, xp.dtype)
+            _check(load().fstu_stu_step_lds_pair(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), rp, fp, R, _p(out), ldy, B, S, d,
+                                                 t, _dt(xp), _stream()), "fstu_stu_step_lds_pair")
             return out
         _check(load().fstu_stu_step_lds_single(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), _p(out), ldy, B, S, d, t,
                                                _dt(xp), _stream()), "fstu_stu_step_lds_single")
@@ -400,7 +416,8 @@ def stu_scan_lds(xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, state: Opt
 
 def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
                     out: Optional[torch.Tensor] = None, xp_out: Optional[torch.Tensor] = None,
-                    co: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    co: Optional[torch.Tensor] = None, ring: Optional[torch.Tensor] = None,
+                    fir: Optional[torch.Tensor] = None) -> torch.Tensor:
     """h (B,K) bf16, Mt = M_inputs^T (d,K): projection + recurrence step in one launch -> y (B,d); with co the step
     of stu_step_lds(pair=True)."""
     _dev(h, Mt, state, a, ce, out, xp_out, co)
@@ -410,13 +427,15 @@ def stu_inproj_step(h: torch.Tensor, Mt: torch.Tensor, state: torch.Tensor, a: t
     assert h.dtype == Mt.dtype == torch.bfloat16 and Mt.shape[1] == K and state.shape == (B, 2, S, d)
     if out is None:
         out = torch.empty(B, d, dtype=h.dtype, device=h.device)
-    _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(co), _p(out), d, _p(xp_out), B, S, d,
-                                       K, t, _stream()), "fstu_stu_inproj_step")
+    rp, fp, R = _fir_args(ring, fir, B, d, h.dtype)
+    _check(load().fstu_stu_inproj_step(_p(h), K, _p(Mt), _p(state), _p(a), _p(ce), _p(co), rp, fp, R, _p(out), d, _p(xp_out), B,
+                                       S, d, K, t, _stream()), "fstu_stu_inproj_step")
     return out
 
 
 def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tensor, eps: float, Mt: torch.Tensor,
-                        state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int, co: Optional[torch.Tensor] = None):
+                        state: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int, co: Optional[torch.Tensor] = None,
+                        ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None):
     """(x', y): x' = x + bf16(sum of the fp32 slices); y = projection + recurrence step of rmsnorm(x') * norm_w."""
     _dev(x, partial, norm_w, Mt, state, a, ce, co)
     B, K = x.shape
@@ -425,8 +444,9 @@ def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Te
     assert x.dtype == Mt.dtype == torch.bfloat16 and partial.dtype == torch.float32 and state.shape == (B, 2, S, d)
     x_out = torch.empty_like(x)
     y = torch.empty(B, d, dtype=x.dtype, device=x.device)
+    rp, fp, R = _fir_args(ring, fir, B, d, x.dtype)
     _check(load().fstu_stu_res_inproj_step(_p(x), _p(partial), partial.shape[0], _p(x_out), _p(norm_w), float(eps), _p(Mt),
-                                           _p(state), _p(a), _p(ce), _p(co), _p(y), d, B, S, d, K, t, _stream()),
+                                           _p(state), _p(a), _p(ce), _p(co), rp, fp, R, _p(y), d, B, S, d, K, t, _stream()),
            "fstu_stu_res_inproj_step")
     return x_out, y
 

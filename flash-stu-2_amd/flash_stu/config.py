@@ -47,6 +47,7 @@ class FlashSTUConfig:
         rms_norm_eps: float = RMS_NORM_EPS,
         stu_decode_mode: str = "auto",       # "history" (exact), "lds" (distilled recurrence), "auto": lds for bf16
         stu_lds_state_dim: int = 64,
+        stu_lds_fir_taps: int = 64,          # exact head of the distilled filter: first lags taken from phi_proj itself (0: off)
         stu_prefill_mode: str = "fft",       # "fft": the reference's convolution; "scan": the distilled recurrence over the prompt
         **kwargs: Any,
     ):
@@ -88,6 +89,9 @@ class FlashSTUConfig:
             raise ValueError(f"stu_decode_mode must be auto|history|lds, got {stu_decode_mode!r}")
         self.stu_decode_mode = stu_decode_mode
         self.stu_lds_state_dim = stu_lds_state_dim
+        if stu_lds_fir_taps and (stu_lds_fir_taps < 8 or stu_lds_fir_taps > 1024 or stu_lds_fir_taps & (stu_lds_fir_taps - 1)):
+            raise ValueError(f"stu_lds_fir_taps must be 0 or a power of two in 8..1024, got {stu_lds_fir_taps}")
+        self.stu_lds_fir_taps = int(stu_lds_fir_taps)
         if stu_prefill_mode not in ("fft", "scan"):
             raise ValueError(f"stu_prefill_mode must be fft|scan, got {stu_prefill_mode!r}")
         self.stu_prefill_mode = stu_prefill_mode

@@ -28,7 +28,7 @@ _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
 class LayerDesc(ctypes.Structure):
     _fields_ = [("kind", _i), ("norm1_w", _vp), ("mlp_norm_w", _vp), ("w_gate", _vp), ("w_up", _vp), ("w_down", _vp),
-                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_co", _vp), ("lds_state", _vp),
+                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_co", _vp), ("lds_state", _vp), ("lds_ring", _vp), ("lds_fir", _vp),
                 ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp),
                 ("wp_gate", _vp), ("wp_up", _vp), ("wp_down", _vp), ("wp_m_inputs", _vp), ("wp_qkv", _vp),
                 ("wp_proj", _vp)]
@@ -37,7 +37,7 @@ class LayerDesc(ctypes.Structure):
 class ModelDesc(ctypes.Structure):
     _fields_ = [("dtype", _i), ("B", _i), ("d", _i), ("I", _i), ("V", _i), ("n_layers", _i), ("n_heads", _i),
                 ("head_dim", _i), ("window", _i), ("kv_cap", _i), ("L", _i), ("hist_cap", _i), ("stu_mode", _i),
-                ("lds_S", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i), ("row0", _i),
+                ("lds_S", _i), ("lds_fir_taps", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i), ("row0", _i),
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
@@ -156,6 +156,7 @@ class DecodeEngine:
         n = len(model.layers)
         arr = (LayerDesc * n)()
         hist_cap = 0
+        fir_taps = 0
         for i, layer in enumerate(model.layers):
             ld = arr[i]
             ld.w_gate = layer.mlp.gate_proj.weight.data_ptr()
@@ -175,6 +176,12 @@ class DecodeEngine:
                     st = state[b0:b1]
                     keep(a), keep(ce), keep(co), keep(st)
                     ld.lds_a, ld.lds_ce, ld.lds_co, ld.lds_state = a.data_ptr(), ce.data_ptr(), co.data_ptr(), st.data_ptr()
+                    fir = stu.lds_fir()
+                    if fir is not None and hist.shape[1] == fir.shape[0] and os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") != "1":
+                        ring = hist[b0:b1]       # in lds mode the history slot of the cache entry is the ring of the last inputs
+                        keep(fir), keep(ring)
+                        ld.lds_ring, ld.lds_fir = ring.data_ptr(), fir.data_ptr()
+                        fir_taps = fir.shape[0]
                 else:
                     hs = hist[b0:b1]
                     if hist_cap and hs.shape[1] != hist_cap:
@@ -204,6 +211,7 @@ class DecodeEngine:
         m.L, m.hist_cap = cfg.seq_len, hist_cap
         m.stu_mode = 1 if mode == "lds" else 0
         m.lds_S = cfg.stu_lds_state_dim
+        m.lds_fir_taps = fir_taps
         m.single_branch = int(cfg.use_hankel_L)
         m.ksplit_down = pick_ksplit_down(I) if dt == torch.bfloat16 else min(8, max(1, I // 512))
         m.hist_nsplit_max = self.HIST_NSPLIT_MAX

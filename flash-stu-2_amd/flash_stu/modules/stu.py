@@ -11,7 +11,8 @@ reference obtains by re-running the whole sequence:
                 per channel and two parity banks of recurrence state replace
                 the history (bounded state; bf16 performance mode).
 
-State tuples are batch-first tensors: (hist (B,cap,d), state (B,2,S,d) fp32, pos (B,) int64 on the host).
+State tuples are batch-first tensors: (hist (B,cap,d), state (B,2,S,d) fp32, pos (B,) int64 on the host); in lds mode
+the history slot holds the ring of the last stu_lds_fir_taps projected inputs (B,R,d), or is empty.
 """
 from __future__ import annotations
 
@@ -121,6 +122,41 @@ class STU(nn.Module):
             dev = self.M_filters.device
             return a.to(dev), ce.to(dev).contiguous(), co.to(dev).contiguous()
         return self._cached("lds", (self.phi, self.M_filters), build)
+
+    def lds_fir(self):
+        """(R,d) fp32: phi_proj minus the fitted filter on the first R = stu_lds_fir_taps lags, the exact head that the
+        two-branch decode step adds to the recurrence from a ring of the last R projected inputs; None when the head
+        is off or does not apply (Hankel-L, exact mode, history mode)."""
+        R = int(getattr(self.config, "stu_lds_fir_taps", 0) or 0)
+        if R == 0 or not self.use_approx or self.use_hankel_L or self.decode_mode() != "lds":
+            return None
+
+        def build():
+            a, ce, co = self.lds_params()
+            f = self.effective_filter().double().cpu()
+            L, d = f.shape
+            fr = torch.zeros(R, d, dtype=torch.float64)
+            fr[: min(R, L)] = f[: min(R, L)]                   # the reference's filter ends at lag L
+            m = torch.arange(R // 2, dtype=torch.float64)
+            V = a.double().cpu()[None, :] ** m[:, None]        # (R/2, S): a_j^m
+            fit = torch.empty(R, d, dtype=torch.float64)
+            fit[0::2] = V @ ce.double().cpu()
+            fit[1::2] = V @ co.double().cpu()
+            return (fr - fit).float().to(self.M_filters.device).contiguous()
+        return self._cached("fir%d" % R, (self.phi, self.M_filters), build)
+
+    def _ring_from_sequence(self, xp: torch.Tensor):
+        """Ring of the last R projected inputs (position p in slot p % R, zeros before the first position), or an
+        empty history slot when the exact head is off."""
+        fir = self.lds_fir()
+        B, T, d = xp.shape
+        if fir is None:
+            return xp.new_empty(B, 0, d)
+        R = fir.shape[0]
+        ring = xp.new_zeros(B, R, d)
+        idx = torch.arange(max(0, T - R), T, device=xp.device)
+        ring[:, idx % R] = xp[:, idx]
+        return ring
 
     def lds_single_params(self):
         """use_hankel_L (one branch over all lags): poles a (S) and per-channel weights ce, co (S,d) fitted to the
@@ -266,7 +302,7 @@ class STU(nn.Module):
                 if not use_cache:
                     return y
                 if self.decode_mode() == "lds":
-                    return y, (xp.new_empty(B, 0, self.d_out), state, torch.full((B,), T, dtype=torch.int64))
+                    return y, (self._ring_from_sequence(xp), state, torch.full((B,), T, dtype=torch.int64))
                 return y, self._state_from_sequence(xp)
             if self.use_approx:
                 xp = self._project(x)
@@ -292,7 +328,7 @@ class STU(nn.Module):
             a = (self.lds_single_params()[0] if self._single_lds_ok() else
                  self.lds_params()[0] if self.use_approx else self.bank_lds_params()[0])
             state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1)
-            return (src.new_empty(B, 0, d), state, pos)
+            return (self._ring_from_sequence(src) if self.use_approx else src.new_empty(B, 0, d), state, pos)
         cap = max(self.config.seq_len, T)
         hist = src.new_zeros(B, cap, d)
         hist[:, :T] = src
@@ -309,7 +345,11 @@ class STU(nn.Module):
                 y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co)
             else:
                 a, ce, co = self.lds_params()
-                y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co, pair=True)
+                fir = self.lds_fir()
+                if fir is not None and hist.shape[1] == fir.shape[0]:
+                    y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co, pair=True, ring=hist, fir=fir)
+                else:
+                    y = _hip.stu_step_lds(state, xp, a, ce, pos, co=co, pair=True)
             return y, (hist, state, pos_t + 1)
         if not self.use_approx and state.numel() > 0:
             # exact mode on the recurrence state: U+- for all K filters, then the two contractions as skinny GEMVs

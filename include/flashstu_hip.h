@@ -132,9 +132,17 @@ int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, co
  * t-1-2m), co (S,d) fitted to phi_proj's odd lags, and
  *   y[b,c] = T( T(E + O) + T(E - O) )
  * i.e. the plus and the minus branch rounded to the model dtype separately before their sum
- * (flash_stu/utils/stu_utils.py:226-228, flash_stu/modules/stu.py:120); fstu_stu_step_lds returns T(2E). */
+ * (flash_stu/utils/stu_utils.py:226-228, flash_stu/modules/stu.py:120); fstu_stu_step_lds returns T(2E).
+ *
+ * Optional exact head of the filter (ring, fir, fir_taps all given, or NULL / NULL / 0): the recurrence reproduces
+ * phi_proj (flash_stu/modules/stu.py:88) only up to its lag-by-lag rounding to the model dtype, which is largest on the
+ * first lags.  fir (fir_taps,d) fp32 holds phi_proj[s,c] minus the fitted filter for the first fir_taps lags (a power of
+ * two, 8..1024), ring (B,fir_taps,d) in the model dtype the last projected inputs (position p in slot p % fir_taps, zero
+ * before the first position): the even lags' correction joins E, the odd lags' O, and the step stores xp in slot
+ * t % fir_taps. */
 int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
-                           void* y, int ldy, int B, int S, int d, int t, int dtype, void* stream);
+                           void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t,
+                           int dtype, void* stream);
 
 /* The same step for the single-branch filters of use_hankel_L=True (flash_stu/utils/stu_utils.py:22-25,229-246:
  * one convolution over ALL lags, no sign branch): ce (S,d) is fitted to the even lags and weighs the bank of parity
@@ -153,18 +161,20 @@ int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, const float* a,
 
 /* Input projection and recurrence step in one launch (bf16, K % 256 == 0):
  *   xp[b,c] = T( h[b,:] . Mt[c,:] )  with Mt = M_inputs^T (d,K) row-major, then the step of
- * fstu_stu_step_lds_pair on xp (co != NULL) or of fstu_stu_step_lds (co == NULL).  xp_out (B,d) receives xp when not NULL.
+ * fstu_stu_step_lds_pair on xp (co != NULL; ring / fir / fir_taps as there) or of fstu_stu_step_lds (co == NULL).
+ * xp_out (B,d) receives xp when not NULL.
  * Replaces `x @ M_inputs` + the convolution at flash_stu/modules/stu.py:87-98,120 for one token. */
 int fstu_stu_inproj_step(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
-                         const float* co, void* y, int ldy, void* xp_out, int B, int S, int d, int K, int t, void* stream);
+                         const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, void* xp_out, int B,
+                         int S, int d, int K, int t, void* stream);
 
 /* The same launch with the residual update and the RMSNorm of its input as the prologue
  * (flash_stu/layers/stu_layer.py:78-82 after the previous layer's :93-97): x' = T(x_in + T(sum of nslices <= 4 fp32
  * (B,K) slices)) goes to x_out (not x_in itself), h = rmsnorm(x') * norm_w feeds the projection.  K % 256 == 0,
  * B*K/8 <= 1024. */
 int fstu_stu_res_inproj_step(const void* x_in, const float* slices, int nslices, void* x_out, const void* norm_w, float eps,
-                             const void* Mt, float* state, const float* a, const float* ce, const float* co, void* y, int ldy,
-                             int B, int S, int d, int K, int t, void* stream);
+                             const void* Mt, float* state, const float* a, const float* ce, const float* co, void* ring,
+                             const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int K, int t, void* stream);
 
 /* The step of fstu_stu_step_lds applied to T consecutive positions t_start .. t_start+T-1 in one launch (scan form
  * of the prefill: no FFT, no history buffer): y[b,t,c] for every position and the state after the last one.
@@ -412,6 +422,8 @@ typedef struct {
   const float* lds_ce;      /* (S,d) even-lag output weights      (lds mode) */
   const float* lds_co;      /* (S,d) odd-lag output weights on the other bank, or NULL: y = T(2E) (lds mode) */
   float* lds_state;         /* (B,2,S,d)                          (lds mode) */
+  void* lds_ring;           /* (B,lds_fir_taps,d) last projected inputs, model dtype, or NULL (lds mode, with lds_co) */
+  const float* lds_fir;     /* (lds_fir_taps,d) phi_proj minus the fitted filter on the first lags, or NULL */
   /* attention */
   const void* w_qkv;        /* (3d,d) */
   const void* w_proj;       /* (d,d) */
@@ -434,6 +446,7 @@ typedef struct {
   int L, hist_cap;
   int stu_mode;             /* 0: history, 1: lds */
   int lds_S;
+  int lds_fir_taps;         /* taps of the layers' lds_fir (a power of two, 8..1024), 0: none */
   int single_branch;        /* use_hankel_L */
   int ksplit_down;          /* K split of the down projection (partial holds ksplit_down*B*d floats) */
   int hist_nsplit_max;      /* eo holds hist_nsplit_max*2*B*d floats */

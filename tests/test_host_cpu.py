@@ -180,6 +180,40 @@ def test_lds_fit_reproduces_hankel_filters_and_rejects_what_it_cannot_fit(L, K):
         check_lds_fit(err, noise)
 
 
+def test_lds_exact_head_closes_the_fit_on_the_first_lags():
+    """STU.lds_fir(): the taps added to the fitted recurrence make the first R lags of the decode filter equal to
+    phi_proj itself (to fp32), for R below and above the filter length; off for Hankel-L, history mode and R = 0."""
+    from flash_stu import FlashSTUConfig
+    from flash_stu.modules.stu import STU
+    for L, R in ((256, 32), (64, 128)):
+        cfg = FlashSTUConfig(n_embd=16, n_heads=2, n_layers=2, seq_len=L, num_eigh=8, vocab_size=11,
+                             torch_dtype=torch.bfloat16, stu_decode_mode="lds", stu_lds_fir_taps=R)
+        phi = torch.tensor(O.get_spectral_filters_f64(L, 8)).to(torch.bfloat16)
+        torch.manual_seed(L)
+        stu = STU(cfg, phi, L)
+        with torch.no_grad():
+            stu.M_filters.copy_(torch.randn_like(stu.M_filters) / 8 ** 0.5)
+        fir = stu.lds_fir()
+        a, ce, co = stu.lds_params()
+        assert fir.shape == (R, 16) and fir.dtype == torch.float32
+        f = stu.effective_filter().detach().double()
+        want = torch.zeros(R, 16, dtype=torch.float64)
+        want[: min(R, L)] = f[: min(R, L)]
+        m = torch.arange(R // 2, dtype=torch.float64)
+        V = a.double()[None, :] ** m[:, None]
+        got = fir.double()
+        got[0::2] += V @ ce.double()
+        got[1::2] += V @ co.double()
+        assert float((got - want).abs().max()) <= 1e-6 * float(f.abs().max())
+        for off in (dict(stu_lds_fir_taps=0), dict(use_hankel_L=True), dict(stu_decode_mode="history")):
+            kw = dict(n_embd=16, n_heads=2, n_layers=2, seq_len=L, num_eigh=8, vocab_size=11, torch_dtype=torch.bfloat16,
+                      stu_decode_mode="lds", stu_lds_fir_taps=R)
+            kw.update(off)
+            assert STU(FlashSTUConfig(**kw), phi, L).lds_fir() is None
+    with pytest.raises(ValueError):
+        FlashSTUConfig(n_embd=16, n_heads=2, n_layers=2, seq_len=64, num_eigh=8, vocab_size=11, stu_lds_fir_taps=48)
+
+
 def test_generate_beyond_seq_len_leaves_the_stateful_paths():
     """prompt + new tokens > seq_len: the decode engine refuses (its state has no counterpart in the reference's
     truncated re-run, model.py:250-255) and FlashSTU.generate takes the recompute loop instead of the engine."""
