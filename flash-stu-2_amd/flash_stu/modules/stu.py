@@ -153,9 +153,10 @@ class STU(nn.Module):
         if fir is None:
             return xp.new_empty(B, 0, d)
         R = fir.shape[0]
+        if T >= R:      # positions T-R .. T-1 to slots p % R: a rotation of the last R rows
+            return torch.roll(xp[:, T - R:], shifts=(T - R) % R, dims=1).contiguous()
         ring = xp.new_zeros(B, R, d)
-        idx = torch.arange(max(0, T - R), T, device=xp.device)
-        ring[:, idx % R] = xp[:, idx]
+        ring[:, :T] = xp
         return ring
 
     def lds_single_params(self):
