@@ -49,12 +49,15 @@ struct NormPrologue {
     return d % 256 == 0 && rows >= 1 && (long long)rows * (d / 8) <= (long long)NXC * NT;
   }
 
-  // phase 1: every load of the prologue, in straight-line code
+  // phase 1: every load of the prologue, in straight-line code.  x_in and delta point at the first of the `rows` rows;
+  // when these are a few rows of taller slices, slice_chunks is the distance between two slices in 8-channel chunks.
   __device__ __forceinline__ void issue(const bf16_t* x_in, const void* delta, int nslices, const bf16_t* norm_w, int rows,
-                                        int d) {
+                                        int d, int slice_chunks = 0) {
     const int nchunk = d >> 3, total = rows * nchunk;
+    const int sstride = slice_chunks > 0 ? slice_chunks : total;
     const fstu_rsrc_t rx = fstu_make_rsrc(x_in, (size_t)total * 16);
-    const fstu_rsrc_t rd = fstu_make_rsrc(delta, NS > 0 ? (size_t)nslices * total * 32 : (size_t)total * 16);
+    const fstu_rsrc_t rd = fstu_make_rsrc(
+        delta, NS > 0 ? (nslices > 0 ? ((size_t)(nslices - 1) * sstride + total) * 32 : 0) : (size_t)total * 16);
     const fstu_rsrc_t rn = fstu_make_rsrc(norm_w, (size_t)d * 2);
     const float inv_nc = 1.0f / (float)nchunk;
 #pragma unroll
@@ -66,7 +69,7 @@ struct NormPrologue {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
           // slices beyond nslices lie beyond the descriptor's range: zeros
-          const unsigned off = q < total ? ((unsigned)s * (unsigned)total + (unsigned)q) * 32u : FSTU_BUF_OOB;
+          const unsigned off = q < total ? ((unsigned)s * (unsigned)sstride + (unsigned)q) * 32u : FSTU_BUF_OOB;
           sv[(j * NS + s) * 2] = fstu_buf_load16(rd, off);
           sv[(j * NS + s) * 2 + 1] = fstu_buf_load16(rd, q < total ? off + 16u : FSTU_BUF_OOB);
         }

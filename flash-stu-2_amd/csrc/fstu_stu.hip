@@ -366,12 +366,17 @@ extern "C" int fstu_stu_bank_step_lds(float* state, const void* x, int ldx, cons
 }
 
 // ---------------------------------------------------------------- input projection + LDS-form step, one launch
-// Workgroup = one tile of 16 channels: x_proj[b, c] = T(h[b,:] . Mt[c,:]) by MFMA (K split over the 4 waves, reduced
-// in LDS), then the recurrence step of those 16 channels for every batch row.  Thread (b, jsub, cq) owns 4 channels
-// (float4) of modes jsub, jsub+8, ...; the 8 mode groups are reduced with wave shuffles.
+// Workgroup = one tile of 16 channels x INPROJ_RB batch rows: x_proj[b, c] = T(h[b,:] . Mt[c,:]) by MFMA (K split over
+// the 4 waves, reduced in LDS), then the recurrence step of those channels and rows.  The three operand streams of the
+// step are dealt to different waves so that every load of the kernel is in flight before the projection and the whole
+// kernel costs one trip to memory: wave 0 advances the bank of the token's parity (even lags), wave 1 reads the other
+// bank (odd lags), waves 2 and 3 the exact head (ring of the last inputs).  Lane (cq, jsub, bsub) of a wave owns 4
+// channels (float4) of row bsub and modes (or lags) jsub, jsub+8, ... (the head: jsub + 8*(wave-2), +16, ...).
 typedef __bf16 stu_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float stu_floatx4_t __attribute__((ext_vector_type(4)));
+#define INPROJ_RB 2
 
+template <int PK /* chunks of 8 channels per thread in the norm prologue: rows * K / 8 <= PK * 256 */>
 __global__ void __launch_bounds__(256)
 stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ Mt /*(d,K) = M_inputs^T*/,
                        float* __restrict__ state, const float* __restrict__ a, const float* __restrict__ ce,
@@ -387,8 +392,9 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
                        bf16_t* __restrict__ ring /*optional (B,R,d), with fir (R,d) and co: exact head of the filter*/,
                        const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn) {
   __shared__ float red[4][64][4];
-  __shared__ float xps[16][16];   // [batch][channel in tile], bf16-rounded values
-  extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (B x (K+8)) bf16
+  __shared__ float xps[INPROJ_RB][16];          // [row][channel in tile], bf16-rounded values
+  __shared__ float part[2][3][INPROJ_RB][16];   // [E | O][wave 0 or 1, wave 2, wave 3][row][channel]
+  extern __shared__ __align__(16) unsigned char inproj_smem[];   // with x_res: h rows (INPROJ_RB x (K+8)) bf16
   if (dyn) parity = dyn[0] & 1;
   if (pos_dyn) t = pos_dyn[0];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -399,36 +405,49 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   int tile = blockIdx.x;
   if ((gridDim.x & 15) == 0) tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const int c0 = tile * 16;
-  // residual update + norm in the prologue
-  typedef NormPrologue<256, 4, 4> Pro;
-  typedef NormPrologue<256, 3, 4> Pro3;   // exact for rows * K / 8 <= 768: one straight line without idle chunks
+  const int b0 = blockIdx.y * INPROJ_RB, rows = min(INPROJ_RB, B - b0);
+  // residual update + norm of this workgroup's rows in the prologue
+  typedef NormPrologue<256, PK, 4> Pro;
   Pro pro;
-  Pro3 pro3;
   const bool merged = x_res != nullptr && slices != nullptr;
-  const bool exact3 = B * (K >> 3) <= 768;
   // ---- projection: A operand = Mt rows (channels), B operand = h rows (batch)
   const int kw = K >> 2;                                    // k range of this wave
   const bf16_t* wp = Mt + (size_t)min(c0 + r, d - 1) * K + w * kw + g * 16;
-  const bool xrow = r < B;
-  const bf16_t* hp = h + (size_t)(xrow ? r : 0) * ldh + w * kw + g * 16;   // re-pointed at LDS by the norm prologue
-  // ---- the recurrence operands of this thread's first batch row go in flight before the projection: they do
-  // not depend on it, and fetched afterwards they would cost a second dependent trip to memory
+  const bool xrow = r < rows;
+  const bf16_t* hp = h + (size_t)(b0 + (xrow ? r : 0)) * ldh + w * kw + g * 16;   // re-pointed at LDS by the norm prologue
+  // ---- the operands of this wave's part of the step go in flight before the projection: they do not depend on it,
+  // and fetched afterwards they would cost a second dependent trip to memory
   constexpr int PJ = 8;
-  const int cq = threadIdx.x & 3, jsub = (threadIdx.x >> 2) & 7, bsub = threadIdx.x >> 5;
+  const int cq = lane & 3, jsub = (lane >> 2) & 7, bsub = lane >> 5;
   const int c = c0 + cq * 4;
-  float4 phv[PJ], pcj[PJ];
+  const bool live = bsub < rows && c < d;
+  const int b = b0 + (live ? bsub : 0), cc = live ? c : 0;
+  const bool head = w >= 2;
+  const int gl = jsub + 8 * (w - 2);   // head: first lag of this lane; the lags of a lane share its parity
+  float4 pa[PJ], pb[PJ];
   float paj[PJ];
-  const bool pre = bsub < B && c < d;
-  {
-    float* st = state + (((size_t)(pre ? bsub : 0) * 2 + parity) * S) * d + (pre ? c : 0);
+  // branch-free inside a role (out-of-range lanes, modes and lags re-read a valid element and ignore it): a conditional
+  // load would reach its use through a copy, and the copy's wait would hold back every load issued after it
+  if (!head) {
+    const float* st = state + (((size_t)b * 2 + (parity ^ w)) * S) * d + cc;
+    const float* cw = ((w == 0 || !co) ? ce : co) + cc;
 #pragma unroll
     for (int k = 0; k < PJ; ++k) {
-      // branch-free (out-of-range lanes and modes re-read a valid element and ignore it): a conditional load would
-      // reach its use through a copy, and the copy's wait would hold back every load issued after it
       const int j = min(jsub + 8 * k, S - 1);
-      phv[k] = *(const float4*)(st + (size_t)j * d);
-      pcj[k] = *(const float4*)(ce + (size_t)j * d + (pre ? c : 0));
+      pa[k] = *(const float4*)(st + (size_t)j * d);
+      pb[k] = *(const float4*)(cw + (size_t)j * d);
       paj[k] = a[j];
+    }
+  } else if (fir) {
+    const bf16_t* rb = ring + (size_t)b * R * d + cc;
+#pragma unroll
+    for (int k = 0; k < PJ; ++k) {
+      const int s = min(gl + 16 * k, R - 1);
+      const uint2 q = *(const uint2*)(rb + (size_t)((t - s) & (R - 1)) * d);
+      pa[k] = make_float4(__uint_as_float(q.x << 16), __uint_as_float(q.x & 0xffff0000u), __uint_as_float(q.y << 16),
+                          __uint_as_float(q.y & 0xffff0000u));
+      pb[k] = *(const float4*)(fir + (size_t)s * d + cc);
+      paj[k] = 0.f;
     }
   }
   stu_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -447,27 +466,28 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
   // loads issued after that point would cost a second trip to memory.  The loads above return first anyway.
   __builtin_amdgcn_sched_barrier(0);
   if (merged) {
-    if (exact3) pro3.issue(x_res, slices, nslices, norm_w, B, K); else pro.issue(x_res, slices, nslices, norm_w, B, K);
-  }
-  if (merged) {
+    const bf16_t* xr = x_res + (size_t)b0 * K;
+    const float* sl = slices + (size_t)b0 * K;
+    const int whole = B * (K >> 3);   // chunks of a whole slice
+    pro.issue(xr, sl, nslices, norm_w, rows, K, whole);
     bf16_t* hs = (bf16_t*)inproj_smem;
     __shared__ float ss_part[Pro::NPART];
-    if (exact3) pro3.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
-    else pro.reduce(ss_part, blockIdx.x == 0 ? x_out : nullptr, B, K);
+    pro.reduce(ss_part, blockIdx.x == 0 ? x_out + (size_t)b0 * K : nullptr, rows, K);
     __syncthreads();
-    if (exact3) pro3.scale(ss_part, hs, ldn, B, K, eps); else pro.scale(ss_part, hs, ldn, B, K, eps);
+    pro.scale(ss_part, hs, ldn, rows, K, eps);
     __syncthreads();
     hp = hs + (size_t)(xrow ? r : 0) * ldn + w * kw + g * 16;
   } else if (x_res) {
-    // h = rmsnorm(x_res) * norm_w for all rows into LDS (every workgroup recomputes it: B*K*2 bytes of input)
+    // h = rmsnorm(x_res) * norm_w for this workgroup's rows into LDS
     bf16_t* hs = (bf16_t*)inproj_smem;
+    const bf16_t* xr = x_res + (size_t)b0 * K;
     const int nchunk = K >> 3;
-    for (int q = threadIdx.x; q < B * nchunk; q += 256) {
+    for (int q = threadIdx.x; q < rows * nchunk; q += 256) {
       const int row = q / nchunk, c8 = (q - row * nchunk) << 3;
-      *(uint4*)(hs + (size_t)row * ldn + c8) = *(const uint4*)(x_res + (size_t)q * 8);
+      *(uint4*)(hs + (size_t)row * ldn + c8) = *(const uint4*)(xr + (size_t)q * 8);
     }
     __syncthreads();
-    for (int row = w; row < B; row += 4) {
+    for (int row = w; row < rows; row += 4) {
       bf16_t* hr = hs + (size_t)row * ldn;
       float ss = 0.f;
       for (int c8 = lane * 8; c8 < K; c8 += 512) {
@@ -528,44 +548,42 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[w][lane][i] = acc[i];
   __syncthreads();
-  if (w == 0) {
+  if (w == 0 && xrow) {
     // D layout: lane holds channels 4*g+i of batch row r
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float v = DT<bf16_t>::rnd(((red[0][lane][i] + red[1][lane][i]) + red[2][lane][i]) + red[3][lane][i]);
       xps[r][4 * g + i] = v;
-      if (xp_out && xrow && c0 + 4 * g + i < d) xp_out[(size_t)r * d + c0 + 4 * g + i] = f32_to_bf16(v);
+      if (xp_out && c0 + 4 * g + i < d) xp_out[(size_t)(b0 + r) * d + c0 + 4 * g + i] = f32_to_bf16(v);
     }
   }
   __syncthreads();
-  // ---- recurrence step of the tile's channels
-  for (int b = bsub; b < B; b += 8) {
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (c < d) {
-      const float x0 = xps[b][cq * 4], x1 = xps[b][cq * 4 + 1], x2 = xps[b][cq * 4 + 2], x3 = xps[b][cq * 4 + 3];
-      float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
-      int jstart = jsub;
-      if (b == bsub) {
+  // ---- this wave's part of the step
+  const int bl = live ? bsub : 0;
+  const float x0 = xps[bl][cq * 4], x1 = xps[bl][cq * 4 + 1], x2 = xps[bl][cq * 4 + 2], x3 = xps[bl][cq * 4 + 3];
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (w == 0) {
+    // even lags: advance the bank of the token's parity
+    float* st = state + (((size_t)b * 2 + parity) * S) * d + cc;
 #pragma unroll
-        for (int k = 0; k < PJ; ++k) {
-          const int j = jsub + 8 * k;
-          if (j < S) {
-            float4 hv = phv[k];
-            hv.x = fmaf(paj[k], hv.x, x0);
-            hv.y = fmaf(paj[k], hv.y, x1);
-            hv.z = fmaf(paj[k], hv.z, x2);
-            hv.w = fmaf(paj[k], hv.w, x3);
-            *(float4*)(st + (size_t)j * d) = hv;
-            sum.x = fmaf(pcj[k].x, hv.x, sum.x);
-            sum.y = fmaf(pcj[k].y, hv.y, sum.y);
-            sum.z = fmaf(pcj[k].z, hv.z, sum.z);
-            sum.w = fmaf(pcj[k].w, hv.w, sum.w);
-          }
-        }
-        jstart = jsub + 8 * PJ;
+    for (int k = 0; k < PJ; ++k) {
+      const int j = jsub + 8 * k;
+      if (j < S && live) {
+        float4 hv = pa[k];
+        hv.x = fmaf(paj[k], hv.x, x0);
+        hv.y = fmaf(paj[k], hv.y, x1);
+        hv.z = fmaf(paj[k], hv.z, x2);
+        hv.w = fmaf(paj[k], hv.w, x3);
+        *(float4*)(st + (size_t)j * d) = hv;
+        sum.x = fmaf(pb[k].x, hv.x, sum.x);
+        sum.y = fmaf(pb[k].y, hv.y, sum.y);
+        sum.z = fmaf(pb[k].z, hv.z, sum.z);
+        sum.w = fmaf(pb[k].w, hv.w, sum.w);
       }
+    }
+    if (live) {
 #pragma unroll 8
-      for (int j = jstart; j < S; j += 8) {
+      for (int j = jsub + 8 * PJ; j < S; j += 8) {
         float4 hv = *(float4*)(st + (size_t)j * d);
         const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
         const float aj = a[j];
@@ -580,60 +598,95 @@ stu_inproj_step_kernel(const bf16_t* __restrict__ h, const bf16_t* __restrict__ 
         sum.w = fmaf(cj.w, hv.w, sum.w);
       }
     }
+  } else if (w == 1) {
     // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (read only)
-    float4 sumo = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (co && c < d) {
+    if (co && live) {
+#pragma unroll
+      for (int k = 0; k < PJ; ++k) {
+        if (jsub + 8 * k < S) {
+          sum.x = fmaf(pb[k].x, pa[k].x, sum.x);
+          sum.y = fmaf(pb[k].y, pa[k].y, sum.y);
+          sum.z = fmaf(pb[k].z, pa[k].z, sum.z);
+          sum.w = fmaf(pb[k].w, pa[k].w, sum.w);
+        }
+      }
       const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
 #pragma unroll 8
-      for (int j = jsub; j < S; j += 8) {
+      for (int j = jsub + 8 * PJ; j < S; j += 8) {
         const float4 hv = *(const float4*)(so + (size_t)j * d);
         const float4 oj = *(const float4*)(co + (size_t)j * d + c);
-        sumo.x = fmaf(oj.x, hv.x, sumo.x);
-        sumo.y = fmaf(oj.y, hv.y, sumo.y);
-        sumo.z = fmaf(oj.z, hv.z, sumo.z);
-        sumo.w = fmaf(oj.w, hv.w, sumo.w);
-      }
-      if (fir) {
-        const float xv[4] = {xps[b][cq * 4], xps[b][cq * 4 + 1], xps[b][cq * 4 + 2], xps[b][cq * 4 + 3]};
-        float f[4] = {0.f, 0.f, 0.f, 0.f};
-        fir_head<bf16_t>(ring, fir, R, t, b, c, d, jsub, xv, f);
-        if (jsub & 1) { sumo.x += f[0]; sumo.y += f[1]; sumo.z += f[2]; sumo.w += f[3]; }
-        else { sum.x += f[0]; sum.y += f[1]; sum.z += f[2]; sum.w += f[3]; }
-        if (jsub == 0) Ring4<bf16_t>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, xv);
+        sum.x = fmaf(oj.x, hv.x, sum.x);
+        sum.y = fmaf(oj.y, hv.y, sum.y);
+        sum.z = fmaf(oj.z, hv.z, sum.z);
+        sum.w = fmaf(oj.w, hv.w, sum.w);
       }
     }
-    // reduce over the 8 mode groups (lanes differing in bits 2..4): two rotations inside the row of 16 lanes, one
-    // swizzle across the two rows
-    auto grp_sum = [](float v) {
-      v += fstu_dpp<0x124>(v);   // row_ror:4
-      v += fstu_dpp<0x128>(v);   // row_ror:8
-      return v + fstu_swz16(v);
-    };
-    sum.x = grp_sum(sum.x);
-    sum.y = grp_sum(sum.y);
-    sum.z = grp_sum(sum.z);
-    sum.w = grp_sum(sum.w);
-    float4 out = make_float4(2.f * sum.x, 2.f * sum.y, 2.f * sum.z, 2.f * sum.w);
-    if (co) {
-      sumo.x = grp_sum(sumo.x);
-      sumo.y = grp_sum(sumo.y);
-      sumo.z = grp_sum(sumo.z);
-      sumo.w = grp_sum(sumo.w);
-      out.x = DT<bf16_t>::rnd(sum.x + sumo.x) + DT<bf16_t>::rnd(sum.x - sumo.x);
-      out.y = DT<bf16_t>::rnd(sum.y + sumo.y) + DT<bf16_t>::rnd(sum.y - sumo.y);
-      out.z = DT<bf16_t>::rnd(sum.z + sumo.z) + DT<bf16_t>::rnd(sum.z - sumo.z);
-      out.w = DT<bf16_t>::rnd(sum.w + sumo.w) + DT<bf16_t>::rnd(sum.w - sumo.w);
-    }
-    if (jsub == 0 && c < d) {
-      bf16_t* yp = y + (size_t)b * ldy + c;
-      if ((ldy & 3) == 0) {
-        *(uint2*)yp = make_uint2(pack2_bf16(out.x, out.y), pack2_bf16(out.z, out.w));
-      } else {
-        yp[0] = f32_to_bf16(out.x);
-        yp[1] = f32_to_bf16(out.y);
-        yp[2] = f32_to_bf16(out.z);
-        yp[3] = f32_to_bf16(out.w);
+  } else if (fir && live) {
+    // exact head: lags gl, gl+16, ... of the ring; a position before the sequence contributes nothing
+#pragma unroll
+    for (int k = 0; k < PJ; ++k) {
+      const int s = gl + 16 * k;
+      if (s < R) {
+        const float m = (t - s >= 0) ? 1.f : 0.f;
+        sum.x = fmaf(pb[k].x, s == 0 ? x0 : m * pa[k].x, sum.x);
+        sum.y = fmaf(pb[k].y, s == 0 ? x1 : m * pa[k].y, sum.y);
+        sum.z = fmaf(pb[k].z, s == 0 ? x2 : m * pa[k].z, sum.z);
+        sum.w = fmaf(pb[k].w, s == 0 ? x3 : m * pa[k].w, sum.w);
       }
+    }
+    const bf16_t* rb = ring + (size_t)b * R * d + c;
+#pragma unroll 4
+    for (int s = gl + 16 * PJ; s < R; s += 16) {
+      float xv[4];
+      Ring4<bf16_t>::ld(rb + (size_t)((t - s) & (R - 1)) * d, xv);
+      const float m = (t - s >= 0) ? 1.f : 0.f;
+      const float4 rv = *(const float4*)(fir + (size_t)s * d + c);
+      sum.x = fmaf(rv.x, m * xv[0], sum.x);
+      sum.y = fmaf(rv.y, m * xv[1], sum.y);
+      sum.z = fmaf(rv.z, m * xv[2], sum.z);
+      sum.w = fmaf(rv.w, m * xv[3], sum.w);
+    }
+    if (gl == 0) {
+      const float xv[4] = {x0, x1, x2, x3};
+      Ring4<bf16_t>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, xv);
+    }
+  }
+  // reduce over the 8 mode groups of a wave (lanes differing in bits 2..4): two rotations inside the row of 16 lanes, one
+  // swizzle across the two rows.  The head keeps even and odd lags apart (the rotation by 4 lanes joins them): its
+  // lanes with jsub 0 end with the even lags' sum, those with jsub 1 with the odd lags'.
+  auto grp_sum = [head](float v) {
+    const float u = v + fstu_dpp<0x124>(v);   // row_ror:4
+    v = head ? v : u;
+    v += fstu_dpp<0x128>(v);   // row_ror:8
+    return v + fstu_swz16(v);
+  };
+  sum.x = grp_sum(sum.x);
+  sum.y = grp_sum(sum.y);
+  sum.z = grp_sum(sum.z);
+  sum.w = grp_sum(sum.w);
+  if (bsub < INPROJ_RB && jsub < (head ? 2 : 1)) {
+    const int eo = head ? jsub : w;          // 0: joins E, 1: joins O
+    const int src = head ? w - 1 : 0;
+    float* pp = &part[eo][src][bsub][cq * 4];
+    pp[0] = sum.x; pp[1] = sum.y; pp[2] = sum.z; pp[3] = sum.w;
+  }
+  __syncthreads();
+  if (w == 0 && jsub == 0 && live) {
+    float o4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float e = (part[0][0][bsub][cq * 4 + i] + part[0][1][bsub][cq * 4 + i]) + part[0][2][bsub][cq * 4 + i];
+      const float o = (part[1][0][bsub][cq * 4 + i] + part[1][1][bsub][cq * 4 + i]) + part[1][2][bsub][cq * 4 + i];
+      o4[i] = co ? DT<bf16_t>::rnd(e + o) + DT<bf16_t>::rnd(e - o) : 2.f * e;
+    }
+    bf16_t* yp = y + (size_t)b * ldy + c;
+    if ((ldy & 3) == 0) {
+      *(uint2*)yp = make_uint2(pack2_bf16(o4[0], o4[1]), pack2_bf16(o4[2], o4[3]));
+    } else {
+      yp[0] = f32_to_bf16(o4[0]);
+      yp[1] = f32_to_bf16(o4[1]);
+      yp[2] = f32_to_bf16(o4[2]);
+      yp[3] = f32_to_bf16(o4[3]);
     }
   }
 }
@@ -664,7 +717,7 @@ int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nsli
   FSTU_REQUIRE(x_in && slices && x_out && norm_w, FSTU_ENULL, "fstu_stu_res_inproj_step: null pointer");
   FSTU_REQUIRE(nslices >= 1 && nslices <= 4, FSTU_EARG, "fstu_stu_res_inproj_step: nslices=%d outside 1..4", nslices);
   FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_stu_res_inproj_step: x_out must not alias x_in");
-  FSTU_REQUIRE((NormPrologue<256, 4, 4>::supported(B, K)), FSTU_ESHAPE, "fstu_stu_res_inproj_step: B=%d K=%d not supported", B, K);
+  FSTU_REQUIRE((NormPrologue<256, 4, 4>::supported(INPROJ_RB, K)), FSTU_ESHAPE, "fstu_stu_res_inproj_step: K=%d not supported", K);
   FSTU_REQUIRE(fstu_aligned(slices, 16) && fstu_aligned(x_out, 16), FSTU_EALIGN, "fstu_stu_res_inproj_step: pointers must be 16-byte aligned");
   return inproj_step_launch(x_in, K, x_in, norm_w, eps, Mt, state, a, ce, co, y, ldy, nullptr, B, S, d, K, t, dyn, stream,
                             FirArgs{ring, fir, fir_taps, dyn ? dyn : pos_dyn}, slices, nslices, x_out);
@@ -680,13 +733,20 @@ static int inproj_step_launch(const void* h, int ldh, const void* x_res, const v
   FSTU_REQUIRE(B >= 1 && B <= FSTU_MAX_DECODE_ROWS && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_inproj_step: B=%d S=%d d=%d", B, S, d);
   FSTU_REQUIRE(K % 256 == 0 && ldh >= K && ldh % 8 == 0 && ldy >= d, FSTU_ESHAPE, "fstu_stu_inproj_step: K=%d must be a multiple of 256 (ldh=%d)", K, ldh);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(Mt, 16) && fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_inproj_step: pointers must be 16-byte aligned");
-  const size_t shm = x_res ? (size_t)B * (K + 8) * 2 : 0;
+  const size_t shm = x_res ? (size_t)INPROJ_RB * (K + 8) * 2 : 0;
   FSTU_REQUIRE(shm <= 56 * 1024, FSTU_ESHAPE, "fstu_stu_inproj_step: B*K too large for the norm prologue");
   FSTU_REQUIRE(fstu_aligned(x_res, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_inproj_step: x_res/norm_w/co must be 16-byte aligned");
-  hipLaunchKernelGGL(stu_inproj_step_kernel, dim3((d + 15) / 16), dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,
-                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,
-                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out, co, (bf16_t*)fa.ring,
-                     fa.fir, fa.taps, t, fa.pos_dyn);
+  const dim3 grid((d + 15) / 16, (B + INPROJ_RB - 1) / INPROJ_RB);
+#define INPROJ_LAUNCH(PK)                                                                                                  \
+  hipLaunchKernelGGL(stu_inproj_step_kernel<PK>, grid, dim3(256), shm, (hipStream_t)stream, (const bf16_t*)h,             \
+                     (const bf16_t*)Mt, state, a, ce, (bf16_t*)y, dyn, t & 1, ldh, ldy, (bf16_t*)xp_out, B, S, d, K,       \
+                     (const bf16_t*)x_res, (const bf16_t*)norm_w, eps, slices, nslices, (bf16_t*)x_out, co,                \
+                     (bf16_t*)fa.ring, fa.fir, fa.taps, t, fa.pos_dyn)
+  const int chunks = INPROJ_RB * (K >> 3);
+  if (chunks <= 256) INPROJ_LAUNCH(1);
+  else if (chunks <= 512) INPROJ_LAUNCH(2);
+  else INPROJ_LAUNCH(4);
+#undef INPROJ_LAUNCH
   FSTU_CHECK_LAUNCH("fstu_stu_inproj_step");
   return FSTU_OK;
 }
