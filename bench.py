@@ -222,6 +222,10 @@ def run_lm(args, torch, _hip, which):
         label = ("BASELINE config 2: FlashSTU 768-d/12-layer/12-head, window 512, K=24, seq_len 2048, vocab 50257, random-init "
                  "bf16 seed 1, batch 8, 512-token prompt, greedy decode")
         metric = METRIC_C2
+        if args.top_k:
+            # not the headline workload: the same model with config 5's sampling, to price the sampler against greedy
+            sampling = dict(temperature=0.8, top_k=args.top_k, top_p=None, do_sample=True, seed=2)
+            label = label.replace("greedy decode", f"top-k {args.top_k} / temperature 0.8 sampling with the seeded stream")
     stu_mode = args.stu_mode if dt == torch.bfloat16 else "history"
     K, W = args.steps, args.warmup
 
@@ -455,6 +459,8 @@ def main():
                     help="prompt pass of the STU layers: the reference's FFT convolution, or the distilled recurrence as a scan")
     ap.add_argument("--batch", type=int, default=0, help="batch rows (default: the workload's own)")
     ap.add_argument("--prompt", type=int, default=0, help="prompt length (default: the workload's own)")
+    ap.add_argument("--top-k", type=int, default=0, dest="top_k",
+                    help="config 2 only: sample with this top-k at temperature 0.8 instead of the greedy pick")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mlp4", action="store_true", dest="no_mlp4", help="skip the second measurement of config 2 at mlp_scale 4")
     ap.add_argument("--graph-steps", type=int, default=8, dest="graph_steps", help="decode steps captured per HIP graph")

@@ -50,6 +50,10 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
+bool fstu_sample_topk_ok(int B, int V, int top_k, int dtype);
+int fstu_sample_topk_dyn(const void* logits, int64_t ldl, void* best_ws, void* samp_ws, int64_t* out, int64_t out_stride, int B,
+                         int V, float temperature, int top_k, float top_p, uint64_t seed, int step, int row0, int* dyn,
+                         int advance, void* stream);
 int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
                                const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
                                const int* pos_dyn, int dtype, void* stream);

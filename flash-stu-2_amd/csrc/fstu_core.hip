@@ -553,7 +553,6 @@ extern "C" int fstu_bias_act(void* y, const void* bias, int64_t rows, int n, int
 // ---------------------------------------------------------------- sampling
 // One workgroup of 1024 threads per row; the row (V logits) is re-read from
 // L2 in each pass instead of being staged.
-#define FSTU_SAMPLE_THREADS 1024
 
 struct SampleShared {
   float redf[16];
@@ -585,8 +584,9 @@ __device__ __forceinline__ float sample_transform(const T* row, int i, float inv
   return DT<T>::rnd(x);
 }
 
+template <int NT>
 __device__ __forceinline__ double block_excl_scan_d(double v, double* red, double* total) {
-  // exclusive scan over 1024 threads (16 waves), fixed order
+  // exclusive scan over NT threads (NT/64 <= 16 waves), fixed order
   int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   double inc = v;
 #pragma unroll
@@ -597,7 +597,7 @@ __device__ __forceinline__ double block_excl_scan_d(double v, double* red, doubl
   if (lane == 63) red[w] = inc;
   __syncthreads();
   double base = 0.0, tot = 0.0;
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NT / 64; ++i) {
     if (i < w) base += red[i];
     tot += red[i];
   }
@@ -647,17 +647,13 @@ __device__ __forceinline__ int select_bin_wave0(const C* h, C base, C need, C* a
 // CACHE (16-bit dtypes, rows of up to 64 K logits): the first pass leaves the transformed logits (temperature, clamp,
 // rounding: themselves 16-bit values) in LDS and every later pass reads them there instead of repeating the
 // division per element from L2.
-template <typename T, bool CACHE>
-__global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
-sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
-              int top_k, float top_p, int do_sample, uint64_t seed, int step, int row0, const int* __restrict__ dyn) {
-  __shared__ SampleShared sh;
-  const int b = blockIdx.x;
-  if (dyn) { out += dyn[0]; step = dyn[1]; }
-  const T* row = logits + (size_t)b * V;
+// One row by the NT threads of a workgroup; the picked token goes to *out_slot.
+template <typename T, bool CACHE, int NT>
+__device__ __forceinline__ void sample_row(SampleShared& sh, unsigned short* tl /*CACHE: V 16-bit words of LDS*/,
+                                           const T* __restrict__ row, int64_t* __restrict__ out_slot, int V, float temperature,
+                                           int top_k, float top_p, int do_sample, uint64_t seed, int step, int rowid) {
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const bool t1 = (temperature == 1.0f);
-  extern __shared__ unsigned short tl[];   // CACHE: transformed logits of the row
   auto tv = [&](int i) -> float {
     return CACHE ? __uint_as_float((unsigned)tl[i] << 16) : sample_transform(row, i, t1, temperature);
   };
@@ -668,18 +664,18 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   {
     // 8 strided loads in flight per thread; indices grow with k, so '>' keeps the lowest index on ties
     int i = tid;
-    for (; i + 7 * FSTU_SAMPLE_THREADS < V; i += 8 * FSTU_SAMPLE_THREADS) {
+    for (; i + 7 * NT < V; i += 8 * NT) {
       float l[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        l[k] = sample_transform(row, i + k * FSTU_SAMPLE_THREADS, t1, temperature);
-        if (CACHE) tl[i + k * FSTU_SAMPLE_THREADS] = (unsigned short)(__float_as_uint(l[k]) >> 16);
+        l[k] = sample_transform(row, i + k * NT, t1, temperature);
+        if (CACHE) tl[i + k * NT] = (unsigned short)(__float_as_uint(l[k]) >> 16);
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        if (besti == 0x7fffffff || l[k] > best) { best = l[k]; besti = i + k * FSTU_SAMPLE_THREADS; }
+        if (besti == 0x7fffffff || l[k] > best) { best = l[k]; besti = i + k * NT; }
     }
-    for (; i < V; i += FSTU_SAMPLE_THREADS) {
+    for (; i < V; i += NT) {
       float l = sample_transform(row, i, t1, temperature);
       if (CACHE) tl[i] = (unsigned short)(__float_as_uint(l) >> 16);
       if (besti == 0x7fffffff || l > best) { best = l; besti = i; }
@@ -696,7 +692,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   if (tid == 0) {
     float bb = sh.redf[0];
     int bi = sh.redi[0];
-    for (int i = 1; i < 16; ++i)
+    for (int i = 1; i < NT / 64; ++i)
       if (sh.redf[i] > bb || (sh.redf[i] == bb && sh.redi[i] < bi)) { bb = sh.redf[i]; bi = sh.redi[i]; }
     sh.redf[0] = bb;
     sh.bcast_i = bi;
@@ -706,7 +702,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   const int arg = sh.bcast_i;
   __syncthreads();
   if (!do_sample) {
-    if (tid == 0) out[(size_t)b * out_stride] = arg;
+    if (tid == 0) *out_slot = arg;
     return;
   }
 
@@ -722,17 +718,17 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   if (top_k > 0 && top_k < V) {
     unsigned prefix = 0, kk = (unsigned)top_k;
     for (int shift = 24; shift >= LOW_SHIFT; shift -= 8) {
-      for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.hist[i] = 0;
+      for (int i = tid; i < 256; i += NT) sh.hist[i] = 0;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
       // 8 strided loads in flight per thread (one load per trip would make every trip a round trip to the L2)
-      for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+      for (int i0 = tid; i0 < V; i0 += 8 * NT) {
         unsigned k[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) k[u] = f32_key(tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1)));
+        for (int u = 0; u < 8; ++u) k[u] = f32_key(tv(min(i0 + u * NT, V - 1)));
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-          if (i0 + u * FSTU_SAMPLE_THREADS < V && (k[u] & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k[u] >> shift) & 255u], 1u);
+          if (i0 + u * NT < V && (k[u] & himask) == (prefix & himask)) atomicAdd(&sh.hist[(k[u] >> shift) & 255u], 1u);
       }
       __syncthreads();
       if (w == 0) {
@@ -758,32 +754,32 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   if (top_p > 0.f && top_p < 1.f) {
     double e = 0.0;
     // (sums stay in index order per thread: the batches only put 8 loads in flight together)
-    for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+    for (int i0 = tid; i0 < V; i0 += 8 * NT) {
       float l[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1));
+      for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * NT, V - 1));
 #pragma unroll
       for (int u = 0; u < 8; ++u)
-        if (i0 + u * FSTU_SAMPLE_THREADS < V && f32_key(l[u]) >= thr_key) e += (double)expf(l[u] - m);
+        if (i0 + u * NT < V && f32_key(l[u]) >= thr_key) e += (double)expf(l[u] - m);
     }
     double Z1;
-    block_excl_scan_d(e, sh.redd, &Z1);
+    block_excl_scan_d<NT>(e, sh.redd, &Z1);
     const double scale = 17592186044416.0 / Z1;  // 2^44 / Z1: fixed-point probabilities
     const unsigned long long target = (unsigned long long)((double)top_p * 17592186044416.0);
     unsigned prefix = 0;
     unsigned long long above = 0;  // mass of keys strictly above the current prefix range
     for (int shift = 24; shift >= LOW_SHIFT; shift -= 8) {
-      for (int i = tid; i < 256; i += FSTU_SAMPLE_THREADS) sh.mass[i] = 0ull;
+      for (int i = tid; i < 256; i += NT) sh.mass[i] = 0ull;
       __syncthreads();
       unsigned himask = (shift == 24) ? 0u : (0xffffffffu << (shift + 8));
-      for (int i0 = tid; i0 < V; i0 += 8 * FSTU_SAMPLE_THREADS) {
+      for (int i0 = tid; i0 < V; i0 += 8 * NT) {
         float l[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * FSTU_SAMPLE_THREADS, V - 1));
+        for (int u = 0; u < 8; ++u) l[u] = tv(min(i0 + u * NT, V - 1));
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const unsigned k = f32_key(l[u]);
-          if (i0 + u * FSTU_SAMPLE_THREADS < V && k >= thr_key && (k & himask) == (prefix & himask))
+          if (i0 + u * NT < V && k >= thr_key && (k & himask) == (prefix & himask))
             atomicAdd(&sh.mass[(k >> shift) & 255u], (unsigned long long)((double)expf(l[u] - m) * scale));
         }
       }
@@ -815,7 +811,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   }
 
   // ---- draw: inverse CDF in index order over contiguous per-thread chunks
-  const int chunk = (V + FSTU_SAMPLE_THREADS - 1) / FSTU_SAMPLE_THREADS;
+  const int chunk = (V + NT - 1) / NT;
   const int i0 = tid * chunk, i1 = min(V, i0 + chunk);
   // tie ranks need an index-ordered count of tokens equal to vb
   double tcount = 0.0;
@@ -823,7 +819,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     for (int i = i0; i < i1; ++i)
       if (f32_key(tv(i)) == vb_key) tcount += 1.0;
   double ttotal = 0.0;
-  double tbase = (tie_keep >= 0) ? block_excl_scan_d(tcount, sh.redd, &ttotal) : 0.0;
+  double tbase = (tie_keep >= 0) ? block_excl_scan_d<NT>(tcount, sh.redd, &ttotal) : 0.0;
   double mysum = 0.0;
   {
     long long rank = (long long)tbase;
@@ -836,10 +832,10 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
     }
   }
   double Z;
-  double mybase = block_excl_scan_d(mysum, sh.redd, &Z);
+  double mybase = block_excl_scan_d<NT>(mysum, sh.redd, &Z);
   // counter-based uniform (splitmix64 finaliser), 24 bits
   unsigned long long z = seed * 0x9E3779B97F4A7C15ull + (unsigned long long)step * 0xBF58476D1CE4E5B9ull +
-                         (unsigned long long)(b + row0) * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
+                         (unsigned long long)rowid * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
   z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
   z = z ^ (z >> 31);
@@ -869,8 +865,348 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
   if (tid == 0) {
     int pick = sh.bcast_i;
     if (pick < 0) pick = arg;  // rounding left the target past the last chunk
-    out[(size_t)b * out_stride] = pick;
+    *out_slot = pick;
   }
+}
+
+#define FSTU_SAMPLE_THREADS 1024
+template <typename T, bool CACHE>
+__global__ void __launch_bounds__(FSTU_SAMPLE_THREADS)
+sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature,
+              int top_k, float top_p, int do_sample, uint64_t seed, int step, int row0, const int* __restrict__ dyn) {
+  __shared__ SampleShared sh;
+  extern __shared__ unsigned short tl[];   // CACHE: transformed logits of the row
+  const int b = blockIdx.x;
+  if (dyn) { out += dyn[0]; step = dyn[1]; }
+  sample_row<T, CACHE, FSTU_SAMPLE_THREADS>(sh, tl, logits + (size_t)b * V, out + (size_t)b * out_stride, V, temperature, top_k,
+                                            top_p, do_sample, seed, step, b + row0);
+}
+
+// ---------------------------------------------------------------- top-k sampling across the chip
+// The same draw as sample_row for 1 <= top_k <= 64 on 16-bit logits, in one launch of (V / 2048) x B workgroups
+// instead of one workgroup per row (reference: flash_stu/model.py:267-299).
+//
+// The head kernel leaves, per row, the maxima of 64 disjoint subsets of the vocabulary (the packed slots of its
+// greedy pick, already temperature-scaled): the top_k-th largest of them is a lower bound Lb of the row's top_k-th
+// largest logit, because top_k different tokens reach it.  Every workgroup transforms one chunk of 2048 logits (one
+// 16-byte load per thread) and leaves the few tokens >= Lb (about 60 of 50 K at top_k 40) in its own part of a
+// workspace, in index order.  The last workgroup of a row to finish (a ticket per row) collects them and one wave
+// does the rest on that short list: exact threshold, optional top-p, inverse-CDF draw in index order, with the
+// arithmetic of sample_row.  A chunk with more than SAMP_CHUNK_CAP candidates (plateaus of equal logits) makes the
+// last workgroup run sample_row on the whole row instead, so every input has an answer.  The counters of the workspace
+// and the slots are zero on entry and zero again on exit; with `advance` the last workgroup of the launch bumps
+// {pos, step}.
+#define SAMP_CHUNK 2048
+#define SAMP_CHUNK_CAP 32
+#define SAMP_MAX_CHUNKS 32
+#define SAMP_MAX_ROWS (2 * FSTU_MAX_DECODE_ROWS)
+struct SampWs {
+  unsigned ticket[SAMP_MAX_ROWS];
+  unsigned done;
+  unsigned pad[31];
+  unsigned cnt[SAMP_MAX_ROWS][SAMP_MAX_CHUNKS];
+  unsigned cand[SAMP_MAX_ROWS][SAMP_MAX_CHUNKS][SAMP_CHUNK_CAP];   // (index << 16) | 16-bit key
+};
+
+// exchanged between workgroups on different XCDs: agent-scope accesses, which the per-XCD L2 does not keep stale
+__device__ __forceinline__ void st_agent(unsigned* p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned ld_agent(const unsigned* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// value of a 16-bit key (the upper half of f32_key of a 16-bit float)
+__device__ __forceinline__ float key16_f32(unsigned k16) {
+  return key_f32((k16 << 16) | ((k16 & 0x8000u) ? 0u : 0xffffu));
+}
+
+__global__ void __launch_bounds__(256)
+sample_topk_kernel(const bf16_t* __restrict__ logits, int64_t ldl, unsigned long long* __restrict__ best,
+                   SampWs* __restrict__ ws, int64_t* __restrict__ out, int64_t out_stride, int V, float temperature, int top_k,
+                   float top_p, uint64_t seed, int step, int row0, int* __restrict__ dyn, int advance) {
+  __shared__ SampleShared sh;
+  __shared__ int s_wtot[4], s_last, s_n, s_over;
+  __shared__ int s_off[SAMP_MAX_CHUNKS + 1];
+  __shared__ unsigned short c_idx[SAMP_MAX_CHUNKS * SAMP_CHUNK_CAP], c_key[SAMP_MAX_CHUNKS * SAMP_CHUNK_CAP];
+  __shared__ float c_e[SAMP_MAX_CHUNKS * SAMP_CHUNK_CAP];
+  __shared__ unsigned long long c_mass[SAMP_MAX_CHUNKS * SAMP_CHUNK_CAP];
+  const int b = blockIdx.y, g = blockIdx.x, G = gridDim.x, nrows = gridDim.y;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  int pos_off = 0;
+  if (dyn) { pos_off = dyn[0]; step = dyn[1]; }
+  const bf16_t* row = logits + (size_t)b * ldl;
+  const unsigned long long slot = best[(size_t)b * 64 + lane];   // every wave: the row's 64 slot maxima
+  // this thread's 8 logits (the row's last vector is moved back inside the row; its first elements then belong to
+  // the thread before and are masked here)
+  const int v0 = (g * 256 + tid) * 8;
+  const int e0 = min(v0, V - 8);
+  uint4 raw;
+  __builtin_memcpy(&raw, row + e0, 16);   // rows start at any even address
+  const unsigned sk = (unsigned)(slot >> 48);
+  unsigned Lb = 0;
+#pragma unroll
+  for (int bit = 15; bit >= 0; --bit) {
+    const unsigned cnd = Lb | (1u << bit);
+    if (__popcll(__ballot(sk >= cnd)) >= top_k) Lb = cnd;
+  }
+  const bool t1 = temperature == 1.0f;
+  const unsigned rw[4] = {raw.x, raw.y, raw.z, raw.w};
+  unsigned keys[8], mask = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float x = __uint_as_float((j & 1) ? (rw[j >> 1] & 0xffff0000u) : (rw[j >> 1] << 16));
+    if (!t1) x = DT<bf16_t>::rnd(x / temperature);
+    x = DT<bf16_t>::rnd(fminf(fmaxf(x, -1e4f), 1e4f));
+    keys[j] = f32_key(x) >> 16;
+    if (e0 + j >= v0 && v0 < V && keys[j] >= Lb) mask |= 1u << j;
+  }
+  // candidates in index order: thread order, then element order
+  const int mine = __popc(mask);
+  int inc = mine;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(inc, o, FSTU_WAVE);
+    if (lane >= o) inc += t;
+  }
+  if (lane == 63) s_wtot[w] = inc;
+  __syncthreads();
+  int at = inc - mine, tot = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (i < w) at += s_wtot[i];
+    tot += s_wtot[i];
+  }
+  unsigned* dst = ws->cand[b][g];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if ((mask >> j) & 1u) {
+      if (at < SAMP_CHUNK_CAP) st_agent(dst + at, ((unsigned)(e0 + j) << 16) | keys[j]);
+      ++at;
+    }
+  if (tid == 0) st_agent(&ws->cnt[b][g], (unsigned)tot);
+  __syncthreads();   // the workgroup's stores have left its waves
+  if (tid == 0) {
+    __threadfence();
+    s_last = atomicAdd(&ws->ticket[b], 1u) == (unsigned)(G - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+
+  // ---- the row's last workgroup
+  int64_t* out_slot = out + pos_off + (size_t)b * out_stride;
+  // every slot of the row's candidate lists is fetched together with the counts that say which of them are filled:
+  // one trip to memory instead of two
+  constexpr int PER = SAMP_MAX_CHUNKS * SAMP_CHUNK_CAP / 256;
+  unsigned val[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int q = tid + u * 256;
+    val[u] = (q / SAMP_CHUNK_CAP < G) ? ld_agent(&ws->cand[b][0][0] + q) : 0u;
+  }
+  if (w == 0) {
+    const int c = lane < G ? (int)ld_agent(&ws->cnt[b][lane]) : 0;
+    int ci = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(ci, o, FSTU_WAVE);
+      if (lane >= o) ci += t;
+    }
+    if (lane <= G) s_off[lane] = ci - c;   // lane G: the total (its own count is 0)
+    if (lane == 63) s_n = ci;
+    const unsigned long long ov = __ballot(c > SAMP_CHUNK_CAP);
+    if (lane == 0) s_over = ov != 0ull;
+    best[(size_t)b * 64 + lane] = 0ull;
+  }
+  __syncthreads();
+  if (s_over) {
+    sample_row<bf16_t, false, 256>(sh, nullptr, row, out_slot, V, temperature, top_k, top_p, 1, seed, step, b + row0);
+  } else {
+    const int n = s_n;
+    {
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int q = tid + u * 256, gq = q / SAMP_CHUNK_CAP, j = q % SAMP_CHUNK_CAP;
+        if (gq < G && j < s_off[gq + 1] - s_off[gq]) {
+          c_idx[s_off[gq] + j] = (unsigned short)(val[u] >> 16);
+          c_key[s_off[gq] + j] = (unsigned short)(val[u] & 0xffffu);
+        }
+      }
+    }
+    __syncthreads();
+    if (w == 0) {
+      // maximum and its lowest index from the slots
+      unsigned long long kb = slot;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long t = __shfl_xor(kb, o, FSTU_WAVE);
+        kb = t > kb ? t : kb;
+      }
+      const float m = key_f32((unsigned)(kb >> 32));
+      const int arg = (int)(0xffffffffu - (unsigned)(kb & 0xffffffffull));
+      // the top_k-th largest key of the row is the top_k-th largest of the candidates
+      unsigned thr = 0;
+      if (n <= 128) {
+        // the usual case: two keys per lane, held in registers (key 0 never counts: every trial value has a bit set)
+        const unsigned k0 = lane < n ? (unsigned)c_key[lane] : 0u, k1 = lane + 64 < n ? (unsigned)c_key[lane + 64] : 0u;
+#pragma unroll
+        for (int bit = 15; bit >= 0; --bit) {
+          const unsigned cnd = thr | (1u << bit);
+          if (__popcll(__ballot(k0 >= cnd)) + __popcll(__ballot(k1 >= cnd)) >= top_k) thr = cnd;
+        }
+      } else {
+        for (int bit = 15; bit >= 0; --bit) {
+          const unsigned cnd = thr | (1u << bit);
+          int c = 0;
+          for (int i0 = 0; i0 < n; i0 += 64) {
+            const int i = i0 + lane;
+            c += __popcll(__ballot(i < n && (unsigned)c_key[i] >= cnd));
+          }
+          if (c >= top_k) thr = cnd;
+        }
+      }
+      for (int i = lane; i < n; i += 64) {
+        const unsigned k = c_key[i];
+        c_e[i] = k >= thr ? expf(key16_f32(k) - m) : 0.f;
+      }
+      // ---- top-p over the survivors: kept set = {key > vb} U {key == vb with tie rank < tie_keep}
+      unsigned vb = thr;
+      long long tie_keep = -1;   // -1: keep every tied token
+      if (top_p > 0.f && top_p < 1.f) {
+        double e = 0.0;
+        for (int i = lane; i < n; i += 64) e += (double)c_e[i];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, FSTU_WAVE);
+        const double scale = 17592186044416.0 / e;   // 2^44 / Z1: fixed-point probabilities
+        const unsigned long long target = (unsigned long long)((double)top_p * 17592186044416.0);
+        for (int i = lane; i < n; i += 64) c_mass[i] = (unsigned long long)((double)c_e[i] * scale);
+        // the largest key whose mass, together with everything above it, exceeds the target
+        unsigned tbest = 0;
+        bool any = false;
+        for (int i0 = 0; i0 < n; i0 += 64) {
+          const int i = i0 + lane;
+          const bool ok = i < n && (unsigned)c_key[i] >= thr;
+          const unsigned ki = ok ? (unsigned)c_key[i] : 0xffffffffu;
+          unsigned long long S = 0ull;
+          for (int j = 0; j < n; ++j)
+            if ((unsigned)c_key[j] >= ki) S += c_mass[j];
+          if (ok && S > target) { any = true; tbest = max(tbest, ki); }
+        }
+        if (__ballot(any) != 0ull) {
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) tbest = max(tbest, (unsigned)__shfl_xor((int)tbest, o, FSTU_WAVE));
+          vb = tbest;
+          unsigned long long above = 0ull;
+          for (int i = lane; i < n; i += 64)
+            if ((unsigned)c_key[i] > vb) above += c_mass[i];
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) above += __shfl_xor(above, o, FSTU_WAVE);
+          unsigned long long pb = (unsigned long long)((double)expf(key16_f32(vb) - m) * scale);
+          if (pb == 0ull) pb = 1ull;
+          tie_keep = (long long)((target - above) / pb) + 1;
+        }
+      }
+      // ---- draw: inverse CDF in index order over contiguous per-lane segments
+      const int seg = (n + 63) / 64, i0 = min(n, lane * seg), i1 = min(n, i0 + seg);
+      int tbase = 0;
+      if (tie_keep >= 0) {
+        int tc = 0;
+        for (int i = i0; i < i1; ++i) tc += (unsigned)c_key[i] == vb;
+        int ti = tc;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const int t = __shfl_up(ti, o, FSTU_WAVE);
+          if (lane >= o) ti += t;
+        }
+        tbase = ti - tc;
+      }
+      double mysum = 0.0;
+      {
+        long long rank = tbase;
+        for (int i = i0; i < i1; ++i) {
+          const unsigned k = c_key[i];
+          bool keep = k > vb;
+          if (k == vb) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
+          if (keep) mysum += (double)c_e[i];
+        }
+      }
+      double si = mysum;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const double t = __shfl_up(si, o, FSTU_WAVE);
+        if (lane >= o) si += t;
+      }
+      const double Z = __shfl(si, 63, FSTU_WAVE), mybase = si - mysum;
+      // counter-based uniform (splitmix64 finaliser), 24 bits
+      unsigned long long z = seed * 0x9E3779B97F4A7C15ull + (unsigned long long)step * 0xBF58476D1CE4E5B9ull +
+                             (unsigned long long)(b + row0) * 0x94D049BB133111EBull + 0x2545F4914F6CDD1Dull;
+      z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+      z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+      z = z ^ (z >> 31);
+      const double tgt = ((double)(z >> 40) / 16777216.0) * Z;
+      int pick = -1;
+      if (mysum > 0.0 && tgt >= mybase && tgt < mybase + mysum) {
+        double acc = mybase;
+        long long rank = tbase;
+        int lastkept = -1;
+        for (int i = i0; i < i1; ++i) {
+          const unsigned k = c_key[i];
+          bool keep = k > vb;
+          if (k == vb) { keep = (tie_keep < 0) || (rank < tie_keep); ++rank; }
+          if (keep) {
+            acc += (double)c_e[i];
+            lastkept = c_idx[i];
+            if (acc > tgt) { pick = c_idx[i]; break; }
+          }
+        }
+        if (pick < 0) pick = lastkept;
+      }
+      const unsigned long long who = __ballot(pick >= 0);
+      if (who != 0ull) pick = __shfl(pick, __ffsll((long long)who) - 1, FSTU_WAVE);
+      else pick = arg;   // rounding left the target past the last segment
+      if (lane == 0) *out_slot = pick;
+    }
+  }
+  // ---- leave the workspace as it was found
+  if (tid < G) ws->cnt[b][tid] = 0u;
+  if (tid == 0) {
+    ws->ticket[b] = 0u;
+    if (atomicAdd(&ws->done, 1u) == (unsigned)(nrows - 1)) {
+      ws->done = 0u;
+      if (dyn && advance) { dyn[0] = pos_off + 1; dyn[1] = step + 1; }
+    }
+  }
+}
+
+extern "C" int64_t fstu_sample_ws_bytes(void) { return (int64_t)sizeof(SampWs); }
+
+bool fstu_sample_topk_ok(int B, int V, int top_k, int dtype) {
+  return dtype == FSTU_BF16 && B >= 1 && B <= SAMP_MAX_ROWS && V >= 1024 && V <= SAMP_CHUNK * SAMP_MAX_CHUNKS && top_k >= 1 &&
+         top_k <= 64;
+}
+
+int fstu_sample_topk_dyn(const void* logits, int64_t ldl, void* best_ws, void* samp_ws, int64_t* out, int64_t out_stride, int B,
+                         int V, float temperature, int top_k, float top_p, uint64_t seed, int step, int row0, int* dyn,
+                         int advance, void* stream) {
+  FSTU_REQUIRE(logits && best_ws && samp_ws && out, FSTU_ENULL, "fstu_sample_topk: null pointer");
+  FSTU_REQUIRE(fstu_sample_topk_ok(B, V, top_k, FSTU_BF16), FSTU_ESHAPE,
+               "fstu_sample_topk: needs 1 <= B <= %d, 1024 <= V <= %d, 1 <= top_k <= 64 (B=%d V=%d top_k=%d)", SAMP_MAX_ROWS,
+               SAMP_CHUNK * SAMP_MAX_CHUNKS, B, V, top_k);
+  FSTU_REQUIRE(temperature > 0.f && ldl >= V && out_stride >= 1, FSTU_EARG, "fstu_sample_topk: bad temperature / ldl / out_stride");
+  FSTU_REQUIRE(fstu_aligned(best_ws, 8) && fstu_aligned(samp_ws, 8) && fstu_aligned(logits, 2), FSTU_EALIGN,
+               "fstu_sample_topk: workspaces must be 8-byte aligned");
+  const dim3 grid((V + SAMP_CHUNK - 1) / SAMP_CHUNK, B);
+  hipLaunchKernelGGL(sample_topk_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)logits, ldl,
+                     (unsigned long long*)best_ws, (SampWs*)samp_ws, out, out_stride, V, temperature, top_k, top_p, seed, step, row0,
+                     dyn, advance);
+  FSTU_CHECK_LAUNCH("fstu_sample_topk");
+  return FSTU_OK;
+}
+
+extern "C" int fstu_sample_topk(const void* logits, int64_t ldl, void* best_ws, void* samp_ws, int64_t* out, int64_t out_stride,
+                                int B, int V, float temperature, int top_k, float top_p, uint64_t seed, int step, void* stream) {
+  return fstu_sample_topk_dyn(logits, ldl, best_ws, samp_ws, out, out_stride, B, V, temperature, top_k, top_p, seed, step, 0, nullptr,
+                              0, stream);
 }
 
 __global__ void advance_dyn_kernel(int* dyn) {

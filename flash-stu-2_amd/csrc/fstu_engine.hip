@@ -138,6 +138,12 @@ static bool chain_ok(const fstu_model_desc* m, int do_sample, const int* dyn) {
          fstu_finish_embed_supported(m->B, m->d, m->emb, m->x, m->layers[0].norm1_w, m->h);
 }
 
+// top-k sampling spread over the chip: needs the head kernel that leaves the packed maxima and the sampler's workspace
+static bool sample_spread_ok(const fstu_model_desc* m, int do_sample, int top_k) {
+  return do_sample && m->best && m->samp_ws && fstu_sample_topk_ok(m->B, m->V, top_k, m->dtype) &&
+         fstu_head_argmax_fused_pick(m->h, m->d, m->emb, m->d, m->dtype);
+}
+
 // 17..32 rows: the MLP, where nearly all the weight bytes are, runs once over all rows on the tiled matrix-core kernel
 // (gate/up with the GLU epilogue, split-K down projection), so every MLP weight is read once per step; the
 // STU recurrence and the window attention, per-row operators, run over all rows in one launch each, and the small
@@ -177,6 +183,15 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
     TIMED(PC_GLU, fstu_gemm_bf16(m->h, d, L.w_gate, L.w_up, nullptr, 0, m->act, I, B, I, d, 1, stream));
     TIMED(PC_DOWN, fstu_gemm_bf16_splitk(m->act, I, L.w_down, m->partial, B, d, I, ks, stream));
     TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, ks, 0, next_w, m->h, B, d, m->eps, dt, stream));
+  }
+  if (sample_spread_ok(m, do_sample, top_k)) {
+    // the head leaves each row's packed maxima, the sampler spreads every row over the chip and advances {pos, step}
+    for (int c = 0; c < 2; ++c)
+      TIMED(PC_HEAD, fstu_head_maxima(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, temperature,
+                                      (char*)m->best + (size_t)c * R * 64 * 8, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_topk_dyn(m->logits, m->V, m->best, m->samp_ws, tok_out, tok_stride, B, m->V, temperature, top_k, top_p,
+                                          seed, step, m->row0, dyn, 1, stream));
+    return FSTU_OK;
   }
   for (int c = 0; c < 2; ++c)
     TIMED(PC_HEAD, fstu_linear_decode(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, dt, stream));
@@ -329,6 +344,10 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   if (!do_sample && m->best) {
     TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
                                         tok_stride, dyn, (chain && g_chain_next) ? -1 : 1, dt, stream));
+  } else if (sample_spread_ok(m, do_sample, top_k)) {
+    TIMED(PC_HEAD, fstu_head_maxima(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, dt, stream));
+    TIMED(PC_SAMPLE, fstu_sample_topk_dyn(m->logits, m->V, m->best, m->samp_ws, tok_out, tok_stride, B, m->V, temperature, top_k, top_p,
+                                          seed, step, m->row0, dyn, 1, stream));
   } else {
     TIMED(PC_HEAD, fstu_linear_decode(m->h, d, m->emb, m->logits, m->V, B, m->V, d, dt, stream));
     TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0, dyn, dt, stream));

@@ -371,6 +371,21 @@ int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, in
   return rc;
 }
 
+extern "C" int fstu_head_maxima(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                                float temperature, void* best_ws, int dtype, void* stream) {
+  int rc = check_common("fstu_head_maxima", x, W, logits, ldx, rows, N, K);
+  if (rc) return rc;
+  FSTU_REQUIRE(best_ws, FSTU_ENULL, "fstu_head_maxima: null workspace");
+  FSTU_REQUIRE(ldy >= N && temperature > 0.f, FSTU_EARG, "fstu_head_maxima: bad ldy / temperature");
+  FSTU_REQUIRE(fstu_aligned(best_ws, 8), FSTU_EALIGN, "fstu_head_maxima: workspace must be 8-byte aligned");
+  FSTU_REQUIRE(fstu_head_argmax_fused_pick(x, ldx, W, K, dtype), FSTU_ESHAPE,
+               "fstu_head_maxima: needs bf16, K %% 256 == 0 and 16-byte aligned rows");
+  LinArgs a{x, ldx, W, nullptr, logits, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
+  launch_mfma<LIN_ARGMAX>(a, 1, (hipStream_t)stream);
+  FSTU_CHECK_LAUNCH("fstu_head_maxima");
+  return FSTU_OK;
+}
+
 // ---------------------------------------------------------------- head + greedy pick without any allocation
 // The packed per-row maxima of the head kernel live in a file-scope device array instead of a caller workspace, for
 // callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid hipMalloc).  Every GPU

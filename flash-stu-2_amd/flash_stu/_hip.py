@@ -56,6 +56,9 @@ SIGNATURES = {
     "fstu_swa_prefill_ws_elems": [_i, _i, _i, _i],
     "fstu_swa_prefill_mfma": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp],
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
+    "fstu_sample_ws_bytes": [],
+    "fstu_head_maxima": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i, _vp],
+    "fstu_sample_topk": [_vp, _i64, _vp, _vp, _vp, _i64, _i, _i, _f, _i, _f, _u64, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
     "fstu_head_argmax_static": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i64, _i, _vp],
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
@@ -108,6 +111,7 @@ def load(path: Optional[str] = None):
         fn.argtypes = args
         fn.restype = ctypes.c_int
     lib.fstu_packed_elems.restype = ctypes.c_int64
+    lib.fstu_sample_ws_bytes.restype = ctypes.c_int64
     lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
     lib.fstu_step_mega_ws_bytes.restype = ctypes.c_size_t
     lib.fstu_lds_sequence_ws_floats.restype = ctypes.c_size_t
@@ -653,6 +657,43 @@ def head_argmax(x: torch.Tensor, W: torch.Tensor, out_tokens: torch.Tensor, best
                                    _p(best_ws), out_tokens.data_ptr(), out_tokens.stride(0), _dt(x), _stream()),
            "fstu_head_argmax")
     return logits
+
+
+def head_maxima(x: torch.Tensor, W: torch.Tensor, best_ws: torch.Tensor, temperature: float = 1.0,
+                logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """logits = x @ W^T (rows<=16, bf16) and, in best_ws (int64 zeros, rows*64 elements), the packed maxima of 64
+    subsets of every row at this temperature: what sample_topk starts from."""
+    rows, ldx = _rows_view(x)
+    _dev(W, best_ws)
+    N, K = W.shape
+    assert x.shape[1] == K and x.dtype == W.dtype
+    if logits is None:
+        logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    assert best_ws.dtype == torch.int64 and best_ws.numel() >= rows * 64
+    _check(load().fstu_head_maxima(_p(x), ldx, _p(W), _p(logits), logits.stride(0), rows, N, K, float(temperature),
+                                   _p(best_ws), _dt(x), _stream()), "fstu_head_maxima")
+    return logits
+
+
+def sample_ws(device) -> torch.Tensor:
+    """Zeroed workspace of sample_topk (allocate once; every call leaves its counters zero again)."""
+    return torch.zeros((int(load().fstu_sample_ws_bytes()) + 7) // 8, dtype=torch.int64, device=device)
+
+
+def sample_topk(logits: torch.Tensor, best_ws: torch.Tensor, samp_ws: torch.Tensor, out: torch.Tensor, top_k: int,
+                temperature: float = 1.0, top_p: Optional[float] = None, seed: int = 0, step: int = 0):
+    """sample() with do_sample=True for bf16 logits and 1 <= top_k <= 64, every row spread over the chip.  best_ws: the
+    maxima head_maxima left for these logits at this temperature; it and samp_ws's counters are zero again afterwards."""
+    _dev(best_ws, samp_ws)
+    if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1 or logits.dtype != torch.bfloat16:
+        raise FlashSTUHipError("sample_topk takes (B,V) bf16 logits with contiguous rows on the GPU")
+    B, V = logits.shape
+    assert out.dtype == torch.int64 and out.is_cuda and out.dim() == 1 and out.shape[0] == B
+    assert best_ws.dtype == torch.int64 and best_ws.numel() >= B * 64
+    _check(load().fstu_sample_topk(_p(logits), logits.stride(0), _p(best_ws), _p(samp_ws), out.data_ptr(), out.stride(0),
+                                   B, V, float(temperature), int(top_k), float(top_p) if top_p else 0.0,
+                                   int(seed) & ((1 << 64) - 1), int(step), _stream()), "fstu_sample_topk")
+    return out
 
 
 def pack_rows(W: torch.Tensor) -> torch.Tensor:

@@ -40,7 +40,7 @@ class ModelDesc(ctypes.Structure):
                 ("lds_S", _i), ("lds_fir_taps", _i), ("single_branch", _i), ("ksplit_down", _i), ("hist_nsplit_max", _i), ("row0", _i),
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
-                ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp),
+                ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp), ("samp_ws", _vp),
                 ("wp_emb", _vp), ("x2", _vp), ("glu_packed", _i), ("down_packed", _i), ("merge_norm", _i),
                 ("mega_ws", _vp)]
 
@@ -232,7 +232,8 @@ class DecodeEngine:
         m.partial = buf(max(m.ksplit_down, 16), B, d, dtype=torch.float32).data_ptr()
         m.eo = buf(self.HIST_NSPLIT_MAX, 2, B, d, dtype=torch.float32).data_ptr()
         m.logits = ch.logits.data_ptr()
-        m.best = buf(16 * 64, dtype=torch.int64).data_ptr()
+        m.best = buf(32 * 64, dtype=torch.int64).data_ptr()
+        m.samp_ws = buf((int(self.lib.fstu_sample_ws_bytes()) + 7) // 8, dtype=torch.int64).data_ptr()
         if dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(B, d, I):
             # gate/up projection over packed weights, one workgroup per CU with equal bytes each
             for i, layer in enumerate(model.layers):

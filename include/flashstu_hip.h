@@ -310,6 +310,24 @@ int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ld
                      float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int dtype,
                      void* stream);
 
+/* The first half of fstu_head_argmax alone (bf16, K % 256 == 0): the logits, and in best_ws (rows*64 64-bit words, zero on
+ * entry) the packed maxima of 64 disjoint subsets of each row: (monotone key of clamp(T(logit/temperature)) << 32) |
+ * ~index.  fstu_sample_topk consumes and clears them.  Replaces lm_head at flash_stu/model.py:176. */
+int fstu_head_maxima(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
+                     float temperature, void* best_ws, int dtype, void* stream);
+
+/* fstu_sample (do_sample = 1) for bf16 logits and 1 <= top_k <= 64, spread over (V / 2048) x B workgroups instead of one
+ * workgroup per row; same draws.  logits: (B, V) rows ldl elements apart; best_ws: the maxima fstu_head_maxima left
+ * for these logits at this temperature; samp_ws: fstu_sample_ws_bytes() bytes, zero-initialised once by the caller.
+ * best_ws and the counters at the start of samp_ws are zero again when the call completes (the candidate lists behind
+ * them keep their last contents, which no later call reads).  1 <= B <= 32, 1024 <= V <= 65536.  The top_k-th largest
+ * of a row's 64 maxima bounds the row's top_k-th largest logit from below, so every workgroup keeps only the few
+ * tokens above that bound and the last one to finish a row draws from that short list; rows with long plateaus of
+ * equal logits are drawn by that workgroup from the whole row instead.  Replaces flash_stu/model.py:267-299. */
+int64_t fstu_sample_ws_bytes(void);
+int fstu_sample_topk(const void* logits, int64_t ldl, void* best_ws, void* samp_ws, int64_t* out, int64_t out_stride,
+                     int B, int V, float temperature, int top_k, float top_p, uint64_t seed, int step, void* stream);
+
 /* fstu_head_argmax for callers that cannot allocate or pass a workspace (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * fstu_head_argmax without best_ws: the packed per-row maxima live in a static device array of the library
@@ -467,6 +485,8 @@ typedef struct {
   float* eo;                /* fp32 */
   void* logits;             /* (B,V) */
   void* best;               /* max(B,16)*64 64-bit words, zero-initialised once by the caller */
+  void* samp_ws;            /* fstu_sample_ws_bytes() bytes, zero-initialised once by the caller, or NULL: top-k sampling
+                               then runs one workgroup per row (fstu_sample) instead of fstu_sample_topk */
   const void* wp_emb;       /* packed tied head (one-launch step) */
   void* x2;                 /* (B,d) second residual buffer (the stream ping-pongs x <-> x2); NULL: the add + norm
                                between sub-layers runs as launches of its own */

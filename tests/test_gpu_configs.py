@@ -190,6 +190,32 @@ def test_c5_shape_sampling_parity_reduced():
     assert torch.equal(got.cpu(), ref)
 
 
+@pytest.mark.parametrize("rows", [8, 32])
+def test_c5_shape_bf16_sampling_spread_over_the_chip(hip, rows):
+    """Config 5's sampling (top-k 40, temperature 0.8) in bf16 through the one-call step, where the head leaves its
+    packed maxima and the sampler spreads every row over the chip: every generated id is the oracle's draw (and the
+    one-workgroup-per-row kernel's) from the logits the step produced, eagerly and under graph replay."""
+    from test_gpu_model import make_pair, prompt
+    ocfg, w, model = make_pair(seed=2, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=256, n_layers=4,
+                               n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
+                               stu_decode_mode="lds")
+    P, N = 20, 40
+    ids = prompt(rows, P, ocfg.vocab_size, 4)
+    got, gl = model.generate(ids.cuda(), max_length=P + N, temperature=0.8, top_k=40, do_sample=True, seed=2,
+                             return_logits=True)
+    again = model.generate(ids.cuda(), max_length=P + N, temperature=0.8, top_k=40, do_sample=True, seed=2)
+    assert torch.equal(again, got)
+    miss = 0
+    for t in range(N):
+        lt = gl[:, t].contiguous()
+        ref = torch.empty(rows, dtype=torch.int64, device="cuda")
+        hip.sample(lt, ref, 0.8, 40, None, True, seed=2, step=t)
+        assert torch.equal(got[:, P + t], ref), t
+        o = O.next_token(lt.cpu(), 0.8, 40, None, True, seed=2, step=t)[:, 0]
+        miss += int((got[:, P + t].cpu() != o).sum())
+    assert miss <= 1, miss
+
+
 @pytest.mark.parametrize("rows", [17, 20, 32])
 def test_c5_shape_bf16_lds_teacher_forced(rows):
     """Same structure in bf16 with the recurrence state, logits within the bf16 tolerance.  17..32 rows step as one

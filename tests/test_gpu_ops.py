@@ -808,6 +808,74 @@ def test_sample_draws_match_oracle(hip, dtype, temperature, top_k, top_p):
     assert agree >= total - 1, (agree, total)
 
 
+SAMP_COUNTER_WORDS = (32 + 32 + 32 * 32) // 2     # tickets, launch counter, per-chunk counts: 32-bit each
+
+
+@pytest.mark.parametrize("V", [50257, 4096, 1031])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 40, None), (0.8, 40, None), (0.8, 1, None), (1.3, 64, None),
+                                                     (0.8, 40, 0.9), (1.0, 7, 0.5)])
+def test_sample_topk_spread_equals_one_workgroup_per_row_and_oracle(hip, V, temperature, top_k, top_p):
+    """The sampler that spreads a row over the chip (head maxima -> candidates -> short-list draw) picks what
+    fstu_sample picks on the same logits, and (without top-p, where the bf16 nucleus rule is the kernel's own) what the
+    oracle's draw picks.  Rows start at odd element offsets (odd V); the maxima and the sampler's counters come back zeroed."""
+    g = gen(41)
+    B, K = 8, 256
+    x = dev((torch.randn(B, K, generator=g)).bfloat16())
+    W = dev((torch.randn(V, K, generator=g) * (3.0 / K ** 0.5)).bfloat16())
+    best = torch.zeros(B * 64, dtype=torch.int64, device="cuda")
+    ws = hip.sample_ws("cuda")
+    agree = total = 0
+    for step in range(12):
+        logits = hip.head_maxima(x, W, best, temperature)
+        assert int((best != 0).sum()) > 0
+        out = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample_topk(logits, best, ws, out, top_k, temperature, top_p, seed=5, step=step)
+        ref = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample(logits, ref, temperature, top_k, top_p, True, seed=5, step=step)
+        assert torch.equal(out, ref), (step, out.tolist(), ref.tolist())
+        assert int((best != 0).sum()) == 0 and int((ws[:SAMP_COUNTER_WORDS] != 0).sum()) == 0
+        if top_p is None:
+            o = O.next_token(logits.cpu(), temperature, top_k, None, True, seed=5, step=step)[:, 0]
+            agree += int((out.cpu() == o).sum())
+            total += B
+    assert agree >= total - 1, (agree, total)
+
+
+def test_sample_topk_spread_plateaus_and_errors(hip):
+    """Long runs of equal logits overflow the per-chunk candidate lists: the row's last workgroup then draws from the
+    whole row, with the same result as fstu_sample.  Arguments outside the fast path are refused."""
+    g = gen(42)
+    B, K, V = 5, 256, 6000
+    x = dev(torch.randn(B, K, generator=g).bfloat16())
+    Wc = (torch.randn(V, K, generator=g) * 0.2).bfloat16()
+    Wc[1000:3000] = Wc[1000]          # 2000 tokens share one logit per row
+    Wc[3500:3600] = Wc[3500]
+    W = dev(Wc)
+    best = torch.zeros(B * 64, dtype=torch.int64, device="cuda")
+    ws = hip.sample_ws("cuda")
+    for step, (top_k, temperature, top_p) in enumerate([(40, 1.0, None), (64, 0.7, None), (40, 0.9, 0.8), (3, 1.0, None)]):
+        logits = hip.head_maxima(x, W, best, temperature)
+        out = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample_topk(logits, best, ws, out, top_k, temperature, top_p, seed=9, step=step)
+        ref = torch.empty(B, dtype=torch.int64, device="cuda")
+        hip.sample(logits, ref, temperature, top_k, top_p, True, seed=9, step=step)
+        assert torch.equal(out, ref), (step, out.tolist(), ref.tolist())
+        assert int((best != 0).sum()) == 0 and int((ws[:SAMP_COUNTER_WORDS] != 0).sum()) == 0
+    # all logits equal: every token is a candidate everywhere
+    xz = torch.zeros(B, K, dtype=torch.bfloat16, device="cuda")
+    logits = hip.head_maxima(xz, W, best, 1.0)
+    out = torch.empty(B, dtype=torch.int64, device="cuda")
+    hip.sample_topk(logits, best, ws, out, 40, 1.0, None, seed=3, step=0)
+    ref = torch.empty(B, dtype=torch.int64, device="cuda")
+    hip.sample(logits, ref, 1.0, 40, None, True, seed=3, step=0)
+    assert torch.equal(out, ref)
+    for bad_k in (0, 65):
+        with pytest.raises(hip.FlashSTUHipError, match="top_k"):
+            hip.sample_topk(logits, best, ws, out, bad_k)
+    with pytest.raises(hip.FlashSTUHipError, match="V="):
+        hip.sample_topk(logits[:, :512].contiguous(), best, ws, out, 40)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_lds_steps_dense(hip, dtype):
     g = gen(13)
