@@ -92,73 +92,129 @@ template <int R> __device__ __forceinline__ void twiddle_powers(cpx (&pw)[R], co
   }
 }
 
-// One radix-R butterfly of a pass over blocks of Nb = R*q elements (q = 1 << lq).  Forward: decimation in
+template <int R> __host__ __device__ constexpr int lg_radix() { return R == 16 ? 4 : R == 8 ? 3 : R == 4 ? 2 : 1; }
+
+// One radix-R butterfly of a pass over blocks of Nb = R*q elements (q = 1 << LQ).  Forward: decimation in
 // frequency, y[k] = w^(r k) * sum_m x[m] W_R^(m k) written where x was read.  Inverse: the exact mirror.
-template <int R, bool INV>
-__device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __restrict__ tw, int u, int lq, int ts) {
-  const int q = 1 << lq;
+// The transform length and the stride are compile-time constants: the R points of a butterfly sit a fixed distance
+// apart in the padded column (q + q/16 slots; q = 1 only occurs with R = 16 on blocks that start at a multiple of
+// 16), so their addresses are one base and immediate offsets.
+template <int R, bool INV, int LQ, int LOGN>
+__device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __restrict__ tw, int u) {
+  constexpr int LR = lg_radix<R>();
+  constexpr int q = 1 << LQ;
+  constexpr int TS = 1 << (LOGN - LQ - LR);   // table stride: w_Nb = tw[TS]
+  constexpr int ST = (LQ >= 4) ? (q + (q >> 4)) : 1;
+  static_assert(LQ == 0 || LQ >= 4, "strides between 2 and 8 would cross a pad slot");
   const int r = u & (q - 1);
-  const int base = ((u >> lq) * R << lq) + r;
+  const int base = ((u >> LQ) << (LQ + LR)) + r;
+  cpx* __restrict__ p = col + phys(base);
   cpx v[R], pw[R];
-  const bool twid = lq > 0;
-  if (twid) twiddle_powers<R>(pw, tw, r * ts);
+  constexpr bool twid = LQ > 0;
+  if (twid) twiddle_powers<R>(pw, tw, r * TS);
   if (!INV) {
 #pragma unroll
-    for (int m = 0; m < R; ++m) v[m] = col[phys(base + (m << lq))];
+    for (int m = 0; m < R; ++m) v[m] = p[m * ST];
     dft_inreg<R>(v);
 #pragma unroll
     for (int k = 0; k < R; ++k) {
       cpx o = v[brev<R>(k)];
       if (twid && k > 0) o = cmul(o, pw[k]);
-      col[phys(base + (k << lq))] = o;
+      p[k * ST] = o;
     }
   } else {
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      cpx o = col[phys(base + (k << lq))];
+      cpx o = p[k * ST];
       if (twid && k > 0) o = cmulc(o, pw[k]);
       v[k] = cconj(o);
     }
     dft_inreg<R>(v);
 #pragma unroll
-    for (int m = 0; m < R; ++m) col[phys(base + (m << lq))] = cconj(v[brev<R>(m)]);
+    for (int m = 0; m < R; ++m) p[m * ST] = cconj(v[brev<R>(m)]);
   }
 }
 
-template <int R, bool INV, int NT>
-__device__ __forceinline__ void run_pass(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn,
-                                         int lNb) {
-  constexpr int LR = (R == 16) ? 4 : (R == 8) ? 3 : (R == 4) ? 2 : 1;
-  const int lq = lNb - LR;           // log2 of the butterfly stride
-  const int lper = logn - LR;        // log2 of butterflies per column
-  const int ts = 1 << (logn - lNb);  // table stride: w_Nb = tw[ts]
-  const int total = cols << lper;
-  for (int w = threadIdx.x; w < total; w += NT) {
-    const int colid = w >> lper;
-    butterfly<R, INV>(lds + (size_t)colid * colstride, tw, w & ((1 << lper) - 1), lq, ts);
-  }
+template <int LOGN> __host__ __device__ constexpr int col_stride() { return (1 << LOGN) + (1 << (LOGN - 4)); }
+
+template <int R, bool INV, int LQ, int LOGN, int NT>
+__device__ __forceinline__ void run_pass(cpx* lds, const cpx* __restrict__ tw, int cols) {
+  constexpr int LPER = LOGN - lg_radix<R>();   // log2 of butterflies per column
+  const int total = cols << LPER;
+  for (int w = threadIdx.x; w < total; w += NT)
+    butterfly<R, INV, LQ, LOGN>(lds + (size_t)(w >> LPER) * col_stride<LOGN>(), tw, w & ((1 << LPER) - 1));
   __syncthreads();
 }
 
-// logn = 4*a + rem: the first forward pass has radix 2^rem (if rem > 0), every other pass radix 16.
-template <int NT>
-__device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn) {
-  int lNb = logn;
-  const int rem = logn & 3;
-  if (rem == 1) run_pass<2, false, NT>(lds, tw, cols, colstride, logn, lNb);
-  if (rem == 2) run_pass<4, false, NT>(lds, tw, cols, colstride, logn, lNb);
-  if (rem == 3) run_pass<8, false, NT>(lds, tw, cols, colstride, logn, lNb);
-  lNb -= rem;
-  for (; lNb >= 4; lNb -= 4) run_pass<16, false, NT>(lds, tw, cols, colstride, logn, lNb);
+// LOGN = 4*a + rem: the first forward pass has radix 2^rem (if rem > 0), every other pass radix 16.  The last forward
+// pass and the first inverse pass work on the same 16 neighbours of a column (stride 1): callers that multiply by a
+// spectrum in between skip both here and do the three steps in registers (fft_middle).
+template <int LOGN, int NT, bool SKIP_LAST>
+__device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw, int cols) {
+  constexpr int REM = LOGN & 3, TOP = LOGN - REM;
+  if constexpr (REM == 1) run_pass<2, false, LOGN - 1, LOGN, NT>(lds, tw, cols);
+  if constexpr (REM == 2) run_pass<4, false, LOGN - 2, LOGN, NT>(lds, tw, cols);
+  if constexpr (REM == 3) run_pass<8, false, LOGN - 3, LOGN, NT>(lds, tw, cols);
+  if constexpr (TOP >= 12) run_pass<16, false, 8, LOGN, NT>(lds, tw, cols);
+  if constexpr (TOP >= 8) run_pass<16, false, 4, LOGN, NT>(lds, tw, cols);
+  if constexpr (!SKIP_LAST) run_pass<16, false, 0, LOGN, NT>(lds, tw, cols);
 }
 
-template <int NT>
-__device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw, int cols, int colstride, int logn) {
-  const int rem = logn & 3;
-  for (int lNb = 4; lNb <= logn - rem; lNb += 4) run_pass<16, true, NT>(lds, tw, cols, colstride, logn, lNb);
-  if (rem == 1) run_pass<2, true, NT>(lds, tw, cols, colstride, logn, logn);
-  if (rem == 2) run_pass<4, true, NT>(lds, tw, cols, colstride, logn, logn);
-  if (rem == 3) run_pass<8, true, NT>(lds, tw, cols, colstride, logn, logn);
+template <int LOGN, int NT, bool SKIP_FIRST>
+__device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw, int cols) {
+  constexpr int REM = LOGN & 3, TOP = LOGN - REM;
+  if constexpr (!SKIP_FIRST) run_pass<16, true, 0, LOGN, NT>(lds, tw, cols);
+  if constexpr (TOP >= 8) run_pass<16, true, 4, LOGN, NT>(lds, tw, cols);
+  if constexpr (TOP >= 12) run_pass<16, true, 8, LOGN, NT>(lds, tw, cols);
+  if constexpr (REM == 1) run_pass<2, true, LOGN - 1, LOGN, NT>(lds, tw, cols);
+  if constexpr (REM == 2) run_pass<4, true, LOGN - 2, LOGN, NT>(lds, tw, cols);
+  if constexpr (REM == 3) run_pass<8, true, LOGN - 3, LOGN, NT>(lds, tw, cols);
+}
+
+// 16 spectrum values of 16 neighbouring positions (128 contiguous bytes)
+__device__ __forceinline__ void load_spec16(const cpx* __restrict__ sp, cpx (&s)[16]) {
+#pragma unroll
+  for (int k = 0; k < 16; k += 2) {
+    const float4 t = *(const float4*)(sp + k);
+    s[k] = make_float2(t.x, t.y);
+    s[k + 1] = make_float2(t.z, t.w);
+  }
+}
+
+// forward stride-1 butterfly of 16 neighbours, left in registers in position order (x[k] belongs to position base + k)
+__device__ __forceinline__ void forward16(const cpx* __restrict__ p, cpx (&x)[16]) {
+  cpx v[16];
+#pragma unroll
+  for (int m = 0; m < 16; ++m) v[m] = p[m];
+  dft_inreg<16>(v);
+#pragma unroll
+  for (int k = 0; k < 16; ++k) x[k] = v[brev<16>(k)];
+}
+
+// x[k] * s[k] through the inverse stride-1 butterfly, written to the 16 neighbours
+__device__ __forceinline__ void product_inverse16(cpx* __restrict__ p, const cpx (&x)[16], const cpx (&s)[16]) {
+  cpx v[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) v[k] = cconj(cmul(x[k], s[k]));
+  dft_inreg<16>(v);
+#pragma unroll
+  for (int m = 0; m < 16; ++m) p[m] = cconj(v[brev<16>(m)]);
+}
+
+// last forward pass, product with the per-column spectra spec[(c0 + col) * n + position], first inverse pass
+template <int LOGN, int NT>
+__device__ __forceinline__ void fft_middle(cpx* lds, const cpx* __restrict__ spec, int c0, int ncol) {
+  constexpr int LPER = LOGN - 4;
+  const int total = ncol << LPER;
+  for (int w = threadIdx.x; w < total; w += NT) {
+    const int colid = w >> LPER, u = w & ((1 << LPER) - 1);
+    cpx* p = lds + (size_t)colid * col_stride<LOGN>() + 17 * u;   // phys(16 u)
+    cpx s[16], x[16];
+    load_spec16(spec + ((size_t)(c0 + colid) << LOGN) + 16 * u, s);
+    forward16(p, x);
+    product_inverse16(p, x, s);
+  }
+  __syncthreads();
 }
 
 // ---------------------------------------------------------------- twiddle table
@@ -173,25 +229,25 @@ __global__ void fft_twiddle_kernel(cpx* __restrict__ tw, int n) {
 // ---------------------------------------------------------------- filter spectra
 // Column j of the filter matrix (element (s, j) at filt[s*f_ls + j*f_cs], taps s < taps) -> spec[j*n + p] =
 // (F[p] + i F[p^8]) / n (both branches) or F[p] / n, p running over the digit-reversed positions.
-template <typename T, int NT>
+template <typename T, int LOGN, int NT>
 __global__ void __launch_bounds__(NT)
 fft_filter_kernel(const T* __restrict__ filt, size_t f_ls, size_t f_cs, cpx* __restrict__ spec,
-                  const cpx* __restrict__ tw, int taps, int ncol_total, int n, int logn, int lcols, int both) {
+                  const cpx* __restrict__ tw, int taps, int ncol_total, int lcols, int both) {
   extern __shared__ cpx fft_lds[];
+  constexpr int n = 1 << LOGN, colstride = col_stride<LOGN>();
   const int cols = 1 << lcols;
-  const int colstride = n + (n >> 4);
   const int c0 = blockIdx.x * cols;
-  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+  for (int idx = threadIdx.x; idx < (cols << LOGN); idx += NT) {
     const int colid = idx & (cols - 1), s = idx >> lcols;
     float v = 0.f;
     if (s < taps && c0 + colid < ncol_total) v = DT<T>::ld(filt + (size_t)s * f_ls + (size_t)(c0 + colid) * f_cs);
     fft_lds[(size_t)colid * colstride + phys(s)] = make_float2(v, 0.f);
   }
   __syncthreads();
-  fft_forward<NT>(fft_lds, tw, cols, colstride, logn);
+  fft_forward<LOGN, NT, false>(fft_lds, tw, cols);
   const float inv_n = 1.0f / (float)n;
-  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
-    const int colid = idx >> logn, p = idx & (n - 1);
+  for (int idx = threadIdx.x; idx < (cols << LOGN); idx += NT) {
+    const int colid = idx >> LOGN, p = idx & (n - 1);
     if (c0 + colid >= ncol_total) continue;
     const cpx* col = fft_lds + (size_t)colid * colstride;
     cpx f = col[phys(p)];
@@ -207,14 +263,14 @@ fft_filter_kernel(const T* __restrict__ filt, size_t f_ls, size_t f_cs, cpx* __r
 // x element (b, t, c) at x[b*x_sb + t*x_st + c*x_sc]; the K outputs of channel c (K = 1: per-channel spectra
 // spec[c]; K > 1: a shared bank spec[k]) go to y[b*y_sb + t*y_st + k*y_sk + c*y_sc] (and y2 likewise).
 // mode 0: y = T(T(re) + T(im));  mode 1: y = T(re);  mode 2: y = T(re), y2 = T(im).
-template <typename T, int NT>
+template <typename T, int LOGN, int NT>
 __global__ void __launch_bounds__(NT)
 fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, const cpx* __restrict__ spec,
                 T* __restrict__ y, T* __restrict__ y2, size_t y_sb, size_t y_st, size_t y_sk, size_t y_sc,
-                const cpx* __restrict__ tw, int Tn, int d, int K, int n, int logn, int lcols, int mode, int xcd_remap) {
+                const cpx* __restrict__ tw, int Tn, int d, int K, int lcols, int mode, int xcd_remap) {
   extern __shared__ cpx fft_lds[];
+  constexpr int n = 1 << LOGN, colstride = col_stride<LOGN>();
   const int cols = 1 << lcols;
-  const int colstride = n + (n >> 4);
   int bx = blockIdx.x;
   if (xcd_remap) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);   // consecutive channel groups share an XCD
   const int c0 = bx * cols;
@@ -223,26 +279,20 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
   const T* xb = x + (size_t)b * x_sb + (size_t)c0 * x_sc;
   const bool t_fast = x_st == 1;   // time-major input: walk t with the lanes
 
-  for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
+  for (int idx = threadIdx.x; idx < (cols << LOGN); idx += NT) {
     int colid, t;
-    if (t_fast) { colid = idx >> logn; t = idx & (n - 1); } else { colid = idx & (cols - 1); t = idx >> lcols; }
+    if (t_fast) { colid = idx >> LOGN; t = idx & (n - 1); } else { colid = idx & (cols - 1); t = idx >> lcols; }
     float v = 0.f;
     if (t < Tn && colid < ncol) v = DT<T>::ld(xb + (size_t)t * x_st + (size_t)colid * x_sc);
     fft_lds[(size_t)colid * colstride + phys(t)] = make_float2(v, 0.f);
   }
   __syncthreads();
-  fft_forward<NT>(fft_lds, tw, cols, colstride, logn);
+  fft_forward<LOGN, NT, true>(fft_lds, tw, cols);
 
   const bool yt_fast = y_st == 1;
   if (K == 1) {
-    for (int idx = threadIdx.x; idx < (cols << logn); idx += NT) {
-      const int colid = idx >> logn, p = idx & (n - 1);
-      if (colid >= ncol) continue;
-      cpx* e = fft_lds + (size_t)colid * colstride + phys(p);
-      *e = cmul(*e, spec[(size_t)(c0 + colid) * n + p]);
-    }
-    __syncthreads();
-    fft_inverse<NT>(fft_lds, tw, cols, colstride, logn);
+    fft_middle<LOGN, NT>(fft_lds, spec, c0, ncol);
+    fft_inverse<LOGN, NT, true>(fft_lds, tw, cols);
     T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc;
     T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc : nullptr;
     for (int idx = threadIdx.x; idx < cols * Tn; idx += NT) {
@@ -260,27 +310,22 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
     return;
   }
 
-  // filter bank: keep the spectrum of the single column in registers and run one inverse per filter
-  constexpr int MAXE = 16;
-  cpx xs[MAXE];
-  const int ept = (n + NT - 1) / NT;   // host guarantees ept <= MAXE and cols == 1
-#pragma unroll
-  for (int j = 0; j < MAXE; ++j)
-    if (j < ept) {
-      const int p = threadIdx.x + j * NT;
-      xs[j] = (p < n) ? fft_lds[phys(p)] : make_float2(0.f, 0.f);
-    }
+  // filter bank (one column per workgroup, n <= 16 * NT): the thread keeps the spectrum of its 16 neighbouring
+  // positions in registers and runs, per filter, the product and the first inverse pass from them
+  const int u = threadIdx.x;
+  const bool act = u < (n >> 4);
+  cpx* p = fft_lds + 17 * (act ? u : 0);
+  cpx xs[16];
+  if (act) forward16(p, xs);
   __syncthreads();
   for (int k = 0; k < K; ++k) {
-    const cpx* sk = spec + (size_t)k * n;
-#pragma unroll
-    for (int j = 0; j < MAXE; ++j)
-      if (j < ept) {
-        const int p = threadIdx.x + j * NT;
-        if (p < n) fft_lds[phys(p)] = cmul(xs[j], sk[p]);
-      }
+    if (act) {
+      cpx s[16];
+      load_spec16(spec + ((size_t)k << LOGN) + 16 * u, s);
+      product_inverse16(p, xs, s);
+    }
     __syncthreads();
-    fft_inverse<NT>(fft_lds, tw, 1, colstride, logn);
+    fft_inverse<LOGN, NT, true>(fft_lds, tw, 1);
     T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk;
     T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk : nullptr;
     for (int t = threadIdx.x; t < Tn; t += NT) {
@@ -342,18 +387,27 @@ extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
   return FSTU_OK;
 }
 
-#define FFT_LAUNCH_NT(NTV, KERNEL, GRID, SHM, NAME, ...)                                             \
-  do {                                                                                               \
-    int rc__ = allow_lds(KERNEL<T, NTV>, SHM, NAME);                                                 \
-    if (rc__) return rc__;                                                                           \
-    hipLaunchKernelGGL((KERNEL<T, NTV>), GRID, dim3(NTV), SHM, (hipStream_t)stream, __VA_ARGS__);    \
+// threads per workgroup follow the transform length: one radix-16 butterfly per thread and pass for n >= 4096
+#define FFT_LAUNCH_ONE(LOGNV, NTV, KERNEL, GRID, SHM, NAME, ...)                                              \
+  do {                                                                                                        \
+    int rc__ = allow_lds(KERNEL<T, LOGNV, NTV>, SHM, NAME);                                                   \
+    if (rc__) return rc__;                                                                                    \
+    hipLaunchKernelGGL((KERNEL<T, LOGNV, NTV>), GRID, dim3(NTV), SHM, (hipStream_t)stream, __VA_ARGS__);      \
   } while (0)
 
-#define FFT_LAUNCH(NT, KERNEL, GRID, SHM, NAME, ...)                                  \
-  do {                                                                                \
-    if ((NT) == 1024) FFT_LAUNCH_NT(1024, KERNEL, GRID, SHM, NAME, __VA_ARGS__);      \
-    else if ((NT) == 512) FFT_LAUNCH_NT(512, KERNEL, GRID, SHM, NAME, __VA_ARGS__);   \
-    else FFT_LAUNCH_NT(256, KERNEL, GRID, SHM, NAME, __VA_ARGS__);                    \
+#define FFT_LAUNCH(LOGN, KERNEL, GRID, SHM, NAME, ...)                                  \
+  do {                                                                                  \
+    switch (LOGN) {                                                                     \
+      case 6: FFT_LAUNCH_ONE(6, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 7: FFT_LAUNCH_ONE(7, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 8: FFT_LAUNCH_ONE(8, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 9: FFT_LAUNCH_ONE(9, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 10: FFT_LAUNCH_ONE(10, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 11: FFT_LAUNCH_ONE(11, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 12: FFT_LAUNCH_ONE(12, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 13: FFT_LAUNCH_ONE(13, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      default: FFT_LAUNCH_ONE(14, 1024, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;   \
+    }                                                                                   \
   } while (0)
 
 extern "C" int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs, float* spec, const float* tw, int taps,
@@ -369,9 +423,8 @@ extern "C" int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs,
   const size_t shm = fft_lds_bytes(n, lcols);
   dim3 grid((ncols + (1 << lcols) - 1) >> lcols);
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_fft_filter",
-                      FFT_LAUNCH(nt, fft_filter_kernel, grid, shm, "fstu_stu_fft_filter", (const T*)filt, (size_t)f_ls,
-                                 (size_t)f_cs, (cpx*)spec, (const cpx*)tw, taps, ncols, n, logn, lcols,
-                                 single_branch ? 0 : 1));
+                      FFT_LAUNCH(logn, fft_filter_kernel, grid, shm, "fstu_stu_fft_filter", (const T*)filt, (size_t)f_ls,
+                                 (size_t)f_cs, (cpx*)spec, (const cpx*)tw, taps, ncols, lcols, single_branch ? 0 : 1));
   FSTU_CHECK_LAUNCH("fstu_stu_fft_filter");
   return FSTU_OK;
 }
@@ -387,15 +440,15 @@ static int conv_fft_launch(const char* name, const void* x, int64_t x_sb, int64_
   int lcols, nt;
   fft_shape(logn, d, &lcols, &nt);
   if (K > 1) lcols = 0;
-  FSTU_REQUIRE(K == 1 || (n + nt - 1) / nt <= 16, FSTU_ESHAPE, "%s: n=%d too long for the bank form", name, n);
+  (void)nt;   // n <= 16 * threads holds for every length: the bank form keeps 16 positions per thread
   const size_t shm = fft_lds_bytes(n, lcols);
   const int gx = (d + (1 << lcols) - 1) >> lcols;
   dim3 grid(gx, B);
   const int remap = (gx % 8 == 0) ? 1 : 0;
   FSTU_DISPATCH_DTYPE(dtype, name,
-                      FFT_LAUNCH(nt, fft_conv_kernel, grid, shm, name, (const T*)x, (size_t)x_sb, (size_t)x_st,
+                      FFT_LAUNCH(logn, fft_conv_kernel, grid, shm, name, (const T*)x, (size_t)x_sb, (size_t)x_st,
                                  (size_t)x_sc, (const cpx*)spec, (T*)y, (T*)y2, (size_t)y_sb, (size_t)y_st, (size_t)y_sk,
-                                 (size_t)y_sc, (const cpx*)tw, T_, d, K, n, logn, lcols, mode, remap));
+                                 (size_t)y_sc, (const cpx*)tw, T_, d, K, lcols, mode, remap));
   FSTU_CHECK_LAUNCH(name);
   return FSTU_OK;
 }
