@@ -50,6 +50,9 @@ int fstu_embed_rmsnorm(const int64_t* ids, int64_t id_stride, const void* table,
 int fstu_sample_dyn(const void* logits, int64_t* out, int64_t out_stride, int B, int V, float temperature, int top_k,
                     float top_p, int do_sample, uint64_t seed, int step, int row0, const int* dyn, int dtype, void* stream);
 int fstu_advance_dyn(int* dyn, void* stream);
+bool fstu_linear_rows32_ok(const void* x, int ldx, const void* W, int K, int dtype);
+int fstu_linear_rows32(const void* x, int ldx, const void* W, void* y, int ldy, int rows, int N, int K, float temperature,
+                       void* best_ws /*NULL: plain projection; else the head's packed maxima, rows*64 words*/, void* stream);
 bool fstu_sample_topk_ok(int B, int V, int top_k, int dtype);
 int fstu_sample_topk_dyn(const void* logits, int64_t ldl, void* best_ws, void* samp_ws, int64_t* out, int64_t out_stride, int B,
                          int V, float temperature, int top_k, float top_p, uint64_t seed, int step, int row0, int* dyn,

@@ -162,21 +162,28 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
   const size_t esz = 2;
   auto rows_of = [&](int c) { return c == 0 ? R : B - R; };
   auto at = [&](void* p, int c, size_t per_row) { return (void*)((char*)p + (size_t)c * R * per_row * esz); };
+  // y = x W^T over all rows: one launch with two row tiles per weight fragment where the operands allow it, else the
+  // 16-row kernel on the two halves of the rows in turn
+  auto proj = [&](void* x, int ldx, const void* W, void* y, int ldy, int N, int K) -> int {
+    if (fstu_linear_rows32_ok(x, ldx, W, K, dt)) return fstu_linear_rows32(x, ldx, W, y, ldy, B, N, K, 1.0f, nullptr, stream);
+    for (int c = 0; c < 2; ++c) {
+      int rc = fstu_linear_decode(at(x, c, ldx), ldx, W, at(y, c, ldy), ldy, rows_of(c), N, K, dt, stream);
+      if (rc) return rc;
+    }
+    return FSTU_OK;
+  };
   TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt, stream, dyn));
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
     if (L.kind == 0) {
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
-      for (int c = 0; c < 2; ++c)
-        TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.m_inputs_t, at(m->xp, c, d), d, rows_of(c), d, d, dt, stream));
+      TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
       TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream));
     } else {
-      for (int c = 0; c < 2; ++c)
-        TIMED(PC_PROJ, fstu_linear_decode(at(m->h, c, d), d, L.w_qkv, at(m->qkv, c, 3 * (size_t)d), 3 * d, rows_of(c), 3 * d, d, dt, stream));
+      TIMED(PC_PROJ, proj(m->h, d, L.w_qkv, m->qkv, 3 * d, 3 * d, d));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
                                          m->window, m->softcap, 1, dyn, dt, stream));
-      for (int c = 0; c < 2; ++c)
-        TIMED(PC_PROJ, fstu_linear_decode(at(m->attn, c, d), d, L.w_proj, at(m->y, c, d), d, rows_of(c), d, d, dt, stream));
+      TIMED(PC_PROJ, proj(m->attn, d, L.w_proj, m->y, d, d, d));
     }
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
     TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
@@ -186,15 +193,17 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
   }
   if (sample_spread_ok(m, do_sample, top_k)) {
     // the head leaves each row's packed maxima, the sampler spreads every row over the chip and advances {pos, step}
-    for (int c = 0; c < 2; ++c)
-      TIMED(PC_HEAD, fstu_head_maxima(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, temperature,
-                                      (char*)m->best + (size_t)c * R * 64 * 8, dt, stream));
+    if (fstu_linear_rows32_ok(m->h, d, m->emb, d, dt))
+      TIMED(PC_HEAD, fstu_linear_rows32(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, stream));
+    else
+      for (int c = 0; c < 2; ++c)
+        TIMED(PC_HEAD, fstu_head_maxima(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, temperature,
+                                        (char*)m->best + (size_t)c * R * 64 * 8, dt, stream));
     TIMED(PC_SAMPLE, fstu_sample_topk_dyn(m->logits, m->V, m->best, m->samp_ws, tok_out, tok_stride, B, m->V, temperature, top_k, top_p,
                                           seed, step, m->row0, dyn, 1, stream));
     return FSTU_OK;
   }
-  for (int c = 0; c < 2; ++c)
-    TIMED(PC_HEAD, fstu_linear_decode(at(m->h, c, d), d, m->emb, at(m->logits, c, (size_t)m->V), m->V, rows_of(c), m->V, d, dt, stream));
+  TIMED(PC_HEAD, proj(m->h, d, m->emb, m->logits, m->V, m->V, d));
   TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, B, m->V, temperature, top_k, top_p, do_sample, seed, step, m->row0,
                                    dyn, dt, stream));
   if (dyn) STEP(fstu_advance_dyn(dyn, stream));

@@ -37,14 +37,17 @@ struct LinArgs {
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
 
 // The arguments are passed one by one (not as a struct) so that the command processor can preload them into SGPRs.
-template <int KSW, int MODE>
+// NB = 2: rows 16..31 are a second B tile of the same weight fragments, so 17..32 rows read every weight once.
+template <int KSW, int MODE, int NB = 1>
 __global__ void __launch_bounds__(256)
 linear_mfma_bf16_kernel(const void* x, const void* W, const void* W2, void* y, unsigned long long* best, int ldx, int ldy,
                         int rows, int N, int K, int kw, float temperature) {
+  static_assert(NB == 1 || MODE == LIN_PLAIN || MODE == LIN_ARGMAX, "two row tiles: plain and head launches only");
   const LinArgs a{x, ldx, W, W2, y, ldy, rows, N, K, kw, best, temperature};
   constexpr int RT = 4 / KSW;
   constexpr int U = 4;  // k steps (of 64) whose loads are issued back to back
-  __shared__ float red[(KSW > 1) ? 4 * 64 * 4 * ((MODE == LIN_GLU) ? 2 : 1) : 1];
+  constexpr int NACC = (MODE == LIN_GLU) ? 2 : NB;   // accumulators per lane: gate + up, or one per row tile
+  __shared__ float red[(KSW > 1) ? 4 * 64 * 4 * NACC : 1];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int rt = w / KSW, ks = w % KSW;
   const int tile = blockIdx.x * RT + rt;
@@ -55,13 +58,20 @@ linear_mfma_bf16_kernel(const void* x, const void* W, const void* W2, void* y, u
   const int k0 = (blockIdx.y * KSW + ks) * a.kw + g * 16;
   const bf16_t* wp = (const bf16_t*)a.W + (size_t)max(n, 0) * a.K + k0;
   const bf16_t* wp2 = (MODE == LIN_GLU) ? (const bf16_t*)a.W2 + (size_t)max(n, 0) * a.K + k0 : nullptr;
-  const bool xrow = r < a.rows;
-  const bf16_t* xp = (const bf16_t*)a.x + (size_t)(xrow ? r : 0) * a.ldx + k0;
-  floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  bool xrow[NB];
+  const bf16_t* xp[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    xrow[j] = 16 * j + r < a.rows;
+    xp[j] = (const bf16_t*)a.x + (size_t)(xrow[j] ? 16 * j + r : 0) * a.ldx + k0;
+  }
+  floatx4_t acc[NACC];
+#pragma unroll
+  for (int j = 0; j < NACC; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
   const int iters = a.kw >> 6;
   if (tile_ok) {
     for (int i0 = 0; i0 < iters; i0 += U) {
-      uint4 wa[U][2], wb[U][2], xa[U][2];
+      uint4 wa[U][2], wb[U][2], xa[NB][U][2];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (i0 + u < iters) {
@@ -73,24 +83,30 @@ linear_mfma_bf16_kernel(const void* x, const void* W, const void* W2, void* y, u
             wb[u][0] = p2[0];
             wb[u][1] = p2[1];
           }
-          if (xrow) {
-            const uint4* q = (const uint4*)(xp + (size_t)(i0 + u) * 64);
-            xa[u][0] = q[0];
-            xa[u][1] = q[1];
-          } else {
-            xa[u][0] = make_uint4(0, 0, 0, 0);
-            xa[u][1] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            if (xrow[j]) {
+              const uint4* q = (const uint4*)(xp[j] + (size_t)(i0 + u) * 64);
+              xa[j][u][0] = q[0];
+              xa[j][u][1] = q[1];
+            } else {
+              xa[j][u][0] = make_uint4(0, 0, 0, 0);
+              xa[j][u][1] = make_uint4(0, 0, 0, 0);
+            }
           }
         }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (i0 + u < iters) {
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][0]), as_bf16x8(xa[u][0]), acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][1]), as_bf16x8(xa[u][1]), acc, 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][0]), as_bf16x8(xa[j][u][0]), acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[u][1]), as_bf16x8(xa[j][u][1]), acc[j], 0, 0, 0);
+          }
           if (MODE == LIN_GLU) {
-            acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][0]), as_bf16x8(xa[u][0]), acc2, 0, 0, 0);
-            acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][1]), as_bf16x8(xa[u][1]), acc2, 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][0]), as_bf16x8(xa[0][u][0]), acc[1], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[u][1]), as_bf16x8(xa[0][u][1]), acc[1], 0, 0, 0);
           }
         }
       }
@@ -98,63 +114,68 @@ linear_mfma_bf16_kernel(const void* x, const void* W, const void* W2, void* y, u
   }
   if (KSW > 1) {
     float* mine = red + (size_t)(w * 64 + lane) * 4;
-    constexpr int GLU_OFF = 4 * 64 * 4;
+    constexpr int OFF = 4 * 64 * 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mine[i] = acc[i];
-      if (MODE == LIN_GLU) mine[GLU_OFF + i] = acc2[i];
-    }
+    for (int j = 0; j < NACC; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[j * OFF + i] = acc[j][i];
     __syncthreads();
     if (ks != 0) return;
 #pragma unroll
     for (int s = 1; s < KSW; ++s) {
       const float* o = red + (size_t)((w + s) * 64 + lane) * 4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[i] += o[i];
-        if (MODE == LIN_GLU) acc2[i] += o[GLU_OFF + i];
-      }
+      for (int j = 0; j < NACC; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] += o[j * OFF + i];
     }
   }
   if (MODE == LIN_ARGMAX) {
     // per batch row: best (value, lowest index) over this wave's 16 features, then one 64-bit atomic max
-    unsigned long long key = 0ull;
-    if (tile_ok && r < a.rows) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int f = tile * 16 + g * 4 + i;
-        if (f < a.N) {
-          float l = DT<bf16_t>::rnd(acc[i]);
-          if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
-          l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
-          unsigned u = __float_as_uint(l);
-          u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-          unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
-          key = k > key ? k : key;
+    for (int j = 0; j < NB; ++j) {
+      const int b = 16 * j + r;
+      unsigned long long key = 0ull;
+      if (tile_ok && b < a.rows) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int f = tile * 16 + g * 4 + i;
+          if (f < a.N) {
+            float l = DT<bf16_t>::rnd(acc[j][i]);
+            if (a.temperature != 1.0f) l = DT<bf16_t>::rnd(l / a.temperature);
+            l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
+            unsigned u = __float_as_uint(l);
+            u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+            unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)f);
+            key = k > key ? k : key;
+          }
         }
       }
+      unsigned long long o = __shfl_xor(key, 16, FSTU_WAVE);
+      key = o > key ? o : key;
+      o = __shfl_xor(key, 32, FSTU_WAVE);
+      key = o > key ? o : key;
+      if (tile_ok && g == 0 && b < a.rows && key != 0ull) atomicMax(a.best + (size_t)b * 64 + (tile & 63), key);  // 64 slots per row spread the contention
     }
-    unsigned long long o = __shfl_xor(key, 16, FSTU_WAVE);
-    key = o > key ? o : key;
-    o = __shfl_xor(key, 32, FSTU_WAVE);
-    key = o > key ? o : key;
-    if (tile_ok && g == 0 && r < a.rows && key != 0ull) atomicMax(a.best + (size_t)r * 64 + (tile & 63), key);  // 64 slots per row spread the contention
   }
   if (!tile_ok) return;
-  // D layout: lane holds features 4*(lane/16)+i, batch row lane%16
-  const int b = r;
-  if (b >= a.rows) return;
+  // D layout: lane holds features 4*(lane/16)+i, batch row lane%16 (of its row tile)
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int f = tile * 16 + g * 4 + i;
-    if (f >= a.N) continue;
-    if (MODE == LIN_PLAIN || MODE == LIN_ARGMAX) {
-      ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(acc[i]);
-    } else if (MODE == LIN_GLU) {
-      float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[i])));
-      ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(ge * DT<bf16_t>::rnd(acc2[i]));
-    } else {
-      ((float*)a.y)[((size_t)blockIdx.y * a.rows + b) * a.N + f] = acc[i];
+  for (int j = 0; j < NB; ++j) {
+    const int b = 16 * j + r;
+    if (b >= a.rows) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int f = tile * 16 + g * 4 + i;
+      if (f >= a.N) continue;
+      if (MODE == LIN_PLAIN || MODE == LIN_ARGMAX) {
+        ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(acc[j][i]);
+      } else if (MODE == LIN_GLU) {
+        float ge = DT<bf16_t>::rnd(gelu_tanh_f32(DT<bf16_t>::rnd(acc[0][i])));
+        ((bf16_t*)a.y)[(size_t)b * a.ldy + f] = f32_to_bf16(ge * DT<bf16_t>::rnd(acc[1][i]));
+      } else {
+        ((float*)a.y)[((size_t)blockIdx.y * a.rows + b) * a.N + f] = acc[j][i];
+      }
     }
   }
 }
@@ -227,7 +248,7 @@ static int pick_ksw(int N, int kper) {
   return 1;
 }
 
-template <int MODE>
+template <int MODE, int NB = 1>
 static int launch_mfma(LinArgs a, int ksplit, hipStream_t s) {
   int kper = a.K / ksplit;
   int ksw = pick_ksw(a.N, kper);
@@ -235,10 +256,29 @@ static int launch_mfma(LinArgs a, int ksplit, hipStream_t s) {
   int tiles = (a.N + 15) / 16;
   int rt = 4 / ksw;
   dim3 grid((tiles + rt - 1) / rt, ksplit);
-  if (ksw == 4) hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
-  else if (ksw == 2) hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
-  else hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, MODE>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
+  if (ksw == 4) hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, MODE, NB>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
+  else if (ksw == 2) hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, MODE, NB>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
+  else hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, MODE, NB>), grid, dim3(256), 0, s, a.x, a.W, a.W2, a.y, a.best, a.ldx, a.ldy, a.rows, a.N, a.K, a.kw, a.temperature);
   return 0;
+}
+
+// 17..32 rows (bf16, K % 64 == 0, 16-byte aligned rows): the plain projection and the head with its packed maxima,
+// every weight read once.  Used by the one-call step for batches beyond FSTU_MAX_DECODE_ROWS.
+bool fstu_linear_rows32_ok(const void* x, int ldx, const void* W, int K, int dtype) {
+  return dtype == FSTU_BF16 && mfma_ok(x, ldx, W, nullptr, K, 1);
+}
+
+int fstu_linear_rows32(const void* x, int ldx, const void* W, void* y, int ldy, int rows, int N, int K, float temperature,
+                       void* best_ws, void* stream) {
+  FSTU_REQUIRE(x && W && y, FSTU_ENULL, "fstu_linear_rows32: null pointer");
+  FSTU_REQUIRE(rows > FSTU_MAX_DECODE_ROWS && rows <= 2 * FSTU_MAX_DECODE_ROWS && N >= 1 && ldx >= K && ldy >= N, FSTU_ESHAPE,
+               "fstu_linear_rows32: rows=%d N=%d K=%d ldx=%d ldy=%d", rows, N, K, ldx, ldy);
+  FSTU_REQUIRE(mfma_ok(x, ldx, W, nullptr, K, 1), FSTU_ESHAPE, "fstu_linear_rows32: needs K %% 64 == 0 and 16-byte aligned rows");
+  LinArgs a{x, ldx, W, nullptr, y, ldy, rows, N, K, K, (unsigned long long*)best_ws, temperature};
+  if (best_ws) launch_mfma<LIN_ARGMAX, 2>(a, 1, (hipStream_t)stream);
+  else launch_mfma<LIN_PLAIN, 2>(a, 1, (hipStream_t)stream);
+  FSTU_CHECK_LAUNCH("fstu_linear_rows32");
+  return FSTU_OK;
 }
 
 template <typename T, int MODE>
