@@ -341,6 +341,121 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
   }
 }
 
+// ---------------------------------------------------------------- convolution, whole 16-byte row pieces per lane
+// The same computation for channel-contiguous (B, T, d) operands with d a multiple of the workgroup's channel count:
+// a workgroup owns CHW = max(COLS, 16 bytes' worth) neighbouring channels, reads them as 16-byte pieces of the rows
+// (all loads in flight at once, kept in registers), transforms COLS of them at a time in LDS, collects the results in
+// registers and writes 16-byte pieces of the output rows.  Global accesses are 8 (bf16) or 4 (fp32) channels wide
+// instead of COLS; for the long transforms (COLS = 1) that is the difference between 2-byte and 16-byte accesses.
+template <typename T> struct RowVec;
+template <> struct RowVec<bf16_t> {
+  static constexpr int CH = 8;
+  template <int E> static __device__ __forceinline__ float get(const unsigned (&w)[4]) {
+    return __uint_as_float((E & 1) ? (w[E >> 1] & 0xffff0000u) : (w[E >> 1] << 16));
+  }
+  template <int E> static __device__ __forceinline__ void put(unsigned (&w)[4], float v) {
+    const unsigned h = f32_to_bf16(v);
+    w[E >> 1] = (E & 1) ? ((w[E >> 1] & 0x0000ffffu) | (h << 16)) : ((w[E >> 1] & 0xffff0000u) | h);
+  }
+};
+template <> struct RowVec<float> {
+  static constexpr int CH = 4;
+  template <int E> static __device__ __forceinline__ float get(const unsigned (&w)[4]) { return __uint_as_float(w[E]); }
+  template <int E> static __device__ __forceinline__ void put(unsigned (&w)[4], float v) { w[E] = __float_as_uint(v); }
+};
+
+// columns in LDS at a time: as many as 34 KB hold (at most 16); n = 4096 takes two with twice the threads (measured
+// 14 % faster than one), n = 8192 one (two with 1024 threads spill registers and were 12 % slower)
+template <int LOGN> __host__ __device__ constexpr int fft_lcols() { return LOGN >= 13 ? 0 : LOGN == 12 ? 1 : (12 - LOGN > 4 ? 4 : 12 - LOGN); }
+
+template <typename T, int LOGN, int NT, int G, int E>
+__device__ __forceinline__ void rows_scatter(cpx* lds, const unsigned (&w)[4], int t, int part) {
+  constexpr int COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, VR = (COLS > CH ? COLS : CH) / CH;
+  if constexpr (E < CH) {
+    // VR == 1: the column is known at compile time; VR > 1 (one group): it follows the row piece
+    if constexpr (VR == 1) {
+      constexpr int col = E - G * COLS;
+      if constexpr (col >= 0 && col < COLS) lds[(size_t)col * col_stride<LOGN>() + phys(t)] = make_float2(RowVec<T>::template get<E>(w), 0.f);
+    } else {
+      lds[(size_t)(part * CH + E) * col_stride<LOGN>() + phys(t)] = make_float2(RowVec<T>::template get<E>(w), 0.f);
+    }
+    rows_scatter<T, LOGN, NT, G, E + 1>(lds, w, t, part);
+  }
+}
+
+template <typename T, int LOGN, int NT, int G, int E>
+__device__ __forceinline__ void rows_gather(const cpx* lds, unsigned (&w)[4], int t, int part, int mode) {
+  constexpr int COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, VR = (COLS > CH ? COLS : CH) / CH;
+  if constexpr (E < CH) {
+    constexpr int col_ct = E - G * COLS;
+    if constexpr (VR > 1 || (col_ct >= 0 && col_ct < COLS)) {
+      const int col = VR > 1 ? part * CH + E : col_ct;
+      const cpx z = lds[(size_t)col * col_stride<LOGN>() + phys(t)];
+      RowVec<T>::template put<E>(w, mode == 0 ? DT<T>::rnd(z.x) + DT<T>::rnd(z.y) : z.x);
+    }
+    rows_gather<T, LOGN, NT, G, E + 1>(lds, w, t, part, mode);
+  }
+}
+
+template <typename T, int LOGN, int NT, int NV, int G>
+__device__ __forceinline__ void rows_groups(cpx* lds, const cpx* __restrict__ spec, const cpx* __restrict__ tw,
+                                            unsigned (&io)[NV][4], int Tn, int c0, int mode) {
+  constexpr int n = 1 << LOGN, COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, CHW = COLS > CH ? COLS : CH;
+  constexpr int VR = CHW / CH, NG = CHW / COLS;
+  if constexpr (G < NG) {
+    if (G > 0) __syncthreads();   // the previous group's results have been collected
+#pragma unroll
+    for (int r = 0; r < NV; ++r) {
+      const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
+      if (t < Tn) rows_scatter<T, LOGN, NT, G, 0>(lds, io[r], t, part);
+    }
+    // zero padding behind the sequence
+    for (int idx = threadIdx.x; idx < COLS * (n - Tn); idx += NT) {
+      const int col = idx / (n - Tn), t = Tn + idx - col * (n - Tn);
+      lds[(size_t)col * col_stride<LOGN>() + phys(t)] = make_float2(0.f, 0.f);
+    }
+    __syncthreads();
+    fft_forward<LOGN, NT, true>(lds, tw, COLS);
+    fft_middle<LOGN, NT>(lds, spec, c0 + G * COLS, COLS);
+    fft_inverse<LOGN, NT, true>(lds, tw, COLS);
+#pragma unroll
+    for (int r = 0; r < NV; ++r) {
+      const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
+      if (t < Tn) rows_gather<T, LOGN, NT, G, 0>(lds, io[r], t, part, mode);   // over the inputs this group consumed
+    }
+    rows_groups<T, LOGN, NT, NV, G + 1>(lds, spec, tw, io, Tn, c0, mode);
+  }
+}
+
+template <typename T, int LOGN, int NT>
+__global__ void __launch_bounds__(NT)
+fft_conv_rows_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, const cpx* __restrict__ spec, T* __restrict__ y,
+                     size_t y_sb, size_t y_st, const cpx* __restrict__ tw, int Tn, int mode, int xcd_remap) {
+  extern __shared__ cpx fft_lds[];
+  constexpr int n = 1 << LOGN, COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, CHW = COLS > CH ? COLS : CH;
+  constexpr int VR = CHW / CH, NV = ((n / 2) * VR + NT - 1) / NT;
+  int bx = blockIdx.x;
+  if (xcd_remap) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);   // consecutive channel groups share an XCD
+  const int c0 = bx * CHW, b = blockIdx.y;
+  const T* xb = x + (size_t)b * x_sb + c0;
+  // the row pieces: inputs at first, each channel's result written over its input once its group is through
+  unsigned io[NV][4];
+#pragma unroll
+  for (int r = 0; r < NV; ++r) {
+    const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
+    // rows behind the sequence re-read its last row (no branch around the load) and are never used
+    const uint4 v = *(const uint4*)(xb + (size_t)min(t, Tn - 1) * x_st + part * CH);
+    io[r][0] = v.x; io[r][1] = v.y; io[r][2] = v.z; io[r][3] = v.w;
+  }
+  rows_groups<T, LOGN, NT, NV, 0>(fft_lds, spec, tw, io, Tn, c0, mode);
+  T* yb = y + (size_t)b * y_sb + c0;
+#pragma unroll
+  for (int r = 0; r < NV; ++r) {
+    const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
+    if (t < Tn) *(uint4*)(yb + (size_t)t * y_st + part * CH) = make_uint4(io[r][0], io[r][1], io[r][2], io[r][3]);
+  }
+}
+
 int ilog2_exact(int n) {
   int l = 0;
   while ((1 << l) < n) ++l;
@@ -410,6 +525,20 @@ extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
     }                                                                                   \
   } while (0)
 
+#define FFT_LAUNCH_ROWS(LOGN, KERNEL, GRID, SHM, NAME, ...)                              \
+  do {                                                                                  \
+    switch (LOGN) {                                                                     \
+      case 6: FFT_LAUNCH_ONE(6, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 7: FFT_LAUNCH_ONE(7, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 8: FFT_LAUNCH_ONE(8, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 9: FFT_LAUNCH_ONE(9, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;      \
+      case 10: FFT_LAUNCH_ONE(10, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 11: FFT_LAUNCH_ONE(11, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 12: FFT_LAUNCH_ONE(12, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      default: FFT_LAUNCH_ONE(13, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+    }                                                                                   \
+  } while (0)
+
 extern "C" int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs, float* spec, const float* tw, int taps,
                                    int ncols, int n, int single_branch, int dtype, void* stream) {
   FSTU_REQUIRE(filt && spec && tw, FSTU_ENULL, "fstu_stu_fft_filter: null pointer");
@@ -440,6 +569,24 @@ static int conv_fft_launch(const char* name, const void* x, int64_t x_sb, int64_
   int lcols, nt;
   fft_shape(logn, d, &lcols, &nt);
   if (K > 1) lcols = 0;
+  {
+    // channel-contiguous operands whose rows split into whole 16-byte pieces per workgroup: the row-piece kernel
+    const int rows_lcols = logn >= 13 ? 0 : logn == 12 ? 1 : (12 - logn > 4 ? 4 : 12 - logn);
+    const int esz = dtype == FSTU_BF16 ? 2 : 4, ch = 16 / esz, cols_full = 1 << rows_lcols;
+    const int chw = cols_full > ch ? cols_full : ch;
+    if (K == 1 && mode != 2 && logn <= 13 && x_sc == 1 && y_sc == 1 && d % chw == 0 && x_st % ch == 0 && y_st % ch == 0 &&
+        x_sb % ch == 0 && y_sb % ch == 0 && fstu_aligned(x, 16) && fstu_aligned(y, 16)) {
+      const size_t shm = fft_lds_bytes(n, rows_lcols);
+      const int gx = d / chw;
+      dim3 grid(gx, B);
+      const int remap = (gx % 8 == 0) ? 1 : 0;
+      FSTU_DISPATCH_DTYPE(dtype, name,
+                          FFT_LAUNCH_ROWS(logn, fft_conv_rows_kernel, grid, shm, name, (const T*)x, (size_t)x_sb, (size_t)x_st,
+                                          (const cpx*)spec, (T*)y, (size_t)y_sb, (size_t)y_st, (const cpx*)tw, T_, mode, remap));
+      FSTU_CHECK_LAUNCH(name);
+      return FSTU_OK;
+    }
+  }
   (void)nt;   // n <= 16 * threads holds for every length: the bank form keeps 16 positions per thread
   const size_t shm = fft_lds_bytes(n, lcols);
   const int gx = (d + (1 << lcols) - 1) >> lcols;
