@@ -134,25 +134,6 @@ template <> struct Ring4<bf16_t> {
     *(uint2*)p = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
   }
 };
-template <typename T>
-__device__ __forceinline__ void fir_head(const T* __restrict__ ring, const float* __restrict__ fir, int R, int tt, int b, int c,
-                                         int d, int g, const float (&x)[4], float (&f)[4]) {
-  const T* rb = ring + (size_t)b * R * d + c;
-  // (all 16 lags of a thread in flight at once was measured slower than four at a time: 0.354 against 0.336 ms per
-  // step at 128 taps)
-#pragma unroll 4
-  for (int s = g; s < R; s += 8) {
-    float xv[4];
-    const int p = tt - s;
-    // a position before the sequence contributes nothing; its slot is read all the same (no branch around the load)
-    Ring4<T>::ld(rb + (size_t)(p & (R - 1)) * d, xv);
-    const float m = (s > 0 && p >= 0) ? 1.f : 0.f;
-    const float4 rv = *(const float4*)(fir + (size_t)s * d + c);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = fmaf(i == 0 ? rv.x : i == 1 ? rv.y : i == 2 ? rv.z : rv.w, s == 0 ? x[i] : m * xv[i], f[i]);
-  }
-}
-
 // ---------------------------------------------------------------- LDS-form step
 // Workgroup = 32 channel quads (128 channels) x 8 mode groups.  Each thread
 // advances S/8 modes of 4 channels (float4 state accesses, 512 contiguous
@@ -176,12 +157,60 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
   const bool ok = c < d;
   float acc[4] = {0.f, 0.f, 0.f, 0.f}, acco[4] = {0.f, 0.f, 0.f, 0.f};
   if (ok) {
+    // Every operand of the thread's first 8 modes of both banks and first 8 lags of the head goes in flight before
+    // anything waits (out-of-range modes and lags re-read a valid element and are ignored): one trip to memory for
+    // S <= 64 and 64 taps; longer states and heads continue in loops.
+    constexpr int PJ = 8;
+    float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
+    const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
+    const bool head = co && fir;
+    const T* rb = head ? ring + (size_t)b * R * d + c : nullptr;
+    float4 ph[PJ], pc[PJ], qh[PJ], qc[PJ], fr[PJ];
+    float pa[PJ], rx[PJ][4];
+#pragma unroll
+    for (int k = 0; k < PJ; ++k) {
+      const int j = min(jg + LDS_JG * k, S - 1);
+      ph[k] = *(const float4*)(st + (size_t)j * d);
+      pc[k] = *(const float4*)(ce + (size_t)j * d + c);
+      pa[k] = a[j];
+    }
+    if (co) {
+#pragma unroll
+      for (int k = 0; k < PJ; ++k) {
+        const int j = min(jg + LDS_JG * k, S - 1);
+        qh[k] = *(const float4*)(so + (size_t)j * d);
+        qc[k] = *(const float4*)(co + (size_t)j * d + c);
+      }
+    }
+    if (head) {
+#pragma unroll
+      for (int k = 0; k < PJ; ++k) {
+        const int sl = min(jg + 8 * k, R - 1);
+        Ring4<T>::ld(rb + (size_t)((t - sl) & (R - 1)) * d, rx[k]);
+        fr[k] = *(const float4*)(fir + (size_t)sl * d + c);
+      }
+    }
     float x[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) x[v] = DT<T>::ld(xp + (size_t)b * ldxp + c + v);
-    float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
+#pragma unroll
+    for (int k = 0; k < PJ; ++k) {
+      const int j = jg + LDS_JG * k;
+      if (j < S) {
+        float4 h = ph[k];
+        h.x = fmaf(pa[k], h.x, x[0]);
+        h.y = fmaf(pa[k], h.y, x[1]);
+        h.z = fmaf(pa[k], h.z, x[2]);
+        h.w = fmaf(pa[k], h.w, x[3]);
+        *(float4*)(st + (size_t)j * d) = h;
+        acc[0] = fmaf(pc[k].x, h.x, acc[0]);
+        acc[1] = fmaf(pc[k].y, h.y, acc[1]);
+        acc[2] = fmaf(pc[k].z, h.z, acc[2]);
+        acc[3] = fmaf(pc[k].w, h.w, acc[3]);
+      }
+    }
 #pragma unroll 4
-    for (int j = jg; j < S; j += LDS_JG) {
+    for (int j = jg + LDS_JG * PJ; j < S; j += LDS_JG) {
       float4 h = *(float4*)(st + (size_t)j * d);
       const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
       const float aj = a[j];
@@ -197,9 +226,17 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
     }
     if (co) {
       // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (not advanced here)
-      const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
+#pragma unroll
+      for (int k = 0; k < PJ; ++k) {
+        if (jg + LDS_JG * k < S) {
+          acco[0] = fmaf(qc[k].x, qh[k].x, acco[0]);
+          acco[1] = fmaf(qc[k].y, qh[k].y, acco[1]);
+          acco[2] = fmaf(qc[k].z, qh[k].z, acco[2]);
+          acco[3] = fmaf(qc[k].w, qh[k].w, acco[3]);
+        }
+      }
 #pragma unroll 4
-      for (int j = jg; j < S; j += LDS_JG) {
+      for (int j = jg + LDS_JG * PJ; j < S; j += LDS_JG) {
         const float4 h = *(const float4*)(so + (size_t)j * d);
         const float4 oj = *(const float4*)(co + (size_t)j * d + c);
         acco[0] = fmaf(oj.x, h.x, acco[0]);
@@ -208,8 +245,30 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
         acco[3] = fmaf(oj.w, h.w, acco[3]);
       }
       if (fir) {
+        // exact head: lags jg, jg+8, ... share the parity of jg; a position before the sequence contributes nothing
         float f[4] = {0.f, 0.f, 0.f, 0.f};
-        fir_head<T>(ring, fir, R, t, b, c, d, jg, x, f);
+#pragma unroll
+        for (int k = 0; k < PJ; ++k) {
+          const int sl = jg + 8 * k;
+          if (sl < R) {
+            const float m = (t - sl >= 0) ? 1.f : 0.f;
+            f[0] = fmaf(fr[k].x, sl == 0 ? x[0] : m * rx[k][0], f[0]);
+            f[1] = fmaf(fr[k].y, sl == 0 ? x[1] : m * rx[k][1], f[1]);
+            f[2] = fmaf(fr[k].z, sl == 0 ? x[2] : m * rx[k][2], f[2]);
+            f[3] = fmaf(fr[k].w, sl == 0 ? x[3] : m * rx[k][3], f[3]);
+          }
+        }
+#pragma unroll 4
+        for (int sl = jg + 8 * PJ; sl < R; sl += 8) {
+          float xv[4];
+          Ring4<T>::ld(rb + (size_t)((t - sl) & (R - 1)) * d, xv);
+          const float m = (t - sl >= 0) ? 1.f : 0.f;
+          const float4 rv = *(const float4*)(fir + (size_t)sl * d + c);
+          f[0] = fmaf(rv.x, m * xv[0], f[0]);
+          f[1] = fmaf(rv.y, m * xv[1], f[1]);
+          f[2] = fmaf(rv.z, m * xv[2], f[2]);
+          f[3] = fmaf(rv.w, m * xv[3], f[3]);
+        }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           if (jg & 1) acco[v] += f[v]; else acc[v] += f[v];
