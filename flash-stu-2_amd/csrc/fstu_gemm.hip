@@ -317,6 +317,7 @@ using TileBig = GemmTile<4, 2, 2, 4, 64, 2>;     // 256 x 256, 8 waves, 128 KB o
 using TileSmall = GemmTile<2, 2, 2, 2, 64, 2>;   // 128 x 128, 4 waves, 64 KB: two workgroups per compute unit
 using TileDeep = GemmTile<2, 2, 2, 2, 64, 4>;    // 128 x 128, 4 waves, 3 tiles in flight: one workgroup per compute unit
 using TileRows32 = GemmTile<2, 1, 2, 1, 64, 4>;  // 128 features x 32 rows, 2 waves, 80 KB: weight streaming, two workgroups per compute unit
+using Tile96 = GemmTile<1, 4, 3, 1, 64, 4>;      // 96 features x 128 rows, 4 waves, 112 KB: N = 768 or 2304 in whole tiles
 using TileK32 = GemmTile<2, 2, 4, 2, 32, 3>;     // 256 x 128, 4 waves, 72 KB, k tiles of 32 for K % 64 != 0
 
 template <int MODE>
@@ -332,6 +333,14 @@ int gemm_launch(const void* A, long long lda, const void* W, const void* W2, con
   const long long big = (long long)((M + 255) / 256) * ((N * nf + 255) / 256);
   const long long small = (long long)((M + 127) / 128) * ((N * nf + 127) / 128);
   if (K >= 1024 && big >= 2 * gemm_cus()) return gemm_launch_tile<TileBig, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  if constexpr (MODE != 1) {
+    // A feature count that is a whole number of 96-wide tiles but leaves compute units idle (or nearly idle in a last
+    // round) with 128-wide ones: the time follows the rounds a compute unit runs times the area of a tile
+    // (N = 768, M = 4096: 192 tiles of 128 x 128 on 256 CUs against 256 tiles of 96 x 128).
+    const long long cus = gemm_cus(), t96 = (long long)((M + 127) / 128) * (N / 96);
+    if (N % 96 == 0 && ((t96 + cus - 1) / cus) * 96 < ((small + cus - 1) / cus) * 128)
+      return gemm_launch_tile<Tile96, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
+  }
   if (K >= 2048 && small <= gemm_cus()) return gemm_launch_tile<TileDeep, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
   return gemm_launch_tile<TileSmall, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
 }

@@ -124,7 +124,7 @@ def test_mlp_decode_chain(hip, dtype, rows, d, I):
 # Prompt-pass GEMM kernel: the three tile shapes (128 x 128; 256 x 256 for K >= 1024 on grids that cover the chip
 # twice; k tiles of 32 for K % 64 != 0), ragged M and N, one- and many-tile grids.
 GEMM_SHAPES = [(4096, 2304, 768), (512, 768, 768), (1000, 772, 96), (17, 4, 32), (300, 200, 1056), (2048, 16384, 1024),
-               (257, 132, 64), (32, 2048, 512), (20, 260, 128), (4096, 768, 3072)]
+               (257, 132, 64), (32, 2048, 512), (20, 260, 128), (4096, 768, 3072), (1000, 288, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
