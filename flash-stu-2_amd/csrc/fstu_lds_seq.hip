@@ -8,8 +8,8 @@
 //   pass 3  (block, batch row): U tile again (x is read twice instead of writing and re-reading U: the same bytes,
 //           no workspace of the size of the sequence), scan from carry[k], Y = H C with H split into a bf16 head and
 //           a bf16 remainder so that the second product keeps the fp32 state's accuracy.
-// Weights are given transposed (B^T (S,d_in), C^T (d_out,S)) so that every MFMA fragment is one 16-byte load.
-#include <mutex>
+// Weights are given transposed (B^T (S,d_in), C^T (d_out,S)) so that every MFMA fragment is one 16-byte piece; both
+// travel through LDS so that the four waves of a workgroup share one fetch.
 #include "fstu_common.h"
 
 namespace {
@@ -32,26 +32,39 @@ __device__ __forceinline__ uint4 buf_load16(rsrc_t rs, unsigned off) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <bool FINAL>
-__global__ void __launch_bounds__(256)
+// NT: state tiles of 16 the instantiation holds registers for (S <= 16 NT).  Two workgroups share a compute unit (a
+// workgroup's life is a chain of short barrier-separated phases, so one alone leaves the unit idle most of the time):
+// at most 256 registers, and U without padding, 128 x S floats = 80 KB at S = 160.  Instead of a pad, the 16-byte slot
+// of element (row, mode) is XOR-ed with bits 1..3 of the row, which keeps the 16 rows of a tile access on 16 different
+// slots; the scan, one thread per mode, follows the same map.
+template <bool FINAL, int NT>
+__global__ void __launch_bounds__(256, NT <= 10 ? 2 : 1)   // beyond S = 160 one workgroup fills the LDS anyway
 lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const bf16_t* __restrict__ BmT,
                const bf16_t* __restrict__ CmT, bf16_t* __restrict__ y, const float* __restrict__ carry,
                float* __restrict__ Eout, int T, int Bt, int d_in, int S, int d_out) {
-  extern __shared__ __align__(16) float Us[];       // LSQ_TB x (S + 4)
-  const int ldu = S + 4;
+  extern __shared__ __align__(16) float Us[];       // LSQ_TB x S
+  const int ldu = S;
+  auto uslot = [](int row, int slot) { return slot ^ ((row >> 1) & 7); };   // 16-byte slot of a row (S/4 slots, a multiple of 8)
   const int blk = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, g = lane >> 4;
   const int t0 = blk * LSQ_TB;
   const int nvalid = min(LSQ_TB, T - t0);
   const int nt = S >> 4;
-  // ---- U = X_blk B: wave w owns positions 32w .. 32w+31 (two tiles of 16)
+  // ---- U = X_blk B: wave w owns positions 32w .. 32w+31 (two tiles of 16).  The four waves need the same weight
+  // fragments: B^T travels through LDS in chunks of 64 k (S rows of 128 bytes, 16-byte pieces XOR-ed with bits of the
+  // row so that the 16 rows of a fragment read fall into 16 different slots), double-buffered in the space that U
+  // takes afterwards, so a workgroup fetches every weight once instead of once per wave (a compute unit's
+  // vector-memory path, not HBM or the matrix cores, is what this kernel runs against).
   {
-    floatx4_t acc[2][LSQ_NTMAX];
+    unsigned char* wst = (unsigned char*)Us;                 // two stages of S * 128 bytes
+    const unsigned wstage = (unsigned)S * 128u;
+    const int npiece = S * 8;                                // 16-byte pieces per chunk
+    constexpr int WPT = (NT * 16 * 8 + 255) / 256;    // pieces per thread at the largest S
+    floatx4_t acc[2][NT];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int n = 0; n < LSQ_NTMAX; ++n) acc[m][n] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    // one descriptor per tile row: positions beyond T read zeros
+      for (int n = 0; n < NT; ++n) acc[m][n] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     const bf16_t* xr[2];
     bool xok[2];
 #pragma unroll
@@ -60,77 +73,98 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
       xok[m] = t < T;
       xr[m] = x + ((size_t)(xok[m] ? t : 0) * Bt + b) * d_in + g * 8;
     }
-    const bf16_t* br = BmT + (size_t)r * d_in + g * 8;
-    // the x fragments of four k steps are in flight while the previous four are multiplied (rows of x lie Bt * d_in
-    // elements apart: every fragment is a trip to memory of its own)
-    constexpr int PF = 4;
-    uint4 xn[PF][2];
+    auto wload = [&](int k0, uint4 (&v)[WPT]) {
 #pragma unroll
-    for (int u = 0; u < PF; ++u)
-#pragma unroll
-      for (int m = 0; m < 2; ++m) xn[u][m] = (xok[m] && 32 * u < d_in) ? *(const uint4*)(xr[m] + 32 * u) : make_uint4(0, 0, 0, 0);
-    // weight fragments of the next k step are requested before the current one is multiplied
-    uint4 wn[LSQ_NTMAX];
-#pragma unroll
-    for (int n = 0; n < LSQ_NTMAX; ++n) wn[n] = n < nt ? *(const uint4*)(br + (size_t)n * 16 * d_in) : make_uint4(0, 0, 0, 0);
-    for (int k0 = 0; k0 < d_in; k0 += 32 * PF) {
-      uint4 xb[PF][2];
-#pragma unroll
-      for (int u = 0; u < PF; ++u)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          xb[u][m] = xn[u][m];
-          const int kn = k0 + 32 * (PF + u);
-          xn[u][m] = (xok[m] && kn < d_in) ? *(const uint4*)(xr[m] + kn) : make_uint4(0, 0, 0, 0);
-        }
-#pragma unroll
-      for (int u = 0; u < PF; ++u) {
-        if (k0 + 32 * u < d_in) {
-          uint4 wa[LSQ_NTMAX];
-          const int kn = k0 + 32 * (u + 1);
-#pragma unroll
-          for (int n = 0; n < LSQ_NTMAX; ++n) {
-            wa[n] = wn[n];
-            if (n < nt) wn[n] = *(const uint4*)(br + (size_t)n * 16 * d_in + (kn < d_in ? kn : 0));
-          }
-#pragma unroll
-          for (int n = 0; n < LSQ_NTMAX; ++n) {
-            if (n < nt) {
-              acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[n]), as_bf16x8(xb[u][0]), acc[0][n], 0, 0, 0);
-              acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[n]), as_bf16x8(xb[u][1]), acc[1][n], 0, 0, 0);
-            }
-          }
-        }
+      for (int i = 0; i < WPT; ++i) {
+        const int q = tid + i * 256, row = q >> 3, c = q & 7;
+        v[i] = (q < npiece && k0 + c * 8 < d_in) ? *(const uint4*)(BmT + (size_t)row * d_in + k0 + c * 8) : make_uint4(0, 0, 0, 0);
       }
+    };
+    auto wstore = [&](int stage, const uint4 (&v)[WPT]) {
+#pragma unroll
+      for (int i = 0; i < WPT; ++i) {
+        const int q = tid + i * 256, row = q >> 3, c = q & 7;
+        if (q < npiece) *(uint4*)(wst + stage * wstage + row * 128 + ((c ^ ((row >> 1) & 7)) << 4)) = v[i];
+      }
+    };
+    auto xload = [&](int k0, uint4 (&v)[2][2]) {             // the two k steps of a chunk, both position tiles
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+          v[kk][m] = (xok[m] && k0 + 32 * kk < d_in) ? *(const uint4*)(xr[m] + k0 + 32 * kk) : make_uint4(0, 0, 0, 0);
+    };
+    // chunks are requested two iterations before the iteration that moves them to LDS (one iteration of MFMAs is
+    // shorter than a trip to memory): wv0 / wv1 and xb / xc hold the next two chunks
+    uint4 wv0[WPT], wv1[WPT], xa[2][2], xb[2][2], xc[2][2];
+    wload(0, wv0);
+    xload(0, xa);
+    wload(64, wv1);
+    xload(64, xb);
+    wstore(0, wv0);
+    wload(128, wv0);
+    xload(128, xc);
+    __syncthreads();
+    // one pass: multiply chunk k0 from stage `cur`, move chunk k0+64 (registers NXT) to the other stage, request
+    // chunk k0+192 into those registers
+#define LSQ_PASS(NXT)                                                                                         \
+    {                                                                                                         \
+      const unsigned char* ws = wst + cur * wstage;                                                           \
+      _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                                                      \
+        _Pragma("unroll") for (int n = 0; n < NT; ++n) {                                                      \
+          if (n < nt) {                                                                                       \
+            const int row = 16 * n + r, c = kk * 4 + g;                                                       \
+            const uint4 wa = *(const uint4*)(ws + row * 128 + ((c ^ ((row >> 1) & 7)) << 4));                 \
+            acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa), as_bf16x8(xa[kk][0]), acc[0][n], 0, 0, 0); \
+            acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa), as_bf16x8(xa[kk][1]), acc[1][n], 0, 0, 0); \
+          }                                                                                                   \
+        }                                                                                                     \
+      }                                                                                                       \
+      if (k0 + 64 < d_in) wstore(cur ^ 1, NXT);                                                               \
+      wload(k0 + 192, NXT);                                                                                   \
+      _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                                                        \
+        _Pragma("unroll") for (int m = 0; m < 2; ++m) { xa[kk][m] = xb[kk][m]; xb[kk][m] = xc[kk][m]; }       \
+      xload(k0 + 192, xc);                                                                                    \
+      __syncthreads();                                                                                        \
+      cur ^= 1;                                                                                               \
+      k0 += 64;                                                                                               \
     }
+    int cur = 0, k0 = 0;
+    while (k0 < d_in) {
+      LSQ_PASS(wv1)
+      if (k0 < d_in) LSQ_PASS(wv0)
+    }
+#undef LSQ_PASS
+    // (the last barrier of the loop: every wave is through with the weight stages, U may overwrite them)
     // D layout: lane (r, g) holds modes 16n + 4g + i of position r of the tile
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int n = 0; n < LSQ_NTMAX; ++n)
+      for (int n = 0; n < NT; ++n)
         if (n < nt)
-          *(float4*)(Us + (size_t)(32 * w + 16 * m + r) * ldu + 16 * n + 4 * g) = make_float4(acc[m][n][0], acc[m][n][1], acc[m][n][2], acc[m][n][3]);
+          *(float4*)(Us + (size_t)(32 * w + 16 * m + r) * ldu + 4 * uslot(32 * w + 16 * m + r, 4 * n + g)) = make_float4(acc[m][n][0], acc[m][n][1], acc[m][n][2], acc[m][n][3]);
   }
   __syncthreads();
   // ---- scan over the block's positions: thread = mode
   if (tid < S) {
     const float a = A[tid];
     float h = FINAL ? carry[((size_t)blk * Bt + b) * S + tid] : 0.f;
-    float* col = Us + tid;
+    // element (p, tid) sits at p * ldu + 4 * uslot(p, tid / 4) + tid % 4
+    auto at = [&](int p_) { return Us + (size_t)p_ * ldu + 4 * uslot(p_, tid >> 2) + (tid & 3); };
     int p = 0;
     for (; p + 8 <= nvalid; p += 8) {
       float u[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) u[i] = col[(size_t)(p + i) * ldu];
+      for (int i = 0; i < 8; ++i) u[i] = *at(p + i);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         h = fmaf(a, h, u[i]);
-        if (FINAL) col[(size_t)(p + i) * ldu] = h;
+        if (FINAL) *at(p + i) = h;
       }
     }
     for (; p < nvalid; ++p) {
-      h = fmaf(a, h, col[(size_t)p * ldu]);
-      if (FINAL) col[(size_t)p * ldu] = h;
+      h = fmaf(a, h, *at(p));
+      if (FINAL) *at(p) = h;
     }
     if (!FINAL) Eout[((size_t)blk * Bt + b) * S + tid] = h;
   }
@@ -138,15 +172,17 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
   __syncthreads();
   // ---- Y = H C: wave w, positions 32w .. 32w+31; H as bf16 head + remainder
   {
-    const int ks2 = S >> 5;        // k steps of 32 modes (<= 8)
-    uint4 hb[2][8], lb[2][8];
+    constexpr int KS = (NT + 1) / 2;   // k steps of 32 modes this instantiation holds registers for
+    const int ks2 = S >> 5;            // k steps of 32 modes (<= KS)
+    uint4 hb[2][KS], lb[2][KS];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-      const float* hr = Us + (size_t)(32 * w + 16 * m + r) * ldu + g * 8;
+      const int hrow = 32 * w + 16 * m + r;
+      const float* hr = Us + (size_t)hrow * ldu;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
+      for (int k = 0; k < KS; ++k) {
         if (k < ks2) {
-          const float4 v0 = *(const float4*)(hr + 32 * k), v1 = *(const float4*)(hr + 32 * k + 4);
+          const float4 v0 = *(const float4*)(hr + 4 * uslot(hrow, 8 * k + 2 * g)), v1 = *(const float4*)(hr + 4 * uslot(hrow, 8 * k + 2 * g + 1));
           const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
           unsigned hi[4], lo[4];
 #pragma unroll
@@ -159,35 +195,70 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
         }
       }
     }
-    const bf16_t* cr = CmT + (size_t)r * S + g * 8;
     const int tA = t0 + 32 * w + r, tB = tA + 16;
     bf16_t* yA = y + ((size_t)min(tA, T - 1) * Bt + b) * d_out + 4 * g;
     bf16_t* yB = y + ((size_t)min(tB, T - 1) * Bt + b) * d_out + 4 * g;
     const int nto = d_out >> 4;
-    uint4 cn[8];
+    // C^T travels through LDS like B^T above, 64 output features (4 tiles) at a time, double-buffered in the space of
+    // U now that every wave holds its H fragments in registers.  Rows are S * 2 + 16 bytes: an odd number of 16-byte
+    // slots, so the 16 rows of a fragment read fall into 16 different slots.
+    __syncthreads();
+    unsigned char* cst = (unsigned char*)Us;
+    const unsigned RS = (unsigned)S * 2u + 16u, cstage = 64u * RS;
+    const int ppr = S >> 3, npc = 64 * ppr;                  // 16-byte pieces per row and per stage
+    constexpr int CPT = (64 * (NT * 16 / 8) + 255) / 256;
+    auto cload = [&](int o0, uint4 (&v)[CPT]) {
 #pragma unroll
-    for (int k = 0; k < 8; ++k) cn[k] = k < ks2 ? *(const uint4*)(cr + 32 * k) : make_uint4(0, 0, 0, 0);
-    for (int ot = 0; ot < nto; ++ot) {
-      floatx4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
-      uint4 wc[8];
-      const int on = ot + 1 < nto ? ot + 1 : ot;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        wc[k] = cn[k];
-        if (k < ks2) cn[k] = *(const uint4*)(cr + (size_t)on * 16 * S + 32 * k);
+      for (int i = 0; i < CPT; ++i) {
+        const int q = tid + i * 256, row = q / ppr, c = q - row * ppr;
+        v[i] = (q < npc && o0 + row < d_out) ? *(const uint4*)(CmT + (size_t)(o0 + row) * S + c * 8) : make_uint4(0, 0, 0, 0);
       }
+    };
+    auto cstore = [&](int stage, const uint4 (&v)[CPT]) {
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        if (k < ks2) {
-          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc[k]), as_bf16x8(hb[0][k]), a0, 0, 0, 0);
-          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc[k]), as_bf16x8(lb[0][k]), a0, 0, 0, 0);
-          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc[k]), as_bf16x8(hb[1][k]), a1, 0, 0, 0);
-          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc[k]), as_bf16x8(lb[1][k]), a1, 0, 0, 0);
-        }
+      for (int i = 0; i < CPT; ++i) {
+        const int q = tid + i * 256, row = q / ppr, c = q - row * ppr;
+        if (q < npc) *(uint4*)(cst + stage * cstage + row * RS + c * 16) = v[i];
       }
-      if (tA < T) *(uint2*)(yA + ot * 16) = make_uint2(pack2_bf16(a0[0], a0[1]), pack2_bf16(a0[2], a0[3]));
-      if (tB < T) *(uint2*)(yB + ot * 16) = make_uint2(pack2_bf16(a1[0], a1[1]), pack2_bf16(a1[2], a1[3]));
+    };
+    uint4 cv0[CPT], cv1[CPT];     // the next two groups of output features
+    cload(0, cv0);
+    cload(64, cv1);
+    cstore(0, cv0);
+    cload(128, cv0);
+    __syncthreads();
+#define LSQ_OUT(NXT)                                                                                          \
+    {                                                                                                         \
+      const unsigned char* cs = cst + cur * cstage;                                                           \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                         \
+        const int ot = (o0 >> 4) + j;                                                                         \
+        if (ot < nto) {                                                                                       \
+          floatx4_t a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};                                     \
+          _Pragma("unroll") for (int k = 0; k < KS; ++k) {                                                    \
+            if (k < ks2) {                                                                                    \
+              const uint4 wc = *(const uint4*)(cs + (16 * j + r) * RS + (32 * k + 8 * g) * 2);                \
+              a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc), as_bf16x8(hb[0][k]), a0, 0, 0, 0);  \
+              a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc), as_bf16x8(lb[0][k]), a0, 0, 0, 0);  \
+              a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc), as_bf16x8(hb[1][k]), a1, 0, 0, 0);  \
+              a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wc), as_bf16x8(lb[1][k]), a1, 0, 0, 0);  \
+            }                                                                                                 \
+          }                                                                                                   \
+          if (tA < T) *(uint2*)(yA + ot * 16) = make_uint2(pack2_bf16(a0[0], a0[1]), pack2_bf16(a0[2], a0[3])); \
+          if (tB < T) *(uint2*)(yB + ot * 16) = make_uint2(pack2_bf16(a1[0], a1[1]), pack2_bf16(a1[2], a1[3])); \
+        }                                                                                                     \
+      }                                                                                                       \
+      if (o0 + 64 < d_out) cstore(cur ^ 1, NXT);                                                              \
+      cload(o0 + 192, NXT);                                                                                   \
+      __syncthreads();                                                                                        \
+      cur ^= 1;                                                                                               \
+      o0 += 64;                                                                                               \
     }
+    int cur = 0, o0 = 0;
+    while (o0 < d_out) {
+      LSQ_OUT(cv1)
+      if (o0 < d_out) LSQ_OUT(cv0)
+    }
+#undef LSQ_OUT
   }
 }
 
@@ -232,23 +303,30 @@ extern "C" int fstu_lds_sequence(float* h, const void* x, const float* A, const 
   const size_t BtS = (size_t)Bt * S;
   float* carry = ws;
   float* E = ws + (size_t)(nblk + 1) * BtS;
-  const size_t shm = (size_t)LSQ_TB * (S + 4) * sizeof(float);
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  std::call_once(once, [&]() {
-    attr_err = hipFuncSetAttribute((const void*)lds_seq_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-    if (attr_err == hipSuccess)
-      attr_err = hipFuncSetAttribute((const void*)lds_seq_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-  });
-  if (attr_err != hipSuccess) { fstu_set_error("fstu_lds_sequence: hipFuncSetAttribute: %s", hipGetErrorString(attr_err)); return (int)attr_err; }
+  const size_t shm = (size_t)LSQ_TB * S * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(nblk, Bt);
-  hipLaunchKernelGGL(lds_seq_kernel<false>, grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT, (const bf16_t*)CmT,
-                     (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);
-  hipLaunchKernelGGL(lds_carry_kernel, dim3((unsigned)((BtS + 255) / 256)), dim3(256), 0, s, h, A, (const float*)E, carry, nblk, T,
-                     (int)BtS, S);
-  hipLaunchKernelGGL(lds_seq_kernel<true>, grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT, (const bf16_t*)CmT,
-                     (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);
+#define LSQ_RUN(NTV)                                                                                                      \
+  do {                                                                                                                    \
+    static const hipError_t e1 = hipFuncSetAttribute((const void*)lds_seq_kernel<false, NTV>,                             \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);            \
+    static const hipError_t e2 = hipFuncSetAttribute((const void*)lds_seq_kernel<true, NTV>,                              \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);            \
+    if (e1 != hipSuccess || e2 != hipSuccess) {                                                                           \
+      fstu_set_error("fstu_lds_sequence: hipFuncSetAttribute: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));       \
+      return (int)(e1 != hipSuccess ? e1 : e2);                                                                           \
+    }                                                                                                                     \
+    hipLaunchKernelGGL((lds_seq_kernel<false, NTV>), grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT,    \
+                       (const bf16_t*)CmT, (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);                    \
+    hipLaunchKernelGGL(lds_carry_kernel, dim3((unsigned)((BtS + 255) / 256)), dim3(256), 0, s, h, A, (const float*)E,     \
+                       carry, nblk, T, (int)BtS, S);                                                                      \
+    hipLaunchKernelGGL((lds_seq_kernel<true, NTV>), grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT,     \
+                       (const bf16_t*)CmT, (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);                    \
+  } while (0)
+  if (S <= 64) LSQ_RUN(4);
+  else if (S <= 160) LSQ_RUN(10);
+  else LSQ_RUN(16);
+#undef LSQ_RUN
   FSTU_CHECK_LAUNCH("fstu_lds_sequence");
   return FSTU_OK;
 }

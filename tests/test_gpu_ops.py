@@ -892,6 +892,32 @@ def test_lds_steps_dense(hip, dtype):
     assert float((h.cpu() - href).abs().max()) < 1e-5 * max(1.0, float(href.abs().max()))
 
 
+@pytest.mark.parametrize("T,Bt,din,S,dout", [(300, 3, 96, 32, 48), (200, 2, 128, 64, 80), (130, 2, 64, 192, 64),
+                                             (257, 1, 256, 256, 144), (129, 4, 160, 160, 16)])
+def test_lds_sequence_on_the_matrix_cores(hip, T, Bt, din, S, dout):
+    """The block-parallel form (bf16, S a multiple of 32: fstu_lds_sequence) at state sizes of every register variant,
+    ragged block counts, d_in of an odd number of 32-wide k steps and output widths that are not whole groups of 64:
+    against the oracle's literal loop, and bit-identical when the sequence is cut at a multiple of 128 positions."""
+    g = gen(15)
+    dtype = torch.bfloat16
+    A = (0.9 + 0.099 * torch.rand(S, generator=g)).float()
+    Bm = (torch.randn(din, S, generator=g) / din ** 0.5).to(dtype)
+    Cm = (torch.randn(S, dout, generator=g) / S).to(dtype)
+    x = torch.randn(T, Bt, din, generator=g).to(dtype)
+    yref, href = O.lds_sequence(x, A, Bm, Cm)
+    Ad, Bd, Cd, xd = dev(A), dev(Bm), dev(Cm), dev(x)
+    h = torch.zeros(Bt, S, device="cuda")
+    y = hip.lds_steps(h, xd, Ad, Bd, Cd)
+    diff = (y.float().cpu() - yref.float()).abs()
+    assert float(diff.max()) <= 2.0 ** -7 * float(yref.float().abs().max())
+    assert float((diff > 0).float().mean()) < 0.05
+    assert float((h.cpu() - href).abs().max()) <= 1e-4 * float(href.abs().max())
+    h2 = torch.zeros(Bt, S, device="cuda")
+    ya = hip.lds_steps(h2, xd[:128], Ad, Bd, Cd)
+    yb = hip.lds_steps(h2, xd[128:], Ad, Bd, Cd)
+    assert torch.equal(torch.cat([ya, yb]), y) and torch.equal(h2, h)
+
+
 def test_argument_errors_do_not_launch(hip):
     x = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
     W = torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda")
