@@ -310,19 +310,25 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
     return;
   }
 
-  // filter bank (one column per workgroup, n <= 16 * NT): the thread keeps the spectrum of its 16 neighbouring
-  // positions in registers and runs, per filter, the product and the first inverse pass from them
-  const int u = threadIdx.x;
-  const bool act = u < (n >> 4);
-  cpx* p = fft_lds + 17 * (act ? u : 0);
-  cpx xs[16];
-  if (act) forward16(p, xs);
+  // filter bank (one column per workgroup): the thread keeps the spectrum of its groups of 16 neighbouring positions
+  // in registers and runs, per filter, the product and the first inverse pass from them
+  constexpr int NB = ((n >> 4) + NT - 1) / NT;     // groups of 16 per thread
+  cpx xs[NB][16];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int u = threadIdx.x + i * NT;
+    if (u < (n >> 4)) forward16(fft_lds + 17 * u, xs[i]);
+  }
   __syncthreads();
   for (int k = 0; k < K; ++k) {
-    if (act) {
-      cpx s[16];
-      load_spec16(spec + ((size_t)k << LOGN) + 16 * u, s);
-      product_inverse16(p, xs, s);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int u = threadIdx.x + i * NT;
+      if (u < (n >> 4)) {
+        cpx s[16];
+        load_spec16(spec + ((size_t)k << LOGN) + 16 * u, s);
+        product_inverse16(fft_lds + 17 * u, xs[i], s);
+      }
     }
     __syncthreads();
     fft_inverse<LOGN, NT, true>(fft_lds, tw, 1);
@@ -502,7 +508,11 @@ extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
   return FSTU_OK;
 }
 
-// threads per workgroup follow the transform length: one radix-16 butterfly per thread and pass for n >= 4096
+// threads per workgroup follow the transform length: one radix-16 butterfly per thread and pass for n = 4096 and
+// 8192, two at 16384 (1024 threads leave 128 registers each, which the bank form's resident spectrum overflows)
+#ifndef FFT_NT14
+#define FFT_NT14 512
+#endif
 #define FFT_LAUNCH_ONE(LOGNV, NTV, KERNEL, GRID, SHM, NAME, ...)                                              \
   do {                                                                                                        \
     int rc__ = allow_lds(KERNEL<T, LOGNV, NTV>, SHM, NAME);                                                   \
@@ -521,7 +531,7 @@ extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
       case 11: FFT_LAUNCH_ONE(11, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
       case 12: FFT_LAUNCH_ONE(12, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
       case 13: FFT_LAUNCH_ONE(13, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
-      default: FFT_LAUNCH_ONE(14, 1024, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;   \
+      default: FFT_LAUNCH_ONE(14, FFT_NT14, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;   \
     }                                                                                   \
   } while (0)
 
