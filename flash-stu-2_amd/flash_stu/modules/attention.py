@@ -69,10 +69,10 @@ class Attention(nn.Module):
             if not use_cache:
                 return y
             cap = W + 1
-            # a prompt of cap positions or more fills every slot of the rings; a shorter one leaves the rest zero
-            alloc = x.new_empty if T >= cap else x.new_zeros
-            kr = alloc(B, H, cap, hd)
-            vr = alloc(B, H, cap, hd)
+            # slots the prompt does not fill are written by the decode step that reaches their position before any
+            # step reads them (a step reads positions below its own only): no zero fill
+            kr = x.new_empty(B, H, cap, hd)
+            vr = x.new_empty(B, H, cap, hd)
             _hip.kv_fill(qkv, kr, vr, 0)
             return y, (kr, vr, torch.full((B,), T, dtype=torch.int64))
         if T != 1:
