@@ -839,14 +839,14 @@ template <> __device__ __forceinline__ float lsh_load<bf16_t>(__amdgpu_buffer_rs
   return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0));
 }
 
-template <typename T, int MAXJ>
-__global__ void __launch_bounds__(256)
+template <typename T, int MAXJ, int NG /* waves of a workgroup, each with up to MAXJ modes of the same 64 channels */>
+__global__ void __launch_bounds__(NG * 64)
 lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__ a, float* __restrict__ state, int S,
                            int d, int t_last, int cap) {
   const int b = blockIdx.y, p = blockIdx.z;
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int jg = threadIdx.x >> 6;
-  const int per = (S + LSH_JG - 1) / LSH_JG;
+  const int per = (S + NG - 1) / NG;
   const int j0 = jg * per;
   if (c >= d) return;
   float h[MAXJ], aj[MAXJ];
@@ -859,20 +859,28 @@ lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__
   const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T*>(hist + (size_t)b * cap * d), 0, (unsigned)((size_t)(t_last + 1) * d * sizeof(T)), 0x00020000);
   const unsigned row = (unsigned)d * (unsigned)sizeof(T), col = (unsigned)c * (unsigned)sizeof(T);
-  float xn[16];
+  // LSH_D batches of 16 positions are in flight: a batch is a quarter of a microsecond of arithmetic, a load a trip to
+  // memory of one to two microseconds
+  constexpr int LSH_D = 4;
+  float xq[LSH_D][16];
 #pragma unroll
-  for (int k = 0; k < 16; ++k) xn[k] = lsh_load<T>(rs, (unsigned)(p + 2 * k) * row + col);
-  for (int tt0 = p; tt0 <= t_last; tt0 += 32) {
-    float xs[16];
+  for (int u = 0; u < LSH_D; ++u)
 #pragma unroll
-    for (int k = 0; k < 16; ++k) xs[k] = xn[k];
+    for (int k = 0; k < 16; ++k) xq[u][k] = lsh_load<T>(rs, (unsigned)(p + 32 * u + 2 * k) * row + col);
+  for (int tt0 = p; tt0 <= t_last; tt0 += 32 * LSH_D) {
 #pragma unroll
-    for (int k = 0; k < 16; ++k) xn[k] = lsh_load<T>(rs, (unsigned)(tt0 + 32 + 2 * k) * row + col);   // next batch in flight
+    for (int u = 0; u < LSH_D; ++u) {
+      float xs[16];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      if (tt0 + 2 * k <= t_last) {      // a step past the end must not decay the state
+      for (int k = 0; k < 16; ++k) xs[k] = xq[u][k];
 #pragma unroll
-        for (int i = 0; i < MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
+      for (int k = 0; k < 16; ++k) xq[u][k] = lsh_load<T>(rs, (unsigned)(tt0 + 32 * (LSH_D + u) + 2 * k) * row + col);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        if (tt0 + 32 * u + 2 * k <= t_last) {      // a step past the end must not decay the state
+#pragma unroll
+          for (int i = 0; i < MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
+        }
       }
     }
   }
@@ -890,14 +898,15 @@ extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, fl
   FSTU_REQUIRE(t_last >= -1 && t_last < cap, FSTU_EARG, "fstu_stu_lds_state_from_hist: t_last=%d cap=%d", t_last, cap);
   FSTU_REQUIRE((size_t)cap * d * 4 < 0xfff00000ull, FSTU_ESHAPE, "fstu_stu_lds_state_from_hist: cap*d too large for 32-bit offsets");
   dim3 grid((d + 63) / 64, B, 2);
-  if (S <= LSH_JG * 16) {
+  if (S <= 64) {
+    // 8 waves of 8 modes: two waves per SIMD cover each other's dependent fused multiply-adds
     FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
-                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, 16>), grid, dim3(256), 0, (hipStream_t)stream,
+                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, 8, 8>), grid, dim3(512), 0, (hipStream_t)stream,
                                            (const T*)hist, a, state, S, d, t_last, cap));
   } else {
     FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
-                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, LSH_MAXJ>), grid, dim3(256), 0, (hipStream_t)stream,
-                                           (const T*)hist, a, state, S, d, t_last, cap));
+                        hipLaunchKernelGGL((lds_state_from_hist_kernel<T, LSH_MAXJ, LSH_JG>), grid, dim3(256), 0,
+                                           (hipStream_t)stream, (const T*)hist, a, state, S, d, t_last, cap));
   }
   FSTU_CHECK_LAUNCH("fstu_stu_lds_state_from_hist");
   return FSTU_OK;
