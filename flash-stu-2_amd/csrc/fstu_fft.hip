@@ -545,7 +545,8 @@ extern "C" int fstu_fft_twiddles(float* tw, int n, void* stream) {
       case 10: FFT_LAUNCH_ONE(10, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
       case 11: FFT_LAUNCH_ONE(11, 256, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
       case 12: FFT_LAUNCH_ONE(12, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
-      default: FFT_LAUNCH_ONE(13, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      case 13: FFT_LAUNCH_ONE(13, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
+      default: FFT_LAUNCH_ONE(14, 512, KERNEL, GRID, SHM, NAME, __VA_ARGS__); break;    \
     }                                                                                   \
   } while (0)
 
@@ -584,7 +585,10 @@ static int conv_fft_launch(const char* name, const void* x, int64_t x_sb, int64_
     const int rows_lcols = logn >= 13 ? 0 : logn == 12 ? 1 : (12 - logn > 4 ? 4 : 12 - logn);
     const int esz = dtype == FSTU_BF16 ? 2 : 4, ch = 16 / esz, cols_full = 1 << rows_lcols;
     const int chw = cols_full > ch ? cols_full : ch;
-    if (K == 1 && mode != 2 && logn <= 13 && x_sc == 1 && y_sc == 1 && d % chw == 0 && x_st % ch == 0 && y_st % ch == 0 &&
+    // (the long transforms take a workgroup's channels one after the other: with fewer than two workgroups per compute
+    // unit the one-column kernel, eight times the workgroups, is the faster one)
+    const bool enough = logn < 13 || (long long)(d / chw) * B >= 512;
+    if (K == 1 && mode != 2 && enough && x_sc == 1 && y_sc == 1 && d % chw == 0 && x_st % ch == 0 && y_st % ch == 0 &&
         x_sb % ch == 0 && y_sb % ch == 0 && fstu_aligned(x, 16) && fstu_aligned(y, 16)) {
       const size_t shm = fft_lds_bytes(n, rows_lcols);
       const int gx = d / chw;
