@@ -901,7 +901,7 @@ sample_kernel(const T* __restrict__ logits, int64_t* __restrict__ out, int64_t o
 #define SAMP_MAX_CHUNKS 32
 #define SAMP_MAX_ROWS (2 * FSTU_MAX_DECODE_ROWS)
 struct SampWs {
-  unsigned ticket[SAMP_MAX_ROWS];
+  unsigned ticket[SAMP_MAX_ROWS][32];   // one 128-byte line per row: atomics on one line are served one after the other
   unsigned done;
   unsigned pad[31];
   unsigned cnt[SAMP_MAX_ROWS][SAMP_MAX_CHUNKS];
@@ -984,14 +984,17 @@ sample_topk_kernel(const bf16_t* __restrict__ logits, int64_t ldl, unsigned long
       ++at;
     }
   if (tid == 0) st_agent(&ws->cnt[b][g], (unsigned)tot);
-  __syncthreads();   // the workgroup's stores have left its waves
+  // Everything another workgroup reads was stored at device scope (written through; such a store is complete once the
+  // wave's store counter has drained), so every wave waits for its own stores, the barrier collects the waves, and the
+  // ticket follows: no write-back or invalidation of the whole L2, which costs microseconds with a row per workgroup
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
   if (tid == 0) {
-    __threadfence();
-    s_last = atomicAdd(&ws->ticket[b], 1u) == (unsigned)(G - 1);
+    s_last = atomicAdd(&ws->ticket[b][0], 1u) == (unsigned)(G - 1);
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // what follows reads the other workgroups' data at device scope
 
   // ---- the row's last workgroup
   int64_t* out_slot = out + pos_off + (size_t)b * out_stride;
@@ -1170,7 +1173,7 @@ sample_topk_kernel(const bf16_t* __restrict__ logits, int64_t ldl, unsigned long
   // ---- leave the workspace as it was found
   if (tid < G) ws->cnt[b][tid] = 0u;
   if (tid == 0) {
-    ws->ticket[b] = 0u;
+    ws->ticket[b][0] = 0u;
     if (atomicAdd(&ws->done, 1u) == (unsigned)(nrows - 1)) {
       ws->done = 0u;
       if (dyn && advance) { dyn[0] = pos_off + 1; dyn[1] = step + 1; }

@@ -809,7 +809,7 @@ def test_sample_draws_match_oracle(hip, dtype, temperature, top_k, top_p):
     assert agree >= total - 1, (agree, total)
 
 
-SAMP_COUNTER_WORDS = (32 + 32 + 32 * 32) // 2     # tickets, launch counter, per-chunk counts: 32-bit each
+SAMP_COUNTER_WORDS = (32 * 32 + 32 + 32 * 32) // 2     # tickets (a line per row), launch counter, per-chunk counts: 32-bit each
 
 
 @pytest.mark.parametrize("V", [50257, 4096, 1031])
