@@ -159,26 +159,37 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
     being served out of the 256 MB Infinity Cache)."""
     d, I = cfg.n_embd, cfg.n_embd * cfg.mlp_scale
     if eng.desc.B > _hip.MAX_DECODE_ROWS:
-        # 17..32 rows: the step's gate/up launch is the tiled GEMM kernel over all rows (weights read once)
+        # 17..32 rows: the step's gate/up launch covers all rows and reads every weight once: the balanced kernel over
+        # packed weights with two row tiles per weight fragment where the shape allows it, else the tiled GEMM kernel
         rows = eng.desc.B
         h = torch.randn(rows, d, device="cuda", dtype=torch.bfloat16)
         act = torch.empty(rows, I, device="cuda", dtype=torch.bfloat16)
         mlps = [l.mlp for l in eng.model.layers]
-        for m_ in mlps[:2]:
-            _hip.gemm(h, m_.gate_proj.weight, up_weight=m_.up_proj.weight, out=act)
+        packed = bool(lib.fstu_mlp_packed_rows32_supported(rows, d, I))
+        if packed:
+            ops = [(eng._pack(m_.gate_proj.weight), eng._pack(m_.up_proj.weight)) for m_ in mlps]
+            launch = lambda o: _hip.glu_packed(h, o[0], o[1], I, out=act)
+            name = ("glu_balanced_kernel<two row tiles> (gate/up projection + gelu*up over all rows, packed weights, "
+                    "one workgroup per compute unit)")
+        else:
+            ops = [(m_.gate_proj.weight, m_.up_proj.weight) for m_ in mlps]
+            launch = lambda o: _hip.gemm(h, o[0], up_weight=o[1], out=act)
+            name = "gemm_bf16_kernel<128 features x 32 rows, gated pair> (gate/up projection + gelu*up over all rows)"
+        for o in ops[:2]:
+            launch(o)
         reps = max(1, 96 // len(mlps))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
-            for m_ in mlps:
-                _hip.gemm(h, m_.gate_proj.weight, up_weight=m_.up_proj.weight, out=act)
+            for o in ops:
+                launch(o)
         e1.record()
         torch.cuda.synchronize()
         n = reps * len(mlps)
         us = e0.elapsed_time(e1) * 1e3 / n
         glu_bytes = 2 * I * d * 2 + rows * d * 2 + rows * I * 2
         gbps = glu_bytes / (us * 1e-6) / 1e9
-        return {"bound": "hbm", "kernel": "gemm_bf16_kernel<128 features x 32 rows, gated pair> (gate/up projection + gelu*up over all rows)",
+        return {"bound": "hbm", "kernel": name,
                 "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
                 "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n, "rows_per_launch": rows}
     ms_c, n_c = ctypes.c_double(), ctypes.c_int()

@@ -134,7 +134,9 @@ struct GluArgs {
 
 // EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T
 // (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
-template <int KSA, int PRO, int EPI>
+// NB = 2 (no prologue): rows 16..31 are a second B tile of the same weight fragments, so 17..32 rows read every weight
+// once; the partial sums of the two row tiles then lie behind each other in dynamic LDS.
+template <int KSA, int PRO, int EPI, int NB = 1>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
                     const void* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
@@ -145,13 +147,17 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
-  __shared__ float red[DA * 8 * 512];
-  extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16
+  static_assert(NB == 1 || (NB == 2 && PRO == 0), "two row tiles: launches without the norm prologue only");
+  constexpr int RED = DA * 8 * 512;                           // partial sums of one row tile
+  __shared__ float red_one[NB == 1 ? RED : 1];
+  extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16; NB 2: the partial sums
+  float* red = NB == 1 ? red_one : (float*)glu_smem;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int wgi = blockIdx.x;
   const bool xrow = r < a.rows;
   uint4 xa[KSA];
+  uint4 xa2[NB == 2 ? KSA : 1];                               // B fragments of rows 16..31
   const int nchunk = a.d >> 3, total = a.rows * nchunk;
   // weight addressing
   // Features are dealt out in groups of 8 (a.fpw == 0): with the packed layout a group of 8 rows is one whole 128-byte
@@ -194,6 +200,11 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
 #pragma unroll
     for (int u = 0; u < KSA; ++u) xa[u] = buf_load16(rh, xrow ? hoff + (unsigned)u * 64u : MLP_OOB);
+    if constexpr (NB == 2) {
+      const bool xrow2 = 16 + r < a.rows;
+#pragma unroll
+      for (int u = 0; u < KSA; ++u) xa2[u] = buf_load16(rh, xrow2 ? hoff + (unsigned)(16 * a.ldh) * 2u + (unsigned)u * 64u : MLP_OOB);
+    }
     load_first();
   } else {
     // x' = T(x + delta) (workgroup 0 also stores it), h = T((x' * rstd) * w) into LDS, then this wave's B fragments.
@@ -274,18 +285,27 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
 #pragma unroll
     for (int j = 0; j < DA; ++j) {
       if (t0 + j >= ta1) continue;   // uniform
-      floatx4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+      floatx4_t acc[NB], acc2[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[nb] = acc2[nb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int u = 0; u < KSA; ++u) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc, 0, 0, 0);
-        if (GLU) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2, 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa[u]), acc[0], 0, 0, 0);
+        if (GLU) acc2[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa[u]), acc2[0], 0, 0, 0);
+        if constexpr (NB == 2) {
+          acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wa[j][u]), as_bf16x8(xa2[u]), acc[1], 0, 0, 0);
+          if (GLU) acc2[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wb[j][u]), as_bf16x8(xa2[u]), acc2[1], 0, 0, 0);
+        }
       }
       if (t0 + DA + j < ta1) load_a(j, t0 + DA + j);   // uniform: a load of nothing still costs its address cycles
-      float* mine = red + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        mine[i] = acc[i];
-        if (GLU) mine[256 + i] = acc2[i];
+      for (int nb = 0; nb < NB; ++nb) {
+        float* mine = red + (size_t)nb * RED + (size_t)((j * 8 + w) * 2 * 64 + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          mine[i] = acc[nb][i];
+          if (GLU) mine[256 + i] = acc2[nb][i];
+        }
       }
     }
     __syncthreads();
@@ -293,40 +313,44 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     if ((w >> 1) < DA && t0 + (w >> 1) < ta1) {
       const int jt = w >> 1, hf = (w & 1) * 2;
       const int tile = t0 + jt;
-      float sg[2] = {0.f, 0.f}, su[2] = {0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const float* o = red + (size_t)((jt * 8 + s) * 2 * 64 + lane) * 4 + hf;
-        const float2 pg = *(const float2*)o;
-        sg[0] += pg.x;
-        sg[1] += pg.y;
-        if (GLU) {
-          const float2 pu = *(const float2*)(o + 256);
-          su[0] += pu.x;
-          su[1] += pu.y;
+      for (int nb = 0; nb < NB; ++nb) {
+        float sg[2] = {0.f, 0.f}, su[2] = {0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          const float* o = red + (size_t)nb * RED + (size_t)((jt * 8 + s) * 2 * 64 + lane) * 4 + hf;
+          const float2 pg = *(const float2*)o;
+          sg[0] += pg.x;
+          sg[1] += pg.y;
+          if (GLU) {
+            const float2 pu = *(const float2*)(o + 256);
+            su[0] += pu.x;
+            su[1] += pu.y;
+          }
         }
-      }
-      const int fb = tile * 16 + g * 4 + hf;
-      float o[2];
+        const int fb = tile * 16 + g * 4 + hf;
+        float o[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        if (GLU) {
-          float ge = DT<bf16_t>::rnd(gelu_tanh_fast(DT<bf16_t>::rnd(sg[i])));
-          o[i] = ge * DT<bf16_t>::rnd(su[i]);
-        } else {
-          o[i] = sg[i];
+        for (int i = 0; i < 2; ++i) {
+          if (GLU) {
+            float ge = DT<bf16_t>::rnd(gelu_tanh_fast(DT<bf16_t>::rnd(sg[i])));
+            o[i] = ge * DT<bf16_t>::rnd(su[i]);
+          } else {
+            o[i] = sg[i];
+          }
         }
-      }
-      // the workgroup's range starts and ends on a multiple of four features, so a pair is inside it or outside it
-      const bool grp_ok = xrow && fb >= f0 && fb < f1;
-      if (grp_ok) {
-        bf16_t* yr = a.act + (size_t)r * a.ldact + fb;
-        if (fb + 2 <= f1 && (a.ldact & 1) == 0) {
-          *(unsigned*)yr = pack2_bf16(o[0], o[1]);
-        } else {
+        // the workgroup's range starts and ends on a multiple of four features, so a pair is inside it or outside it
+        const int row = 16 * nb + r;
+        const bool grp_ok = row < a.rows && fb >= f0 && fb < f1;
+        if (grp_ok) {
+          bf16_t* yr = a.act + (size_t)row * a.ldact + fb;
+          if (fb + 2 <= f1 && (a.ldact & 1) == 0) {
+            *(unsigned*)yr = pack2_bf16(o[0], o[1]);
+          } else {
 #pragma unroll
-          for (int i = 0; i < 2; ++i)
-            if (fb + i < f1) yr[i] = f32_to_bf16(o[i]);
+            for (int i = 0; i < 2; ++i)
+              if (fb + i < f1) yr[i] = f32_to_bf16(o[i]);
+          }
         }
       }
     }
@@ -345,13 +369,15 @@ struct DownSkArgs {
   int rows, d, I, ldact, KS, tpw, tiles_out, kch;
 };
 
-template <int KSB>
+// NB = 2: rows 16..31 as a second B tile of the same weight fragments (17..32 rows read every weight once).
+template <int KSB, int NB = 1>
 __global__ void __launch_bounds__(512)
 down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* partial, int rows, int d, int I, int ldact, int KS,
                             int tpw, int tiles_out, int kch) {
   const DownSkArgs a{act, wp_down, partial, rows, d, I, ldact, KS, tpw, tiles_out, kch};
   constexpr int DB = KSB <= 3 ? 4 : (KSB == 4 ? 3 : (KSB <= 8 ? 2 : 1));
-  __shared__ float red[DB * 8 * 256];
+  constexpr int RED = DB * 8 * 256;                          // partial sums of one row tile
+  __shared__ float red[NB * RED];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const bool xrow = r < a.rows;
@@ -364,8 +390,15 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
   const rsrc_t rx = make_rsrc(a.act, ((size_t)(a.rows - 1) * a.ldact + a.I) * 2);
   const unsigned xbase = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldact + (unsigned)(chunk * a.kch + ksb0) * 32u + (unsigned)g * 8u) * 2u;
   uint4 xb[KSB];
+  uint4 xb2[NB == 2 ? KSB : 1];                               // B fragments of rows 16..31
 #pragma unroll
   for (int u = 0; u < KSB; ++u) xb[u] = buf_load16(rx, (xrow && u < nks) ? xbase + (unsigned)u * 64u : MLP_OOB);
+  if constexpr (NB == 2) {
+    const bool xrow2 = 16 + r < a.rows;
+#pragma unroll
+    for (int u = 0; u < KSB; ++u)
+      xb2[u] = buf_load16(rx, (xrow2 && u < nks) ? xbase + (unsigned)(16 * a.ldact) * 2u + (unsigned)u * 64u : MLP_OOB);
+  }
   const rsrc_t rdn = make_rsrc(a.wp_down, (size_t)a.tiles_out * tsb * 16);
   const unsigned bbase = ((unsigned)(chunk * a.kch + ksb0) * 64 + lane) * 16u;
   uint4 wd[DB][KSB];
@@ -388,14 +421,22 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
 #pragma unroll
       for (int j = 0; j < DB; ++j) {
         if (t0 + j >= tb1) continue;
-        floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+        floatx4_t acc[NB];
 #pragma unroll
-        for (int u = 0; u < KSB; ++u)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc, 0, 0, 0);
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KSB; ++u) {
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb[u]), acc[0], 0, 0, 0);
+          if constexpr (NB == 2)
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wd[j][u]), as_bf16x8(xb2[u]), acc[1], 0, 0, 0);
+        }
         if (t0 + DB + j < tb1) load_b(j, t0 + DB + j);
-        float* mine = red + (size_t)((j * 8 + w) * 64 + lane) * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) mine[i] = acc[i];
+        for (int nb = 0; nb < NB; ++nb) {
+          float* mine = red + (size_t)nb * RED + (size_t)((j * 8 + w) * 64 + lane) * 4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[i] = acc[nb][i];
+        }
       }
     }
     __syncthreads();
@@ -403,15 +444,18 @@ down_splitk_balanced_kernel(const bf16_t* act, const uint4* wp_down, float* part
     if ((w >> 1) < DB && t0 + (w >> 1) < tb1) {
       const int jt = w >> 1, hf = (w & 1) * 2;
       const int tile = t0 + jt;
-      float sd[2] = {0.f, 0.f};
-      for (int s = 0; s < nact; ++s) {
-        const float2 o = *(const float2*)(red + (size_t)((jt * 8 + s) * 64 + lane) * 4 + hf);
-        sd[0] += o.x;
-        sd[1] += o.y;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        float sd[2] = {0.f, 0.f};
+        for (int s = 0; s < nact; ++s) {
+          const float2 o = *(const float2*)(red + (size_t)nb * RED + (size_t)((jt * 8 + s) * 64 + lane) * 4 + hf);
+          sd[0] += o.x;
+          sd[1] += o.y;
+        }
+        // D layout: features tile*16 + 4g + i of batch row r of the row tile
+        const int fb = tile * 16 + 4 * g + hf, row = 16 * nb + r;
+        if (row < a.rows && fb < a.d) *(float2*)(a.partial + ((size_t)chunk * a.rows + row) * a.d + fb) = make_float2(sd[0], sd[1]);
       }
-      // D layout: features tile*16 + 4g + i of batch row r
-      const int fb = tile * 16 + 4 * g + hf;
-      if (xrow && fb < a.d) *(float2*)(a.partial + ((size_t)chunk * a.rows + r) * a.d + fb) = make_float2(sd[0], sd[1]);
     }
     if (t0 + DB < tb1) __syncthreads();
   }
@@ -436,6 +480,13 @@ extern "C" int fstu_glu_packed_supported(int rows, int d, int I) {
          I >= 16 && (size_t)I * d * 2 < 0xfff00000ull;
 }
 
+// 17..32 rows: fstu_glu_packed and fstu_down_packed_splitk take them as two row tiles per weight fragment (the launches
+// with a norm prologue do not)
+extern "C" int fstu_mlp_packed_rows32_supported(int rows, int d, int I) {
+  return rows > FSTU_MAX_DECODE_ROWS && rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(FSTU_MAX_DECODE_ROWS, d, I) &&
+         I % 512 == 0 && (size_t)rows * I * 2 < 0x7ff00000ull;
+}
+
 template <int KSA>
 static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const char* name, hipStream_t s) {
 #define GLU_GO(PRO, GLUF)                                                                                        \
@@ -448,6 +499,18 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,    \
                        a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);                    \
   } while (0)
+  if (a.rows > FSTU_MAX_DECODE_ROWS) {
+    // two row tiles: the partial sums of both lie in dynamic LDS
+    constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
+    const size_t red2 = (size_t)2 * DA * 8 * 512 * sizeof(float);
+    FSTU_REQUIRE(pro == 0 && epi == 0, FSTU_ESHAPE, "%s: more than %d rows only without the norm prologue", name, FSTU_MAX_DECODE_ROWS);
+    static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, 0, 0, 2>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)red2);
+    FSTU_REQUIRE(attr_err == hipSuccess, (int)attr_err, "%s: %zu bytes of dynamic LDS refused", name, red2);
+    hipLaunchKernelGGL((glu_balanced_kernel<KSA, 0, 0, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,
+                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);
+    return FSTU_OK;
+  }
   if (pro == 2) GLU_GO(2, 1);
   else if (pro && epi == 0) GLU_GO(1, 0);
   else if (pro) GLU_GO(1, 1);
@@ -490,7 +553,8 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
 extern "C" int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
                                int I, int d, void* stream) {
   FSTU_REQUIRE(h && wp_gate && wp_up && act, FSTU_ENULL, "fstu_glu_packed: null pointer");
-  FSTU_REQUIRE(fstu_glu_packed_supported(rows, d, I), FSTU_ESHAPE, "fstu_glu_packed: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, d, I) || fstu_mlp_packed_rows32_supported(rows, d, I), FSTU_ESHAPE,
+               "fstu_glu_packed: unsupported shape rows=%d d=%d I=%d", rows, d, I);
   FSTU_REQUIRE(ldh >= d && ldh % 8 == 0 && ldact >= I && ldact % 4 == 0, FSTU_ESHAPE, "fstu_glu_packed: ldh=%d ldact=%d", ldh, ldact);
   FSTU_REQUIRE(fstu_aligned(h, 16) && fstu_aligned(wp_gate, 16) && fstu_aligned(wp_up, 16) && fstu_aligned(act, 8), FSTU_EALIGN,
                "fstu_glu_packed: pointers must be 16-byte aligned");
@@ -567,8 +631,8 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   // *ksplit_io on entry: the number of K slices wanted (4, 8 or 16; anything else: 16); on return: the number written
   const int want = ksplit_io ? *ksplit_io : 16;
   const int KS = (want == 4 || want == 8) ? want : 16;
-  FSTU_REQUIRE(rows >= 1 && rows <= FSTU_MAX_DECODE_ROWS && d >= 16 && d % 16 == 0 && I >= KS * 32 && I % (KS * 32) == 0 &&
-                   (size_t)I * d * 2 < 0xfff00000ull,
+  FSTU_REQUIRE(rows >= 1 && rows <= 2 * FSTU_MAX_DECODE_ROWS && d >= 16 && d % 16 == 0 && I >= KS * 32 && I % (KS * 32) == 0 &&
+                   (size_t)I * d * 2 < 0xfff00000ull && (size_t)rows * ldact * 2 < 0x7ff00000ull,
                FSTU_ESHAPE, "fstu_down_packed_splitk: unsupported shape rows=%d d=%d I=%d", rows, d, I);
   FSTU_REQUIRE(ldact >= I && ldact % 8 == 0, FSTU_ESHAPE, "fstu_down_packed_splitk: ldact=%d", ldact);
   FSTU_REQUIRE(fstu_aligned(act, 16) && fstu_aligned(wp_down, 16) && fstu_aligned(partial, 16), FSTU_EALIGN,
@@ -587,14 +651,24 @@ extern "C" int fstu_down_packed_splitk(const void* act, int ldact, const void* w
   FSTU_REQUIRE(ksb <= 12, FSTU_ESHAPE, "fstu_down_packed_splitk: I=%d too large", I);
   dim3 grid(ngroups * KS);
   hipStream_t s = (hipStream_t)stream;
-  if (ksb <= 1) hipLaunchKernelGGL(down_splitk_balanced_kernel<1>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb == 2) hipLaunchKernelGGL(down_splitk_balanced_kernel<2>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb == 3) hipLaunchKernelGGL(down_splitk_balanced_kernel<3>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb == 4) hipLaunchKernelGGL(down_splitk_balanced_kernel<4>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb <= 6) hipLaunchKernelGGL(down_splitk_balanced_kernel<6>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb <= 8) hipLaunchKernelGGL(down_splitk_balanced_kernel<8>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else if (ksb == 9) hipLaunchKernelGGL(down_splitk_balanced_kernel<9>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
-  else hipLaunchKernelGGL(down_splitk_balanced_kernel<12>, grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);
+#define DOWN_GO(KSB)                                                                                                          \
+  do {                                                                                                                         \
+    if (rows > FSTU_MAX_DECODE_ROWS)                                                                                           \
+      hipLaunchKernelGGL((down_splitk_balanced_kernel<KSB, 2>), grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, \
+                         a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);                                                       \
+    else                                                                                                                       \
+      hipLaunchKernelGGL((down_splitk_balanced_kernel<KSB, 1>), grid, dim3(512), 0, s, a.act, a.wp_down, a.partial, a.rows, a.d, \
+                         a.I, a.ldact, a.KS, a.tpw, a.tiles_out, a.kch);                                                       \
+  } while (0)
+  if (ksb <= 1) DOWN_GO(1);
+  else if (ksb == 2) DOWN_GO(2);
+  else if (ksb == 3) DOWN_GO(3);
+  else if (ksb == 4) DOWN_GO(4);
+  else if (ksb <= 6) DOWN_GO(6);
+  else if (ksb <= 8) DOWN_GO(8);
+  else if (ksb == 9) DOWN_GO(9);
+  else DOWN_GO(12);
+#undef DOWN_GO
   FSTU_CHECK_LAUNCH("fstu_down_packed_splitk");
   if (ksplit_io) *ksplit_io = KS;
   return FSTU_OK;

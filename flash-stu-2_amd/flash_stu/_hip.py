@@ -64,6 +64,7 @@ SIGNATURES = {
     "fstu_pack_rows": [_vp, _vp, _i, _i, _vp],
     "fstu_packed_elems": [_i, _i],
     "fstu_glu_packed_supported": [_i, _i, _i],
+    "fstu_mlp_packed_rows32_supported": [_i, _i, _i],
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
@@ -710,11 +711,12 @@ def pack_rows(W: torch.Tensor) -> torch.Tensor:
 
 def glu_packed(x: torch.Tensor, wp_gate: torch.Tensor, wp_up: torch.Tensor, I: int,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Gate/up projection + GLU over packed weights (rows <= 16, bf16): x (rows,d) -> act (rows,I)."""
+    """Gate/up projection + GLU over packed weights (rows <= 32, bf16): x (rows,d) -> act (rows,I)."""
     _dev(wp_gate, wp_up, out)
     rows, ldx = _rows_view(x)
     d = x.shape[1]
-    if x.dtype != torch.bfloat16 or not load().fstu_glu_packed_supported(rows, d, I):
+    if x.dtype != torch.bfloat16 or not (load().fstu_glu_packed_supported(rows, d, I) or
+                                         load().fstu_mlp_packed_rows32_supported(rows, d, I)):
         raise FlashSTUHipError(f"fstu_glu_packed does not support rows={rows} d={d} I={I} dtype={x.dtype}")
     if out is None:
         out = torch.empty(rows, I, dtype=x.dtype, device=x.device)

@@ -253,6 +253,12 @@ class DecodeEngine:
                         if isinstance(layer, AttentionLayer):
                             arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
                     m.merge_norm = 1
+        if dt == torch.bfloat16 and self.lib.fstu_mlp_packed_rows32_supported(B, d, I):
+            # 17..32 rows: the MLP streams packed weights as two row tiles per weight fragment
+            for i, layer in enumerate(model.layers):
+                arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
+                arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
+                arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
         ch.arr, ch.desc = arr, m
         ch.mega = None
         if B > _hip.MAX_DECODE_ROWS:

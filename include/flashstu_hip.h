@@ -385,10 +385,14 @@ int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
 
 /* Gate/up projection with the GLU epilogue over packed weights, one workgroup per CU with equal bytes each
  * (4-feature granularity) and every weight fragment in flight from the first instruction:
- *   act[r,f] = T( T(gelu_tanh(T(h[r,:].Wg[f,:]))) * T(h[r,:].Wu[f,:]) ),  rows <= 16, bf16.
+ *   act[r,f] = T( T(gelu_tanh(T(h[r,:].Wg[f,:]))) * T(h[r,:].Wu[f,:]) ),  rows <= 16 (32: below), bf16.
  * Same contract as fstu_glu_decode (flash_stu/modules/swiglu.py:23-26); wp_* from fstu_pack_rows.
- * fstu_glu_packed_supported tells whether a shape is covered (d in {256,512,768,1024,2048}, I % 4 == 0). */
+ * fstu_glu_packed_supported tells whether a shape is covered (d in {256,512,768,1024,2048}, I % 4 == 0).
+ * 17..32 rows (fstu_mlp_packed_rows32_supported: such a d, I % 512 == 0): fstu_glu_packed and fstu_down_packed_splitk
+ * take them as two row tiles per weight fragment, so every weight is still read once; the launches with a norm
+ * prologue (fstu_glu_packed_norm, fstu_linear_packed, fstu_linear_packed_res) stay at 16 rows. */
 int fstu_glu_packed_supported(int rows, int d, int I);
+int fstu_mlp_packed_rows32_supported(int rows, int d, int I);
 int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
                     int I, int d, void* stream);
 /* The same launch with the sub-layer's residual add and mlp_norm as its prologue (stu_layer.py:93-96,
@@ -406,7 +410,7 @@ int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, co
 /* Split-K form of the down projection over packed weights (reference: flash_stu/modules/swiglu.py:22-29, down_proj):
  * partial receives *ksplit_io fp32 slices (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1) or the norm prologue of
  * the next projection sums in slice order.  *ksplit_io on entry: slices wanted (4, 8 or 16; anything else: 16); on
- * return: slices written.  d % 16 == 0, I % (32 * slices) == 0, rows <= 16, bf16.  Same values as
+ * return: slices written.  d % 16 == 0, I % (32 * slices) == 0, rows <= 32, bf16.  Same values as
  * fstu_linear_decode_splitk up to the summation order. */
 int fstu_down_packed_splitk(const void* act, int ldact, const void* wp_down, float* partial, int rows, int d, int I,
                             int* ksplit_io, void* stream);

@@ -992,10 +992,11 @@ def test_stu_step_lds_with_the_reference_lds_fixture(hip):
 
 
 @pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (1, 256, 512), (16, 512, 1000), (5, 1024, 4096), (8, 2048, 24576),
-                                      (3, 768, 20)])
+                                      (3, 768, 20), (32, 768, 9216), (17, 256, 512), (24, 2048, 8192), (32, 1024, 4096)])
 def test_glu_packed_balanced(hip, rows, d, I):
     """Balanced packed gate/up GEMV == the row-major GLU kernel bit for bit is not required (other K split), but both
-    must match the oracle within one bf16 ulp; ragged I (not a multiple of 16 or of the grid)."""
+    must match the oracle within one bf16 ulp; ragged I (not a multiple of 16 or of the grid).  17..32 rows run as two
+    row tiles per weight fragment and equal two launches of 16 rows bit for bit."""
     dtype = torch.bfloat16
     g = gen(60)
     x = torch.randn(rows, d, generator=g).to(dtype)
@@ -1014,7 +1015,12 @@ def test_glu_packed_balanced(hip, rows, d, I):
         assert bool((diff <= b.abs() * 2.0 ** -6 + 1e-3 * 2.0 ** -7 * float(b.abs().max())).all())
         assert float((diff > 0).float().mean()) <= frac
     close(out, ref, 0.05)
-    close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
+    if rows <= 16:
+        close(out, hip.glu_decode(dev(x), dev(wg), dev(wu)), 0.02)     # the row-major kernel, other K split
+    else:
+        pg, pu = hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu))
+        halves = torch.cat([hip.glu_packed(dev(x[:16]), pg, pu, I), hip.glu_packed(dev(x[16:]), pg, pu, I)])
+        assert torch.equal(out, halves)
 
 
 @pytest.mark.parametrize("rows,d,I", [(8, 768, 9216), (3, 256, 512), (16, 1024, 4096), (8, 2048, 8192),
@@ -1109,9 +1115,11 @@ def test_stu_bank_step_lds(hip, dtype):
     assert worst <= tol * float(rp.float().abs().max()), worst
 
 
-@pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8)])
+@pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8),
+                                         (32, 768, 9216, 16), (19, 1024, 4096, 8), (32, 2048, 24576, 16), (17, 48, 1024, 4)])
 def test_down_packed_splitk(hip, rows, d, I, ks):
-    """Balanced split-K down projection: the 4, 8 or 16 slices sum to the float64-accumulated product."""
+    """Balanced split-K down projection: the 4, 8 or 16 slices sum to the float64-accumulated product (17..32 rows: two
+    row tiles per weight fragment, slice for slice equal to two launches of 16 rows)."""
     dtype = torch.bfloat16
     g = gen(64)
     act = torch.randn(rows, I, generator=g).to(dtype)
@@ -1121,6 +1129,10 @@ def test_down_packed_splitk(hip, rows, d, I, ks):
     assert part.shape[0] == ks
     got = part.double().sum(0).cpu()
     assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max())
+    if rows > 16:
+        wp = hip.pack_rows(dev(wd))
+        halves = torch.cat([hip.down_packed_splitk(dev(act[:16]), wp, d, ks), hip.down_packed_splitk(dev(act[16:]), wp, d, ks)], 1)
+        assert torch.equal(part, halves)
 
 
 def test_kernels_against_committed_known_answers(hip):
