@@ -30,6 +30,24 @@ template <> __device__ __forceinline__ void load_vec<bf16_t, 32>(const bf16_t* p
   load_vec<bf16_t, 16>(p, o);
   load_vec<bf16_t, 16>(p + 16, o + 16);
 }
+// the same for data read exactly once per launch (the rings of a decode step): non-temporal, so that the stream does
+// not push the step's weights and activations out of the caches
+typedef unsigned swa_u32x4_t __attribute__((ext_vector_type(4)));
+template <typename T, int N>
+__device__ __forceinline__ void load_vec_stream(const T* p, float* o) { load_vec<T, N>(p, o); }
+template <> __device__ __forceinline__ void load_vec_stream<bf16_t, 8>(const bf16_t* p, float* o) {
+  const swa_u32x4_t v = __builtin_nontemporal_load((const swa_u32x4_t*)p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(v[i] << 16); o[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u); }
+}
+template <> __device__ __forceinline__ void load_vec_stream<bf16_t, 16>(const bf16_t* p, float* o) {
+  load_vec_stream<bf16_t, 8>(p, o);
+  load_vec_stream<bf16_t, 8>(p + 8, o + 8);
+}
+template <> __device__ __forceinline__ void load_vec_stream<bf16_t, 32>(const bf16_t* p, float* o) {
+  load_vec_stream<bf16_t, 16>(p, o);
+  load_vec_stream<bf16_t, 16>(p + 16, o + 16);
+}
 template <> __device__ __forceinline__ void load_vec<float, 4>(const float* p, float* o) {
   float4 v = *(const float4*)p;
   o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
@@ -229,8 +247,10 @@ extern "C" int fstu_kv_append(const void* qkv, void* kring, void* vring, int B, 
 // sweep in flight at once.  With append != 0 the workgroup stores the new token's
 // k,v (read from the qkv row) into ring slot pos % cap and attends to that key
 // straight from the qkv row, so the ring sweep covers the older keys only.
+// STREAM: the ring loads are non-temporal.  The rings of a step that fit the memory-side cache next to the weights are
+// found there again by the next step and are read with ordinary loads; larger ones only push other data out.
 #define SWA_U 4
-template <typename T, int HD, int NWAVES>
+template <typename T, int HD, int NWAVES, bool STREAM = false>
 __global__ void __launch_bounds__(NWAVES * 64)
 swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__ out, const float* __restrict__ slopes,
                   const int* __restrict__ dyn /* early in the list: within the preloaded argument dwords */, int H, int cap,
@@ -288,8 +308,13 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
       const int j = min(jb + u, j_end - 1);
       int slot = slot_lo + (j - lo);
       slot = slot >= cap ? slot - cap : slot;
-      load_vec<T, DPL>(kb + (size_t)slot * HD, kk[u]);
-      load_vec<T, DPL>(vb + (size_t)slot * HD, vv[u]);
+      if constexpr (STREAM) {
+        load_vec_stream<T, DPL>(kb + (size_t)slot * HD, kk[u]);
+        load_vec_stream<T, DPL>(vb + (size_t)slot * HD, vv[u]);
+      } else {
+        load_vec<T, DPL>(kb + (size_t)slot * HD, kk[u]);
+        load_vec<T, DPL>(vb + (size_t)slot * HD, vv[u]);
+      }
     }
     float sc[SWA_U], mit = -INFINITY;
 #pragma unroll
@@ -388,9 +413,17 @@ int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, c
   FSTU_REQUIRE(B <= 65535, FSTU_ESHAPE, "fstu_swa_decode: B too large");
   hipStream_t s = (hipStream_t)stream;
   const int nkeys = dyn ? window + 1 : (pos < window ? pos : window) + 1;
-#define SWA_LAUNCH(HD, NW)                                                                                      \
-  hipLaunchKernelGGL((swa_decode_kernel<T, HD, NW>), dim3(H, B), dim3(NW * 64), 0, s, (const T*)qkv, (T*)kring, \
-                     (T*)vring, (T*)out, slopes, dyn, H, cap, pos, window, softcap, append)
+  // keys and values one launch reads: from 64 MB on (a quarter of the memory-side cache) they are streamed
+  const bool stream_ring = (size_t)B * H * nkeys * hd * 2 * (dtype == FSTU_BF16 ? 2 : 4) >= ((size_t)64 << 20);
+#define SWA_LAUNCH(HD, NW)                                                                                              \
+  do {                                                                                                                  \
+    if (stream_ring)                                                                                                    \
+      hipLaunchKernelGGL((swa_decode_kernel<T, HD, NW, true>), dim3(H, B), dim3(NW * 64), 0, s, (const T*)qkv, (T*)kring, \
+                         (T*)vring, (T*)out, slopes, dyn, H, cap, pos, window, softcap, append);                        \
+    else                                                                                                                \
+      hipLaunchKernelGGL((swa_decode_kernel<T, HD, NW, false>), dim3(H, B), dim3(NW * 64), 0, s, (const T*)qkv, (T*)kring, \
+                         (T*)vring, (T*)out, slopes, dyn, H, cap, pos, window, softcap, append);                        \
+  } while (0)
   FSTU_DISPATCH_DTYPE(dtype, "fstu_swa_decode", {
     if (hd == 32) { if (nkeys > 128) SWA_LAUNCH(32, 16); else SWA_LAUNCH(32, 4); }
     // head dim 64, long windows: 8 waves (16 measured 1.5 us per decode step slower at window 512, 4 waves 3 us slower)

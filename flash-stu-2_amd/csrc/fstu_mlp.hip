@@ -132,7 +132,9 @@ struct GluArgs {
   int nslices;
 };
 
-// EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T
+// EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus, per row, the packed maxima
+// (value key of the logit at `eps` as temperature, ~index) of 64 subsets of the features, into `x_out` as 64-bit words
+// (the tied head in front of the greedy pick or of the spread sampler)
 // (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
 // NB = 2 (no prologue): rows 16..31 are a second B tile of the same weight fragments, so 17..32 rows read every weight
 // once; the partial sums of the two row tiles then lie behind each other in dynamic LDS.
@@ -342,6 +344,32 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         // the workgroup's range starts and ends on a multiple of four features, so a pair is inside it or outside it
         const int row = 16 * nb + r;
         const bool grp_ok = row < a.rows && fb >= f0 && fb < f1;
+        if constexpr (EPI == 2) {
+          // best (value, lowest index) over the wave's 8 features of this row, then one 64-bit atomic max into the
+          // slot of the tile (64 slots per row spread the contention; the two halves of a tile share a slot)
+          unsigned long long* best = (unsigned long long*)a.x_out;
+          const float temperature = a.eps;
+          unsigned long long key = 0ull;
+          if (grp_ok) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              if (fb + i < f1) {
+                float l = DT<bf16_t>::rnd(o[i]);
+                if (temperature != 1.0f) l = DT<bf16_t>::rnd(l / temperature);
+                l = DT<bf16_t>::rnd(fminf(fmaxf(l, -1e4f), 1e4f));
+                unsigned u = __float_as_uint(l);
+                u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                const unsigned long long k = ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (unsigned)(fb + i));
+                key = k > key ? k : key;
+              }
+            }
+          }
+          unsigned long long ok = __shfl_xor(key, 16, 64);
+          key = ok > key ? ok : key;
+          ok = __shfl_xor(key, 32, 64);
+          key = ok > key ? ok : key;
+          if (g == 0 && row < a.rows && key != 0ull) atomicMax(best + (size_t)row * 64 + (tile & 63), key);
+        }
         if (grp_ok) {
           bf16_t* yr = a.act + (size_t)row * a.ldact + fb;
           if (fb + 2 <= f1 && (a.ldact & 1) == 0) {
@@ -503,18 +531,24 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
     // two row tiles: the partial sums of both lie in dynamic LDS
     constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
     const size_t red2 = (size_t)2 * DA * 8 * 512 * sizeof(float);
-    FSTU_REQUIRE(pro == 0 && epi == 0, FSTU_ESHAPE, "%s: more than %d rows only without the norm prologue", name, FSTU_MAX_DECODE_ROWS);
-    static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, 0, 0, 2>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)red2);
-    FSTU_REQUIRE(attr_err == hipSuccess, (int)attr_err, "%s: %zu bytes of dynamic LDS refused", name, red2);
-    hipLaunchKernelGGL((glu_balanced_kernel<KSA, 0, 0, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,
-                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);
+    FSTU_REQUIRE(pro == 0, FSTU_ESHAPE, "%s: more than %d rows only without the norm prologue", name, FSTU_MAX_DECODE_ROWS);
+#define GLU_GO2(EPI)                                                                                                       \
+  do {                                                                                                                     \
+    static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, 0, EPI, 2>),    \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)red2);               \
+    FSTU_REQUIRE(attr_err == hipSuccess, (int)attr_err, "%s: %zu bytes of dynamic LDS refused", name, red2);               \
+    hipLaunchKernelGGL((glu_balanced_kernel<KSA, 0, EPI, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act,  \
+                       a.x_in, a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);      \
+  } while (0)
+    if (epi == 0) GLU_GO2(0); else if (epi == 2) GLU_GO2(2); else GLU_GO2(1);
+#undef GLU_GO2
     return FSTU_OK;
   }
   if (pro == 2) GLU_GO(2, 1);
   else if (pro && epi == 0) GLU_GO(1, 0);
   else if (pro) GLU_GO(1, 1);
   else if (epi == 0) GLU_GO(0, 0);
+  else if (epi == 2) GLU_GO(0, 2);
   else GLU_GO(0, 1);
 #undef GLU_GO
   return FSTU_OK;
@@ -588,7 +622,9 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
 extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                                   int rows, int N, int K, void* stream) {
   FSTU_REQUIRE(x && wp && y, FSTU_ENULL, "fstu_linear_packed: null pointer");
-  FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N), FSTU_ESHAPE, "fstu_linear_packed: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N) ||
+                   (norm_w == nullptr && rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(FSTU_MAX_DECODE_ROWS, K, N)),
+               FSTU_ESHAPE, "fstu_linear_packed: unsupported shape rows=%d K=%d N=%d", rows, K, N);
   FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && ldy % 4 == 0, FSTU_ESHAPE, "fstu_linear_packed: ldx=%d ldy=%d", ldx, ldy);
   FSTU_REQUIRE(norm_w == nullptr || ldx == K, FSTU_ESHAPE, "fstu_linear_packed: the norm prologue needs dense rows");
   FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(wp, 16) && fstu_aligned(y, 8), FSTU_EALIGN,
@@ -599,6 +635,24 @@ extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, fl
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
   if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
   return glu_launch(a, norm_w != nullptr ? 1 : 0, 1, "fstu_linear_packed", (hipStream_t)stream);
+}
+
+// The tied head over a packed embedding: logits = T(x W^T) for rows <= 32 and the rows' packed maxima at `temperature`
+// into best_ws (rows x 64 words, zero on entry), as fstu_head_maxima leaves them.
+extern "C" int fstu_head_maxima_packed(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                                       float temperature, void* best_ws, void* stream) {
+  FSTU_REQUIRE(x && wp && logits && best_ws, FSTU_ENULL, "fstu_head_maxima_packed: null pointer");
+  FSTU_REQUIRE(rows >= 1 && rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(rows > FSTU_MAX_DECODE_ROWS ? FSTU_MAX_DECODE_ROWS : rows, K, N),
+               FSTU_ESHAPE, "fstu_head_maxima_packed: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && temperature > 0.f, FSTU_ESHAPE, "fstu_head_maxima_packed: ldx=%d ldy=%d temperature=%g",
+               ldx, ldy, (double)temperature);
+  FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(wp, 16) && fstu_aligned(logits, 2) && fstu_aligned(best_ws, 8), FSTU_EALIGN,
+               "fstu_head_maxima_packed: x and wp must be 16-byte aligned, best_ws 8");
+  GluArgs a = {};
+  a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)logits; a.h = (const bf16_t*)x;
+  a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy;
+  a.x_out = (bf16_t*)best_ws; a.eps = temperature;     // EPI 2 reads them as the maxima and the temperature
+  return glu_launch(a, 0, 2, "fstu_head_maxima_packed", (hipStream_t)stream);
 }
 
 // y = T(h W^T) with h = rmsnorm(x') * norm_w and x' = T(x_in + T(sum of nslices fp32 slices)): the add+norm launch

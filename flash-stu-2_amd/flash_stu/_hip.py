@@ -58,6 +58,7 @@ SIGNATURES = {
     "fstu_sample": [_vp, _vp, _i64, _i, _i, _f, _i, _f, _i, _u64, _i, _i, _vp],
     "fstu_sample_ws_bytes": [],
     "fstu_head_maxima": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i, _vp],
+    "fstu_head_maxima_packed": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp],
     "fstu_sample_topk": [_vp, _i64, _vp, _vp, _vp, _i64, _i, _i, _f, _i, _f, _u64, _i, _vp],
     "fstu_head_argmax": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _i64, _i, _vp],
     "fstu_head_argmax_static": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp, _i64, _i, _vp],
@@ -673,6 +674,20 @@ def head_maxima(x: torch.Tensor, W: torch.Tensor, best_ws: torch.Tensor, tempera
     assert best_ws.dtype == torch.int64 and best_ws.numel() >= rows * 64
     _check(load().fstu_head_maxima(_p(x), ldx, _p(W), _p(logits), logits.stride(0), rows, N, K, float(temperature),
                                    _p(best_ws), _dt(x), _stream()), "fstu_head_maxima")
+    return logits
+
+
+def head_maxima_packed(x: torch.Tensor, wp: torch.Tensor, N: int, best_ws: torch.Tensor, temperature: float = 1.0,
+                       logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """head_maxima over a packed copy of the (N,K) head weight (pack_rows), rows <= 32."""
+    rows, ldx = _rows_view(x)
+    _dev(wp, best_ws)
+    K = x.shape[1]
+    if logits is None:
+        logits = torch.empty(rows, N, dtype=x.dtype, device=x.device)
+    assert x.dtype == torch.bfloat16 and best_ws.dtype == torch.int64 and best_ws.numel() >= rows * 64
+    _check(load().fstu_head_maxima_packed(_p(x), ldx, _p(wp), _p(logits), logits.stride(0), rows, N, K, float(temperature),
+                                          _p(best_ws), _stream()), "fstu_head_maxima_packed")
     return logits
 
 

@@ -259,6 +259,10 @@ class DecodeEngine:
                 arr[i].wp_gate = self._pack(layer.mlp.gate_proj.weight).data_ptr()
                 arr[i].wp_up = self._pack(layer.mlp.up_proj.weight).data_ptr()
                 arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
+                if isinstance(layer, AttentionLayer):
+                    arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+        if dt == torch.bfloat16 and B > _hip.MAX_DECODE_ROWS and self.lib.fstu_glu_packed_supported(_hip.MAX_DECODE_ROWS, d, V):
+            m.wp_emb = self._pack(model.lm_head.weight).data_ptr()      # 17..32 rows: the head streams a packed copy
         ch.arr, ch.desc = arr, m
         ch.mega = None
         if B > _hip.MAX_DECODE_ROWS:
@@ -288,8 +292,6 @@ class DecodeEngine:
                             "fstu_step_mega_prepare")
                 m.mega_ws = ws.data_ptr()
                 ch.mega = ws
-            else:
-                m.wp_emb = None
 
     # ------------------------------------------------------------------ eager step
     def step(self, tokens: torch.Tensor, pos: int, temperature, top_k, top_p, do_sample, seed, step_idx):

@@ -316,6 +316,13 @@ int fstu_head_argmax(const void* x, int ldx, const void* W, void* logits, int ld
 int fstu_head_maxima(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                      float temperature, void* best_ws, int dtype, void* stream);
 
+/* The same over a packed copy of the head weight (fstu_pack_rows of the (N,K) embedding; K in {256,512,768,1024,2048},
+ * bf16, rows <= 32): one workgroup per CU streams an equal share of the vocabulary against activations it holds in
+ * registers, so the activations are not fetched again for every 16 vocabulary rows.  Same logits as fstu_head_maxima up
+ * to the summation order over K; the same contract for best_ws.  Replaces lm_head at flash_stu/model.py:176. */
+int fstu_head_maxima_packed(const void* x, int ldx, const void* wp, void* logits, int ldy, int rows, int N, int K,
+                            float temperature, void* best_ws, void* stream);
+
 /* fstu_sample (do_sample = 1) for bf16 logits and 1 <= top_k <= 64, spread over (V / 2048) x B workgroups instead of one
  * workgroup per row; same draws.  logits: (B, V) rows ldl elements apart; best_ws: the maxima fstu_head_maxima left
  * for these logits at this temperature; samp_ws: fstu_sample_ws_bytes() bytes, zero-initialised once by the caller.
@@ -404,7 +411,8 @@ int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const
 
 /* y = T(x W^T) over packed W (N,K) with the same balanced launch; with norm_w != NULL, x is the residual stream
  * (dense rows) and h = rmsnorm(x) * norm_w is formed in the prologue (the sub-layer norm of stu_layer.py:81 /
- * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, rows <= 16, bf16. */
+ * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, bf16, rows <= 16
+ * (without norm_w: rows <= 32, the second 16 as another row tile of the same weight fragments). */
 int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                        int rows, int N, int K, void* stream);
 /* Split-K form of the down projection over packed weights (reference: flash_stu/modules/swiglu.py:22-29, down_proj):
@@ -491,7 +499,7 @@ typedef struct {
   void* best;               /* max(B,16)*64 64-bit words, zero-initialised once by the caller */
   void* samp_ws;            /* fstu_sample_ws_bytes() bytes, zero-initialised once by the caller, or NULL: top-k sampling
                                then runs one workgroup per row (fstu_sample) instead of fstu_sample_topk */
-  const void* wp_emb;       /* packed tied head (one-launch step) */
+  const void* wp_emb;       /* packed tied head (fstu_pack_rows of emb) or NULL: the head then reads emb row-major */
   void* x2;                 /* (B,d) second residual buffer (the stream ping-pongs x <-> x2); NULL: the add + norm
                                between sub-layers runs as launches of its own */
   int glu_packed;           /* != 0: layers with wp_gate and wp_up run their gate/up projection through fstu_glu_packed */

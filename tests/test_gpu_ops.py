@@ -842,6 +842,45 @@ def test_sample_topk_spread_equals_one_workgroup_per_row_and_oracle(hip, V, temp
     assert agree >= total - 1, (agree, total)
 
 
+@pytest.mark.parametrize("rows,K,V,temperature", [(32, 2048, 50257, 0.8), (8, 768, 50257, 1.0), (19, 1024, 4099, 1.3),
+                                                  (1, 256, 1031, 1.0), (16, 512, 6000, 0.7)])
+def test_head_maxima_over_packed_embedding(hip, rows, K, V, temperature):
+    """The head over a packed copy of the embedding (rows <= 32): logits within bf16 rounding of the float64 product;
+    the packed maxima name, per row, the first index of the largest transformed logit and every slot holds an element
+    of its row; fed to the spread sampler they give what fstu_sample draws from the same logits."""
+    g = gen(43)
+    x = dev(torch.randn(rows, K, generator=g).bfloat16())
+    Wc = (torch.randn(V, K, generator=g) * (3.0 / K ** 0.5)).bfloat16()
+    W = dev(Wc)
+    wp = hip.pack_rows(W)
+    best = torch.zeros(32 * 64, dtype=torch.int64, device="cuda")
+    logits = hip.head_maxima_packed(x, wp, V, best, temperature)
+    ref = x.double() @ W.double().t()
+    assert float((logits.double() - ref).abs().max()) <= 2.0 ** -8 * float(ref.abs().max()) * 1.01
+    t = logits.float()
+    if temperature != 1.0:
+        t = (t / temperature).bfloat16().float()
+    t = t.clamp(-1e4, 1e4).bfloat16().float()
+    b = best.view(32, 64)
+    assert int((b[rows:] != 0).sum()) == 0
+    idx_of = lambda w: 0xffffffff - (w & 0xffffffff)
+    top = b[:rows].max(dim=1).values
+    for r in range(rows):
+        i = int(idx_of(top[r]))
+        assert float(t[r, i]) == float(t[r].max()) and i == int((t[r] == t[r].max()).nonzero()[0])
+        slots = b[r][b[r] != 0]
+        ids = idx_of(slots)
+        assert int(ids.max()) < V and len(set(ids.tolist())) == len(ids)
+    if V >= 1024:
+        ws = hip.sample_ws("cuda")
+        out = torch.empty(rows, dtype=torch.int64, device="cuda")
+        hip.sample_topk(logits, best, ws, out, 40, temperature, None, seed=11, step=3)
+        want = torch.empty(rows, dtype=torch.int64, device="cuda")
+        hip.sample(logits, want, temperature, 40, None, True, seed=11, step=3)
+        assert torch.equal(out, want)
+        assert int((best != 0).sum()) == 0
+
+
 def test_sample_topk_spread_plateaus_and_errors(hip):
     """Long runs of equal logits overflow the per-chunk candidate lists: the row's last workgroup then draws from the
     whole row, with the same result as fstu_sample.  Arguments outside the fast path are refused."""
