@@ -41,6 +41,7 @@ int fstu_swa_decode_impl(const void* qkv, void* kring, void* vring, void* out, c
 int fstu_head_argmax_dyn(const void* x, int ldx, const void* W, void* logits, int ldy, int rows, int N, int K,
                          float temperature, void* best_ws, int64_t* tok_out, int64_t tok_stride, int* dyn, int advance,
                          int dtype, void* stream);
+int fstu_argmax_finish_launch(void* best_ws, int64_t* tok_out, int64_t tok_stride, int rows, int* dyn, int advance, void* stream);
 bool fstu_finish_embed_supported(int rows, int d, const void* table, const void* x, const void* w, const void* h);
 int fstu_finish_embed_rmsnorm(void* best_ws, int64_t* tok_out, int64_t tok_stride, const void* table, void* x, const void* w,
                               void* h, int* dyn, int rows, int d, int vocab, float eps, void* stream);

@@ -205,8 +205,7 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
   if (sample_spread_ok(m, do_sample, top_k)) {
     // the head leaves each row's packed maxima, the sampler spreads every row over the chip and advances {pos, step}
     // over the packed copy of the embedding where the model holds one: a workgroup keeps the activations in registers
-    // instead of fetching the 32 rows again for every 16 vocabulary rows (42 against 75 us at 2048-d; at 16 rows and
-    // fewer the row-major kernel is the faster one: 17.6 against 24 us at 768-d)
+    // instead of fetching the 32 rows again for every 16 vocabulary rows (40 against 75 us at 2048-d)
     if (m->wp_emb && fstu_glu_packed_supported(R, d, m->V))
       TIMED(PC_HEAD, fstu_head_maxima_packed(m->h, d, m->wp_emb, m->logits, m->V, B, m->V, d, temperature, m->best, stream));
     else if (fstu_linear_rows32_ok(m->h, d, m->emb, d, dt))
@@ -366,11 +365,22 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
     }
     TIMED(PC_NORM, fstu_add_rmsnorm(xc, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
+  // the head over the packed copy of the embedding where the model holds one: a workgroup keeps the activations in
+  // registers for its whole share of the vocabulary and issues one atomic per row (768-d, 8 rows: 14.2 us against
+  // 17.4 us for the row-major kernel, whose workgroups own 16 vocabulary rows each)
+  const bool head_packed = dt == FSTU_BF16 && m->wp_emb && m->best && fstu_glu_packed_supported(B, d, m->V);
   if (!do_sample && m->best) {
-    TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out,
-                                        tok_stride, dyn, (chain && g_chain_next) ? -1 : 1, dt, stream));
+    const int adv = (chain && g_chain_next) ? -1 : 1;   // < 0: the next step's first launch reduces the maxima
+    if (head_packed) {
+      TIMED(PC_HEAD, fstu_head_maxima_packed(m->h, d, m->wp_emb, m->logits, m->V, B, m->V, d, temperature, m->best, stream));
+      if (adv >= 0) STEP(fstu_argmax_finish_launch(m->best, tok_out, tok_stride, B, dyn, adv, stream));
+    } else {
+      TIMED(PC_HEAD, fstu_head_argmax_dyn(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, tok_out, tok_stride, dyn,
+                                          adv, dt, stream));
+    }
   } else if (sample_spread_ok(m, do_sample, top_k)) {
-    TIMED(PC_HEAD, fstu_head_maxima(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, dt, stream));
+    if (head_packed) TIMED(PC_HEAD, fstu_head_maxima_packed(m->h, d, m->wp_emb, m->logits, m->V, B, m->V, d, temperature, m->best, stream));
+    else TIMED(PC_HEAD, fstu_head_maxima(m->h, d, m->emb, m->logits, m->V, B, m->V, d, temperature, m->best, dt, stream));
     TIMED(PC_SAMPLE, fstu_sample_topk_dyn(m->logits, m->V, m->best, m->samp_ws, tok_out, tok_stride, B, m->V, temperature, top_k, top_p,
                                           seed, step, m->row0, dyn, 1, stream));
   } else {

@@ -283,6 +283,9 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     for (int u = 0; u < KSA; ++u) xa[u] = xrow ? *(const uint4*)(hl + u * 32) : make_uint4(0, 0, 0, 0);
   }
 
+  unsigned long long run_key[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) run_key[nb] = 0ull;
   for (int t0 = ta0; t0 < ta1; t0 += DA) {
 #pragma unroll
     for (int j = 0; j < DA; ++j) {
@@ -345,9 +348,8 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         const int row = 16 * nb + r;
         const bool grp_ok = row < a.rows && fb >= f0 && fb < f1;
         if constexpr (EPI == 2) {
-          // best (value, lowest index) over the wave's 8 features of this row, then one 64-bit atomic max into the
-          // slot of the tile (64 slots per row spread the contention; the two halves of a tile share a slot)
-          unsigned long long* best = (unsigned long long*)a.x_out;
+          // best (value, lowest index) of this lane's features so far; the workgroup's lanes are merged after its
+          // last tile
           const float temperature = a.eps;
           unsigned long long key = 0ull;
           if (grp_ok) {
@@ -364,11 +366,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
               }
             }
           }
-          unsigned long long ok = __shfl_xor(key, 16, 64);
-          key = ok > key ? ok : key;
-          ok = __shfl_xor(key, 32, 64);
-          key = ok > key ? ok : key;
-          if (g == 0 && row < a.rows && key != 0ull) atomicMax(best + (size_t)row * 64 + (tile & 63), key);
+          run_key[nb] = key > run_key[nb] ? key : run_key[nb];
         }
         if (grp_ok) {
           bf16_t* yr = a.act + (size_t)row * a.ldact + fb;
@@ -383,6 +381,35 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       }
     }
     if (t0 + DA < ta1) __syncthreads();
+  }
+  if constexpr (EPI == 2) {
+    // Per row: the best of the workgroup's whole feature range, then ONE 64-bit atomic max per row and workgroup into
+    // slot (workgroup & 63) of the row: the slots stay disjoint subsets of the vocabulary (4 workgroups each on a
+    // grid of 256), and the launch issues a few thousand atomics instead of one per row and half tile
+    unsigned long long* best = (unsigned long long*)a.x_out;
+    unsigned long long* keys = (unsigned long long*)red;          // 8 waves x NB x 16 rows
+    __syncthreads();                                              // the last reduction has read `red`
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      unsigned long long key = run_key[nb];
+      unsigned long long ok = __shfl_xor(key, 16, 64);
+      key = ok > key ? ok : key;
+      ok = __shfl_xor(key, 32, 64);
+      key = ok > key ? ok : key;
+      if (g == 0) keys[(w * NB + nb) * 16 + r] = key;
+    }
+    __syncthreads();
+    if (threadIdx.x < NB * 16) {
+      const int nb = threadIdx.x >> 4, rr = threadIdx.x & 15;
+      unsigned long long key = 0ull;
+#pragma unroll
+      for (int ww = 0; ww < 8; ++ww) {
+        const unsigned long long o = keys[(ww * NB + nb) * 16 + rr];
+        key = o > key ? o : key;
+      }
+      const int row = 16 * nb + rr;
+      if (row < a.rows && key != 0ull) atomicMax(best + (size_t)row * 64 + (wgi & 63), key);
+    }
   }
 }
 
@@ -560,6 +587,9 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
   // Features are dealt out in groups of 8: no 128-byte line is shared between two workgroups (HBM traffic of the
   // gate/up launch 1.00x the algorithmic bytes instead of 1.125x with groups of 4), at the price of workgroups of 32
   // and 40 features instead of 36 each.
+  // the head (thousands of tiles, one weight matrix: half the bytes in flight per workgroup of the gated pair) runs two
+  // workgroups per compute unit where registers and LDS allow it
+  if (epi == 2 && a.rows <= FSTU_MAX_DECODE_ROWS && a.d <= 1024) G *= 2;
   if (G > (a.I + 7) / 8) G = (a.I + 7) / 8;
   // a plain projection narrower than 16 features per CU (QKV at d = 768: 2304 features) gets one whole tile per
   // workgroup rather than half tiles on every CU: every workgroup repeats the norm prologue, and its operands come
