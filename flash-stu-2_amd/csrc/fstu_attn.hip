@@ -62,6 +62,30 @@ template <> __device__ __forceinline__ void load_vec<float, 32>(const float* p, 
   load_vec<float, 16>(p, o); load_vec<float, 16>(p + 16, o + 16);
 }
 
+// A head-dim vector dealt to the 8 lanes of a key group in 16-byte pieces: piece p of lane gl holds elements
+// p*8*E + gl*E .. +E (E = elements per 16 bytes), so every load instruction of the group covers 128 contiguous bytes of
+// the row.  (With DPL consecutive elements per lane a 256-byte row was touched in every other 16 bytes by each of the
+// two instructions: every line fetched twice.)
+template <typename T, int DPL, bool STREAM>
+__device__ __forceinline__ void load_pieces(const T* vec, int gl, float* o) {
+  constexpr int E = 16 / (int)sizeof(T);
+  if constexpr (DPL < E) {          // a row of less than 128 bytes: one short piece per lane
+    load_vec<T, DPL>(vec + gl * DPL, o);
+  } else {
+#pragma unroll
+    for (int p = 0; p < DPL / E; ++p) {
+      if constexpr (STREAM) load_vec_stream<T, E>(vec + p * 8 * E + gl * E, o + p * E);
+      else load_vec<T, E>(vec + p * 8 * E + gl * E, o + p * E);
+    }
+  }
+}
+template <typename T, int DPL>
+__device__ __forceinline__ int piece_elem(int gl, int i) {   // element of the head-dim vector held in slot i of lane gl
+  constexpr int E = 16 / (int)sizeof(T);
+  if constexpr (DPL < E) return gl * DPL + i;
+  return (i / E) * 8 * E + gl * E + (i % E);
+}
+
 // Online-softmax partial of one 8-lane key group.
 template <int DPL>
 struct Partial {
@@ -270,13 +294,13 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   const int at = (int)threadIdx.x - (NWAVES * 64 - HD);
   const T app_k = row[d + max(at, 0)], app_v = row[2 * d + max(at, 0)];
   float q[DPL];
-  load_vec<T, DPL>(row + gl * DPL, q);
+  load_pieces<T, DPL, false>(row, gl, q);
   const bool self_grp = append && (G == NGRP - 1);   // this group also takes the new token's own key
   // every group reads the new token's key and value (no branch, so nothing waits for them before the ring loads are
   // out); only the last group of the last wave gives them a weight
   float kself[DPL], vself[DPL];
-  load_vec<T, DPL>(row + d + gl * DPL, kself);
-  load_vec<T, DPL>(row + 2 * d + gl * DPL, vself);
+  load_pieces<T, DPL, false>(row + d, gl, kself);
+  load_pieces<T, DPL, false>(row + 2 * d, gl, vself);
   // Every wave keeps ONE running maximum for its 8 key groups (wave-wide max of the scores of an iteration), so the
   // groups of a wave merge by plain sums across lanes; only the NWAVES wave partials go through LDS.
   constexpr bool FAST = sizeof(T) == 2;
@@ -284,8 +308,8 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   const float scale = rsqrtf((float)HD), slope = slopes[h];
   const float inv_cap2l = softcap > 0.f ? 2.8853900817779268f / softcap : 0.f;
   const int j_end = append ? pos : pos + 1, slot_lo = lo % cap;
-  const T* kb = kring + hbase + gl * DPL;
-  const T* vb = vring + hbase + gl * DPL;
+  const T* kb = kring + hbase;
+  const T* vb = vring + hbase;
   float M = -INFINITY, l = 0.f, acc[DPL];
 #pragma unroll
   for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
@@ -308,13 +332,8 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
       const int j = min(jb + u, j_end - 1);
       int slot = slot_lo + (j - lo);
       slot = slot >= cap ? slot - cap : slot;
-      if constexpr (STREAM) {
-        load_vec_stream<T, DPL>(kb + (size_t)slot * HD, kk[u]);
-        load_vec_stream<T, DPL>(vb + (size_t)slot * HD, vv[u]);
-      } else {
-        load_vec<T, DPL>(kb + (size_t)slot * HD, kk[u]);
-        load_vec<T, DPL>(vb + (size_t)slot * HD, vv[u]);
-      }
+      load_pieces<T, DPL, STREAM>(kb + (size_t)slot * HD, gl, kk[u]);
+      load_pieces<T, DPL, STREAM>(vb + (size_t)slot * HD, gl, vv[u]);
     }
     float sc[SWA_U], mit = -INFINITY;
 #pragma unroll
@@ -362,7 +381,7 @@ swa_decode_kernel(const T* __restrict__ qkv, T* kring, T* vring, T* __restrict__
   __shared__ float wacc[NWAVES][HD];
   if (lane < 8) {
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) wacc[w][gl * DPL + i] = acc[i];
+    for (int i = 0; i < DPL; ++i) wacc[w][piece_elem<T, DPL>(gl, i)] = acc[i];
     if (lane == 0) { wm[w] = M; wl[w] = l; }
   }
   __syncthreads();
