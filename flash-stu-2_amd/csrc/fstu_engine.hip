@@ -178,14 +178,16 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
     const fstu_layer_desc& L = m->layers[l];
     if (L.kind == 0) {
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
-      TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
+      if (packed_mlp && L.wp_m_inputs) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_m_inputs, m->xp, d, B, d, d, stream));
+      else TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
       TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream));
     } else {
       if (packed_mlp && L.wp_qkv) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.w_qkv, m->qkv, 3 * d, 3 * d, d));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
                                          m->window, m->softcap, 1, dyn, dt, stream));
-      TIMED(PC_PROJ, proj(m->attn, d, L.w_proj, m->y, d, d, d));
+      if (packed_mlp && L.wp_proj) TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
+      else TIMED(PC_PROJ, proj(m->attn, d, L.w_proj, m->y, d, d, d));
     }
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
     TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));

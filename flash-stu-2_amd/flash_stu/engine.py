@@ -261,6 +261,9 @@ class DecodeEngine:
                 arr[i].wp_down = self._pack(layer.mlp.down_proj.weight).data_ptr()
                 if isinstance(layer, AttentionLayer):
                     arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
+                    arr[i].wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
+                elif mode == "lds":
+                    arr[i].wp_m_inputs = self._pack(layer.stu.m_inputs_t()).data_ptr()
         if dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(min(B, _hip.MAX_DECODE_ROWS), d, V):
             m.wp_emb = self._pack(model.lm_head.weight).data_ptr()      # the head streams a packed copy of the embedding
         ch.arr, ch.desc = arr, m
