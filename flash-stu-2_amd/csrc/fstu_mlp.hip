@@ -130,10 +130,13 @@ struct GluArgs {
   const bf16_t* norm_w;
   float eps;
   int nslices;
+  // EPI 2: per-row packed maxima (rows x 64 words, zero on entry) of the logits at this temperature
+  unsigned long long* best;
+  float temperature;
 };
 
 // EPI 0: act = gelu(gate)*up (two matrices);  1: y = x W^T;  2: y = x W^T plus, per row, the packed maxima
-// (value key of the logit at `eps` as temperature, ~index) of 64 subsets of the features, into `x_out` as 64-bit words
+// (value key of the logit at `temperature`, ~index) of 64 subsets of the features, into `best` as 64-bit words
 // (the tied head in front of the greedy pick or of the spread sampler)
 // (arguments passed one by one so that the command processor can preload the leading ones into SGPRs)
 // NB = 2 (no prologue): rows 16..31 are a second B tile of the same weight fragments, so 17..32 rows read every weight
@@ -142,10 +145,11 @@ template <int KSA, int PRO, int EPI, int NB = 1>
 __global__ void __launch_bounds__(512)
 glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, bf16_t* act, const bf16_t* x_in,
                     const void* delta, bf16_t* x_out, const bf16_t* norm_w, int rows, int d, int I, int ldh, int ldact,
-                    int fpw, float eps, int nslices) {
+                    int fpw, float eps, int nslices, unsigned long long* best, float temperature) {
   GluArgs a;
   a.h = h; a.wp_gate = wp_gate; a.wp_up = wp_up; a.act = act; a.rows = rows; a.d = d; a.I = I; a.ldh = ldh; a.ldact = ldact;
   a.fpw = fpw; a.x_in = x_in; a.delta = delta; a.x_out = x_out; a.norm_w = norm_w; a.eps = eps; a.nslices = nslices;
+  a.best = best; a.temperature = temperature;
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
@@ -350,7 +354,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         if constexpr (EPI == 2) {
           // best (value, lowest index) of this lane's features so far; the workgroup's lanes are merged after its
           // last tile
-          const float temperature = a.eps;
+          const float temperature = a.temperature;
           unsigned long long key = 0ull;
           if (grp_ok) {
 #pragma unroll
@@ -386,7 +390,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
     // Per row: the best of the workgroup's whole feature range, then ONE 64-bit atomic max per row and workgroup into
     // slot (workgroup & 63) of the row: the slots stay disjoint subsets of the vocabulary (4 workgroups each on a
     // grid of 256), and the launch issues a few thousand atomics instead of one per row and half tile
-    unsigned long long* best = (unsigned long long*)a.x_out;
+    unsigned long long* best = a.best;
     unsigned long long* keys = (unsigned long long*)red;          // 8 waves x NB x 16 rows
     __syncthreads();                                              // the last reduction has read `red`
 #pragma unroll
@@ -552,7 +556,7 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
       FSTU_REQUIRE(e == hipSuccess, (int)e, "%s: %zu bytes of dynamic LDS refused", name, shm);                  \
     }                                                                                                            \
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, GLUF>), dim3(G), dim3(512), shm, s, a.h, a.wp_gate, a.wp_up, a.act, a.x_in,    \
-                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);                    \
+                       a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices, a.best, a.temperature); \
   } while (0)
   if (a.rows > FSTU_MAX_DECODE_ROWS) {
     // two row tiles: the partial sums of both lie in dynamic LDS
@@ -565,7 +569,8 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)red2);               \
     FSTU_REQUIRE(attr_err == hipSuccess, (int)attr_err, "%s: %zu bytes of dynamic LDS refused", name, red2);               \
     hipLaunchKernelGGL((glu_balanced_kernel<KSA, 0, EPI, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act,  \
-                       a.x_in, a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices);      \
+                       a.x_in, a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices, a.best,  \
+                       a.temperature);                                                                                      \
   } while (0)
     if (epi == 0) GLU_GO2(0); else if (epi == 2) GLU_GO2(2); else GLU_GO2(1);
 #undef GLU_GO2
@@ -681,7 +686,7 @@ extern "C" int fstu_head_maxima_packed(const void* x, int ldx, const void* wp, v
   GluArgs a = {};
   a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)logits; a.h = (const bf16_t*)x;
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy;
-  a.x_out = (bf16_t*)best_ws; a.eps = temperature;     // EPI 2 reads them as the maxima and the temperature
+  a.best = (unsigned long long*)best_ws; a.temperature = temperature;
   return glu_launch(a, 0, 2, "fstu_head_maxima_packed", (hipStream_t)stream);
 }
 
