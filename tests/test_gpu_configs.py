@@ -219,7 +219,8 @@ def test_c5_shape_bf16_sampling_spread_over_the_chip(hip, rows):
 @pytest.mark.parametrize("rows", [17, 20, 32])
 def test_c5_shape_bf16_lds_teacher_forced(rows):
     """Same structure in bf16 with the recurrence state, logits within the bf16 tolerance.  17..32 rows step as one
-    chunk: the MLP once over all rows on the tiled GEMM kernel, the state operators on the two halves of the rows."""
+    chunk: projections, MLP and head once over all rows on the packed-weight kernels (two row tiles per weight
+    fragment), the state operators over all rows in one launch each."""
     from test_gpu_model import make_pair, prompt, _teacher_forced
     ocfg, w, model = make_pair(seed=2, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=256, n_layers=4,
                                n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
@@ -234,16 +235,18 @@ def test_c5_shape_bf16_lds_teacher_forced(rows):
     assert float(err.max()) <= 2e-2
 
 
-@pytest.mark.parametrize("d,heads", [(1024, 8), (2048, 16)])
-def test_c5_width_bf16_step_kernels(d, heads):
+@pytest.mark.parametrize("d,heads,rows", [(1024, 8, 8), (2048, 16, 8), (2048, 16, 32), (1024, 8, 21)])
+def test_c5_width_bf16_step_kernels(d, heads, rows):
     """Config 5's widths through the whole one-call step (head dim 128, d=2048 takes the 8-k-step variants of the
-    balanced gate/up kernel and its norm prologue): two layers, bf16, logits against the teacher-forced oracle."""
+    balanced gate/up kernel and its norm prologue; 17..32 rows take the packed-weight kernels with two row tiles per
+    weight fragment for the MLP, the small projections and the head): two layers, bf16, logits against the
+    teacher-forced oracle."""
     from test_gpu_model import make_pair, prompt, _teacher_forced
     ocfg, w, model = make_pair(seed=4, init="healthy", dtype=torch.bfloat16, mlp_scale=4, n_embd=d, n_layers=2,
                                n_heads=heads, window_size=32, num_eigh=24, seq_len=128, vocab_size=1511,
                                stu_decode_mode="lds")
     P, N = 12, 28
-    ids = prompt(8, P, ocfg.vocab_size, 6)
+    ids = prompt(rows, P, ocfg.vocab_size, 6)
     got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
     again = model.generate(ids.cuda(), max_length=P + N, do_sample=False)        # graph replay
     assert torch.equal(again, got)
@@ -254,7 +257,7 @@ def test_c5_width_bf16_step_kernels(d, heads):
 
 def test_c5_full_architecture_decode_against_full_sequence_recompute():
     """BASELINE config 5's full architecture (d=2048, 24 layers, 16 heads of 128, window 1024, L=8192, mlp_scale 12:
-    3.98 B parameters) at batch 32 (two row chunks of 16 on concurrent streams) with its sampler (top-k 40,
+    3.98 B parameters) at batch 32 (one chunk of 32 rows that reads every weight once) with its sampler (top-k 40,
     temperature 0.8, seeded stream); the CPU oracle is out of reach at this size, so the checks are size-independent:
     graph replay equals the kernel-by-kernel loop token for token, a second run reproduces the ids, and the stateful
     logits equal those of a full-sequence forward over the same tokens within the bf16 tolerance.  The prompt is
