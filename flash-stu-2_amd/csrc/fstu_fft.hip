@@ -71,6 +71,44 @@ template <int R> __device__ __forceinline__ void dft_inreg(cpx (&v)[R]) {
   }
 }
 
+// a * exp(-2 pi i k / 16) for a real a (the values mul_root16 gives for z = (a, 0))
+__device__ __forceinline__ cpx mul_root16_real(float a, int k) {
+  const float s = 0.70710678118654752f, c1 = 0.92387953251128674f, s1 = 0.38268343236508977f;
+  switch (k) {
+    case 0: return make_float2(a, 0.f);
+    case 1: return make_float2(c1 * a, -s1 * a);
+    case 2: return make_float2(a * s, -a * s);
+    case 3: return make_float2(s1 * a, -c1 * a);
+    case 4: return make_float2(0.f, -a);
+    case 5: return make_float2(-s1 * a, -c1 * a);
+    case 6: return make_float2(-a * s, -a * s);
+    default: return make_float2(-c1 * a, -s1 * a);
+  }
+}
+
+// The R-point DFT of a real input whose upper half is zero (a zero-padded signal in the first pass of its transform):
+// the first stage adds and subtracts nothing, v[j + R/2] = x[j] W_R^j, and the other stages run as always.
+// in: x[0 .. R/2) ; out: as dft_inreg.
+template <int R> __device__ __forceinline__ void dft_inreg_real_half(const float (&x)[R / 2], cpx (&v)[R]) {
+#pragma unroll
+  for (int j = 0; j < R / 2; ++j) {
+    v[j] = make_float2(x[j], 0.f);
+    v[j + R / 2] = mul_root16_real(x[j], j * (16 / R));
+  }
+#pragma unroll
+  for (int h = R / 4; h >= 1; h >>= 1) {
+#pragma unroll
+    for (int b0 = 0; b0 < R; b0 += 2 * h) {
+#pragma unroll
+      for (int j = 0; j < h; ++j) {
+        cpx a = v[b0 + j], b = v[b0 + j + h];
+        v[b0 + j] = cadd(a, b);
+        v[b0 + j + h] = mul_root16(csub(a, b), j * (8 / h));
+      }
+    }
+  }
+}
+
 // powers 1..R-1 of w = tw[r*ts] : the binary powers come from the table, the rest are products of two of them
 template <int R> __device__ __forceinline__ void twiddle_powers(cpx (&pw)[R], const cpx* __restrict__ tw, int e) {
   pw[0] = make_float2(1.f, 0.f);
@@ -99,8 +137,13 @@ template <int R> __host__ __device__ constexpr int lg_radix() { return R == 16 ?
 // The transform length and the stride are compile-time constants: the R points of a butterfly sit a fixed distance
 // apart in the padded column (q + q/16 slots; q = 1 only occurs with R = 16 on blocks that start at a multiple of
 // 16), so their addresses are one base and immediate offsets.
-template <int R, bool INV, int LQ, int LOGN>
+// HALF 1 (forward, first pass of a transform): the inputs are real and the upper half of the column is zero (a signal
+// of at most n/2 samples): only the lower half's real parts are read.  HALF 2 (inverse, last pass): only the lower
+// half of the column is wanted afterwards, the other outputs are neither stored nor (their last stage) computed.
+template <int R, bool INV, int LQ, int LOGN, int HALF = 0>
 __device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __restrict__ tw, int u) {
+  static_assert(HALF == 0 || (HALF == 1 && !INV) || (HALF == 2 && INV), "half-column passes: forward first, inverse last");
+  static_assert(HALF == 0 || LQ + lg_radix<R>() == LOGN, "half-column passes span the whole column");
   constexpr int LR = lg_radix<R>();
   constexpr int q = 1 << LQ;
   constexpr int TS = 1 << (LOGN - LQ - LR);   // table stride: w_Nb = tw[TS]
@@ -113,9 +156,16 @@ __device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __re
   constexpr bool twid = LQ > 0;
   if (twid) twiddle_powers<R>(pw, tw, r * TS);
   if (!INV) {
+    if constexpr (HALF == 1) {
+      float xr[R / 2];
 #pragma unroll
-    for (int m = 0; m < R; ++m) v[m] = p[m * ST];
-    dft_inreg<R>(v);
+      for (int m = 0; m < R / 2; ++m) xr[m] = p[m * ST].x;
+      dft_inreg_real_half<R>(xr, v);
+    } else {
+#pragma unroll
+      for (int m = 0; m < R; ++m) v[m] = p[m * ST];
+      dft_inreg<R>(v);
+    }
 #pragma unroll
     for (int k = 0; k < R; ++k) {
       cpx o = v[brev<R>(k)];
@@ -131,44 +181,50 @@ __device__ __forceinline__ void butterfly(cpx* __restrict__ col, const cpx* __re
     }
     dft_inreg<R>(v);
 #pragma unroll
-    for (int m = 0; m < R; ++m) p[m * ST] = cconj(v[brev<R>(m)]);
+    for (int m = 0; m < (HALF == 2 ? R / 2 : R); ++m) p[m * ST] = cconj(v[brev<R>(m)]);
   }
 }
 
 template <int LOGN> __host__ __device__ constexpr int col_stride() { return (1 << LOGN) + (1 << (LOGN - 4)); }
 
-template <int R, bool INV, int LQ, int LOGN, int NT>
+template <int R, bool INV, int LQ, int LOGN, int NT, int HALF = 0>
 __device__ __forceinline__ void run_pass(cpx* lds, const cpx* __restrict__ tw, int cols) {
   constexpr int LPER = LOGN - lg_radix<R>();   // log2 of butterflies per column
   const int total = cols << LPER;
   for (int w = threadIdx.x; w < total; w += NT)
-    butterfly<R, INV, LQ, LOGN>(lds + (size_t)(w >> LPER) * col_stride<LOGN>(), tw, w & ((1 << LPER) - 1));
+    butterfly<R, INV, LQ, LOGN, HALF>(lds + (size_t)(w >> LPER) * col_stride<LOGN>(), tw, w & ((1 << LPER) - 1));
   __syncthreads();
 }
 
 // LOGN = 4*a + rem: the first forward pass has radix 2^rem (if rem > 0), every other pass radix 16.  The last forward
 // pass and the first inverse pass work on the same 16 neighbours of a column (stride 1): callers that multiply by a
 // spectrum in between skip both here and do the three steps in registers (fft_middle).
-template <int LOGN, int NT, bool SKIP_LAST>
+// HALF_COL: the columns hold real signals of at most n/2 samples (forward: the pass that spans the whole column reads
+// only those; inverse: only the lower half of the result is produced).
+template <int LOGN, int NT, bool SKIP_LAST, bool HALF_COL = false>
 __device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw, int cols) {
   constexpr int REM = LOGN & 3, TOP = LOGN - REM;
-  if constexpr (REM == 1) run_pass<2, false, LOGN - 1, LOGN, NT>(lds, tw, cols);
-  if constexpr (REM == 2) run_pass<4, false, LOGN - 2, LOGN, NT>(lds, tw, cols);
-  if constexpr (REM == 3) run_pass<8, false, LOGN - 3, LOGN, NT>(lds, tw, cols);
-  if constexpr (TOP >= 12) run_pass<16, false, 8, LOGN, NT>(lds, tw, cols);
-  if constexpr (TOP >= 8) run_pass<16, false, 4, LOGN, NT>(lds, tw, cols);
+  constexpr int H = HALF_COL ? 1 : 0;
+  constexpr int H16A = (REM == 0 && TOP == 12) ? H : 0, H16B = (REM == 0 && TOP == 8) ? H : 0;
+  if constexpr (REM == 1) run_pass<2, false, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 2) run_pass<4, false, LOGN - 2, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 3) run_pass<8, false, LOGN - 3, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (TOP >= 12) run_pass<16, false, 8, LOGN, NT, H16A>(lds, tw, cols);
+  if constexpr (TOP >= 8) run_pass<16, false, 4, LOGN, NT, H16B>(lds, tw, cols);
   if constexpr (!SKIP_LAST) run_pass<16, false, 0, LOGN, NT>(lds, tw, cols);
 }
 
-template <int LOGN, int NT, bool SKIP_FIRST>
+template <int LOGN, int NT, bool SKIP_FIRST, bool HALF_COL = false>
 __device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw, int cols) {
   constexpr int REM = LOGN & 3, TOP = LOGN - REM;
+  constexpr int H = HALF_COL ? 2 : 0;
+  constexpr int H16A = (REM == 0 && TOP == 12) ? H : 0, H16B = (REM == 0 && TOP == 8) ? H : 0;
   if constexpr (!SKIP_FIRST) run_pass<16, true, 0, LOGN, NT>(lds, tw, cols);
-  if constexpr (TOP >= 8) run_pass<16, true, 4, LOGN, NT>(lds, tw, cols);
-  if constexpr (TOP >= 12) run_pass<16, true, 8, LOGN, NT>(lds, tw, cols);
-  if constexpr (REM == 1) run_pass<2, true, LOGN - 1, LOGN, NT>(lds, tw, cols);
-  if constexpr (REM == 2) run_pass<4, true, LOGN - 2, LOGN, NT>(lds, tw, cols);
-  if constexpr (REM == 3) run_pass<8, true, LOGN - 3, LOGN, NT>(lds, tw, cols);
+  if constexpr (TOP >= 8) run_pass<16, true, 4, LOGN, NT, H16B>(lds, tw, cols);
+  if constexpr (TOP >= 12) run_pass<16, true, 8, LOGN, NT, H16A>(lds, tw, cols);
+  if constexpr (REM == 1) run_pass<2, true, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 2) run_pass<4, true, LOGN - 2, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 3) run_pass<8, true, LOGN - 3, LOGN, NT, H>(lds, tw, cols);
 }
 
 // 16 spectrum values of 16 neighbouring positions (128 contiguous bytes)
@@ -292,7 +348,7 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
   const bool yt_fast = y_st == 1;
   if (K == 1) {
     fft_middle<LOGN, NT>(fft_lds, spec, c0, ncol);
-    fft_inverse<LOGN, NT, true>(fft_lds, tw, cols);
+    fft_inverse<LOGN, NT, true, true>(fft_lds, tw, cols);   // outputs t < Tn <= n/2 only
     T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc;
     T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc : nullptr;
     for (int idx = threadIdx.x; idx < cols * Tn; idx += NT) {
@@ -331,7 +387,7 @@ fft_conv_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, size_t x_sc, 
       }
     }
     __syncthreads();
-    fft_inverse<LOGN, NT, true>(fft_lds, tw, 1);
+    fft_inverse<LOGN, NT, true, true>(fft_lds, tw, 1);      // outputs t < Tn <= n/2 only
     T* yb = y + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk;
     T* yb2 = (mode == 2) ? y2 + (size_t)b * y_sb + (size_t)c0 * y_sc + (size_t)k * y_sk : nullptr;
     for (int t = threadIdx.x; t < Tn; t += NT) {
@@ -415,15 +471,21 @@ __device__ __forceinline__ void rows_groups(cpx* lds, const cpx* __restrict__ sp
       const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
       if (t < Tn) rows_scatter<T, LOGN, NT, G, 0>(lds, io[r], t, part);
     }
-    // zero padding behind the sequence
-    for (int idx = threadIdx.x; idx < COLS * (n - Tn); idx += NT) {
-      const int col = idx / (n - Tn), t = Tn + idx - col * (n - Tn);
+    // zero padding behind the sequence, up to half the column: the first forward pass knows that the upper half of a
+    // column is zero and the inputs real and reads neither, the last inverse pass produces the lower half only.
+    // (At 8192 points only the inverse: the forward pass has radix 2 there and little to save, and the kernel with it
+    // needs 139 registers instead of 126, which leaves one workgroup per compute unit instead of two: 3.0 against
+    // 2.6 ms.)
+    constexpr bool HF = LOGN != 13, HI = true;
+    constexpr int pad_to = HF ? n / 2 : n;
+    for (int idx = threadIdx.x; idx < COLS * (pad_to - Tn); idx += NT) {
+      const int col = idx / (pad_to - Tn), t = Tn + idx - col * (pad_to - Tn);
       lds[(size_t)col * col_stride<LOGN>() + phys(t)] = make_float2(0.f, 0.f);
     }
     __syncthreads();
-    fft_forward<LOGN, NT, true>(lds, tw, COLS);
+    fft_forward<LOGN, NT, true, HF>(lds, tw, COLS);
     fft_middle<LOGN, NT>(lds, spec, c0 + G * COLS, COLS);
-    fft_inverse<LOGN, NT, true>(lds, tw, COLS);
+    fft_inverse<LOGN, NT, true, HI>(lds, tw, COLS);
 #pragma unroll
     for (int r = 0; r < NV; ++r) {
       const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
