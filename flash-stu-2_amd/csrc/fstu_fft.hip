@@ -201,12 +201,14 @@ __device__ __forceinline__ void run_pass(cpx* lds, const cpx* __restrict__ tw, i
 // spectrum in between skip both here and do the three steps in registers (fft_middle).
 // HALF_COL: the columns hold real signals of at most n/2 samples (forward: the pass that spans the whole column reads
 // only those; inverse: only the lower half of the result is produced).
-template <int LOGN, int NT, bool SKIP_LAST, bool HALF_COL = false>
+// NO_R2 (lengths with a radix-2 pass): the caller performs that pass itself while it writes the column (forward) or
+// collects the results (inverse).
+template <int LOGN, int NT, bool SKIP_LAST, bool HALF_COL = false, bool NO_R2 = false>
 __device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw, int cols) {
   constexpr int REM = LOGN & 3, TOP = LOGN - REM;
   constexpr int H = HALF_COL ? 1 : 0;
   constexpr int H16A = (REM == 0 && TOP == 12) ? H : 0, H16B = (REM == 0 && TOP == 8) ? H : 0;
-  if constexpr (REM == 1) run_pass<2, false, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 1 && !NO_R2) run_pass<2, false, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
   if constexpr (REM == 2) run_pass<4, false, LOGN - 2, LOGN, NT, H>(lds, tw, cols);
   if constexpr (REM == 3) run_pass<8, false, LOGN - 3, LOGN, NT, H>(lds, tw, cols);
   if constexpr (TOP >= 12) run_pass<16, false, 8, LOGN, NT, H16A>(lds, tw, cols);
@@ -214,7 +216,7 @@ __device__ __forceinline__ void fft_forward(cpx* lds, const cpx* __restrict__ tw
   if constexpr (!SKIP_LAST) run_pass<16, false, 0, LOGN, NT>(lds, tw, cols);
 }
 
-template <int LOGN, int NT, bool SKIP_FIRST, bool HALF_COL = false>
+template <int LOGN, int NT, bool SKIP_FIRST, bool HALF_COL = false, bool NO_R2 = false>
 __device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw, int cols) {
   constexpr int REM = LOGN & 3, TOP = LOGN - REM;
   constexpr int H = HALF_COL ? 2 : 0;
@@ -222,7 +224,7 @@ __device__ __forceinline__ void fft_inverse(cpx* lds, const cpx* __restrict__ tw
   if constexpr (!SKIP_FIRST) run_pass<16, true, 0, LOGN, NT>(lds, tw, cols);
   if constexpr (TOP >= 8) run_pass<16, true, 4, LOGN, NT, H16B>(lds, tw, cols);
   if constexpr (TOP >= 12) run_pass<16, true, 8, LOGN, NT, H16A>(lds, tw, cols);
-  if constexpr (REM == 1) run_pass<2, true, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
+  if constexpr (REM == 1 && !NO_R2) run_pass<2, true, LOGN - 1, LOGN, NT, H>(lds, tw, cols);
   if constexpr (REM == 2) run_pass<4, true, LOGN - 2, LOGN, NT, H>(lds, tw, cols);
   if constexpr (REM == 3) run_pass<8, true, LOGN - 3, LOGN, NT, H>(lds, tw, cols);
 }
@@ -430,32 +432,43 @@ template <> struct RowVec<float> {
 // 14 % faster than one), n = 8192 one (two with 1024 threads spill registers and were 12 % slower)
 template <int LOGN> __host__ __device__ constexpr int fft_lcols() { return LOGN >= 13 ? 0 : LOGN == 12 ? 1 : (12 - LOGN > 4 ? 4 : 12 - LOGN); }
 
-template <typename T, int LOGN, int NT, int G, int E>
-__device__ __forceinline__ void rows_scatter(cpx* lds, const unsigned (&w)[4], int t, int part) {
+// R2: the radix-2 first pass of the forward transform happens here.  Its butterfly pairs sample t with the zero at
+// t + n/2, so position t keeps x and position t + n/2 receives x * w^t (wt = tw[t]): the same values the pass would
+// leave, without its trip through LDS and its barrier.
+template <typename T, int LOGN, int NT, int G, int E, bool R2 = false>
+__device__ __forceinline__ void rows_scatter(cpx* lds, const unsigned (&w)[4], int t, int part, cpx wt = make_float2(1.f, 0.f)) {
   constexpr int COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, VR = (COLS > CH ? COLS : CH) / CH;
+  constexpr int n = 1 << LOGN;
   if constexpr (E < CH) {
     // VR == 1: the column is known at compile time; VR > 1 (one group): it follows the row piece
-    if constexpr (VR == 1) {
-      constexpr int col = E - G * COLS;
-      if constexpr (col >= 0 && col < COLS) lds[(size_t)col * col_stride<LOGN>() + phys(t)] = make_float2(RowVec<T>::template get<E>(w), 0.f);
-    } else {
-      lds[(size_t)(part * CH + E) * col_stride<LOGN>() + phys(t)] = make_float2(RowVec<T>::template get<E>(w), 0.f);
+    constexpr int col_ct = E - G * COLS;
+    if constexpr (VR > 1 || (col_ct >= 0 && col_ct < COLS)) {
+      const int col = VR > 1 ? part * CH + E : col_ct;
+      const float xv = RowVec<T>::template get<E>(w);
+      cpx* c = lds + (size_t)col * col_stride<LOGN>();
+      c[phys(t)] = make_float2(xv, 0.f);
+      if constexpr (R2) c[phys(t + n / 2)] = make_float2(xv * wt.x, xv * wt.y);
     }
-    rows_scatter<T, LOGN, NT, G, E + 1>(lds, w, t, part);
+    rows_scatter<T, LOGN, NT, G, E + 1, R2>(lds, w, t, part, wt);
   }
 }
 
-template <typename T, int LOGN, int NT, int G, int E>
-__device__ __forceinline__ void rows_gather(const cpx* lds, unsigned (&w)[4], int t, int part, int mode) {
+// R2: the radix-2 last pass of the inverse transform happens here, for the wanted lower half only:
+// y[t] = u[t] + u[t + n/2] * conj(w^t).
+template <typename T, int LOGN, int NT, int G, int E, bool R2 = false>
+__device__ __forceinline__ void rows_gather(const cpx* lds, unsigned (&w)[4], int t, int part, int mode, cpx wt = make_float2(1.f, 0.f)) {
   constexpr int COLS = 1 << fft_lcols<LOGN>(), CH = RowVec<T>::CH, VR = (COLS > CH ? COLS : CH) / CH;
+  constexpr int n = 1 << LOGN;
   if constexpr (E < CH) {
     constexpr int col_ct = E - G * COLS;
     if constexpr (VR > 1 || (col_ct >= 0 && col_ct < COLS)) {
       const int col = VR > 1 ? part * CH + E : col_ct;
-      const cpx z = lds[(size_t)col * col_stride<LOGN>() + phys(t)];
+      const cpx* c = lds + (size_t)col * col_stride<LOGN>();
+      cpx z = c[phys(t)];
+      if constexpr (R2) z = cadd(z, cmulc(c[phys(t + n / 2)], wt));
       RowVec<T>::template put<E>(w, mode == 0 ? DT<T>::rnd(z.x) + DT<T>::rnd(z.y) : z.x);
     }
-    rows_gather<T, LOGN, NT, G, E + 1>(lds, w, t, part, mode);
+    rows_gather<T, LOGN, NT, G, E + 1, R2>(lds, w, t, part, mode, wt);
   }
 }
 
@@ -466,37 +479,46 @@ __device__ __forceinline__ void rows_groups(cpx* lds, const cpx* __restrict__ sp
   constexpr int VR = CHW / CH, NG = CHW / COLS;
   if constexpr (G < NG) {
     if (G > 0) __syncthreads();   // the previous group's results have been collected
+    constexpr bool R2 = (LOGN & 3) == 1;   // the radix-2 pass of these lengths rides on the scatter and the gather
 #pragma unroll
     for (int r = 0; r < NV; ++r) {
       const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
-      if (t < Tn) rows_scatter<T, LOGN, NT, G, 0>(lds, io[r], t, part);
+      if (t < Tn) {
+        if constexpr (R2) rows_scatter<T, LOGN, NT, G, 0, true>(lds, io[r], t, part, tw[t]);
+        else rows_scatter<T, LOGN, NT, G, 0>(lds, io[r], t, part);
+      }
     }
     // zero padding behind the sequence, up to half the column: the first forward pass knows that the upper half of a
     // column is zero and the inputs real and reads neither, the last inverse pass produces the lower half only.
-    // (At 8192 points only the inverse: the forward pass has radix 2 there and little to save, and the kernel with it
-    // needs 139 registers instead of 126, which leaves one workgroup per compute unit instead of two: 3.0 against
-    // 2.6 ms.)
-    constexpr bool HF = LOGN != 13, HI = true;
-    constexpr int pad_to = HF ? n / 2 : n;
+    // (At 512 and 8192 points those passes have radix 2: they are not run at all, the scatter above and the gather
+    // below do their work on the way.)
+    constexpr bool HF = !R2, HI = !R2;
+    constexpr int pad_to = n / 2;
     for (int idx = threadIdx.x; idx < COLS * (pad_to - Tn); idx += NT) {
       const int col = idx / (pad_to - Tn), t = Tn + idx - col * (pad_to - Tn);
-      lds[(size_t)col * col_stride<LOGN>() + phys(t)] = make_float2(0.f, 0.f);
+      cpx* c = lds + (size_t)col * col_stride<LOGN>();
+      c[phys(t)] = make_float2(0.f, 0.f);
+      if constexpr (R2) c[phys(t + n / 2)] = make_float2(0.f, 0.f);   // what the radix-2 pass makes of a zero pair
     }
     __syncthreads();
-    fft_forward<LOGN, NT, true, HF>(lds, tw, COLS);
+    fft_forward<LOGN, NT, true, HF, R2>(lds, tw, COLS);
     fft_middle<LOGN, NT>(lds, spec, c0 + G * COLS, COLS);
-    fft_inverse<LOGN, NT, true, HI>(lds, tw, COLS);
+    fft_inverse<LOGN, NT, true, HI, R2>(lds, tw, COLS);
 #pragma unroll
     for (int r = 0; r < NV; ++r) {
       const int q = threadIdx.x + r * NT, t = q / VR, part = q % VR;
-      if (t < Tn) rows_gather<T, LOGN, NT, G, 0>(lds, io[r], t, part, mode);   // over the inputs this group consumed
+      if (t < Tn) {                                   // over the inputs this group consumed
+        if constexpr (R2) rows_gather<T, LOGN, NT, G, 0, true>(lds, io[r], t, part, mode, tw[t]);
+        else rows_gather<T, LOGN, NT, G, 0>(lds, io[r], t, part, mode);
+      }
     }
     rows_groups<T, LOGN, NT, NV, G + 1>(lds, spec, tw, io, Tn, c0, mode);
   }
 }
 
+// (8192 points: two workgroups of 512 threads share a compute unit, 70 KB of LDS each, so a thread may hold 128 registers)
 template <typename T, int LOGN, int NT>
-__global__ void __launch_bounds__(NT)
+__global__ void __launch_bounds__(NT, LOGN == 13 ? 4 : 1)
 fft_conv_rows_kernel(const T* __restrict__ x, size_t x_sb, size_t x_st, const cpx* __restrict__ spec, T* __restrict__ y,
                      size_t y_sb, size_t y_st, const cpx* __restrict__ tw, int Tn, int mode, int xcd_remap) {
   extern __shared__ cpx fft_lds[];

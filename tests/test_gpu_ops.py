@@ -234,7 +234,8 @@ def test_stu_conv_direct(hip, dtype, B, T, d, L):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("B,T,d,L", [(2, 100, 96, 128), (1, 64, 256, 1024), (3, 120, 100, 128), (2, 17, 5, 64),
                                      (2, 512, 64, 512), (1, 1000, 48, 1024), (1, 2048, 32, 2048), (1, 4096, 8, 4096),
-                                     (1, 3000, 4, 8192), (1, 8192, 2, 8192), (4, 4096, 1024, 4096), (4, 8192, 1024, 8192)])
+                                     (1, 3000, 4, 8192), (1, 8192, 2, 8192), (4, 4096, 1024, 4096), (4, 8192, 1024, 8192),
+                                     (2, 200, 64, 256), (3, 256, 96, 256), (2, 3500, 2048, 4096)])
 def test_stu_conv_fft(hip, dtype, B, T, d, L):
     """The FFT form against the oracle's rfft/irfft convolution, every transform length 64..16384
     (radix splits 4*16, 8*16, 16*16, 2*16*16 ... 4*16*16*16), ragged channel counts, T < L and T == L; the last two
