@@ -59,7 +59,8 @@ def decode_step_bytes(cfg, B, t, mode, S):
 def timed_decode(eng, tokens, pos, step_idx, W, K, S, torch, temperature=1.0, top_k=None, top_p=None, do_sample=False, seed=0,
                  use_graph=True):
     """W warm-up steps, then K timed steps starting at position `pos`.  Returns (seconds for the K steps, next position).
-    Graph replay: graphs of S steps, the remainders (W % S before, K % S after) as single-step graphs."""
+    Graph replay: graphs of S steps; the warm-up's remainder (W % S) as single-step graphs, the timed steps' remainder
+    (K % S) as one more graph of that many steps."""
     if not use_graph:
         def run(n, p):
             for i in range(n):
@@ -74,6 +75,9 @@ def timed_decode(eng, tokens, pos, step_idx, W, K, S, torch, temperature=1.0, to
     eng.graph_begin(tokens, pos, step_idx, temperature, top_k, top_p, do_sample, seed, steps_per_graph=1)
     if w8 + k8 > 0 and S > 1:
         eng.graph_begin(tokens, pos + w1, step_idx + w1, temperature, top_k, top_p, do_sample, seed, steps_per_graph=S, keep=True)
+    if k1 > 1:
+        eng.graph_begin(tokens, pos + W + k8 * S, step_idx + W + k8 * S, temperature, top_k, top_p, do_sample, seed,
+                        steps_per_graph=k1, keep=True)
     for _ in range(w1):
         eng.graph_step(1)
     for _ in range(w8):
@@ -84,8 +88,8 @@ def timed_decode(eng, tokens, pos, step_idx, W, K, S, torch, temperature=1.0, to
     t0 = time.perf_counter()
     for _ in range(k8):
         eng.graph_step(S)
-    for _ in range(k1):
-        eng.graph_step(1)
+    if k1:
+        eng.graph_step(k1)
     eng.graph_sync()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
