@@ -1155,6 +1155,39 @@ def test_stu_bank_step_lds(hip, dtype):
     assert worst <= tol * float(rp.float().abs().max()), worst
 
 
+def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
+    """More than 32 rows, 17..32 rows with a norm prologue, and widths outside the packed kernels' set are refused on
+    the host before any launch."""
+    g = gen(66)
+    d, I = 256, 512
+    wg = dev((torch.randn(I, d, generator=g) / 16).bfloat16())
+    pg = hip.pack_rows(wg)
+    pd = hip.pack_rows(dev((torch.randn(d, I, generator=g) / 16).bfloat16()))
+    nw = dev(torch.ones(d).bfloat16())
+    x33 = dev(torch.randn(33, d, generator=g).bfloat16())
+    x20 = dev(torch.randn(20, d, generator=g).bfloat16())
+    best = torch.zeros(64 * 64, dtype=torch.int64, device="cuda")
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.glu_packed(x33, pg, pg, I)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.down_packed_splitk(dev(torch.randn(33, I, generator=g).bfloat16()), pd, d, 16)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.linear_packed(x33, pg, I)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.linear_packed(x20, pg, I, nw, 1e-6)             # the norm prologue stops at 16 rows
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.glu_packed_norm(x20, None, nw, 1e-6, pg, pg, I)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.head_maxima_packed(x33, pg, I, best)
+    x320 = dev(torch.randn(20, 320, generator=g).bfloat16())    # K = 320 is not one of the packed kernels' widths
+    w320 = hip.pack_rows(dev((torch.randn(I, 320, generator=g) / 16).bfloat16()))
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.linear_packed(x320, w320, I)
+    # and what they do take at 20 rows still runs
+    assert hip.linear_packed(x20, pg, I).shape == (20, I)
+    assert hip.glu_packed(x20, pg, pg, I).shape == (20, I)
+
+
 @pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8),
                                          (32, 768, 9216, 16), (19, 1024, 4096, 8), (32, 2048, 24576, 16), (17, 48, 1024, 4)])
 def test_down_packed_splitk(hip, rows, d, I, ks):
