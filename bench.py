@@ -193,8 +193,11 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
         us = e0.elapsed_time(e1) * 1e3 / n
         glu_bytes = 2 * I * d * 2 + rows * d * 2 + rows * I * 2
         gbps = glu_bytes / (us * 1e-6) / 1e9
+        # HBM bytes per launch from two rocprofv3 --pmc runs (FETCH_SIZE x2.000, WRITE_SIZE x1.000 against the library's
+        # plain copy kernel), measured offline for config 5's shape: profiles/decode_c5_hbm_traffic_pmc.txt
+        traffic = 204052787 if packed and (d, I, rows) == (2048, 24576, 32) else None
         return {"bound": "hbm", "kernel": name,
-                "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+                "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
                 "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n, "rows_per_launch": rows}
     ms_c, n_c = ctypes.c_double(), ctypes.c_int()
     torch.cuda.synchronize()
