@@ -281,7 +281,6 @@ def run_lm(args, torch, _hip, which):
             res["prefill_tokens_per_s"] = B * P / statistics.median(warm)
         use_graph = eng.graph_supported() and not args.no_graph
         dt_s, pos = timed_decode(eng, tokens, P, 1, W, K, args.graph_steps, torch, use_graph=use_graph, **sampling)
-        eng.check_status()
         res["ms_per_step"] = dt_s / K * 1e3
         res["value"] = B * K / dt_s
         S = cfg.stu_lds_state_dim
@@ -302,8 +301,7 @@ def run_lm(args, torch, _hip, which):
         "config": {"workload": label, "mlp_scale": cfg.mlp_scale, "params": res["params"], "batch": B, "prompt": P,
                    "stu_decode_mode": stu_mode, "stu_prefill_mode": args.stu_prefill, "hip_graph": res["hip_graph"],
                    "graph_steps": args.graph_steps, "stu_state_dim": cfg.stu_lds_state_dim if stu_mode == "lds" else None,
-                   "stu_fir_taps": cfg.stu_lds_fir_taps if stu_mode == "lds" else None,
-                   "one_launch_step": os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") == "1"},
+                   "stu_fir_taps": cfg.stu_lds_fir_taps if stu_mode == "lds" else None},
         "step_roofline": res["step_roofline"],
         "prefill_tokens_per_s": res.get("prefill_tokens_per_s"), "prefill_ms": res.get("prefill_ms"),
         "prefill_first_call_ms": res["prefill_first_call_ms"],

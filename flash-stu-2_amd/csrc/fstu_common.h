@@ -68,12 +68,6 @@ int fstu_stu_res_inproj_step_dyn(const void* x_in, const float* slices, int nsli
                                  const void* Mt, float* state, const float* a, const float* ce, const float* co, void* ring,
                                  const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int K, int t,
                                  const int* dyn, const int* pos_dyn, void* stream);
-// the whole step as one persistent launch: tokens / tok_out are the column-0 bases of the input and output views, the
-// step reads column `pos` (dyn[0] when dyn is given) of the first and writes the same column of the second
-bool fstu_step_mega_ok(const fstu_model_desc* m);
-int fstu_step_mega_launch(const fstu_model_desc* m, int64_t* tokens, int64_t* tok_out, int64_t tok_stride, int pos,
-                          float temperature, int greedy, int* dyn, void* stream);
-
 static inline bool fstu_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 // the optional exact head of the distilled filter: ring, taps and their count go together; count a power of two in 8..1024
 static inline bool fstu_fir_ok(const void* ring, const float* fir, int taps) {

@@ -259,19 +259,6 @@ static int decode_step_impl(const fstu_model_desc* m, const int64_t* tok_in, int
   }
   if (m->B > FSTU_MAX_DECODE_ROWS)
     return decode_step_wide(m, tok_in, tok_out, tok_stride, pos, temperature, top_k, top_p, do_sample, seed, step, dyn, stream);
-  if (fstu_step_mega_ok(m)) {
-    // the whole step as one persistent launch; sampling (when asked for) reads the logits it leaves
-    const int greedy = do_sample ? 0 : 1;
-    int64_t* in0 = const_cast<int64_t*>(tok_in) - (dyn ? 0 : pos);
-    int64_t* out0 = tok_out - (dyn ? 0 : pos);
-    TIMED(PC_GLU, fstu_step_mega_launch(m, in0, out0, tok_stride, pos, temperature, greedy, dyn, stream));
-    if (!greedy) {
-      TIMED(PC_SAMPLE, fstu_sample_dyn(m->logits, tok_out, tok_stride, m->B, m->V, temperature, top_k, top_p, do_sample, seed, step,
-                                       m->row0, dyn, m->dtype, stream));
-      if (dyn) STEP(fstu_advance_dyn(dyn, stream));
-    }
-    return FSTU_OK;
-  }
   // x = embedding rows, h = norm(x) with the first layer's norm weight
   const bool chain = chain_ok(m, do_sample, dyn);
   if (chain && g_chain_prev)
@@ -416,9 +403,8 @@ extern "C" int fstu_decode_graph_create(const fstu_model_desc* m, int64_t* token
   FSTU_REQUIRE(pos0 >= 0 && nsteps >= 1 && nsteps <= 64, FSTU_EARG, "fstu_decode_graph_create: pos0=%d nsteps=%d (1..64)", pos0, nsteps);
   hipStream_t s = (hipStream_t)stream;
   // One graph per parity of the first position: the STU launches carry their parity as an argument.  A graph of an
-  // even number of steps always starts on the parity of pos0, so the other one is not captured.  (The one-launch step
-  // reads the position on the device: one graph serves both parities.)
-  const bool baked = m->stu_mode == 1 && !fstu_step_mega_ok(m);
+  // even number of steps always starts on the parity of pos0, so the other one is not captured.
+  const bool baked = m->stu_mode == 1;
   fstu_graph* h = new fstu_graph{{nullptr, nullptr}, {nullptr, nullptr}, pos0, nsteps, baked};
   for (int par = 0; par < 2; ++par) {
     if (!baked && par == 1) break;

@@ -71,9 +71,6 @@ SIGNATURES = {
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed_res": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
-    "fstu_step_mega_ws_bytes": [_vp],
-    "fstu_step_mega_prepare": [_vp, _vp, _vp],
-    "fstu_step_mega_status": [_vp, _vp],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
     "fstu_decode_graph_create": [_vp, _vp, _i64, _vp, _i, _i, _f, _i, _f, _i, _u64, _vp, _vp],
     "fstu_decode_graph_launch": [_vp, _vp],
@@ -115,7 +112,6 @@ def load(path: Optional[str] = None):
     lib.fstu_packed_elems.restype = ctypes.c_int64
     lib.fstu_sample_ws_bytes.restype = ctypes.c_int64
     lib.fstu_swa_prefill_ws_elems.restype = ctypes.c_int64
-    lib.fstu_step_mega_ws_bytes.restype = ctypes.c_size_t
     lib.fstu_lds_sequence_ws_floats.restype = ctypes.c_size_t
     if path is None:
         _lib = lib

@@ -41,8 +41,7 @@ class ModelDesc(ctypes.Structure):
                 ("eps", _f), ("softcap", _f), ("emb", _vp), ("final_norm_w", _vp), ("layers", ctypes.POINTER(LayerDesc)),
                 ("x", _vp), ("h", _vp), ("qkv", _vp), ("attn", _vp), ("act", _vp), ("xp", _vp), ("y", _vp),
                 ("partial", _vp), ("eo", _vp), ("logits", _vp), ("best", _vp), ("samp_ws", _vp),
-                ("wp_emb", _vp), ("x2", _vp), ("glu_packed", _i), ("down_packed", _i), ("merge_norm", _i),
-                ("mega_ws", _vp)]
+                ("wp_emb", _vp), ("x2", _vp), ("glu_packed", _i), ("down_packed", _i), ("merge_norm", _i)]
 
 
 def pick_ksplit_down(I: int) -> int:
@@ -177,7 +176,7 @@ class DecodeEngine:
                     keep(a), keep(ce), keep(co), keep(st)
                     ld.lds_a, ld.lds_ce, ld.lds_co, ld.lds_state = a.data_ptr(), ce.data_ptr(), co.data_ptr(), st.data_ptr()
                     fir = stu.lds_fir()
-                    if fir is not None and hist.shape[1] == fir.shape[0] and os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") != "1":
+                    if fir is not None and hist.shape[1] == fir.shape[0]:
                         ring = hist[b0:b1]       # in lds mode the history slot of the cache entry is the ring of the last inputs
                         keep(fir), keep(ring)
                         ld.lds_ring, ld.lds_fir = ring.data_ptr(), fir.data_ptr()
@@ -267,34 +266,12 @@ class DecodeEngine:
         if dt == torch.bfloat16 and self.lib.fstu_glu_packed_supported(min(B, _hip.MAX_DECODE_ROWS), d, V):
             m.wp_emb = self._pack(model.lm_head.weight).data_ptr()      # the head streams a packed copy of the embedding
         ch.arr, ch.desc = arr, m
-        ch.mega = None
         if B > _hip.MAX_DECODE_ROWS:
             # first use of the tiled kernels outside any graph capture (their launch set-up raises an LDS limit once)
             wx = torch.zeros(B, 64, dtype=dt, device=dev)
             ww = torch.zeros(8, 64, dtype=dt, device=dev)
             _hip.gemm(wx, ww, up_weight=ww)
             _hip.gemm_splitk(wx, ww, 1)
-        if (dt == torch.bfloat16 and mode == "lds" and m.glu_packed and m.down_packed and not cfg.use_hankel_L
-                and os.environ.get("FSTU_ONE_LAUNCH_STEP", "0") == "1"):
-            # opt-in: the whole step as one persistent launch (packed copies of every weight, one workspace for the
-            # tagged hand-over between the phases).  Correct and tested, but measured slower than the chain of launches
-            # (0.52 against 0.32 ms per step at 768-d, batch 8): a hand-over through memory costs a phase 3-5 us once
-            # the arrival skew of 256 polling workgroups is counted, as much as a kernel boundary
-            for i, layer in enumerate(model.layers):
-                if isinstance(layer, STULayer):
-                    arr[i].wp_m_inputs = self._pack(layer.stu.m_inputs_t()).data_ptr()
-                else:
-                    arr[i].wp_qkv = self._pack(layer.attn.c_attn.weight).data_ptr()
-                    arr[i].wp_proj = self._pack(layer.attn.c_proj.weight).data_ptr()
-            m.wp_emb = self._pack(model.lm_head.weight).data_ptr()
-            nbytes = int(self.lib.fstu_step_mega_ws_bytes(ctypes.byref(m)))
-            if nbytes > 0:
-                ws = torch.zeros(nbytes // 8 + 32, dtype=torch.int64, device=dev)
-                keep(ws)
-                _hip._check(self.lib.fstu_step_mega_prepare(ctypes.byref(m), ws.data_ptr(), torch.cuda.current_stream().cuda_stream),
-                            "fstu_step_mega_prepare")
-                m.mega_ws = ws.data_ptr()
-                ch.mega = ws
 
     # ------------------------------------------------------------------ eager step
     def step(self, tokens: torch.Tensor, pos: int, temperature, top_k, top_p, do_sample, seed, step_idx):
@@ -327,9 +304,7 @@ class DecodeEngine:
             self.graph_end()
         n = int(steps_per_graph)
         self.graph_steps = n
-        # a persistent one-launch step needs every compute unit: row chunks then replay one after the other
-        concurrent = not any(getattr(ch, "mega", None) is not None for ch in self.chunks)
-        n_streams = len(self.chunks) if concurrent else 1
+        n_streams = len(self.chunks)
         if not self._gstreams:
             self._gstreams = [torch.cuda.Stream(device=tokens.device) for _ in range(n_streams)]
         stride = tokens.stride(0)
@@ -361,16 +336,6 @@ class DecodeEngine:
         length have advanced the device-side position in between)."""
         for ch in self.chunks:
             _hip._check(self.lib.fstu_decode_graph_seek(ch.graphs[int(steps_per_graph)], int(pos)), "fstu_decode_graph_seek")
-
-    def check_status(self):
-        """Raises when a wait inside the one-launch step timed out (synchronises the device)."""
-        for ch in self.chunks:
-            if getattr(ch, "mega", None) is not None:
-                err = ctypes.c_int(0)
-                _hip._check(self.lib.fstu_step_mega_status(ch.mega.data_ptr(), ctypes.byref(err)), "fstu_step_mega_status")
-                if err.value:
-                    raise _hip.FlashSTUHipError(f"one-launch decode step: a wait timed out in phase {err.value - 0x100} "
-                                                "(is another process using the GPU?)")
 
     def graph_sync(self):
         """Blocks until every chunk's replay stream has drained."""

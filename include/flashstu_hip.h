@@ -509,25 +509,7 @@ typedef struct {
                                attention layers, B*d <= 8192): the down projection leaves 4 split-K slices and the next
                                layer's first projection adds and normalises them in its prologue
                                (fstu_stu_res_inproj_step / fstu_linear_packed_res); one add+norm launch less per layer */
-  void* mega_ws;            /* != NULL: workspace of the one-launch step (fstu_step_mega_ws_bytes, fstu_step_mega_prepare);
-                               fstu_decode_step and the graphs then run the whole step as ONE persistent kernel when
-                               the model is covered (bf16, recurrence STU state with lds_co, packed copies of every
-                               weight incl. wp_m_inputs / wp_qkv / wp_proj / wp_emb, B <= 16, d % 256 == 0) */
 } fstu_model_desc;
-
-/* ---- the decode step as one persistent launch ------------------------------------
- * No counterpart in the reference (its token loop, flash_stu/model.py:245-302, launches every op of every layer
- * separately).  One grid of one workgroup per compute unit walks all layers; the hand-over between the phases moves
- * through tagged 64-bit words in the workspace (payload + tag of the producing phase, polled with agent-scope
- * loads), so a step costs one launch instead of about fifty.  Nothing else may run on the GPU at the same time (all
- * workgroups must be resident); every wait is bounded and a timeout is reported by fstu_step_mega_status.
- * fstu_step_mega_ws_bytes: size of the workspace, 0 when the model is not covered.
- * fstu_step_mega_prepare: zeroes the workspace and stores the layer table (synchronises `stream`); call it once per
- *   descriptor, and again whenever a pointer of the descriptor changes.
- * fstu_step_mega_status: *err_out = 0, or 0x100 + the phase whose wait timed out (synchronous read). */
-size_t fstu_step_mega_ws_bytes(const fstu_model_desc* m);
-int fstu_step_mega_prepare(const fstu_model_desc* m, void* ws, void* stream);
-int fstu_step_mega_status(const void* ws, int* err_out);
 
 /* tok_in[b*tok_stride] is the token at absolute position pos; the sampled next
  * token is written to tok_out[b*tok_stride].  `step` indexes the sampling

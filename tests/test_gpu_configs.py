@@ -261,8 +261,8 @@ def test_c5_full_architecture_decode_against_full_sequence_recompute():
     temperature 0.8, seeded stream); the CPU oracle is out of reach at this size, so the checks are size-independent:
     graph replay equals the kernel-by-kernel loop token for token, a second run reproduces the ids, and the stateful
     logits equal those of a full-sequence forward over the same tokens within the bf16 tolerance.  The prompt is
-    cut to 192 tokens to keep the test short (the window of 1024 is not reached; the ring wrap is covered at
-    config 2's full size and in test_window_wraps_the_ring_bf16)."""
+    cut to 1100 tokens to keep the test short: longer than the 1025-slot ring, so the prompt pass fills a wrapped
+    ring and every decode step reads the full window through the streamed head-dim-128 attention kernel."""
     from flash_stu import FlashSTU, FlashSTUConfig
     from test_gpu_model import prompt
     torch.manual_seed(2)
@@ -272,7 +272,7 @@ def test_c5_full_architecture_decode_against_full_sequence_recompute():
         model = FlashSTU(cfg)
     model = model.cuda().eval()
     assert abs(model.get_num_params() - 3.98e9) < 0.05e9
-    B, P, N = 32, 192, 24
+    B, P, N = 32, 1100, 24
     ids = prompt(B, P, cfg.vocab_size, 2).cuda()
     kw = dict(max_length=P + N, do_sample=True, top_k=40, temperature=0.8, seed=2)
     eager, logits = model.generate(ids, return_logits=True, **kw)

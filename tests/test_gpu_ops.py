@@ -687,6 +687,74 @@ def test_swa_ring_decode_and_prefill(hip, dtype, B, H, hd, W, T):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,hd,W,T", [(8, 16, 128, 1024, 1100), (2, 16, 128, 512, 560), (4, 12, 64, 512, 540)])
+def test_swa_decode_long_window_past_the_ring_wrap(hip, dtype, B, H, hd, W, T):
+    """The long-window instances of the decode kernel (8 waves per head; head dim 128 deals a 256-byte ring row to
+    the 8 lanes of a key in 16-byte pieces) on a ring that has wrapped, against the oracle on the last queries
+    only.  B=8, H=16, hd=128, W=1024 is config 5's attention shape at a quarter of its batch: one launch reads
+    2*B*H*(W+1)*hd elements = 64 MB or more in either dtype, which selects the instance with streamed
+    (non-temporal) ring loads.  The rings start out filled with NaN: no slot may be read before it is written."""
+    g = gen(31)
+    d = H * hd
+    nq = 6
+    qkv = torch.randn(B, T, 3 * d, generator=g).to(dtype)
+    slopes = O.alibi_slopes(H)
+    q, k, v = (t.reshape(B, T, H, hd) for t in torch.chunk(qkv, 3, dim=2))
+    lo = T - nq - W - 1          # the oldest key any of the checked queries sees is at T - nq - W
+    full = O.attention_core(q[:, T - nq:], k[:, lo:], v[:, lo:], W, slopes, 50.0).reshape(B, nq, d)
+    cap = W + 1
+    assert T - nq > cap          # the prompt alone wraps the ring
+    if hd == 128 and W == 1024:
+        assert 2 * B * H * cap * hd * qkv.element_size() >= 64 << 20
+    kr = torch.full((B, H, cap, hd), float("nan"), dtype=dtype, device="cuda")
+    vr = torch.full_like(kr, float("nan"))
+    qd = dev(qkv)
+    hip.kv_fill(qd[:, :T - nq].contiguous(), kr, vr, 0)
+    sd = dev(slopes)
+    scale = float(full.abs().max())
+    for i, pos in enumerate(range(T - nq, T)):
+        row = qd[:, pos].contiguous()
+        if i % 2 == 0:           # fused append + decode and the two separate calls in turn
+            o = hip.swa_decode(row, kr, vr, sd, pos, W, 50.0, append=True)
+        else:
+            hip.kv_append(row, kr, vr, pos)
+            o = hip.swa_decode(row, kr, vr, sd, pos, W, 50.0)
+        assert bool(torch.isfinite(o).all())
+        check(o, full[:, i], dtype, frac=0.05, scale=scale)
+    # the ring holds exactly the last cap positions, each in slot position % cap
+    want = torch.empty(B, H, cap, hd, dtype=dtype)
+    pos = torch.arange(T - cap, T)
+    want[:, :, pos % cap] = k[:, T - cap:].transpose(1, 2)
+    assert torch.equal(kr.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,hd,W", [(2, 4, 64, 16), (1, 16, 128, 160), (8, 12, 64, 512)])
+def test_swa_decode_never_reads_a_slot_before_it_is_written(hip, dtype, B, H, hd, W):
+    """Rings are allocated uninitialised by the attention module.  A prompt shorter than the window leaves most
+    slots unwritten; with those slots set to NaN every decode step up to and past the wrap must give the finite
+    values of a zero-filled ring, bit for bit (a masked slot read with weight 0 would give 0 * NaN)."""
+    g = gen(32)
+    d = H * hd
+    P, T = 5, W + 9
+    qkv = dev(torch.randn(B, T, 3 * d, generator=g).to(dtype))
+    sd = dev(O.alibi_slopes(H))
+    rings = []
+    for fill in (0.0, float("nan")):
+        kr = torch.full((B, H, W + 1, hd), fill, dtype=dtype, device="cuda")
+        vr = torch.full_like(kr, fill)
+        hip.kv_fill(qkv[:, :P].contiguous(), kr, vr, 0)
+        rings.append((kr, vr))
+    for pos in range(P, T):
+        row = qkv[:, pos].contiguous()
+        o0 = hip.swa_decode(row, *rings[0], sd, pos, W, 50.0, append=True)
+        o1 = hip.swa_decode(row, *rings[1], sd, pos, W, 50.0, append=True)
+        assert bool(torch.isfinite(o1).all()), pos
+        assert torch.equal(o0, o1), pos
+    assert torch.equal(rings[0][0], rings[1][0]) and torch.equal(rings[0][1], rings[1][1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_sample_greedy_matches_oracle_ties_included(hip, dtype):
     g = gen(11)
     B, V = 8, 50257
