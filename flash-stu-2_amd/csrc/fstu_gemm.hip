@@ -302,6 +302,219 @@ int gemm_launch_tile(const void* A, long long lda, const void* W, const void* W2
   return 0;
 }
 
+// ---------------------------------------------------------------- transposed activations
+// C[b][m, n] = sum_k A[b][k, m] W[n, k]: the activations come as a slab with the REDUCTION index slowest (k rows of
+// lda elements, m contiguous) — the time-major U+- of the exact-mode STU operator (flash_stu/modules/stu.py:107-120:
+// tensordot of U (B, L, K, d) with M_phi (K, d, d) over (K, d); the filter-bank kernel writes U as (B, K*d, L) so
+// that its stores are whole lines).  Same tiles, pipeline and epilogues as gemm_bf16_kernel (mode 0 and 2); what
+// differs is the activation tile: LDS rows are k (BK rows of BT*2 bytes, filled 16 bytes = 8 consecutive m per lane),
+// and the MFMA B fragment — 8 consecutive k of one m per lane — is gathered by two transposing reads
+// (ds_read_b64_tr_b16: in a block of 16 lanes, lane i supplies the address of 4 consecutive m of row i/4 starting at
+// column 4*(i%4), and receives column i of the 4 rows).  The 64-byte column groups of a row are XOR-ed with the row's
+// low two bits, so the four rows of a read fall into different banks.  `nbatch` slabs run as one grid.
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ __forceinline__ u32x2_t lds_read_tr8(unsigned addr) {
+  u32x2_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int N, int STEP, int I = 0>
+__device__ __forceinline__ void lds_read_tr_cols(u32x2_t* f, const unsigned* addr) {   // N column tiles, rows k..k+3 and k+4..k+7
+  if constexpr (I < N) {
+    f[2 * I] = lds_read_tr8<0>(addr[I]);
+    f[2 * I + 1] = lds_read_tr8<4 * STEP>(addr[I]);
+    lds_read_tr_cols<N, STEP, I + 1>(f, addr);
+  }
+}
+template <int LEFT>
+__device__ __forceinline__ void lds_wait_n() { asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(LEFT)); }
+template <int N> __device__ __forceinline__ void pin4(u32x4_t* f) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+}
+template <int N> __device__ __forceinline__ void pin2(u32x2_t* f) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+}
+
+template <class G, int MODE>
+__global__ void __launch_bounds__(G::THREADS)
+gemm_ta_bf16_kernel(const bf16_t* __restrict__ A, long long lda, long long sa, const bf16_t* __restrict__ W,
+                    const bf16_t* __restrict__ R, long long ldr, long long sr, bf16_t* __restrict__ C, long long ldc,
+                    long long sc, int M, int N, int K, int mt, int nt, int share, int nbatch) {
+  constexpr int FI = G::FI, TJ = G::TJ, BF = G::BF, BT = G::BT, WL = G::WL, AL = G::AL, NS = G::NS, KK = G::KK;
+  constexpr unsigned STAGE = G::STAGE;
+  constexpr int RBT = BT * 2, CPRT = BT / 8;              // bytes and 16-byte chunks of an activation row (one k)
+  constexpr int NRD = FI + 2 * TJ;                        // LDS reads per k step
+  static_assert(G::BK == 64 && BT >= 128, "k tile of 64, at least 128 columns");
+  static_assert((MODE == 0 || MODE == 2), "plain or residual epilogue");
+  extern __shared__ __align__(16) unsigned char gm_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int wf = w % G::WFN, wt = w / G::WFN;
+  int o = (int)(blockIdx.x & 7) * share + (int)(blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= share || o >= mt * nt * nbatch) return;
+  const int batch = o / (mt * nt);
+  o -= batch * (mt * nt);
+  const int per_panel = mt * GM_PANEL;
+  const int panel = o / per_panel, in_panel = o - panel * per_panel;
+  const int pw = min(GM_PANEL, nt - panel * GM_PANEL);
+  const int bt = in_panel / pw, bf = panel * GM_PANEL + in_panel % pw;
+  const int m0 = bt * BT, n0 = bf * BF;
+  A += (size_t)batch * sa;
+  C += (size_t)batch * sc;
+  if (MODE == 2) R += (size_t)batch * sr;
+  const int wv = __builtin_amdgcn_readfirstlane(w);
+  const int rows_w = min(BF, N - n0);
+  const rsrc_t rs_w = make_rsrc(W + (size_t)n0 * K, (size_t)rows_w * K * 2);
+  const rsrc_t rs_a = make_rsrc(A + m0, ((size_t)(K - 1) * lda + BT) * 2);     // M % BT == 0: whole rows of BT columns
+  unsigned wvoff[WL], avoff[AL];
+#pragma unroll
+  for (int j = 0; j < WL; ++j) {
+    const int slot = (wv * WL + j) * 64 + lane, row = slot / G::CPR;
+    const int ch = (int)((G::swz(row, slot % G::CPR) - (unsigned)row * G::RB) >> 4);
+    wvoff[j] = (unsigned)row * (unsigned)K * 2u + (unsigned)ch * 16u;
+  }
+#pragma unroll
+  for (int j = 0; j < AL; ++j) {
+    const int slot = (wv * AL + j) * 64 + lane, kr = slot / CPRT, pc = slot % CPRT;
+    const int lc = pc ^ (4 * (kr & 3));                  // the XOR is its own inverse
+    avoff[j] = (unsigned)kr * (unsigned)lda * 2u + (unsigned)lc * 16u;
+  }
+  const unsigned wslot = (unsigned)(wv * WL) * 1024u, aslot = (unsigned)BF * G::RB + (unsigned)(wv * AL) * 1024u;
+#define GT_FETCH(stage_, k0)                                                                                 \
+  {                                                                                                          \
+    unsigned char* st_ = gm_smem + (unsigned)(stage_) * STAGE;                                               \
+    const unsigned sw_ = (unsigned)(k0) * 2u;                                                                \
+    const unsigned sa_ = (unsigned)((size_t)(k0) * (size_t)lda * 2u);                                        \
+    _Pragma("unroll") for (int j = 0; j < WL; ++j) buf_load16_to_lds(rs_w, wvoff[j], sw_, st_ + wslot + j * 1024); \
+    _Pragma("unroll") for (int j = 0; j < AL; ++j) buf_load16_to_lds(rs_a, avoff[j], sa_, st_ + aslot + j * 1024); \
+  }
+  struct Frag8 { u32x2_t lo, hi; };
+#define GT_MFMAS(fw_, fx_)                                                                                   \
+  _Pragma("unroll") for (int i = 0; i < FI; ++i)                                                             \
+    _Pragma("unroll") for (int j = 0; j < TJ; ++j) {                                                         \
+      const Frag8 b_ = {fx_[2 * j], fx_[2 * j + 1]};                                                         \
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fw_[i]),              \
+                                                          __builtin_bit_cast(bf16x8_t, b_), acc[i][j], 0, 0, 0); \
+    }
+  const int l32 = lane & 31, lh = lane >> 5;
+  unsigned fw_off[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) fw_off[kk] = G::swz(wf * (32 * FI) + l32, kk * 2 + lh);
+  // transposing reads: this lane's address inside a stage for column tile j at k step 0, rows k..k+3
+  const int blk = lane >> 4, i16 = lane & 15, key = i16 >> 2;
+  unsigned ta_off[TJ];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j)
+    ta_off[j] = (unsigned)BF * G::RB + (unsigned)(8 * (blk >> 1) + key) * RBT + (unsigned)(((wt * TJ + j) ^ key) << 6) +
+                (unsigned)(2 * (blk & 1) + ((i16 & 3) >> 1)) * 16u + (unsigned)(i16 & 1) * 8u;
+  floatx16_t acc[FI][TJ];
+#pragma unroll
+  for (int i = 0; i < FI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  const int nkt = K / G::BK;
+  constexpr int LPT = WL + AL;
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t)
+    if (t < nkt) GT_FETCH(t, t * G::BK)
+  const unsigned smem0 = lds_addr(gm_smem);
+  if (NS - 2 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  if (NS - 1 < nkt) GT_FETCH(NS - 1, (NS - 1) * G::BK)
+  u32x4_t wa_[FI], wb_[FI];                           // weight fragments of alternate k steps
+  u32x2_t xa_[2 * TJ], xb_[2 * TJ];                   // activation fragments (two halves per column tile)
+  unsigned ta[TJ];
+#define GT_READ(fw_, fx_, base_, kk_)                                                                        \
+  {                                                                                                          \
+    lds_read_rows<FI, 32 * G::RB>(fw_, (base_) + fw_off[kk_]);                                               \
+    _Pragma("unroll") for (int j = 0; j < TJ; ++j) ta[j] = (base_) + ta_off[j] + (unsigned)(kk_) * 16u * RBT; \
+    lds_read_tr_cols<TJ, RBT>(fx_, ta);                                                                      \
+  }
+#define GT_WAIT(left_, fw_, fx_)                                                                             \
+  {                                                                                                          \
+    lds_wait_n<left_>();                                                                                     \
+    pin4<FI>(fw_);                                                                                           \
+    pin2<2 * TJ>(fx_);                                                                                       \
+  }
+  GT_READ(wa_, xa_, smem0, 0)
+  int cur = 0;
+  for (int kt = 0; kt < nkt; ++kt) {
+    const unsigned cb = smem0 + (unsigned)cur * STAGE;
+    const int nxt = cur + 1 == NS ? 0 : cur + 1;
+    __builtin_amdgcn_sched_barrier(0);
+    GT_READ(wb_, xb_, cb, 1)
+    GT_WAIT(NRD, wa_, xa_)
+    GT_MFMAS(wa_, xa_)
+    __builtin_amdgcn_sched_barrier(0);
+    GT_READ(wa_, xa_, cb, 2)
+    GT_WAIT(NRD, wb_, xb_)
+    GT_MFMAS(wb_, xb_)
+    __builtin_amdgcn_sched_barrier(0);
+    GT_READ(wb_, xb_, cb, 3)
+    GT_WAIT(NRD, wa_, xa_)
+    GT_MFMAS(wa_, xa_)
+    __builtin_amdgcn_sched_barrier(0);
+    GT_WAIT(0, wb_, xb_)                              // this wave has left the stage of tile kt
+    if (kt + 1 < nkt) {
+      if (kt + NS - 1 < nkt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPT) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      if (kt + NS < nkt) GT_FETCH(cur, (kt + NS) * G::BK)
+      const unsigned nb = smem0 + (unsigned)nxt * STAGE;
+      GT_READ(wa_, xa_, nb, 0)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    GT_MFMAS(wb_, xb_)
+    cur = nxt;
+  }
+#undef GT_FETCH
+#undef GT_MFMAS
+#undef GT_READ
+#undef GT_WAIT
+  // ---- epilogue: lane l holds row (position) l % 32 and features 8*(e/4) + 4*(l/32) + e%4 of a 32x32 tile
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) {
+    const int m = m0 + wt * (32 * TJ) + j * 32 + l32;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < FI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int f = n0 + wf * (32 * FI) + i * 32 + q * 8 + lh * 4;
+        if (f >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+        if (MODE == 2) {
+          const uint2 rv = *(const uint2*)(R + (size_t)m * ldr + f);
+          v[0] = __uint_as_float(rv.x << 16) + rnd_bf16(v[0]);
+          v[1] = __uint_as_float(rv.x & 0xffff0000u) + rnd_bf16(v[1]);
+          v[2] = __uint_as_float(rv.y << 16) + rnd_bf16(v[2]);
+          v[3] = __uint_as_float(rv.y & 0xffff0000u) + rnd_bf16(v[3]);
+        }
+        *(uint2*)(C + (size_t)m * ldc + f) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+      }
+  }
+}
+
+template <class G, int MODE>
+int gemm_ta_launch_tile(const void* A, long long lda, long long sa, const void* W, const void* R, long long ldr, long long sr,
+                        void* C, long long ldc, long long sc, int M, int N, int K, int nbatch, hipStream_t s) {
+  static hipError_t attr_err = hipFuncSetAttribute((const void*)gemm_ta_bf16_kernel<G, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS);
+  if (attr_err != hipSuccess) { fstu_set_error("fstu_gemm_bf16_ta: hipFuncSetAttribute: %s", hipGetErrorString(attr_err)); return (int)attr_err; }
+  const int mt = M / G::BT, nt = (N + G::BF - 1) / G::BF;
+  const long long tiles = (long long)mt * nt * nbatch;
+  const int share = (int)((tiles + 7) / 8);
+  hipLaunchKernelGGL((gemm_ta_bf16_kernel<G, MODE>), dim3((unsigned)share * 8u), dim3(G::THREADS), G::LDS, s, (const bf16_t*)A, lda, sa,
+                     (const bf16_t*)W, (const bf16_t*)R, ldr, sr, (bf16_t*)C, ldc, sc, M, N, K, mt, nt, share, nbatch);
+  return 0;
+}
+
 int gemm_cus() {
   static int cus = [] {
     int dev = 0;
@@ -381,5 +594,40 @@ extern "C" int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const v
   else rc = gemm_launch<2>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
   if (rc) return rc;
   FSTU_CHECK_LAUNCH("fstu_gemm_bf16");
+  return FSTU_OK;
+}
+
+// C[b] = T(A[b]^T W^T) (mode 0) or T(R[b] + T(A[b]^T W^T)) (mode 2) for nbatch slabs A[b] of shape (K, M) with row
+// stride lda (elements; the reduction index slowest, M contiguous), W (N, K) row-major.  M must be a multiple of 128.
+extern "C" int fstu_gemm_bf16_ta(const void* A, int64_t lda, int64_t batch_stride_a, const void* W, const void* R, int64_t ldr,
+                                 int64_t batch_stride_r, void* C, int64_t ldc, int64_t batch_stride_c, int M, int N, int K,
+                                 int nbatch, int mode, void* stream) {
+  FSTU_REQUIRE(A && W && C, FSTU_ENULL, "fstu_gemm_bf16_ta: null pointer");
+  FSTU_REQUIRE(mode == 0 || mode == 2, FSTU_EARG, "fstu_gemm_bf16_ta: mode %d (0: plain, 2: residual add)", mode);
+  FSTU_REQUIRE(mode != 2 || R, FSTU_ENULL, "fstu_gemm_bf16_ta: mode 2 needs R");
+  FSTU_REQUIRE(M >= 128 && M % 128 == 0 && N >= 4 && N % 4 == 0 && K >= 64 && K % 64 == 0 && nbatch >= 1, FSTU_ESHAPE,
+               "fstu_gemm_bf16_ta: need M %% 128 == 0, N %% 4 == 0, K %% 64 == 0 (M=%d N=%d K=%d nbatch=%d)", M, N, K, nbatch);
+  FSTU_REQUIRE(lda >= M && lda % 8 == 0 && ldc >= N && ldc % 4 == 0 && (mode != 2 || (ldr >= N && ldr % 4 == 0)), FSTU_ESHAPE,
+               "fstu_gemm_bf16_ta: row strides (lda=%lld ldc=%lld ldr=%lld)", (long long)lda, (long long)ldc, (long long)ldr);
+  // 32-bit byte offsets inside a slab (buffer addressing) and inside W
+  FSTU_REQUIRE((unsigned long long)K * (unsigned long long)lda * 2ull < 0xfff00000ull && (unsigned long long)N * K * 2ull < 0xfff00000ull,
+               FSTU_ESHAPE, "fstu_gemm_bf16_ta: a slab (K*lda) or W (N*K) exceeds 4 GB of 32-bit offsets");
+  FSTU_REQUIRE(batch_stride_a % 8 == 0 && batch_stride_c % 4 == 0 && batch_stride_r % 4 == 0, FSTU_ESHAPE,
+               "fstu_gemm_bf16_ta: batch strides must keep the alignment");
+  FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(C, 8) && fstu_aligned(R, 8), FSTU_EALIGN,
+               "fstu_gemm_bf16_ta: pointers must be 16-byte aligned (C, R: 8)");
+  hipStream_t s = (hipStream_t)stream;
+  const long long big = (long long)(M / 256) * ((N + 255) / 256) * nbatch;
+  int rc;
+#define TA_GO(TILE)                                                                                                              \
+  (mode == 0 ? gemm_ta_launch_tile<TILE, 0>(A, lda, batch_stride_a, W, R, ldr, batch_stride_r, C, ldc, batch_stride_c, M, N, K,  \
+                                            nbatch, s)                                                                           \
+             : gemm_ta_launch_tile<TILE, 2>(A, lda, batch_stride_a, W, R, ldr, batch_stride_r, C, ldc, batch_stride_c, M, N, K,  \
+                                            nbatch, s))
+  if (M % 256 == 0 && K >= 1024 && big >= 2 * gemm_cus()) rc = TA_GO(TileBig);
+  else rc = TA_GO(TileSmall);
+#undef TA_GO
+  if (rc) return rc;
+  FSTU_CHECK_LAUNCH("fstu_gemm_bf16_ta");
   return FSTU_OK;
 }

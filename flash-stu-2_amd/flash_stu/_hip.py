@@ -82,6 +82,7 @@ SIGNATURES = {
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
     "fstu_gemm_bf16": [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
     "fstu_gemm_bf16_splitk": [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_gemm_bf16_ta": [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_sequence_ws_floats": [_i, _i, _i],
     "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -294,6 +295,34 @@ def gemm(x2: torch.Tensor, weight: torch.Tensor, up_weight: Optional[torch.Tenso
         mode, ldr = 2, residual.stride(0)
     _check(load().fstu_gemm_bf16(_p(x2), x2.stride(0), _p(weight), _p(up_weight), _p(residual), ldr, _p(out), out.stride(0),
                                  M, N, K, mode, _stream()), "fstu_gemm_bf16")
+    return out
+
+
+def gemm_ta(slabs: torch.Tensor, weight: torch.Tensor, residual: Optional[torch.Tensor] = None,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[b] = T(slabs[b]^T @ weight^T) (+ residual[b], rounded again) for slabs (nb, K, M) whose last index is
+    contiguous (the reduction index is the slow one: the time-major U of the exact-mode STU operator), weight (N, K).
+    M must be a multiple of 128; slab rows may be strided (a view of a wider buffer)."""
+    _dev(weight)
+    for t in (slabs, residual, out):
+        if t is not None and not t.is_cuda:
+            raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    if slabs.dim() != 3 or slabs.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or slabs.stride(2) != 1:
+        raise FlashSTUHipError("gemm_ta: slabs must be (nb, K, M) bf16 with M contiguous")
+    nb, K, M = slabs.shape
+    N = weight.shape[0]
+    if weight.shape != (N, K) or not weight.is_contiguous():
+        raise FlashSTUHipError("gemm_ta: weight must be (N, K) contiguous")
+    if out is None:
+        out = torch.empty(nb, M, N, dtype=slabs.dtype, device=slabs.device)
+    for t, name in ((out, "out"), (residual, "residual")):
+        if t is not None and (t.shape != (nb, M, N) or t.stride(2) != 1 or t.dtype != slabs.dtype):
+            raise FlashSTUHipError(f"gemm_ta: {name} must be (nb, M, N) with contiguous rows")
+    mode = 2 if residual is not None else 0
+    _check(load().fstu_gemm_bf16_ta(_p(slabs), slabs.stride(1), slabs.stride(0) if nb > 1 else 0, _p(weight), _p(residual),
+                                    residual.stride(1) if residual is not None else 0,
+                                    residual.stride(0) if residual is not None and nb > 1 else 0, _p(out), out.stride(1),
+                                    out.stride(0) if nb > 1 else 0, M, N, K, nb, mode, _stream()), "fstu_gemm_bf16_ta")
     return out
 
 

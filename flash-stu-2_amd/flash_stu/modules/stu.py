@@ -241,9 +241,9 @@ class STU(nn.Module):
 
     def _exact_sequence(self, x: torch.Tensor) -> torch.Tensor:
         """use_approx=False: U+-[b,t,k,i] for the whole filter bank (one forward transform per channel, one
-        inverse per filter), then the (K*d_in, d_out) contractions as library GEMMs with the reference's
-        rounding points (stu.py:107-120).  The FFT form writes U time-major, (B, K*d, T), which the GEMM
-        consumes as a transposed operand; x is never expanded K-fold."""
+        inverse per filter), then the (K*d_in, d_out) contractions on the matrix cores with the reference's
+        rounding points, T(T(U+ M+) + T(U- M-)) (stu.py:107-120).  The FFT form writes U time-major, (B, K*d, T),
+        which fstu_gemm_bf16_ta consumes as it lies; x is never expanded K-fold."""
         B, T, d = x.shape
         wp, wm = self.exact_flat_weights()
         n = _hip.fft_length(T) if T >= FFT_MIN_T else 0
@@ -255,19 +255,29 @@ class STU(nn.Module):
             if Um is not None:
                 y = y + torch.matmul(Um.reshape(B * T, self.K * d), wm)
             return y.reshape(B, T, self.d_out)
-        Up = torch.empty(B, self.K, d, T, dtype=x.dtype, device=x.device)
+        # Slabs of (K*d, Tp) per batch row with Tp = T rounded up to the contraction's 128-position tiles; the filter
+        # bank writes positions below T, the contraction's rows beyond T are cut off again (each output row depends
+        # on its own column of the slab only, so what the padding holds never reaches a kept row).
+        Tp = (T + 127) // 128 * 128
+        Kd = self.K * d
+        Up = torch.empty(B, self.K, d, Tp, dtype=x.dtype, device=x.device)
         Um = None if self.use_hankel_L else torch.empty_like(Up)
         xt = x.transpose(1, 2).contiguous().transpose(1, 2)            # time-major copy: coalesced column loads
-        _hip.stu_conv_bank_fft(xt, self.filter_spectrum(n), Up.permute(0, 3, 1, 2),
-                               None if Um is None else Um.permute(0, 3, 1, 2))
-        # U is the transposed operand of the contraction.  One GEMM per batch row takes the (K*d, T) slab as it lies
-        # (a batched matmul over the 3-D view would first copy all of U into row-major order: 2 x 3.7 ms at
-        # B=4, T=8192, K*d=24576)
+        _hip.stu_conv_bank_fft(xt, self.filter_spectrum(n), Up[..., :T].permute(0, 3, 1, 2),
+                               None if Um is None else Um[..., :T].permute(0, 3, 1, 2))
+        if x.dtype == torch.bfloat16 and Kd % 64 == 0 and self.d_out % 4 == 0:
+            wpt, wmt = self.exact_flat_weights_t()
+            y = _hip.gemm_ta(Up.view(B, Kd, Tp), wpt)
+            if Um is not None:
+                _hip.gemm_ta(Um.view(B, Kd, Tp), wmt, residual=y, out=y)
+            return y if Tp == T else y[:, :T].contiguous()
+        # fp32 (the parity path) and widths the matrix-core kernel does not take: one library GEMM per batch row on
+        # the (K*d, T) slab as a transposed operand
         y = torch.empty(B, T, self.d_out, dtype=x.dtype, device=x.device)
         for b in range(B):
-            torch.mm(Up[b].reshape(self.K * d, T).t(), wp, out=y[b])
+            torch.mm(Up[b].reshape(Kd, Tp)[:, :T].t(), wp, out=y[b])
             if Um is not None:
-                y[b] += torch.mm(Um[b].reshape(self.K * d, T).t(), wm)
+                y[b] += torch.mm(Um[b].reshape(Kd, Tp)[:, :T].t(), wm)
         return y
 
     def forward_differentiable(self, x: torch.Tensor) -> torch.Tensor:

@@ -364,6 +364,17 @@ int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, co
 int fstu_gemm_bf16_splitk(const void* A, int64_t lda, const void* W, float* partial, int M, int N, int K, int ksplit,
                           void* stream);
 
+/* The contraction of the exact-mode STU operator (flash_stu/modules/stu.py:107-120: tensordot of U+- (B,L,K,d) with
+ * M_phi+- (K,d,d) over (K,d)) with U stored as the filter-bank kernel writes it, time-major: nbatch slabs A[b] of shape
+ * (K, M) — the reduction index slowest, M contiguous, row stride lda, slab stride batch_stride_a (elements) — against
+ * W (N, K) row-major (M_phi flattened to (K*d, N) and transposed once at model-prepare time):
+ *   mode 0  C[b] = T(A[b]^T W^T)            mode 2  C[b] = T(R[b] + T(A[b]^T W^T))   (the sum of the two sign branches)
+ * C, R (nbatch, M, N) with row strides ldc / ldr and slab strides batch_stride_c / batch_stride_r; C may alias R.
+ * M % 128 == 0, K % 64 == 0, N % 4 == 0, lda % 8 == 0, K*lda*2 and N*K*2 below 4 GB; A, W 16-byte aligned. */
+int fstu_gemm_bf16_ta(const void* A, int64_t lda, int64_t batch_stride_a, const void* W, const void* R, int64_t ldr,
+                      int64_t batch_stride_r, void* C, int64_t ldc, int64_t batch_stride_c, int M, int N, int K, int nbatch,
+                      int mode, void* stream);
+
 /* ---- dense LDS (mini_stu/lds.py:95-101) ------------------------------------
  * T_steps consecutive steps with the fp32 state h (Bt,S) carried in place:
  *   h <- h*A + x_t @ Bm ;  y_t = T(h @ Cm)

@@ -144,6 +144,38 @@ def test_gemm_bf16_plain_and_residual(hip, M, N, K):
     check(rd, (res.float() + ref.float()).bfloat16(), torch.bfloat16, frac=0.05, atol=2.0 ** -7 * float(ref.float().abs().max()))
 
 
+@pytest.mark.parametrize("nb,M,N,K", [(1, 128, 64, 64), (3, 256, 132, 192), (2, 1024, 1024, 1536), (4, 512, 260, 2048),
+                                      (1, 4096, 768, 3072)])
+def test_gemm_bf16_transposed_activations(hip, nb, M, N, K):
+    """fstu_gemm_bf16_ta (the exact-mode contraction over time-major slabs, reference stu.py:107-120): every slab
+    (K, M) with M contiguous against F.linear of its transpose in fp32 rounded once; the residual form adds in place;
+    slab rows that are a view of a wider buffer (row stride > M); and bit-identity with fstu_gemm_bf16 on a row-major
+    copy of the same operand (same tiles, same summation order)."""
+    g = gen(63)
+    A = torch.randn(nb, K, M, generator=g).bfloat16()
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    res = torch.randn(nb, M, N, generator=g).bfloat16()
+    ref = torch.stack([F.linear(A[b].t().float(), W.float()) for b in range(nb)]).bfloat16()
+    Ad, Wd = dev(A), dev(W)
+    got = hip.gemm_ta(Ad, Wd)
+    check(got, ref, torch.bfloat16)
+    rd = dev(res.clone())
+    out = hip.gemm_ta(Ad, Wd, residual=rd, out=rd)
+    assert out.data_ptr() == rd.data_ptr()
+    check(rd, (res.float() + ref.float()).bfloat16(), torch.bfloat16, frac=0.05, atol=2.0 ** -7 * float(ref.float().abs().max()))
+    wide = torch.full((nb, K, M + 256), float("nan"), dtype=torch.bfloat16, device="cuda")
+    wide[:, :, :M] = Ad
+    assert torch.equal(hip.gemm_ta(wide[:, :, :M], Wd), got)
+    if K % 64 == 0 and M > 32:
+        rowmajor = torch.stack([hip.gemm(Ad[b].t().contiguous(), Wd) for b in range(nb)])
+        frac = float((rowmajor != got).float().mean())
+        assert frac <= 1e-3, frac            # another tile shape may be picked: same values up to rare rounding flips
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.gemm_ta(Ad[:, :, :100], Wd)      # M not a multiple of 128
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.gemm_ta(Ad.transpose(1, 2), Wd)  # M not the contiguous index
+
+
 @pytest.mark.parametrize("M,d,I", [(4096, 768, 3072), (300, 256, 1000), (2048, 1024, 8192), (100, 96, 132)])
 def test_gemm_bf16_gated_pair(hip, M, d, I):
     """Mode 1: T(T(gelu_tanh(T(x Wg^T))) * T(x Wu^T)) in one kernel equals the three-step bf16 chain of the reference
