@@ -4,7 +4,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["fstu_core.hip", "fstu_linear.hip", "fstu_stu.hip", "fstu_fft.hip", "fstu_attn.hip", "fstu_attn_mfma.hip", "fstu_gemv.hip", "fstu_mlp.hip", "fstu_lds_seq.hip", "fstu_gemm.hip", "fstu_engine.hip"]
+SOURCES = ["fstu_core.hip", "fstu_linear.hip", "fstu_stu.hip", "fstu_fft.hip", "fstu_attn.hip", "fstu_attn_mfma.hip", "fstu_pack.hip", "fstu_mlp.hip", "fstu_lds_seq.hip", "fstu_gemm.hip", "fstu_gemm_any.hip", "fstu_engine.hip"]
 LIB = os.path.join(HERE, "libflashstu_hip.so")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          # packed fp32 instructions are kept out of the generated code

@@ -82,6 +82,7 @@ SIGNATURES = {
     "fstu_prof_glu_loop": [_vp, _i, _vp, _vp, _vp],
     "fstu_gemm_bf16": [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
     "fstu_gemm_bf16_splitk": [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_gemm_any": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
     "fstu_gemm_bf16_ta": [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_sequence_ws_floats": [_i, _i, _i],
     "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -298,6 +299,28 @@ def gemm(x2: torch.Tensor, weight: torch.Tensor, up_weight: Optional[torch.Tenso
     return out
 
 
+def gemm_any(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out (M,N) = T(a @ w^T) for ANY strided 2-D views a (M,K) and w (N,K) of one dtype (fp32 or bf16): the general
+    kernel behind everything the bf16 matrix-core GEMM does not take.  fp32 accumulation, one rounding."""
+    for t in (a, w, out):
+        if t is not None and not t.is_cuda:
+            raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1] or a.dtype != w.dtype:
+        raise FlashSTUHipError(f"gemm_any: operands {tuple(a.shape)} {a.dtype} x {tuple(w.shape)} {w.dtype}")
+    M, K = a.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty(M, N, dtype=a.dtype, device=a.device)
+    if out.shape != (M, N) or out.stride(1) != 1 or out.dtype != a.dtype:
+        raise FlashSTUHipError("gemm_any: out must be (M,N) with contiguous rows")
+    # a size-1 dimension may carry any stride: give it a positive one
+    sam, sak = max(a.stride(0), 1), max(a.stride(1), 1)
+    swn, swk = max(w.stride(0), 1), max(w.stride(1), 1)
+    _check(load().fstu_gemm_any(_p(a), sam, sak, _p(w), swn, swk, _p(out), out.stride(0), M, N, K, _dt(a), _stream()),
+           "fstu_gemm_any")
+    return out
+
+
 def gemm_ta(slabs: torch.Tensor, weight: torch.Tensor, residual: Optional[torch.Tensor] = None,
             out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[b] = T(slabs[b]^T @ weight^T) (+ residual[b], rounded again) for slabs (nb, K, M) whose last index is
@@ -344,8 +367,9 @@ def gemm_splitk(x2: torch.Tensor, weight: torch.Tensor, ksplit: int, partial: Op
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x (..., K) @ weight (N,K)^T (+ bias): the skinny GEMV kernel for up to 16 rows, the matrix-core GEMM kernel for
-    more rows in bf16; other dtypes and shapes the kernel does not take go to a library GEMM."""
+    """x (..., K) @ weight (N,K)^T (+ bias): the skinny GEMV kernel for up to 16 rows, the bf16 matrix-core GEMM kernel
+    for more rows, the general kernel (fstu_gemm_any: fp32, odd shapes, strided weights) for everything else.  No
+    library GEMM."""
     shape = x.shape
     x2 = x.reshape(-1, shape[-1])
     if x2.shape[0] <= MAX_DECODE_ROWS:
@@ -356,10 +380,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         y = gemm(x2, weight)
         if bias is not None:
             bias_act(y, bias)
-    elif bias is not None:
-        y = torch.addmm(bias, x2, weight.t())
     else:
-        y = torch.matmul(x2, weight.t())
+        y = gemm_any(x2, weight)
+        if bias is not None:
+            bias_act(y, bias)
     return y.reshape(*shape[:-1], weight.shape[0])
 
 

@@ -75,9 +75,14 @@ class STU(nn.Module):
         return (not self.use_approx and self.decode_mode() == "lds" and self.phi.shape[0] % 2 == 0 and self.K <= 32)
 
     def effective_filter(self) -> torch.Tensor:
-        """phi_proj = phi @ M_filters, (L,d) in the model dtype (stu.py:88)."""
-        return self._cached("filt", (self.phi, self.M_filters),
-                            lambda: torch.matmul(self.phi, self.M_filters).contiguous())
+        """phi_proj = phi @ M_filters, (L,d) in the model dtype (stu.py:88).  On the GPU the general contraction
+        kernel; the host-side filter fit (lds_params / lds_fir in float64) may ask for it before the module has been
+        moved to the GPU, and then it is a host matmul like the rest of that fit."""
+        def build():
+            if self.phi.is_cuda:
+                return _hip.gemm_any(self.phi, self.M_filters.t())
+            return torch.matmul(self.phi, self.M_filters).contiguous()
+        return self._cached("filt", (self.phi, self.M_filters), build)
 
     def filter_spectrum(self, n: int) -> torch.Tensor:
         """Spectra of the convolution filters for transform length n, (d,n,2) fp32 in approx mode, (K,n,2) in
@@ -227,7 +232,7 @@ class STU(nn.Module):
         x2 = x.reshape(B * T, d)
         if _hip.gemm_supported(x2, self.m_inputs_t()):
             return _hip.gemm(x2, self.m_inputs_t()).reshape(B, T, self.d_out)
-        return torch.matmul(x, self.m_inputs_eff())
+        return _hip.gemm_any(x2, self.m_inputs_t()).reshape(B, T, self.d_out)
 
     def _convolve(self, xp: torch.Tensor) -> torch.Tensor:
         """Approx-mode convolution of the projected inputs with phi_proj (stu.py:89-98,120): the FFT form of
@@ -251,9 +256,10 @@ class STU(nn.Module):
             Up = torch.empty(B, T, self.K, d, dtype=x.dtype, device=x.device)
             Um = None if self.use_hankel_L else torch.empty_like(Up)
             _hip.stu_conv_bank(x, self.phi, Up, Um)
-            y = torch.matmul(Up.reshape(B * T, self.K * d), wp)
+            wpt, wmt = self.exact_flat_weights_t()
+            y = _hip.linear(Up.reshape(B * T, self.K * d), wpt)
             if Um is not None:
-                y = y + torch.matmul(Um.reshape(B * T, self.K * d), wm)
+                y = y + _hip.linear(Um.reshape(B * T, self.K * d), wmt)
             return y.reshape(B, T, self.d_out)
         # Slabs of (K*d, Tp) per batch row with Tp = T rounded up to the contraction's 128-position tiles; the filter
         # bank writes positions below T, the contraction's rows beyond T are cut off again (each output row depends
@@ -271,13 +277,13 @@ class STU(nn.Module):
             if Um is not None:
                 _hip.gemm_ta(Um.view(B, Kd, Tp), wmt, residual=y, out=y)
             return y if Tp == T else y[:, :T].contiguous()
-        # fp32 (the parity path) and widths the matrix-core kernel does not take: one library GEMM per batch row on
-        # the (K*d, T) slab as a transposed operand
+        # fp32 (the parity path) and widths the matrix-core kernel does not take: the general kernel per batch row on
+        # the (K*d, T) slab as a strided operand
         y = torch.empty(B, T, self.d_out, dtype=x.dtype, device=x.device)
         for b in range(B):
-            torch.mm(Up[b].reshape(Kd, Tp)[:, :T].t(), wp, out=y[b])
+            _hip.gemm_any(Up[b].reshape(Kd, Tp)[:, :T].t(), wp.t(), out=y[b])
             if Um is not None:
-                y[b] += torch.mm(Um[b].reshape(Kd, Tp)[:, :T].t(), wm)
+                y[b] += _hip.gemm_any(Um[b].reshape(Kd, Tp)[:, :T].t(), wm.t())
         return y
 
     def forward_differentiable(self, x: torch.Tensor) -> torch.Tensor:

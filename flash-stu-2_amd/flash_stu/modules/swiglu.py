@@ -44,8 +44,9 @@ class MLP(nn.Module):
                 return None
             out = _hip.gemm(act, self.down_proj.weight)
         else:
-            g = torch.matmul(x2, self.gate_proj.weight.t())
-            u = torch.matmul(x2, self.up_proj.weight.t())
+            # fp32 (the parity configuration) and shapes the bf16 matrix-core kernel does not take: the general kernel
+            g = _hip.gemm_any(x2, self.gate_proj.weight)
+            u = _hip.gemm_any(x2, self.up_proj.weight)
             act = _hip.gelu_mul(g, u, out=g)
-            out = torch.matmul(act, self.down_proj.weight.t())
+            out = _hip.gemm_any(act, self.down_proj.weight)
         return out.reshape(shape)

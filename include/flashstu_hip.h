@@ -364,6 +364,15 @@ int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const void* W2, co
 int fstu_gemm_bf16_splitk(const void* A, int64_t lda, const void* W, float* partial, int M, int N, int K, int ksplit,
                           void* stream);
 
+/* General contraction for what fstu_gemm_bf16 does not take: fp32 (the reference's fp32 configuration,
+ * flash_stu/model.py:108-205 with torch_dtype float32: every nn.Linear of the prompt pass), bf16 shapes with
+ * K % 32 != 0 or unaligned rows, and operands given by strides (phi @ M_filters, flash_stu/modules/stu.py:88; the
+ * fp32 slabs of exact mode, stu.py:107-120).  C (M,N; row stride ldc) = T(A W^T), A element (m,k) at A[m*sam + k*sak],
+ * W element (n,k) at W[n*swn + k*swk] (strides in elements, positive); fp32 accumulation on the fp32 matrix
+ * instruction, one rounding to `dtype`.  Any M, N, K >= 1. */
+int fstu_gemm_any(const void* A, int64_t sam, int64_t sak, const void* W, int64_t swn, int64_t swk, void* C, int64_t ldc,
+                  int M, int N, int K, int dtype, void* stream);
+
 /* The contraction of the exact-mode STU operator (flash_stu/modules/stu.py:107-120: tensordot of U+- (B,L,K,d) with
  * M_phi+- (K,d,d) over (K,d)) with U stored as the filter-bank kernel writes it, time-major: nbatch slabs A[b] of shape
  * (K, M) — the reduction index slowest, M contiguous, row stride lda, slab stride batch_stride_a (elements) — against

@@ -144,6 +144,36 @@ def test_gemm_bf16_plain_and_residual(hip, M, N, K):
     check(rd, (res.float() + ref.float()).bfloat16(), torch.bfloat16, frac=0.05, atol=2.0 ** -7 * float(ref.float().abs().max()))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(64, 256, 256), (1000, 772, 100), (17, 3, 5), (300, 200, 1056), (1, 1, 1), (129, 65, 33),
+                                   (4096, 768, 256)])
+def test_gemm_any_against_float64(hip, dtype, M, N, K):
+    """fstu_gemm_any (every dense contraction the bf16 prompt GEMM does not take: the fp32 configuration, odd shapes,
+    strided operands) against a float64 matmul rounded once: fp32 within summation-order noise, bf16 within one ulp;
+    row-major, transposed (k slowest) and padded views of either operand give the same values."""
+    g = gen(64)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    ref = (x.double() @ W.double().t()).to(dtype)
+    xd, Wd = dev(x), dev(W)
+    got = hip.gemm_any(xd, Wd)
+    check(got, ref, dtype)
+    xt = xd.t().contiguous().t()                      # element (m,k) at k*M + m
+    Wt = Wd.t().contiguous().t()
+    assert torch.equal(hip.gemm_any(xt, Wt), got)
+    wide = torch.full((M, K + 3), float("nan"), dtype=dtype, device="cuda")
+    wide[:, :K] = xd
+    out = torch.full((M, N + 5), float("nan"), dtype=dtype, device="cuda")
+    hip.gemm_any(wide[:, :K], Wd, out=out[:, :N])
+    assert torch.equal(out[:, :N], got) and bool(torch.isnan(out[:, N:]).all())
+    # the dispatcher takes what the bf16 matrix-core kernel refuses (and fp32 beyond 16 rows) to this kernel
+    if M > 16:
+        check(hip.linear(xd, Wd), ref, dtype)
+        b = torch.randn(N, generator=g).to(dtype)
+        check(hip.linear(xd, Wd, dev(b)), (ref.float() + b.float()).to(dtype), dtype, frac=0.05,
+              atol=2.0 ** -7 * float(ref.float().abs().max()))
+
+
 @pytest.mark.parametrize("nb,M,N,K", [(1, 128, 64, 64), (3, 256, 132, 192), (2, 1024, 1024, 1536), (4, 512, 260, 2048),
                                       (1, 4096, 768, 3072)])
 def test_gemm_bf16_transposed_activations(hip, nb, M, N, K):
