@@ -439,13 +439,13 @@ def run_c4(args, torch, _hip):
     torch.cuda.synchronize()
     dt_s = time.perf_counter() - t0
     ms = dt_s / K * 1e3
-    alg = 2 * T * Bt * d * 2 + (2 * d * S * 2 + S * 4) + 2 * Bt * S * 4
+    alg = 2 * T * Bt * d * 2 + (2 * d * S * 2 + S * 4) + 2 * Bt * S * 4      # x in, y out, weights, state
     gbps = alg / (ms * 1e-3) / 1e9
     # launch by launch (one position per launch, state carried in HBM)
     n1 = 512
     h.zero_()
     tr = (Bm.t().contiguous(), Cm.t().contiguous())
-    ws1 = torch.empty(3 * Bt * S, dtype=torch.float32, device="cuda")
+    ws1 = torch.empty(int(_hip.load().fstu_lds_sequence_ws_floats(1, Bt, S)), dtype=torch.float32, device="cuda")
     for t in range(16):
         _hip.lds_steps(h, x[t:t + 1], A, Bm, Cm, y[t:t + 1], transposed=tr, ws=ws1)
     torch.cuda.synchronize()
@@ -460,7 +460,7 @@ def run_c4(args, torch, _hip):
             "config": {"workload": "BASELINE config 4: dense LDS step, batch 64, d_in=d_out=1024, state 160, A~U(0.9,0.999) fp32, "
                                    "B~N(0,1/d), C~N(0,1/160) bf16, 4096 consecutive steps in one launch (a bench step = one launch)",
                        "positions_per_launch": T, "us_per_position_one_launch": ms * 1e3 / T, "us_per_position_launch_by_launch": us_launch},
-            "roofline": {"bound": "hbm", "kernel": "lds_seq_kernel x2 + lds_carry_kernel (blocks of 128 positions on the matrix cores; x is read twice)", "achieved": gbps,
+            "roofline": {"bound": "hbm", "kernel": "lds_seq_kernel (blocks of 128 positions on the matrix cores, the state handed from block to block inside the launch; x is read once)", "achieved": gbps,
                          "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": alg}}
 
 

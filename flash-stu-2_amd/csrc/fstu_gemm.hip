@@ -549,9 +549,11 @@ int gemm_launch(const void* A, long long lda, const void* W, const void* W2, con
   if constexpr (MODE != 1) {
     // A feature count that is a whole number of 96-wide tiles but leaves compute units idle (or nearly idle in a last
     // round) with 128-wide ones: the time follows the rounds a compute unit runs times the area of a tile
-    // (N = 768, M = 4096: 192 tiles of 128 x 128 on 256 CUs against 256 tiles of 96 x 128).
+    // (N = 768, M = 4096: 192 tiles of 128 x 128 on 256 CUs against 256 tiles of 96 x 128).  Only where the 128-wide
+    // grid does not fill the chip: with several rounds per compute unit two resident workgroups of 128 x 128 cover
+    // each other's start and end (N = 2304, M = 4096: 28.5 us against 35.2 us for the 96-wide tile).
     const long long cus = gemm_cus(), t96 = (long long)((M + 127) / 128) * (N / 96);
-    if (N % 96 == 0 && ((t96 + cus - 1) / cus) * 96 < ((small + cus - 1) / cus) * 128)
+    if (N % 96 == 0 && small <= cus && ((t96 + cus - 1) / cus) * 96 < ((small + cus - 1) / cus) * 128)
       return gemm_launch_tile<Tile96, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);
   }
   if (K >= 2048 && small <= gemm_cus()) return gemm_launch_tile<TileDeep, MODE>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, s);

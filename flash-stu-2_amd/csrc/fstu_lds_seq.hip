@@ -1,13 +1,16 @@
 // Dense LDS over a whole sequence on the matrix cores (bf16): the loop of mini_stu/lds.py:95-101,
 //   h <- h * A + x_t @ B ;  y_t = T(h @ C),   t = 0 .. T-1, state h (Bt,S) fp32 carried,
-// cut into blocks of 128 positions that run in parallel.  x_t @ B does not depend on the state, so a block forms
-// U = X_blk B with MFMA tiles and scans it in LDS; the state that enters a block is handed over by a short chain:
-//   pass 1  (block, batch row): U tile, scan from zero, the block's end state E
-//   pass 2  per (row, mode): carry[k+1] = E[k] + A^len(k) * carry[k], carry[0] = the caller's h; the last carry is the
-//           new h.  Splitting a sequence at a multiple of 128 therefore gives bit-identical states and outputs.
-//   pass 3  (block, batch row): U tile again (x is read twice instead of writing and re-reading U: the same bytes,
-//           no workspace of the size of the sequence), scan from carry[k], Y = H C with H split into a bf16 head and
-//           a bf16 remainder so that the second product keeps the fp32 state's accuracy.
+// cut into blocks of 128 positions that run in parallel, x read ONCE.  x_t @ B does not depend on the state, so a
+// workgroup (block, batch row) forms U = X_blk B with MFMA tiles and keeps it in LDS from then on:
+//   1  scan U from zero: the block's end state E, published at once as tagged 64-bit words (value, tag of the call)
+//   2  the state that enters the block: carry = h, then carry = E[j] + A^128 * carry over the blocks j in front of it,
+//      read from what those blocks published (they are earlier in launch order, so they are resident or done, and
+//      they publish before they wait for anything: the wait ends; it is bounded all the same and reports a
+//      time-out through a status word instead of hanging).  The chain is the same fused multiply-adds in the same
+//      order for every block, so splitting a sequence at a multiple of 128 gives bit-identical states and outputs.
+//      The last block of a row also forms the state behind the sequence.
+//   3  scan U again from the carry (now the true states H), Y = H C with H split into a bf16 head and a bf16
+//      remainder so that the second product keeps the fp32 state's accuracy.
 // Weights are given transposed (B^T (S,d_in), C^T (d_out,S)) so that every MFMA fragment is one 16-byte piece; both
 // travel through LDS so that the four waves of a workgroup share one fetch.
 #include "fstu_common.h"
@@ -37,11 +40,15 @@ __device__ __forceinline__ uint4 buf_load16(rsrc_t rs, unsigned off) {
 // at most 256 registers, and U without padding, 128 x S floats = 80 KB at S = 160.  Instead of a pad, the 16-byte slot
 // of element (row, mode) is XOR-ed with bits 1..3 of the row, which keeps the 16 rows of a tile access on 16 different
 // slots; the scan, one thread per mode, follows the same map.
-template <bool FINAL, int NT>
+#define LSQ_SPIN_LIMIT (1 << 18)   // polls of one batch of published states before the wait gives up
+#define LSQ_LOOK 8                 // published states requested at a time
+
+template <int NT>
 __global__ void __launch_bounds__(256, NT <= 10 ? 2 : 1)   // beyond S = 160 one workgroup fills the LDS anyway
 lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const bf16_t* __restrict__ BmT,
-               const bf16_t* __restrict__ CmT, bf16_t* __restrict__ y, const float* __restrict__ carry,
-               float* __restrict__ Eout, int T, int Bt, int d_in, int S, int d_out) {
+               const bf16_t* __restrict__ CmT, bf16_t* __restrict__ y, const float* __restrict__ h0,
+               float* __restrict__ hnew, unsigned long long* __restrict__ etag, unsigned* __restrict__ status, unsigned tag,
+               int T, int Bt, int d_in, int S, int d_out) {
   extern __shared__ __align__(16) float Us[];       // LSQ_TB x S
   const int ldu = S;
   auto uslot = [](int row, int slot) { return slot ^ ((row >> 1) & 7); };   // 16-byte slot of a row (S/4 slots, a multiple of 8)
@@ -148,9 +155,55 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
   // ---- scan over the block's positions: thread = mode
   if (tid < S) {
     const float a = A[tid];
-    float h = FINAL ? carry[((size_t)blk * Bt + b) * S + tid] : 0.f;
     // element (p, tid) sits at p * ldu + 4 * uslot(p, tid / 4) + tid % 4
     auto at = [&](int p_) { return Us + (size_t)p_ * ldu + 4 * uslot(p_, tid >> 2) + (tid & 3); };
+    // 1: the block's end state from zero, published as (tag, value)
+    float e = 0.f;
+    {
+      int p = 0;
+      for (; p + 8 <= nvalid; p += 8) {
+        float u[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u[i] = *at(p + i);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e = fmaf(a, e, u[i]);
+      }
+      for (; p < nvalid; ++p) e = fmaf(a, e, *at(p));
+    }
+    const size_t rowbase = (size_t)b * gridDim.x * S;
+    __hip_atomic_store(etag + rowbase + (size_t)blk * S + tid, ((unsigned long long)tag << 32) | __float_as_uint(e),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // 2: the state that enters this block (every block in front of it is a full one)
+    const double ad = (double)a;
+    const float ap_full = (float)pow(ad, (double)LSQ_TB);
+    float h = h0[(size_t)b * S + tid];
+    bool timed_out = false;
+    for (int j0 = 0; j0 < blk; j0 += LSQ_LOOK) {
+      unsigned long long wv[LSQ_LOOK];
+      int spins = 0;
+      bool ok;
+      do {
+        ok = true;
+#pragma unroll
+        for (int i = 0; i < LSQ_LOOK; ++i) {
+          const int j = min(j0 + i, blk - 1);
+          wv[i] = __hip_atomic_load(etag + rowbase + (size_t)j * S + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int i = 0; i < LSQ_LOOK; ++i) ok = ok && (unsigned)(wv[i] >> 32) == tag;
+        if (!ok) __builtin_amdgcn_s_sleep(4);
+      } while (!ok && ++spins < LSQ_SPIN_LIMIT);
+      timed_out = timed_out || !ok;
+#pragma unroll
+      for (int i = 0; i < LSQ_LOOK; ++i)
+        if (j0 + i < blk) h = fmaf(ap_full, h, __uint_as_float((unsigned)wv[i]));
+    }
+    if (timed_out) atomicOr(status, 1u);
+    if (blk == (int)gridDim.x - 1) {
+      const float ap = nvalid == LSQ_TB ? ap_full : (float)pow(ad, (double)nvalid);
+      hnew[(size_t)b * S + tid] = fmaf(ap, h, e);
+    }
+    // 3: the true states of the block's positions
     int p = 0;
     for (; p + 8 <= nvalid; p += 8) {
       float u[8];
@@ -159,16 +212,14 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         h = fmaf(a, h, u[i]);
-        if (FINAL) *at(p + i) = h;
+        *at(p + i) = h;
       }
     }
     for (; p < nvalid; ++p) {
       h = fmaf(a, h, *at(p));
-      if (FINAL) *at(p) = h;
+      *at(p) = h;
     }
-    if (!FINAL) Eout[((size_t)blk * Bt + b) * S + tid] = h;
   }
-  if (!FINAL) return;
   __syncthreads();
   // ---- Y = H C: wave w, positions 32w .. 32w+31; H as bf16 head + remainder
   {
@@ -262,31 +313,24 @@ lds_seq_kernel(const bf16_t* __restrict__ x, const float* __restrict__ A, const 
   }
 }
 
-// carry[0] = h; carry[k+1] = E[k] + A^len(k) * carry[k]; h = carry[nblk]
-__global__ void __launch_bounds__(256)
-lds_carry_kernel(float* __restrict__ h, const float* __restrict__ A, const float* __restrict__ E, float* __restrict__ carry,
-                 int nblk, int T, int BtS, int S) {
+// clears the published states of the call about to start
+__global__ void __launch_bounds__(256) lds_seq_clear_kernel(unsigned long long* __restrict__ etag, size_t n, unsigned* __restrict__ status) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) etag[i] = 0ull;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *status = 0u;
+}
+// the state behind the sequence replaces the caller's h (every block has read h by the time this launch starts)
+__global__ void __launch_bounds__(256) lds_seq_finish_kernel(float* __restrict__ h, const float* __restrict__ hnew, int n) {
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= BtS) return;
-  const double a = (double)A[i % S];
-  const float ap_full = (float)pow(a, (double)LSQ_TB);
-  float c = h[i];
-  carry[i] = c;
-  for (int k = 0; k < nblk; ++k) {
-    const int len = min(LSQ_TB, T - k * LSQ_TB);
-    const float ap = len == LSQ_TB ? ap_full : (float)pow(a, (double)len);
-    c = fmaf(ap, c, E[(size_t)k * BtS + i]);
-    carry[(size_t)(k + 1) * BtS + i] = c;
-  }
-  h[i] = c;
+  if (i < n) h[i] = hnew[i];
 }
 
 }  // namespace
 
+// workspace: 64 floats of header (status word), the published block states (nblk * Bt * S 64-bit words), the new h
 extern "C" size_t fstu_lds_sequence_ws_floats(int T, int Bt, int S) {
   if (T < 0 || Bt < 1 || S < 1) return 0;
   const size_t nblk = (size_t)(T + LSQ_TB - 1) / LSQ_TB;
-  return (2 * nblk + 1) * (size_t)Bt * S;
+  return 64 + (2 * nblk + 1) * (size_t)Bt * S;
 }
 
 extern "C" int fstu_lds_sequence(float* h, const void* x, const float* A, const void* BmT, const void* CmT, void* y, float* ws,
@@ -301,32 +345,43 @@ extern "C" int fstu_lds_sequence(float* h, const void* x, const float* A, const 
   if (T == 0) return FSTU_OK;
   const int nblk = (T + LSQ_TB - 1) / LSQ_TB;
   const size_t BtS = (size_t)Bt * S;
-  float* carry = ws;
-  float* E = ws + (size_t)(nblk + 1) * BtS;
+  unsigned* status = (unsigned*)ws;
+  unsigned long long* etag = (unsigned long long*)(ws + 64);
+  float* hnew = ws + 64 + 2 * (size_t)nblk * BtS;
   const size_t shm = (size_t)LSQ_TB * S * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(nblk, Bt);
+  const size_t nwords = (size_t)nblk * BtS;
+  unsigned cgrid = (unsigned)((nwords + 255) / 256);
+  if (cgrid > 1024u) cgrid = 1024u;
 #define LSQ_RUN(NTV)                                                                                                      \
   do {                                                                                                                    \
-    static const hipError_t e1 = hipFuncSetAttribute((const void*)lds_seq_kernel<false, NTV>,                             \
+    static const hipError_t e1 = hipFuncSetAttribute((const void*)lds_seq_kernel<NTV>,                                    \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);            \
-    static const hipError_t e2 = hipFuncSetAttribute((const void*)lds_seq_kernel<true, NTV>,                              \
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);            \
-    if (e1 != hipSuccess || e2 != hipSuccess) {                                                                           \
-      fstu_set_error("fstu_lds_sequence: hipFuncSetAttribute: %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));       \
-      return (int)(e1 != hipSuccess ? e1 : e2);                                                                           \
+    if (e1 != hipSuccess) {                                                                                               \
+      fstu_set_error("fstu_lds_sequence: hipFuncSetAttribute: %s", hipGetErrorString(e1));                                \
+      return (int)e1;                                                                                                     \
     }                                                                                                                     \
-    hipLaunchKernelGGL((lds_seq_kernel<false, NTV>), grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT,    \
-                       (const bf16_t*)CmT, (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);                    \
-    hipLaunchKernelGGL(lds_carry_kernel, dim3((unsigned)((BtS + 255) / 256)), dim3(256), 0, s, h, A, (const float*)E,     \
-                       carry, nblk, T, (int)BtS, S);                                                                      \
-    hipLaunchKernelGGL((lds_seq_kernel<true, NTV>), grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT,     \
-                       (const bf16_t*)CmT, (bf16_t*)y, (const float*)carry, E, T, Bt, d_in, S, d_out);                    \
+    hipLaunchKernelGGL(lds_seq_clear_kernel, dim3(cgrid), dim3(256), 0, s, etag, nwords, status);                         \
+    hipLaunchKernelGGL((lds_seq_kernel<NTV>), grid, dim3(256), shm, s, (const bf16_t*)x, A, (const bf16_t*)BmT,           \
+                       (const bf16_t*)CmT, (bf16_t*)y, (const float*)h, hnew, etag, status, 1u, T, Bt, d_in, S, d_out);   \
+    hipLaunchKernelGGL(lds_seq_finish_kernel, dim3((unsigned)((BtS + 255) / 256)), dim3(256), 0, s, h, (const float*)hnew, \
+                       (int)BtS);                                                                                         \
   } while (0)
   if (S <= 64) LSQ_RUN(4);
   else if (S <= 160) LSQ_RUN(10);
   else LSQ_RUN(16);
 #undef LSQ_RUN
   FSTU_CHECK_LAUNCH("fstu_lds_sequence");
+  return FSTU_OK;
+}
+
+// 0, or 1 when a wait of the last fstu_lds_sequence call on this workspace ran out (synchronous read of the status word)
+extern "C" int fstu_lds_sequence_status(const float* ws, int* err_out) {
+  FSTU_REQUIRE(ws && err_out, FSTU_ENULL, "fstu_lds_sequence_status: null pointer");
+  unsigned v = 0;
+  hipError_t e = hipMemcpy(&v, ws, sizeof(v), hipMemcpyDeviceToHost);
+  if (e != hipSuccess) { fstu_set_error("fstu_lds_sequence_status: %s", hipGetErrorString(e)); return (int)e; }
+  *err_out = (int)v;
   return FSTU_OK;
 }

@@ -85,6 +85,7 @@ SIGNATURES = {
     "fstu_gemm_any": [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i, _i, _i, _i, _vp],
     "fstu_gemm_bf16_ta": [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_sequence_ws_floats": [_i, _i, _i],
+    "fstu_lds_sequence_status": [_vp, _vp],
     "fstu_lds_sequence": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_lds_steps": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
@@ -840,11 +841,13 @@ def linear_packed_res(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Tens
 
 
 def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tensor, Cm: torch.Tensor,
-              out: Optional[torch.Tensor] = None, transposed=None, ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+              out: Optional[torch.Tensor] = None, transposed=None, ws: Optional[torch.Tensor] = None,
+              check_status: bool = False) -> torch.Tensor:
     """Dense LDS: h fp32 (Bt,S) carried in place over x (T,Bt,d_in) -> y (T,Bt,d_out).  bf16 with MFMA-friendly shapes
     runs on the matrix cores (fstu_lds_sequence); `transposed` = (Bm^T, Cm^T) contiguous copies and `ws` (fp32,
     lds_sequence_ws_floats elements) may be passed by callers that step position by position, to keep the two
-    transposes and the allocation out of every call."""
+    transposes and the allocation out of every call.  check_status: synchronise and raise if a wait inside the
+    sequence kernel ran out."""
     _dev(h, x, A, Bm, Cm, out, ws)
     T, Bt, d_in = x.shape
     S = A.numel()
@@ -865,6 +868,11 @@ def lds_steps(h: torch.Tensor, x: torch.Tensor, A: torch.Tensor, Bm: torch.Tenso
         assert bmt.shape == (S, d_in) and cmt.shape == (d_out, S) and bmt.is_contiguous() and cmt.is_contiguous()
         _check(lib.fstu_lds_sequence(_p(h), _p(x), _p(A), _p(bmt), _p(cmt), _p(out), _p(ws), T, Bt, d_in, S, d_out, _stream()),
                "fstu_lds_sequence")
+        if check_status:
+            err = ctypes.c_int(0)
+            _check(lib.fstu_lds_sequence_status(_p(ws), ctypes.byref(err)), "fstu_lds_sequence_status")
+            if err.value:
+                raise FlashSTUHipError("fstu_lds_sequence: a block waited in vain for the state of the blocks in front of it")
         return out
     _check(load().fstu_lds_steps(_p(h), _p(x), _p(A), _p(Bm), _p(Cm), _p(out), T, Bt, d_in, S, d_out, _dt(x), _stream()),
            "fstu_lds_steps")

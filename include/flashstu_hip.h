@@ -394,10 +394,15 @@ int fstu_lds_steps(float* h, const void* x, const float* A, const void* Bm, cons
 
 /* The same loop over a whole sequence on the matrix cores (bf16): blocks of 128 positions run in parallel (x_t @ Bm
  * does not depend on the state), a short chain hands the state from block to block.  Weights are given TRANSPOSED:
- * BmT (S,d_in), CmT (d_out,S).  ws: fstu_lds_sequence_ws_floats(T,Bt,S) floats, owned by the caller.  d_in % 32 == 0,
+ * BmT (S,d_in), CmT (d_out,S).  ws: fstu_lds_sequence_ws_floats(T,Bt,S) floats, owned by the caller (any contents; calls
+ * that share a workspace must not overlap).  d_in % 32 == 0,
  * S % 32 == 0, S <= 256, d_out % 16 == 0.  Same values as fstu_lds_steps up to the fp32 summation order; a sequence
- * split at a multiple of 128 positions into two calls gives bit-identical outputs and states. */
+ * split at a multiple of 128 positions into two calls gives bit-identical outputs and states.  x is read once: a
+ * block takes the state that enters it from what the blocks in front of it publish inside the same launch; that wait
+ * is bounded, and fstu_lds_sequence_status (a synchronous read) returns *err_out = 1 when it ran out in the last call
+ * on that workspace (the outputs of that call are then not valid), 0 otherwise. */
 size_t fstu_lds_sequence_ws_floats(int T, int Bt, int S);
+int fstu_lds_sequence_status(const float* ws, int* err_out);
 int fstu_lds_sequence(float* h, const void* x, const float* A, const void* BmT, const void* CmT, void* y, float* ws,
                       int T, int Bt, int d_in, int S, int d_out, void* stream);
 

@@ -147,8 +147,8 @@ def test_c4_lds_step_parity_at_full_width(hip):
     A, Bm, Cm, x = _c4_tensors(T)
     yref, href = O.lds_sequence(x, A, Bm, Cm)
     h = torch.zeros(64, 160, device="cuda")
-    y1 = hip.lds_steps(h, x[:100].cuda(), A.cuda(), Bm.cuda(), Cm.cuda())
-    y2 = hip.lds_steps(h, x[100:].cuda(), A.cuda(), Bm.cuda(), Cm.cuda())
+    y1 = hip.lds_steps(h, x[:100].cuda(), A.cuda(), Bm.cuda(), Cm.cuda(), check_status=True)
+    y2 = hip.lds_steps(h, x[100:].cuda(), A.cuda(), Bm.cuda(), Cm.cuda(), check_status=True)
     y = torch.cat([y1, y2]).float().cpu()
     diff = (y - yref.float()).abs()
     assert float(diff.max()) <= 2.0 ** -7 * float(yref.float().abs().max())
@@ -164,10 +164,10 @@ def test_c4_4096_steps_state_is_the_closed_form(hip):
     xs = x.expand(T, 64, 1024).contiguous().cuda()
     Ad, Bd, Cd = A.cuda(), Bm.cuda(), Cm.cuda()
     h1 = torch.zeros(64, 160, device="cuda")
-    y_full = hip.lds_steps(h1, xs, Ad, Bd, Cd)
+    y_full = hip.lds_steps(h1, xs, Ad, Bd, Cd, check_status=True)
     h2 = torch.zeros(64, 160, device="cuda")
-    ya = hip.lds_steps(h2, xs[:2048], Ad, Bd, Cd)
-    yb = hip.lds_steps(h2, xs[2048:], Ad, Bd, Cd)
+    ya = hip.lds_steps(h2, xs[:2048], Ad, Bd, Cd, check_status=True)
+    yb = hip.lds_steps(h2, xs[2048:], Ad, Bd, Cd, check_status=True)
     torch.cuda.synchronize()
     assert torch.equal(torch.cat([ya, yb]), y_full) and torch.equal(h1, h2)
     u = x[0].float() @ Bm.float()                                   # (64,160)

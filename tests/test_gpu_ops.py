@@ -1078,14 +1078,14 @@ def test_lds_sequence_on_the_matrix_cores(hip, T, Bt, din, S, dout):
     yref, href = O.lds_sequence(x, A, Bm, Cm)
     Ad, Bd, Cd, xd = dev(A), dev(Bm), dev(Cm), dev(x)
     h = torch.zeros(Bt, S, device="cuda")
-    y = hip.lds_steps(h, xd, Ad, Bd, Cd)
+    y = hip.lds_steps(h, xd, Ad, Bd, Cd, check_status=True)
     diff = (y.float().cpu() - yref.float()).abs()
     assert float(diff.max()) <= 2.0 ** -7 * float(yref.float().abs().max())
     assert float((diff > 0).float().mean()) < 0.05
     assert float((h.cpu() - href).abs().max()) <= 1e-4 * float(href.abs().max())
     h2 = torch.zeros(Bt, S, device="cuda")
-    ya = hip.lds_steps(h2, xd[:128], Ad, Bd, Cd)
-    yb = hip.lds_steps(h2, xd[128:], Ad, Bd, Cd)
+    ya = hip.lds_steps(h2, xd[:128], Ad, Bd, Cd, check_status=True)
+    yb = hip.lds_steps(h2, xd[128:], Ad, Bd, Cd, check_status=True)
     assert torch.equal(torch.cat([ya, yb]), y) and torch.equal(h2, h)
 
 
