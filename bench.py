@@ -201,6 +201,7 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
         traffic = 204052787 if packed and (d, I, rows) == (2048, 24576, 32) else None
         return {"bound": "hbm", "kernel": name,
                 "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
+                "traffic_source": "profiles/decode_c5_hbm_traffic_pmc.txt (counter runs of this kernel, not of this run)" if traffic else None,
                 "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n, "rows_per_launch": rows}
     ms_c, n_c = ctypes.c_double(), ctypes.c_int()
     torch.cuda.synchronize()
@@ -213,9 +214,11 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
     # HBM bytes per launch from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE, each scaled by what the same counter
     # reads for the library's plain 256 MiB copy kernel: x2.000 and x1.000); measured offline for the default workload,
     # summary and commands in profiles/glu_c2_hbm_traffic_pmc.txt
-    traffic = 28876800 if (cfg.n_embd, cfg.mlp_scale, rows) == (768, 12, 8) else None
+    default_shape = (cfg.n_embd, cfg.mlp_scale, rows) == (768, 12, 8)
+    traffic = 28870625 if default_shape else None
     return {"bound": "hbm", "kernel": "glu_balanced_kernel<PRO> (residual add + mlp_norm + gate/up projection + gelu*up)",
             "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
+            "traffic_source": "profiles/glu_c2_hbm_traffic_pmc.txt (counter runs of this kernel, not of this run)" if default_shape else None,
             "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n_c.value, "rows_per_launch": rows}
 
 
@@ -517,9 +520,9 @@ def run_ref(args, torch, _hip):
                        "batch": B, "L": L, "d": d, "K": Kf,
                        "published": {"ms_per_call": published_ms, "hardware": "NVIDIA H100 PCIe (another GPU: context, not a like-for-like bar)",
                                      "source": "tests/tilling/standard_memory_profile.txt:48-59"}},
-            "kernels_ms": {"x @ M_inputs (gemm_bf16_kernel)": ms_proj, "spectral convolution (fft_conv_rows_kernel)": ms_conv,
+            "kernels_ms": {"x @ M_inputs (gemm_bf16_kernel)": ms_proj, "spectral convolution (fft_conv_kernel)": ms_conv,
                            "projection_tflops": flops / (ms_proj * 1e-3) / 1e12},
-            "roofline": {"bound": "hbm", "kernel": "fft_conv_rows_kernel (spectral convolution of the projected inputs, both sign branches)",
+            "roofline": {"bound": "hbm", "kernel": "fft_conv_kernel (spectral convolution of the projected inputs, both sign branches, one column per workgroup)",
                          "achieved": conv_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": conv_gbps / HBM_PEAK_GBPS,
                          "traffic": None, "bytes_per_launch": conv_bytes, "avg_launch_us": ms_conv * 1e3}}
 

@@ -27,6 +27,10 @@ typedef float floatx16_t __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 
 #define GM_PANEL 8     // feature tiles per panel of the tile order
+// A workgroup addresses its tile through a buffer descriptor whose base is the tile's first row (64-bit arithmetic) and a
+// 32-bit byte offset per lane of at most 256 rows * row stride * 2 bytes: row strides (lda, and K for the weights) stay
+// below 2^22 elements so that this offset cannot wrap; what lies beyond a tile's rows is cut off by the descriptor's range
+#define GM_MAX_LD (1 << 22)
 
 __device__ __forceinline__ float rnd_bf16(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 __device__ __forceinline__ float gelu_tanh_fast(float x) {
@@ -571,6 +575,8 @@ extern "C" int fstu_gemm_bf16_splitk(const void* A, int64_t lda, const void* W, 
                "fstu_gemm_bf16_splitk: M=%d N=%d (N %% 4 == 0) lda=%lld", M, N, (long long)lda);
   FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(partial, 16), FSTU_EALIGN,
                "fstu_gemm_bf16_splitk: pointers must be 16-byte aligned");
+  FSTU_REQUIRE(lda < GM_MAX_LD && K < GM_MAX_LD, FSTU_ESHAPE, "fstu_gemm_bf16_splitk: lda=%lld / K=%d beyond the 32-bit tile offsets",
+               (long long)lda, K);
   int rc;
   if (M <= 32) rc = gemm_launch_tile<TileRows32, 3>(A, lda, W, nullptr, nullptr, 0, partial, N, M, N, K, (hipStream_t)stream, ksplit);
   else rc = gemm_launch_tile<TileSmall, 3>(A, lda, W, nullptr, nullptr, 0, partial, N, M, N, K, (hipStream_t)stream, ksplit);
@@ -590,6 +596,8 @@ extern "C" int fstu_gemm_bf16(const void* A, int64_t lda, const void* W, const v
                "fstu_gemm_bf16: row strides (lda=%lld ldc=%lld ldr=%lld)", (long long)lda, (long long)ldc, (long long)ldr);
   FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(W2, 16) && fstu_aligned(C, 8) && fstu_aligned(R, 8),
                FSTU_EALIGN, "fstu_gemm_bf16: pointers must be 16-byte aligned (C, R: 8)");
+  FSTU_REQUIRE(lda < GM_MAX_LD && K < GM_MAX_LD, FSTU_ESHAPE, "fstu_gemm_bf16: lda=%lld / K=%d beyond the 32-bit tile offsets",
+               (long long)lda, K);
   int rc;
   if (mode == 0) rc = gemm_launch<0>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
   else if (mode == 1) rc = gemm_launch<1>(A, lda, W, W2, R, ldr, C, ldc, M, N, K, (hipStream_t)stream);
@@ -614,6 +622,8 @@ extern "C" int fstu_gemm_bf16_ta(const void* A, int64_t lda, int64_t batch_strid
   // 32-bit byte offsets inside a slab (buffer addressing) and inside W
   FSTU_REQUIRE((unsigned long long)K * (unsigned long long)lda * 2ull < 0xfff00000ull && (unsigned long long)N * K * 2ull < 0xfff00000ull,
                FSTU_ESHAPE, "fstu_gemm_bf16_ta: a slab (K*lda) or W (N*K) exceeds 4 GB of 32-bit offsets");
+  FSTU_REQUIRE(lda < GM_MAX_LD && K < GM_MAX_LD, FSTU_ESHAPE, "fstu_gemm_bf16_ta: lda=%lld / K=%d beyond the 32-bit tile offsets",
+               (long long)lda, K);
   FSTU_REQUIRE(batch_stride_a % 8 == 0 && batch_stride_c % 4 == 0 && batch_stride_r % 4 == 0, FSTU_ESHAPE,
                "fstu_gemm_bf16_ta: batch strides must keep the alignment");
   FSTU_REQUIRE(fstu_aligned(A, 16) && fstu_aligned(W, 16) && fstu_aligned(C, 8) && fstu_aligned(R, 8), FSTU_EALIGN,
