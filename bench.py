@@ -442,6 +442,8 @@ def run_c4(args, torch, _hip):
     torch.cuda.synchronize()
     dt_s = time.perf_counter() - t0
     ms = dt_s / K * 1e3
+    _hip.lds_steps(h, x, A, Bm, Cm, y, check_status=True)      # raises if a block's wait for its predecessors ran out
+    assert bool(torch.isfinite(y.float()).all())
     alg = 2 * T * Bt * d * 2 + (2 * d * S * 2 + S * 4) + 2 * Bt * S * 4      # x in, y out, weights, state
     gbps = alg / (ms * 1e-3) / 1e9
     # launch by launch (one position per launch, state carried in HBM)
