@@ -40,6 +40,26 @@ def _exact_stu(dtype, d, L, K, seed):
     return stu.cuda(), phi, p
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T", [200, 384, 20])
+def test_c3_exact_mode_ragged_lengths_and_both_dtypes(dtype, T):
+    """The exact-mode operator on sequences shorter than the filters and not a multiple of the contraction's
+    128-position tiles (the slabs are padded to whole tiles and the padding's rows cut off again), in bf16 (matrix-core
+    contraction over the time-major slabs) and fp32 (the general kernel on the slab as a strided operand), and below
+    the shortest transform (time-domain filter bank, row-major U): all against the oracle on the same inputs."""
+    stu, phi, p = _exact_stu(dtype, 64, 512, 8, 7)
+    x = torch.randn(3, T, 64, generator=torch.Generator().manual_seed(8)).to(dtype)
+    ref = O.stu_forward(x, phi, p, 1024, use_approx=False).float()
+    y = stu(x.cuda()).float().cpu()
+    assert y.shape == ref.shape and bool(torch.isfinite(y).all())
+    scale = float(ref.abs().max())
+    if dtype == torch.float32:
+        assert float((y - ref).abs().max()) <= 2e-4 * scale
+    else:
+        assert float((y - ref).abs().max()) <= 3e-2 * scale
+        assert float((y - ref).abs().mean()) <= 3e-3 * scale
+
+
 def test_c3_exact_mode_prefill_parity_reduced():
     """Config 3's operator (use_approx=False, K=24, M_phi ~ N(0,1/sqrt(d))) at B=2, L=1024, d=128, bf16."""
     dtype = torch.bfloat16
