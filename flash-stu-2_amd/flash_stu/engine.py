@@ -14,7 +14,6 @@ consecutive row chunks of 16 against the same weights and batch-first state.
 from __future__ import annotations
 
 import ctypes
-import os
 from typing import List, Optional
 
 import torch
