@@ -105,11 +105,14 @@ extern "C" int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* st
   } while (0)
 
 // recurrence step on m->xp: both sign branches rounded separately when the layer carries odd-lag weights
-static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, const int* pos_dyn, void* stream) {
+// (stream_x: the residual stream; the step then adds its output to it in place instead of leaving it in m->y)
+static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, const int* pos_dyn, void* stream,
+                    void* stream_x = nullptr) {
   if (L.lds_co)
     return fstu_stu_step_lds_pair_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, L.lds_co, L.lds_ring, L.lds_fir,
-                                      L.lds_fir ? m->lds_fir_taps : 0, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, pos_dyn,
-                                      m->dtype, stream);
+                                      L.lds_fir ? m->lds_fir_taps : 0, stream_x ? stream_x : m->y, m->d, m->B, m->lds_S, m->d, pos,
+                                      dyn, pos_dyn, m->dtype, stream, stream_x);
+  if (stream_x) return FSTU_EARG;
   return fstu_stu_step_lds_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, m->dtype,
                                stream);
 }
@@ -176,26 +179,35 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
   TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt, stream, dyn));
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
+    // Where the layer's MLP streams packed weights, the sub-layer's last launch adds its output to the residual stream
+    // itself (m->x in place) and the gate/up launch normalises the stream in its own fragments: no add+norm launch
+    // between them.
+    const bool join = packed_mlp && L.wp_gate && L.wp_up && (L.kind == 0 ? L.lds_co != nullptr : L.wp_proj != nullptr);
     if (L.kind == 0) {
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
       if (packed_mlp && L.wp_m_inputs) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_m_inputs, m->xp, d, B, d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
-      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream));
+      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream, join ? m->x : nullptr));
     } else {
       if (packed_mlp && L.wp_qkv) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.w_qkv, m->qkv, 3 * d, 3 * d, d));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
                                          m->window, m->softcap, 1, dyn, dt, stream));
-      if (packed_mlp && L.wp_proj) TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
+      if (join) TIMED(PC_PROJ, fstu_linear_packed_add(m->attn, d, L.wp_proj, m->x, m->x, B, d, d, stream));
+      else if (packed_mlp && L.wp_proj) TIMED(PC_PROJ, fstu_linear_packed(m->attn, d, nullptr, 0.f, L.wp_proj, m->y, d, B, d, d, stream));
       else TIMED(PC_PROJ, proj(m->attn, d, L.w_proj, m->y, d, d, d));
     }
     const void* next_w = (l + 1 < m->n_layers) ? m->layers[l + 1].norm1_w : m->final_norm_w;
-    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
     // the MLP over packed weights where the model holds them (contiguous streams, one workgroup per compute unit with
     // equal bytes each: measured 33 against 46 us for the 201 MB of a 2048-d gate/up pair), else the tiled GEMM
     int nsl = ks;
-    if (packed_mlp && L.wp_gate && L.wp_up) TIMED(PC_GLU, fstu_glu_packed(m->h, d, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
-    else TIMED(PC_GLU, fstu_gemm_bf16(m->h, d, L.w_gate, L.w_up, nullptr, 0, m->act, I, B, I, d, 1, stream));
+    if (join) {
+      TIMED(PC_GLU, fstu_glu_packed_norm(m->x, nullptr, nullptr, L.mlp_norm_w, m->eps, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
+    } else {
+      TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->y, 0, 1, 0, L.mlp_norm_w, m->h, B, d, m->eps, dt, stream));
+      if (packed_mlp && L.wp_gate && L.wp_up) TIMED(PC_GLU, fstu_glu_packed(m->h, d, L.wp_gate, L.wp_up, m->act, I, B, I, d, stream));
+      else TIMED(PC_GLU, fstu_gemm_bf16(m->h, d, L.w_gate, L.w_up, nullptr, 0, m->act, I, B, I, d, 1, stream));
+    }
     if (packed_mlp && L.wp_down) {
       nsl = 16;
       TIMED(PC_DOWN, fstu_down_packed_splitk(m->act, I, L.wp_down, m->partial, B, d, I, &nsl, stream));

@@ -153,7 +153,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
   constexpr bool GLU = EPI == 0;
   constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
   constexpr int NXC = 4;
-  static_assert(NB == 1 || (NB == 2 && PRO == 0), "two row tiles: launches without the norm prologue only");
+  static_assert(PRO == 3 ? NB == 2 : (NB == 1 || PRO == 0), "two row tiles: no prologue, or the in-register one (PRO 3)");
   constexpr int RED = DA * 8 * 512;                           // partial sums of one row tile
   __shared__ float red_one[NB == 1 ? RED : 1];
   extern __shared__ __align__(16) unsigned char glu_smem[];   // PRO: h rows (rows x (d+8)) bf16; NB 2: the partial sums
@@ -200,7 +200,7 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       if (ta0 + j < ta1) load_a(j, ta0 + j);
   };
 
-  if (!PRO) {
+  if constexpr (PRO == 0) {
     // activations first (they are consumed first), then the weights
     const rsrc_t rh = make_rsrc(a.h, ((size_t)(a.rows - 1) * a.ldh + a.d) * 2);
     const unsigned hoff = ((unsigned)(xrow ? r : 0) * (unsigned)a.ldh + (unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
@@ -212,6 +212,92 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
       for (int u = 0; u < KSA; ++u) xa2[u] = buf_load16(rh, xrow2 ? hoff + (unsigned)(16 * a.ldh) * 2u + (unsigned)u * 64u : MLP_OOB);
     }
     load_first();
+  } else if constexpr (PRO == 3) {
+    // Two row tiles (17..32 dense rows of stride d), x_in = the residual stream with the sub-layer's output already
+    // added: h = T((x * rstd) * w) is formed in the B fragments themselves.  A row's sum of squares goes over the
+    // four lane groups by shuffles and over the 8 waves (which split K) through LDS, as do the norm weights (kept in
+    // registers next to both row tiles and the weight fragments they would spill).  All of it happens while the
+    // weights, requested right behind the activations, are on their way.
+    __shared__ float ss_part[8][32];
+    __shared__ __align__(16) unsigned nw_s[128 * KSA];
+    constexpr int NWD = (KSA + 3) / 4;
+    unsigned nwt[NWD];
+    const rsrc_t rxi = make_rsrc(a.x_in, (size_t)a.rows * a.d * 2), rnw = make_rsrc(a.norm_w, (size_t)a.d * 2);
+    const unsigned koff = ((unsigned)(w * KSA) * 32u + (unsigned)g * 8u) * 2u;
+    const unsigned o1 = (unsigned)r * (unsigned)a.d * 2u + koff, o2 = o1 + 16u * (unsigned)a.d * 2u;
+    const bool xrow2 = 16 + r < a.rows;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) xa[u] = buf_load16(rxi, xrow ? o1 + (unsigned)u * 64u : MLP_OOB);
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) xa2[u] = buf_load16(rxi, xrow2 ? o2 + (unsigned)u * 64u : MLP_OOB);
+#pragma unroll
+    for (int k = 0; k < NWD; ++k) {
+      const unsigned i = threadIdx.x + k * 512u;
+      nwt[k] = __builtin_amdgcn_raw_buffer_load_b32(rnw, i < 128u * KSA ? i * 4u : MLP_OOB, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the activations' requests stay in front of the weights'
+    // One tile of weights (16 KB per wave) goes out behind them, the others after the rows are scaled: with every
+    // tile of every workgroup queued at once the activations come back late (38.3 against 36.5 us for the launch
+    // at 2048 x 24576).
+    load_a(0, ta0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    auto squares = [](uint4 v, float& ss) {
+      const unsigned vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(vw[i] << 16), hi = __uint_as_float(vw[i] & 0xffff0000u);
+        ss = fmaf(lo, lo, ss);
+        ss = fmaf(hi, hi, ss);
+      }
+    };
+    float ss1 = 0.f, ss2 = 0.f;
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) {
+      squares(xa[u], ss1);
+      squares(xa2[u], ss2);
+    }
+    // the rows stay packed until they are scaled: without this the unpacked values of the squares above (twice the
+    // registers) are kept for the scaling below and spill
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) {
+      asm volatile("" : "+v"(xa[u].x), "+v"(xa[u].y), "+v"(xa[u].z), "+v"(xa[u].w));
+      asm volatile("" : "+v"(xa2[u].x), "+v"(xa2[u].y), "+v"(xa2[u].z), "+v"(xa2[u].w));
+    }
+    ss1 += __shfl_xor(ss1, 16, 64);
+    ss1 += __shfl_xor(ss1, 32, 64);
+    ss2 += __shfl_xor(ss2, 16, 64);
+    ss2 += __shfl_xor(ss2, 32, 64);
+    if (g == 0) { ss_part[w][r] = ss1; ss_part[w][16 + r] = ss2; }
+#pragma unroll
+    for (int k = 0; k < NWD; ++k) {
+      const unsigned i = threadIdx.x + k * 512u;
+      if (i < 128u * KSA) nw_s[i] = nwt[k];
+    }
+    __syncthreads();
+    float t1 = 0.f, t2 = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) { t1 += ss_part[s][r]; t2 += ss_part[s][16 + r]; }
+    const float rs1 = rsqrtf(t1 / (float)a.d + a.eps), rs2 = rsqrtf(t2 / (float)a.d + a.eps);
+    auto scale8 = [](uint4 v, uint4 wv, float rstd) {
+      unsigned vw[4] = {v.x, v.y, v.z, v.w};
+      const unsigned ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        vw[i] = pack2_bf16((__uint_as_float(vw[i] << 16) * rstd) * __uint_as_float(ww[i] << 16),
+                           (__uint_as_float(vw[i] & 0xffff0000u) * rstd) * __uint_as_float(ww[i] & 0xffff0000u));
+      return make_uint4(vw[0], vw[1], vw[2], vw[3]);
+    };
+#pragma unroll
+    for (int u = 0; u < KSA; ++u) {
+      const uint4 nwv = *(const uint4*)(nw_s + (w * KSA + u) * 16 + g * 4);
+      xa[u] = scale8(xa[u], nwv, rs1);
+      xa2[u] = scale8(xa2[u], nwv, rs2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 1; j < DA; ++j)
+      if (ta0 + j < ta1) load_a(j, ta0 + j);
   } else {
     // x' = T(x + delta) (workgroup 0 also stores it), h = T((x' * rstd) * w) into LDS, then this wave's B fragments.
     // The 24 KB of x and delta are requested and consumed BEFORE the weights are requested: they return at
@@ -317,6 +403,22 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
         }
       }
     }
+    // EPI 1 with x_out: the projection's output joins the residual stream here, x_out = T(x_in + T(y)) (rows of stride
+    // ldact in both); the pairs of x_in this wave will need are requested before the barrier
+    unsigned resw[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) resw[nb] = 0u;
+    if constexpr (EPI == 1 && PRO == 0) {
+      if (a.x_out) {
+        const int fbp = (t0 + (w >> 1)) * 16 + g * 4 + (w & 1) * 2;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int row = 16 * nb + r;
+          const bool okp = (w >> 1) < DA && row < a.rows && fbp >= f0 && fbp + 2 <= f1;
+          resw[nb] = okp ? *(const unsigned*)(a.x_in + (size_t)row * a.ldact + fbp) : 0u;
+        }
+      }
+    }
     __syncthreads();
     // reduction over the 8 K slices and the epilogue: wave w takes half a tile (two of a lane's four features)
     if ((w >> 1) < DA && t0 + (w >> 1) < ta1) {
@@ -372,7 +474,14 @@ glu_balanced_kernel(const bf16_t* h, const uint4* wp_gate, const uint4* wp_up, b
           }
           run_key[nb] = key > run_key[nb] ? key : run_key[nb];
         }
-        if (grp_ok) {
+        if (EPI == 1 && PRO == 0 && a.x_out) {
+          // (feature ranges start and end on multiples of 8 and ldact is even here: whole pairs only)
+          if (grp_ok) {
+            const float y0 = DT<bf16_t>::rnd(o[0]), y1 = DT<bf16_t>::rnd(o[1]);
+            *(unsigned*)(a.x_out + (size_t)row * a.ldact + fb) =
+                pack2_bf16(__uint_as_float(resw[nb] << 16) + y0, __uint_as_float(resw[nb] & 0xffff0000u) + y1);
+          }
+        } else if (grp_ok) {
           bf16_t* yr = a.act + (size_t)row * a.ldact + fb;
           if (fb + 2 <= f1 && (a.ldact & 1) == 0) {
             *(unsigned*)yr = pack2_bf16(o[0], o[1]);
@@ -562,17 +671,18 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
     // two row tiles: the partial sums of both lie in dynamic LDS
     constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
     const size_t red2 = (size_t)2 * DA * 8 * 512 * sizeof(float);
-    FSTU_REQUIRE(pro == 0, FSTU_ESHAPE, "%s: more than %d rows only without the norm prologue", name, FSTU_MAX_DECODE_ROWS);
-#define GLU_GO2(EPI)                                                                                                       \
+    FSTU_REQUIRE(pro == 0 || (pro == 3 && epi == 0), FSTU_ESHAPE, "%s: more than %d rows: no prologue, or the gated pair with the in-register one",
+                 name, FSTU_MAX_DECODE_ROWS);
+#define GLU_GO2(PRO, EPI)                                                                                                  \
   do {                                                                                                                     \
-    static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, 0, EPI, 2>),    \
+    static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(glu_balanced_kernel<KSA, PRO, EPI, 2>),  \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)red2);               \
     FSTU_REQUIRE(attr_err == hipSuccess, (int)attr_err, "%s: %zu bytes of dynamic LDS refused", name, red2);               \
-    hipLaunchKernelGGL((glu_balanced_kernel<KSA, 0, EPI, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act,  \
+    hipLaunchKernelGGL((glu_balanced_kernel<KSA, PRO, EPI, 2>), dim3(G), dim3(512), red2, s, a.h, a.wp_gate, a.wp_up, a.act, \
                        a.x_in, a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices, a.best,  \
                        a.temperature);                                                                                      \
   } while (0)
-    if (epi == 0) GLU_GO2(0); else if (epi == 2) GLU_GO2(2); else GLU_GO2(1);
+    if (pro == 3) GLU_GO2(3, 0); else if (epi == 0) GLU_GO2(0, 0); else if (epi == 2) GLU_GO2(0, 2); else GLU_GO2(0, 1);
 #undef GLU_GO2
     return FSTU_OK;
   }
@@ -601,7 +711,7 @@ static int glu_launch(GluArgs& a, int pro, int epi, const char* name, hipStream_
   // out of one L2 per XCD
   if (epi != 0 && G > (a.I + 15) / 16) G = (a.I + 15) / 16;
   a.fpw = 0;
-  const size_t shm = pro ? (size_t)a.rows * (a.d + 8) * 2 : 0;
+  const size_t shm = (pro == 1 || pro == 2) ? (size_t)a.rows * (a.d + 8) * 2 : 0;
   int rc;
   switch (a.d / 256) {
     case 1: rc = glu_launch_ksa<1>(a, pro, epi, G, shm, name, s); break;
@@ -637,19 +747,25 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
                                     const void* wp_gate, const void* wp_up, void* act, int ldact, int rows, int I, int d,
                                     void* stream) {
   FSTU_REQUIRE(x_in && norm_w && wp_gate && wp_up && act, FSTU_ENULL, "fstu_glu_packed_norm: null pointer");
-  FSTU_REQUIRE(fstu_glu_packed_supported(rows, d, I), FSTU_ESHAPE, "fstu_glu_packed_norm: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  // 17..32 rows: the norm is formed in the matrix-core fragments (two row tiles) of a stream that already holds the
+  // sub-layer's output (fstu_linear_packed_add, the recurrence step with a residual): no delta, nothing stored
+  const bool wide = rows > FSTU_MAX_DECODE_ROWS;
+  FSTU_REQUIRE(wide ? fstu_mlp_packed_rows32_supported(rows, d, I) : fstu_glu_packed_supported(rows, d, I), FSTU_ESHAPE,
+               "fstu_glu_packed_norm: unsupported shape rows=%d d=%d I=%d", rows, d, I);
+  FSTU_REQUIRE(!wide || (delta == nullptr && x_out == nullptr), FSTU_EARG,
+               "fstu_glu_packed_norm: more than %d rows take the summed stream (delta and x_out must be NULL)", FSTU_MAX_DECODE_ROWS);
   FSTU_REQUIRE(ldact >= I && ldact % 4 == 0, FSTU_ESHAPE, "fstu_glu_packed_norm: ldact=%d", ldact);
-  FSTU_REQUIRE(x_out != x_in, FSTU_EARG, "fstu_glu_packed_norm: x_out must not alias x_in (other workgroups still read it)");
+  FSTU_REQUIRE(wide || x_out != x_in, FSTU_EARG, "fstu_glu_packed_norm: x_out must not alias x_in (other workgroups still read it)");
   FSTU_REQUIRE(fstu_aligned(x_in, 16) && fstu_aligned(delta, 16) && fstu_aligned(x_out, 16) && fstu_aligned(norm_w, 16) &&
                    fstu_aligned(wp_gate, 16) && fstu_aligned(wp_up, 16) && fstu_aligned(act, 8),
                FSTU_EALIGN, "fstu_glu_packed_norm: pointers must be 16-byte aligned");
-  FSTU_REQUIRE((size_t)rows * (d + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_glu_packed_norm: rows*d too large for LDS");
+  FSTU_REQUIRE(wide || (size_t)rows * (d + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_glu_packed_norm: rows*d too large for LDS");
   GluArgs a = {};
   a.wp_gate = (const uint4*)wp_gate; a.wp_up = (const uint4*)wp_up; a.act = (bf16_t*)act;
   a.rows = rows; a.d = d; a.I = I; a.ldh = d; a.ldact = ldact;
   a.x_in = (const bf16_t*)x_in; a.delta = delta; a.x_out = (bf16_t*)x_out; a.norm_w = (const bf16_t*)norm_w;
   a.eps = eps;
-  return glu_launch(a, 1, 0, "fstu_glu_packed_norm", (hipStream_t)stream);
+  return glu_launch(a, wide ? 3 : 1, 0, "fstu_glu_packed_norm", (hipStream_t)stream);
 }
 
 // y = T(x W^T) over packed W (N,K): x given normalised (norm_w == NULL, x = h with row stride ldx) or as the residual
@@ -670,6 +786,25 @@ extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, fl
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
   if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
   return glu_launch(a, norm_w != nullptr ? 1 : 0, 1, "fstu_linear_packed", (hipStream_t)stream);
+}
+
+// The same projection joining the residual stream: res_out = T(res_in + T(x W^T)), rows of stride N in both (res_out
+// may be res_in: every pair is read and written by the same lane).  The launch that normalises the stream afterwards
+// (fstu_glu_packed_norm at 17..32 rows) then needs no add of its own.
+extern "C" int fstu_linear_packed_add(const void* x, int ldx, const void* wp, const void* res_in, void* res_out, int rows, int N,
+                                      int K, void* stream) {
+  FSTU_REQUIRE(x && wp && res_in && res_out, FSTU_ENULL, "fstu_linear_packed_add: null pointer");
+  FSTU_REQUIRE(rows >= 1 && rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(rows > FSTU_MAX_DECODE_ROWS ? FSTU_MAX_DECODE_ROWS : rows, K, N) &&
+                   N % 8 == 0,
+               FSTU_ESHAPE, "fstu_linear_packed_add: unsupported shape rows=%d K=%d N=%d", rows, K, N);
+  FSTU_REQUIRE(ldx >= K && ldx % 8 == 0, FSTU_ESHAPE, "fstu_linear_packed_add: ldx=%d", ldx);
+  FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(wp, 16) && fstu_aligned(res_in, 4) && fstu_aligned(res_out, 4), FSTU_EALIGN,
+               "fstu_linear_packed_add: x and wp must be 16-byte aligned, the residual rows 4");
+  GluArgs a = {};
+  a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)res_out; a.h = (const bf16_t*)x;
+  a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = N;
+  a.x_in = (const bf16_t*)res_in; a.x_out = (bf16_t*)res_out;
+  return glu_launch(a, 0, 1, "fstu_linear_packed_add", (hipStream_t)stream);
 }
 
 // The tied head over a packed embedding: logits = T(x W^T) for rows <= 32 and the rows' packed maxima at `temperature`

@@ -146,7 +146,8 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
                     float scale, T* __restrict__ y, int ldy, int S, int d, int parity, const int* __restrict__ dyn,
                     int pair /* != 0 (needs co): y = T(T(E+O) + T(E-O)), the two sign branches rounded separately */,
                     T* __restrict__ ring /*optional (B,R,d), with fir (R,d) and co: exact head of the filter*/,
-                    const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn) {
+                    const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn,
+                    const T* res /*optional, rows of stride ldy: y = T(res + T(output)); may be y itself*/) {
   __shared__ float sh[LDS_JG][32][4];
   __shared__ float sho[LDS_JG][32][4];
   if (dyn) parity = dyn[0] & 1;
@@ -156,7 +157,10 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
   const int c = (blockIdx.x * 32 + q) * 4;
   const bool ok = c < d;
   float acc[4] = {0.f, 0.f, 0.f, 0.f}, acco[4] = {0.f, 0.f, 0.f, 0.f};
+  float rsd[4] = {0.f, 0.f, 0.f, 0.f};
   if (ok) {
+    // the residual row piece the epilogue adds: the oldest request, so no wait for a later one depends on the branch
+    if (res) Ring4<T>::ld(res + (size_t)b * ldy + c, rsd);
     // Every operand of the thread's first 8 modes of both banks and first 8 lags of the head goes in flight before
     // anything waits (out-of-range modes and lags re-read a valid element and are ignored): one trip to memory for
     // S <= 64 and 64 taps; longer states and heads continue in loops.
@@ -287,7 +291,7 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
 #pragma unroll
       for (int g = 0; g < LDS_JG; ++g) { e += sh[g][q][v]; o += sho[g][q][v]; }
       const float out = pair ? DT<T>::rnd(e + o) + DT<T>::rnd(e - o) : scale * (e + o);
-      DT<T>::st(y + (size_t)b * ldy + c + v, out);
+      DT<T>::st(y + (size_t)b * ldy + c + v, res ? rsd[v] + DT<T>::rnd(out) : out);
     }
   }
 }
@@ -300,7 +304,7 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
                                void* stream, int pair = 0, void* ring = nullptr, const float* fir = nullptr, int R = 0,
-                               const int* pos_dyn = nullptr);
+                               const int* pos_dyn = nullptr, const void* res = nullptr);
 
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
@@ -319,26 +323,38 @@ extern "C" int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, co
                                       const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S,
                                       int d, int t, int dtype, void* stream) {
   return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
-                                    stream);
+                                    stream, nullptr);
 }
 
 // ring / fir / fir_taps: optional exact head of the filter (all three or none).  dyn: device-side {position, step} that
 // supplies the parity; pos_dyn: the same words where only the ring slot is read from them (the parity then comes with t)
 int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
                                const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
-                               const int* pos_dyn, int dtype, void* stream) {
+                               const int* pos_dyn, int dtype, void* stream, const void* res) {
   FSTU_REQUIRE(co, FSTU_ENULL, "fstu_stu_step_lds_pair: null pointer");
   FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_pair: co must be 16-byte aligned");
   FSTU_REQUIRE(fstu_fir_ok(ring, fir, fir_taps), FSTU_EARG,
                "fstu_stu_step_lds_pair: ring, fir and fir_taps (a power of two, 8..1024) go together, 16-byte aligned");
   return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, dyn, dtype, stream, 1, ring, fir, fir_taps,
-                             dyn ? dyn : pos_dyn);
+                             dyn ? dyn : pos_dyn, res);
+}
+
+// The same step joining the residual stream: y = T(res + T(step output)), rows of stride ldy in both; y may be res
+// (every element is read and written by the same thread).
+extern "C" int fstu_stu_step_lds_pair_add(float* state, const void* xp, int ldxp, const float* a, const float* ce,
+                                          const float* co, void* ring, const float* fir, int fir_taps, const void* res, void* y,
+                                          int ldy, int B, int S, int d, int t, int dtype, void* stream) {
+  FSTU_REQUIRE(res, FSTU_ENULL, "fstu_stu_step_lds_pair_add: res is null");
+  return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
+                                    stream, res);
 }
 
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream, int pair, void* ring, const float* fir, int R, const int* pos_dyn) {
+                               void* stream, int pair, void* ring, const float* fir, int R, const int* pos_dyn, const void* res) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
+  FSTU_REQUIRE(!res || (fstu_aligned(res, 16) && ldy % 4 == 0), FSTU_EALIGN,
+               "fstu_stu_step_lds: the residual rows must be 16-byte aligned with a stride that is a multiple of 4");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
   FSTU_REQUIRE(ldxp >= d && ldy >= d, FSTU_ESHAPE, "fstu_stu_step_lds: row stride smaller than d");
   FSTU_REQUIRE(t >= 0, FSTU_EARG, "fstu_stu_step_lds: t<0");
@@ -347,7 +363,7 @@ static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const flo
   FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
                       hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
                                          (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair, (T*)ring, fir, R,
-                                         t, pos_dyn));
+                                         t, pos_dyn, (const T*)res));
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }

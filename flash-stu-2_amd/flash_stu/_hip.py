@@ -35,6 +35,7 @@ SIGNATURES = {
     "fstu_stu_step_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_pair": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_pair_add": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_single": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
@@ -69,6 +70,7 @@ SIGNATURES = {
     "fstu_glu_packed": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_glu_packed_norm": [_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_packed": [_vp, _i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
+    "fstu_linear_packed_add": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _vp],
     "fstu_linear_packed_res": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_down_packed_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _vp, _vp],
     "fstu_decode_step": [_vp, _vp, _vp, _i64, _i, _f, _i, _f, _i, _u64, _i, _vp],
@@ -417,11 +419,13 @@ def _fir_args(ring, fir, B, d, dtype):
 
 def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
                  out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None, pair: bool = False,
-                 ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None,
+                 res: Optional[torch.Tensor] = None) -> torch.Tensor:
     """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d) = T(2E), E = ce . bank(t).  With co (S,d) and
     O = co . other bank: the single-branch form y = T(E+O) (use_hankel_L), or with pair=True the two sign branches
     rounded separately, y = T(T(E+O) + T(E-O)).  pair=True with ring (B,R,d) and fir (R,d): the exact head of the
-    filter on the first R lags (the ring is updated in place)."""
+    filter on the first R lags (the ring is updated in place).  pair=True with res (B,d): the step joins the residual
+    stream, y = T(res + T(output)); out may be res."""
     _dev(state, a, ce, co)
     B, two, S, d = state.shape
     assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
@@ -436,6 +440,13 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
         assert co.dtype == torch.float32 and co.shape == (S, d)
         if pair:
             rp, fp, R = _fir_args(ring, fir, B, d, xp.dtype)
+            if res is not None:
+                _dev(res)
+                assert res.dtype == xp.dtype and res.shape == (B, d) and _rows_view(res)[1] == ldy
+                _check(load().fstu_stu_step_lds_pair_add(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), rp, fp, R, _p(res),
+                                                         _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
+                       "fstu_stu_step_lds_pair_add")
+                return out
             _check(load().fstu_stu_step_lds_pair(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), rp, fp, R, _p(out), ldy, B, S, d,
                                                  t, _dt(xp), _stream()), "fstu_stu_step_lds_pair")
             return out
@@ -795,10 +806,15 @@ def glu_packed_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torc
     """(x + delta, act) with act = GLU(rmsnorm(x + delta) * norm_w): residual add, norm and gate/up in one launch."""
     _dev(x, delta, norm_w, wp_gate, wp_up)
     rows, d = x.shape
-    if x.dtype != torch.bfloat16 or not load().fstu_glu_packed_supported(rows, d, I):
+    wide = rows > 16 and delta is None and bool(load().fstu_mlp_packed_rows32_supported(rows, d, I))
+    if x.dtype != torch.bfloat16 or not (wide or load().fstu_glu_packed_supported(rows, d, I)):
         raise FlashSTUHipError(f"fstu_glu_packed_norm does not support rows={rows} d={d} I={I} dtype={x.dtype}")
-    x_out = torch.empty_like(x)
     act = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    if wide:      # 17..32 rows: x is the summed stream, nothing is stored
+        _check(load().fstu_glu_packed_norm(_p(x), None, None, _p(norm_w), float(eps), _p(wp_gate), _p(wp_up),
+                                           _p(act), I, rows, I, d, _stream()), "fstu_glu_packed_norm")
+        return x, act
+    x_out = torch.empty_like(x)
     _check(load().fstu_glu_packed_norm(_p(x), _p(delta), _p(x_out), _p(norm_w), float(eps), _p(wp_gate), _p(wp_up),
                                        _p(act), I, rows, I, d, _stream()), "fstu_glu_packed_norm")
     return x_out, act
@@ -812,6 +828,21 @@ def linear_packed(x: torch.Tensor, wp: torch.Tensor, N: int, norm_w: Optional[to
     out = torch.empty(rows, N, dtype=x.dtype, device=x.device)
     _check(load().fstu_linear_packed(_p(x), ldx, _p(norm_w), float(eps), _p(wp), _p(out), N, rows, N, K, _stream()),
            "fstu_linear_packed")
+    return out
+
+
+def linear_packed_add(x: torch.Tensor, wp: torch.Tensor, res: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """T(res + T(x (rows,K) @ W^T)) over packed W (N,K): the projection joins the residual stream res (rows,N), dense
+    rows; out may be res."""
+    _dev(wp, res, out)
+    rows, ldx = _rows_view(x)
+    K = x.shape[1]
+    N = res.shape[1]
+    assert res.shape == (rows, N) and res.is_contiguous() and res.dtype == x.dtype
+    if out is None:
+        out = torch.empty_like(res)
+    assert out.shape == res.shape and out.is_contiguous() and out.dtype == res.dtype
+    _check(load().fstu_linear_packed_add(_p(x), ldx, _p(wp), _p(res), _p(out), rows, N, K, _stream()), "fstu_linear_packed_add")
     return out
 
 

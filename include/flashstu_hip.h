@@ -143,6 +143,11 @@ int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, co
 int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                            void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t,
                            int dtype, void* stream);
+/* The same step joining the residual stream (flash_stu/layers/stu_layer.py:93, x = x + stu(stu_norm(x))):
+ * y = T(res + T(step output)), rows of stride ldy in both, 16-byte aligned; y may be res. */
+int fstu_stu_step_lds_pair_add(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                               void* ring, const float* fir, int fir_taps, const void* res, void* y, int ldy, int B, int S,
+                               int d, int t, int dtype, void* stream);
 
 /* The same step for the single-branch filters of use_hankel_L=True (flash_stu/utils/stu_utils.py:22-25,229-246:
  * one convolution over ALL lags, no sign branch): ce (S,d) is fitted to the even lags and weighs the bank of parity
@@ -421,15 +426,17 @@ int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
  * Same contract as fstu_glu_decode (flash_stu/modules/swiglu.py:23-26); wp_* from fstu_pack_rows.
  * fstu_glu_packed_supported tells whether a shape is covered (d in {256,512,768,1024,2048}, I % 4 == 0).
  * 17..32 rows (fstu_mlp_packed_rows32_supported: such a d, I % 512 == 0): fstu_glu_packed and fstu_down_packed_splitk
- * take them as two row tiles per weight fragment, so every weight is still read once; the launches with a norm
- * prologue (fstu_glu_packed_norm, fstu_linear_packed, fstu_linear_packed_res) stay at 16 rows. */
+ * take them as two row tiles per weight fragment, so every weight is still read once; of the launches with a norm
+ * prologue fstu_glu_packed_norm takes them too (see there), fstu_linear_packed and fstu_linear_packed_res stay at 16 rows. */
 int fstu_glu_packed_supported(int rows, int d, int I);
 int fstu_mlp_packed_rows32_supported(int rows, int d, int I);
 int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
                     int I, int d, void* stream);
 /* The same launch with the sub-layer's residual add and mlp_norm as its prologue (stu_layer.py:93-96,
  * attention_layer.py:59-62): x' = T(x_in + delta) (delta may be NULL), h = rmsnorm(x') * norm_w recomputed by every
- * workgroup while its weight loads are in flight; x' is stored to x_out (may be NULL; must not alias x_in). */
+ * workgroup while its weight loads are in flight; x' is stored to x_out (may be NULL; must not alias x_in).
+ * 17..32 rows: x_in is the stream with the sub-layer's output already added (fstu_linear_packed_add,
+ * fstu_stu_step_lds_pair_add), delta and x_out must be NULL; the norm is formed in the matrix-core fragments. */
 int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const void* norm_w, float eps,
                          const void* wp_gate, const void* wp_up, void* act, int ldact, int rows, int I, int d,
                          void* stream);
@@ -440,6 +447,11 @@ int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const
  * (without norm_w: rows <= 32, the second 16 as another row tile of the same weight fragments). */
 int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                        int rows, int N, int K, void* stream);
+/* The same projection joining the residual stream (flash_stu/layers/attention_layer.py:57, x = x + attn(attn_norm(x))
+ * with c_proj as the projection): res_out = T(res_in + T(x W^T)), rows of stride N in both; res_out may be res_in.
+ * rows <= 32, N % 8 == 0, K as above, bf16. */
+int fstu_linear_packed_add(const void* x, int ldx, const void* wp, const void* res_in, void* res_out, int rows, int N,
+                           int K, void* stream);
 /* Split-K form of the down projection over packed weights (reference: flash_stu/modules/swiglu.py:22-29, down_proj):
  * partial receives *ksplit_io fp32 slices (slice, rows, d) that fstu_add_rmsnorm(delta_mode 1) or the norm prologue of
  * the next projection sums in slice order.  *ksplit_io on entry: slices wanted (4, 8 or 16; anything else: 16); on

@@ -607,6 +607,25 @@ def test_stu_step_lds_pair_keeps_the_reference_rounding_points(hip):
     assert bad_pair <= 0.22 * total and bad_pair < 0.6 * bad_2e, (bad_pair / total, bad_2e / total)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_stu_step_lds_pair_joins_the_residual_stream(hip, dtype):
+    """The pair step with a residual row: y = T(res + T(step output)), bit for bit the plain step followed by an add
+    in the model dtype, in place on the stream and with identical states."""
+    B, d, S = 3, 384, 64
+    g = gen(91)
+    a = dev(torch.rand(S, generator=g) * 0.9)
+    ce, co = dev(torch.randn(S, d, generator=g) / 8), dev(torch.randn(S, d, generator=g) / 8)
+    st1 = torch.zeros(B, 2, S, d, device="cuda")
+    st2 = torch.zeros(B, 2, S, d, device="cuda")
+    stream = dev(torch.randn(B, d, generator=g).to(dtype))
+    for t in range(5):
+        xt = dev(torch.randn(B, d, generator=g).to(dtype))
+        want = stream + hip.stu_step_lds(st1, xt, a, ce, t, co=co, pair=True)
+        got = hip.stu_step_lds(st2, xt, a, ce, t, co=co, pair=True, res=stream, out=stream)
+        assert got is stream and torch.equal(stream, want)
+    assert torch.equal(st1, st2)
+
+
 @pytest.mark.parametrize("R", [8, 32, 128, 256])
 def test_stu_step_lds_exact_head(hip, R):
     """The exact head of the distilled filter: fir[s] = phi_proj[s] - fitted filter for the first R lags, applied to a
@@ -1219,6 +1238,51 @@ def test_glu_packed_norm_prologue(hip, rows, d, I):
     assert torch.equal(x_out2.cpu(), x)
 
 
+@pytest.mark.parametrize("rows,d,I", [(32, 2048, 4096), (17, 2048, 1024), (24, 1024, 2048), (32, 768, 1536), (29, 256, 512)])
+def test_glu_packed_norm_two_row_tiles(hip, rows, d, I):
+    """17..32 rows: the RMSNorm of the (already summed) residual stream formed in the matrix-core fragments of the
+    gate/up launch.  The activations meet the float64 reference like the 16-row prologue's, and the separate norm
+    launch followed by the plain gate/up launch almost everywhere bit for bit (the row's sum of squares is gathered in
+    another order, so a normalised value may round the other way now and then)."""
+    dtype = torch.bfloat16
+    g = gen(67)
+    x = torch.randn(rows, d, generator=g).to(dtype)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype)
+    wg = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    wu = (torch.randn(I, d, generator=g) / math.sqrt(d)).to(dtype)
+    pg, pu = hip.pack_rows(dev(wg)), hip.pack_rows(dev(wu))
+    xd = dev(x)
+    x_out, act = hip.glu_packed_norm(xd, None, dev(nw), O.RMS_EPS_DEFAULT, pg, pu, I)
+    assert x_out is xd and torch.equal(xd.cpu(), x)
+    h_ref = O.rms_norm(x, nw, O.RMS_EPS_DEFAULT)
+    gate = (h_ref.double() @ wg.double().t()).to(dtype)
+    up = (h_ref.double() @ wu.double().t()).to(dtype)
+    ref = torch.nn.functional.gelu(gate.float(), approximate="tanh").to(dtype) * up
+    diff = (act.float().cpu() - ref.float()).abs()
+    assert bool((diff <= ref.float().abs() * 2.0 ** -6 + 2.0 ** -7 * 2e-2 * float(ref.float().abs().max())).all())
+    assert float((diff > 0).float().mean()) <= 0.10
+    h = hip.add_rmsnorm(xd.clone(), None, dev(nw), O.RMS_EPS_DEFAULT)
+    two = hip.glu_packed(h, pg, pu, I)
+    assert float((two != act).float().mean()) <= 0.01
+
+
+@pytest.mark.parametrize("rows,K,N", [(32, 2048, 2048), (8, 768, 768), (19, 1024, 512), (32, 256, 64)])
+def test_linear_packed_add_joins_the_residual_stream(hip, rows, K, N):
+    """res_out = T(res + T(x W^T)) == the plain packed projection followed by a bf16 add, bit for bit; in place too."""
+    dtype = torch.bfloat16
+    g = gen(68)
+    x = dev(torch.randn(rows, K, generator=g).to(dtype))
+    res = dev(torch.randn(rows, N, generator=g).to(dtype))
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    wp = hip.pack_rows(dev(W))
+    want = res + hip.linear_packed(x, wp, N)
+    assert torch.equal(hip.linear_packed_add(x, wp, res), want)
+    r2 = res.clone()
+    assert hip.linear_packed_add(x, wp, r2, out=r2) is r2 and torch.equal(r2, want)
+    ref = (res.double().cpu() + (x.double().cpu() @ W.double().t()).to(dtype).double()).to(dtype)
+    check(want, ref, dtype)
+
+
 @pytest.mark.parametrize("rows,K,N,ns", [(8, 768, 2304, 4), (4, 256, 96, 3), (2, 1024, 3072, 1)])
 def test_linear_packed_res_equals_add_norm_then_linear(hip, rows, K, N, ns):
     dtype = torch.bfloat16
@@ -1286,8 +1350,8 @@ def test_stu_bank_step_lds(hip, dtype):
 
 
 def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
-    """More than 32 rows, 17..32 rows with a norm prologue, and widths outside the packed kernels' set are refused on
-    the host before any launch."""
+    """More than 32 rows, 17..32 rows with a norm prologue that would have to add a delta, and widths outside the packed
+    kernels' set are refused on the host before any launch."""
     g = gen(66)
     d, I = 256, 512
     wg = dev((torch.randn(I, d, generator=g) / 16).bfloat16())
@@ -1306,7 +1370,11 @@ def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
     with pytest.raises(hip.FlashSTUHipError):
         hip.linear_packed(x20, pg, I, nw, 1e-6)             # the norm prologue stops at 16 rows
     with pytest.raises(hip.FlashSTUHipError):
-        hip.glu_packed_norm(x20, None, nw, 1e-6, pg, pg, I)
+        hip.glu_packed_norm(x20, x20, nw, 1e-6, pg, pg, I)  # 17..32 rows take the summed stream only: no delta
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.glu_packed_norm(x33, None, nw, 1e-6, pg, pg, I)
+    with pytest.raises(hip.FlashSTUHipError):
+        hip.linear_packed_add(x33, pg, dev(torch.zeros(33, I).bfloat16()))
     with pytest.raises(hip.FlashSTUHipError):
         hip.head_maxima_packed(x33, pg, I, best)
     x320 = dev(torch.randn(20, 320, generator=g).bfloat16())    # K = 320 is not one of the packed kernels' widths
@@ -1316,6 +1384,7 @@ def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
     # and what they do take at 20 rows still runs
     assert hip.linear_packed(x20, pg, I).shape == (20, I)
     assert hip.glu_packed(x20, pg, pg, I).shape == (20, I)
+    assert hip.glu_packed_norm(x20, None, nw, 1e-6, pg, pg, I)[1].shape == (20, I)
 
 
 @pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8),
