@@ -174,10 +174,11 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
         mlps = [l.mlp for l in eng.model.layers]
         packed = bool(lib.fstu_mlp_packed_rows32_supported(rows, d, I))
         if packed:
-            ops = [(eng._pack(m_.gate_proj.weight), eng._pack(m_.up_proj.weight)) for m_ in mlps]
-            launch = lambda o: _hip.glu_packed(h, o[0], o[1], I, out=act)
-            name = ("glu_balanced_kernel<two row tiles> (gate/up projection + gelu*up over all rows, packed weights, "
-                    "one workgroup per compute unit)")
+            # as the step launches it: mlp_norm of the summed residual stream formed in the launch's own fragments
+            ops = [(eng._pack(l.mlp.gate_proj.weight), eng._pack(l.mlp.up_proj.weight), l.mlp_norm.weight) for l in eng.model.layers]
+            launch = lambda o: _hip.glu_packed_norm(h, None, o[2], cfg.rms_norm_eps, o[0], o[1], I, out=act)
+            name = ("glu_balanced_kernel<two row tiles, norm in the fragments> (mlp_norm + gate/up projection + gelu*up over "
+                    "all rows, packed weights, one workgroup per compute unit)")
         else:
             ops = [(m_.gate_proj.weight, m_.up_proj.weight) for m_ in mlps]
             launch = lambda o: _hip.gemm(h, o[0], up_weight=o[1], out=act)
@@ -201,7 +202,7 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
         traffic = 204052787 if packed and (d, I, rows) == (2048, 24576, 32) else None
         return {"bound": "hbm", "kernel": name,
                 "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
-                "traffic_source": "profiles/decode_c5_hbm_traffic_pmc.txt (counter runs of this kernel, not of this run)" if traffic else None,
+                "traffic_source": "profiles/decode_c5_hbm_traffic_pmc.txt (counter runs of this launch without its norm, not of this run)" if traffic else None,
                 "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n, "rows_per_launch": rows}
     ms_c, n_c = ctypes.c_double(), ctypes.c_int()
     torch.cuda.synchronize()

@@ -802,14 +802,15 @@ def glu_packed(x: torch.Tensor, wp_gate: torch.Tensor, wp_up: torch.Tensor, I: i
 
 
 def glu_packed_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
-                    wp_gate: torch.Tensor, wp_up: torch.Tensor, I: int):
+                    wp_gate: torch.Tensor, wp_up: torch.Tensor, I: int, out: Optional[torch.Tensor] = None):
     """(x + delta, act) with act = GLU(rmsnorm(x + delta) * norm_w): residual add, norm and gate/up in one launch."""
     _dev(x, delta, norm_w, wp_gate, wp_up)
     rows, d = x.shape
     wide = rows > 16 and delta is None and bool(load().fstu_mlp_packed_rows32_supported(rows, d, I))
     if x.dtype != torch.bfloat16 or not (wide or load().fstu_glu_packed_supported(rows, d, I)):
         raise FlashSTUHipError(f"fstu_glu_packed_norm does not support rows={rows} d={d} I={I} dtype={x.dtype}")
-    act = torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    act = out if out is not None else torch.empty(rows, I, dtype=x.dtype, device=x.device)
+    assert act.shape == (rows, I) and act.dtype == x.dtype and act.is_contiguous() and act.is_cuda
     if wide:      # 17..32 rows: x is the summed stream, nothing is stored
         _check(load().fstu_glu_packed_norm(_p(x), None, None, _p(norm_w), float(eps), _p(wp_gate), _p(wp_up),
                                            _p(act), I, rows, I, d, _stream()), "fstu_glu_packed_norm")
