@@ -50,10 +50,17 @@ def decode_step_bytes(cfg, B, t, mode, S):
     weights = (cfg.n_layers * (3 * d * I + 2 * d) + n_att * 4 * d * d + n_stu * d * d + d + V * d) * w
     kv = n_att * B * 2 * d * w * (min(t, cfg.window_left + 1) + 1)
     if mode == "lds":
-        stu = n_stu * (B * S * d * 4 * 3 + 2 * S * d * 4)      # both parity banks read, one written; ce and co
         R = int(getattr(cfg, "stu_lds_fir_taps", 0) or 0)
-        if R and not cfg.use_hankel_L:
-            stu += n_stu * (B * R * d * w + B * d * w + R * d * 4)   # ring of the last R inputs read, one row written; taps
+        if B > 16 and w == 2 and not cfg.use_hankel_L:
+            # 17..32 rows: the odd-lag sum is handed from step to step, so a step reads and writes ONE parity bank
+            # (plus that sum, B x d fp32 read and written) and the even-lag half of the ring
+            stu = n_stu * (B * S * d * 4 * 2 + 2 * B * d * 4 + 2 * S * d * 4)
+            if R:
+                stu += n_stu * (B * (R // 2) * d * w + B * d * w + R * d * 4)
+        else:
+            stu = n_stu * (B * S * d * 4 * 3 + 2 * S * d * 4)      # both parity banks read, one written; ce and co
+            if R and not cfg.use_hankel_L:
+                stu += n_stu * (B * R * d * w + B * d * w + R * d * 4)   # ring of the last R inputs read, one row written; taps
     else:
         stu = n_stu * (B * (t + 1) * d * w + (t + 1) * d * w)
     return weights + kv + stu + B * V * w

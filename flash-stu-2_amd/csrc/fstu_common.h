@@ -61,7 +61,8 @@ int fstu_sample_topk_dyn(const void* logits, int64_t ldl, void* best_ws, void* s
 int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
                                const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
                                const int* pos_dyn, int dtype, void* stream,
-                               const void* res = nullptr /*y = T(res + T(output)), rows of stride ldy*/);
+                               const void* res = nullptr /*y = T(res + T(output)), rows of stride ldy*/,
+                               float* ocache = nullptr /*(B,d): the odd-lag sum handed from step to step*/);
 int fstu_stu_inproj_step_dyn(const void* h, int ldh, const void* Mt, float* state, const float* a, const float* ce,
                              const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, void* xp_out, int B,
                              int S, int d, int K, int t, const int* dyn, const int* pos_dyn, void* stream);

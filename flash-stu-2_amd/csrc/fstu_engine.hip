@@ -106,12 +106,13 @@ extern "C" int fstu_prof_copy(void* dst, const void* src, size_t bytes, void* st
 
 // recurrence step on m->xp: both sign branches rounded separately when the layer carries odd-lag weights
 // (stream_x: the residual stream; the step then adds its output to it in place instead of leaving it in m->y)
+// (wide: the 17..32-row step, which hands the odd-lag sum from step to step where the layer carries lds_ocache)
 static int stu_step(const fstu_layer_desc& L, const fstu_model_desc* m, int pos, const int* dyn, const int* pos_dyn, void* stream,
-                    void* stream_x = nullptr) {
+                    void* stream_x = nullptr, bool wide = false) {
   if (L.lds_co)
     return fstu_stu_step_lds_pair_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, L.lds_co, L.lds_ring, L.lds_fir,
                                       L.lds_fir ? m->lds_fir_taps : 0, stream_x ? stream_x : m->y, m->d, m->B, m->lds_S, m->d, pos,
-                                      dyn, pos_dyn, m->dtype, stream, stream_x);
+                                      dyn, pos_dyn, m->dtype, stream, stream_x, wide ? L.lds_ocache : nullptr);
   if (stream_x) return FSTU_EARG;
   return fstu_stu_step_lds_dyn(L.lds_state, m->xp, m->d, L.lds_a, L.lds_ce, m->y, m->d, m->B, m->lds_S, m->d, pos, dyn, m->dtype,
                                stream);
@@ -187,7 +188,7 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
       if (packed_mlp && L.wp_m_inputs) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_m_inputs, m->xp, d, B, d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
-      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream, join ? m->x : nullptr));
+      TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream, join ? m->x : nullptr, true));
     } else {
       if (packed_mlp && L.wp_qkv) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.w_qkv, m->qkv, 3 * d, 3 * d, d));

@@ -138,8 +138,29 @@ template <> struct Ring4<bf16_t> {
 // Workgroup = 32 channel quads (128 channels) x 8 mode groups.  Each thread
 // advances S/8 modes of 4 channels (float4 state accesses, 512 contiguous
 // bytes per mode row and wave half), then the 8 mode groups are reduced in LDS.
+//
+// omode (with co and ocache (B,d) fp32): the odd-lag sum O of a step weighs the bank the PREVIOUS step advanced, which
+// nothing has touched since, and the odd lags of the exact head reach the inputs the previous step already held.  So
+// a step can form the next step's O while it has its own bank in registers and leave it in ocache:
+//   omode 1  O of this step comes from ocache; the next step's O is formed on this bank after its advance (the same
+//            products in the same order as the plain step would form them one step later: bit-identical) and stored.
+//            The other bank is not read: a third less state traffic.
+//   omode 2  priming for position t (the last position of a prompt): nothing is advanced and nothing is written but
+//            ocache, which receives what a step at position t would have left for position t+1; x is taken from the
+//            ring (or not at all without the exact head).
 #define LDS_JG 8
-template <typename T>
+// state rows of the wide step: read once and written once per two steps, far more than the caches hold in between
+typedef float f32x4_nt __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld_state_nt(const float* p) {
+  const f32x4_nt v = __builtin_nontemporal_load((const f32x4_nt*)p);
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st_state_nt(float* p, float4 h) {
+  const f32x4_nt v = {h.x, h.y, h.z, h.w};
+  __builtin_nontemporal_store(v, (f32x4_nt*)p);
+}
+// (OM: the mode as a template parameter, so that each instance holds only the operands its mode requests)
+template <typename T, int OM>
 __global__ void __launch_bounds__(256)
 stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldxp, const float* __restrict__ a,
                     const float* __restrict__ ce, const float* __restrict__ co /*optional: weights of the other bank*/,
@@ -147,34 +168,42 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
                     int pair /* != 0 (needs co): y = T(T(E+O) + T(E-O)), the two sign branches rounded separately */,
                     T* __restrict__ ring /*optional (B,R,d), with fir (R,d) and co: exact head of the filter*/,
                     const float* __restrict__ fir, int R, int t, const int* __restrict__ pos_dyn,
-                    const T* res /*optional, rows of stride ldy: y = T(res + T(output)); may be y itself*/) {
+                    const T* res /*optional, rows of stride ldy: y = T(res + T(output)); may be y itself*/,
+                    float* ocache) {
+  constexpr int omode = OM;
   __shared__ float sh[LDS_JG][32][4];
   __shared__ float sho[LDS_JG][32][4];
+  __shared__ float shf[LDS_JG][32][4];   // omode: the exact head's share of the next step's O, in the odd slots
   if (dyn) parity = dyn[0] & 1;
   if (pos_dyn) t = pos_dyn[0];
   const int b = blockIdx.y;
   const int q = threadIdx.x & 31, jg = threadIdx.x >> 5;
   const int c = (blockIdx.x * 32 + q) * 4;
   const bool ok = c < d;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acco[4] = {0.f, 0.f, 0.f, 0.f};
-  float rsd[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool head = co && fir;
+  constexpr bool prime = OM == 2;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acco[4] = {0.f, 0.f, 0.f, 0.f}, fnx[4] = {0.f, 0.f, 0.f, 0.f};
+  float rsd[4] = {0.f, 0.f, 0.f, 0.f}, ocur[4] = {0.f, 0.f, 0.f, 0.f};
   if (ok) {
-    // the residual row piece the epilogue adds: the oldest request, so no wait for a later one depends on the branch
+    // the residual row piece the epilogue adds and the cached O: the oldest requests, so no wait for a later one
+    // depends on these branches
     if (res) Ring4<T>::ld(res + (size_t)b * ldy + c, rsd);
+    if constexpr (OM == 1) Ring4<float>::ld(ocache + (size_t)b * d + c, ocur);
     // Every operand of the thread's first 8 modes of both banks and first 8 lags of the head goes in flight before
     // anything waits (out-of-range modes and lags re-read a valid element and are ignored): one trip to memory for
     // S <= 64 and 64 taps; longer states and heads continue in loops.
     constexpr int PJ = 8;
     float* st = state + (((size_t)b * 2 + parity) * S) * d + c;
     const float* so = state + (((size_t)b * 2 + (parity ^ 1)) * S) * d + c;
-    const bool head = co && fir;
     const T* rb = head ? ring + (size_t)b * R * d + c : nullptr;
-    float4 ph[PJ], pc[PJ], qh[PJ], qc[PJ], fr[PJ];
+    // omode: only the even mode groups take lags (the even ones, for this step's E and, shifted by one, the next O)
+    const bool lags = head && (omode == 0 || (jg & 1) == 0);
+    float4 ph[PJ], pc[PJ], qh[PJ], qc[PJ], fr[PJ], fr2[PJ];
     float pa[PJ], rx[PJ][4];
 #pragma unroll
     for (int k = 0; k < PJ; ++k) {
       const int j = min(jg + LDS_JG * k, S - 1);
-      ph[k] = *(const float4*)(st + (size_t)j * d);
+      ph[k] = OM == 1 ? ld_state_nt(st + (size_t)j * d) : *(const float4*)(st + (size_t)j * d);
       pc[k] = *(const float4*)(ce + (size_t)j * d + c);
       pa[k] = a[j];
     }
@@ -182,84 +211,121 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
 #pragma unroll
       for (int k = 0; k < PJ; ++k) {
         const int j = min(jg + LDS_JG * k, S - 1);
-        qh[k] = *(const float4*)(so + (size_t)j * d);
+        if constexpr (OM == 0) qh[k] = *(const float4*)(so + (size_t)j * d);
         qc[k] = *(const float4*)(co + (size_t)j * d + c);
       }
     }
-    if (head) {
+    if (lags) {
 #pragma unroll
       for (int k = 0; k < PJ; ++k) {
         const int sl = min(jg + 8 * k, R - 1);
         Ring4<T>::ld(rb + (size_t)((t - sl) & (R - 1)) * d, rx[k]);
         fr[k] = *(const float4*)(fir + (size_t)sl * d + c);
+        if constexpr (OM != 0) fr2[k] = *(const float4*)(fir + (size_t)min(sl + 1, R - 1) * d + c);
       }
     }
-    float x[4];
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (!prime) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) x[v] = DT<T>::ld(xp + (size_t)b * ldxp + c + v);
+      for (int v = 0; v < 4; ++v) x[v] = DT<T>::ld(xp + (size_t)b * ldxp + c + v);
+    } else if (head) {
+      Ring4<T>::ld(rb + (size_t)(t & (R - 1)) * d, x);
+    }
 #pragma unroll
     for (int k = 0; k < PJ; ++k) {
       const int j = jg + LDS_JG * k;
       if (j < S) {
         float4 h = ph[k];
-        h.x = fmaf(pa[k], h.x, x[0]);
-        h.y = fmaf(pa[k], h.y, x[1]);
-        h.z = fmaf(pa[k], h.z, x[2]);
-        h.w = fmaf(pa[k], h.w, x[3]);
-        *(float4*)(st + (size_t)j * d) = h;
-        acc[0] = fmaf(pc[k].x, h.x, acc[0]);
-        acc[1] = fmaf(pc[k].y, h.y, acc[1]);
-        acc[2] = fmaf(pc[k].z, h.z, acc[2]);
-        acc[3] = fmaf(pc[k].w, h.w, acc[3]);
+        if constexpr (!prime) {
+          h.x = fmaf(pa[k], h.x, x[0]);
+          h.y = fmaf(pa[k], h.y, x[1]);
+          h.z = fmaf(pa[k], h.z, x[2]);
+          h.w = fmaf(pa[k], h.w, x[3]);
+          if constexpr (OM == 1) st_state_nt(st + (size_t)j * d, h); else *(float4*)(st + (size_t)j * d) = h;
+          acc[0] = fmaf(pc[k].x, h.x, acc[0]);
+          acc[1] = fmaf(pc[k].y, h.y, acc[1]);
+          acc[2] = fmaf(pc[k].z, h.z, acc[2]);
+          acc[3] = fmaf(pc[k].w, h.w, acc[3]);
+        }
+        if constexpr (OM != 0) {   // the next step's odd-lag sum on this bank
+          acco[0] = fmaf(qc[k].x, h.x, acco[0]);
+          acco[1] = fmaf(qc[k].y, h.y, acco[1]);
+          acco[2] = fmaf(qc[k].z, h.z, acco[2]);
+          acco[3] = fmaf(qc[k].w, h.w, acco[3]);
+        }
       }
     }
 #pragma unroll 4
     for (int j = jg + LDS_JG * PJ; j < S; j += LDS_JG) {
       float4 h = *(float4*)(st + (size_t)j * d);
-      const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
-      const float aj = a[j];
-      h.x = fmaf(aj, h.x, x[0]);
-      h.y = fmaf(aj, h.y, x[1]);
-      h.z = fmaf(aj, h.z, x[2]);
-      h.w = fmaf(aj, h.w, x[3]);
-      *(float4*)(st + (size_t)j * d) = h;
-      acc[0] = fmaf(cj.x, h.x, acc[0]);
-      acc[1] = fmaf(cj.y, h.y, acc[1]);
-      acc[2] = fmaf(cj.z, h.z, acc[2]);
-      acc[3] = fmaf(cj.w, h.w, acc[3]);
-    }
-    if (co) {
-      // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (not advanced here)
-#pragma unroll
-      for (int k = 0; k < PJ; ++k) {
-        if (jg + LDS_JG * k < S) {
-          acco[0] = fmaf(qc[k].x, qh[k].x, acco[0]);
-          acco[1] = fmaf(qc[k].y, qh[k].y, acco[1]);
-          acco[2] = fmaf(qc[k].z, qh[k].z, acco[2]);
-          acco[3] = fmaf(qc[k].w, qh[k].w, acco[3]);
-        }
+      if constexpr (!prime) {
+        const float4 cj = *(const float4*)(ce + (size_t)j * d + c);
+        const float aj = a[j];
+        h.x = fmaf(aj, h.x, x[0]);
+        h.y = fmaf(aj, h.y, x[1]);
+        h.z = fmaf(aj, h.z, x[2]);
+        h.w = fmaf(aj, h.w, x[3]);
+        *(float4*)(st + (size_t)j * d) = h;
+        acc[0] = fmaf(cj.x, h.x, acc[0]);
+        acc[1] = fmaf(cj.y, h.y, acc[1]);
+        acc[2] = fmaf(cj.z, h.z, acc[2]);
+        acc[3] = fmaf(cj.w, h.w, acc[3]);
       }
-#pragma unroll 4
-      for (int j = jg + LDS_JG * PJ; j < S; j += LDS_JG) {
-        const float4 h = *(const float4*)(so + (size_t)j * d);
+      if constexpr (OM != 0) {
         const float4 oj = *(const float4*)(co + (size_t)j * d + c);
         acco[0] = fmaf(oj.x, h.x, acco[0]);
         acco[1] = fmaf(oj.y, h.y, acco[1]);
         acco[2] = fmaf(oj.z, h.z, acco[2]);
         acco[3] = fmaf(oj.w, h.w, acco[3]);
       }
-      if (fir) {
-        // exact head: lags jg, jg+8, ... share the parity of jg; a position before the sequence contributes nothing
+    }
+    if (co) {
+      if constexpr (OM == 0) {
+        // odd lags: lag 2m+1 reaches position t-1-2m, which the bank of the other parity holds (not advanced here)
+#pragma unroll
+        for (int k = 0; k < PJ; ++k) {
+          if (jg + LDS_JG * k < S) {
+            acco[0] = fmaf(qc[k].x, qh[k].x, acco[0]);
+            acco[1] = fmaf(qc[k].y, qh[k].y, acco[1]);
+            acco[2] = fmaf(qc[k].z, qh[k].z, acco[2]);
+            acco[3] = fmaf(qc[k].w, qh[k].w, acco[3]);
+          }
+        }
+#pragma unroll 4
+        for (int j = jg + LDS_JG * PJ; j < S; j += LDS_JG) {
+          const float4 h = *(const float4*)(so + (size_t)j * d);
+          const float4 oj = *(const float4*)(co + (size_t)j * d + c);
+          acco[0] = fmaf(oj.x, h.x, acco[0]);
+          acco[1] = fmaf(oj.y, h.y, acco[1]);
+          acco[2] = fmaf(oj.z, h.z, acco[2]);
+          acco[3] = fmaf(oj.w, h.w, acco[3]);
+        }
+      }
+      if (lags) {
+        // exact head: lags jg, jg+8, ... share the parity of jg; a position before the sequence contributes nothing.
+        // omode: the same inputs, weighted with the next lag's taps, are the odd lags of the next step (lag sl+1 of
+        // position t+1 is lag sl of position t), summed in the order the plain step uses for its odd mode groups.
         float f[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int k = 0; k < PJ; ++k) {
           const int sl = jg + 8 * k;
           if (sl < R) {
             const float m = (t - sl >= 0) ? 1.f : 0.f;
-            f[0] = fmaf(fr[k].x, sl == 0 ? x[0] : m * rx[k][0], f[0]);
-            f[1] = fmaf(fr[k].y, sl == 0 ? x[1] : m * rx[k][1], f[1]);
-            f[2] = fmaf(fr[k].z, sl == 0 ? x[2] : m * rx[k][2], f[2]);
-            f[3] = fmaf(fr[k].w, sl == 0 ? x[3] : m * rx[k][3], f[3]);
+            float xv[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) xv[v] = sl == 0 ? x[v] : m * rx[k][v];
+            if constexpr (!prime) {
+              f[0] = fmaf(fr[k].x, xv[0], f[0]);
+              f[1] = fmaf(fr[k].y, xv[1], f[1]);
+              f[2] = fmaf(fr[k].z, xv[2], f[2]);
+              f[3] = fmaf(fr[k].w, xv[3], f[3]);
+            }
+            if (OM != 0 && sl + 1 < R) {
+              fnx[0] = fmaf(fr2[k].x, xv[0], fnx[0]);
+              fnx[1] = fmaf(fr2[k].y, xv[1], fnx[1]);
+              fnx[2] = fmaf(fr2[k].z, xv[2], fnx[2]);
+              fnx[3] = fmaf(fr2[k].w, xv[3], fnx[3]);
+            }
           }
         }
 #pragma unroll 4
@@ -267,32 +333,57 @@ stu_step_lds_kernel(float* __restrict__ state, const T* __restrict__ xp, int ldx
           float xv[4];
           Ring4<T>::ld(rb + (size_t)((t - sl) & (R - 1)) * d, xv);
           const float m = (t - sl >= 0) ? 1.f : 0.f;
-          const float4 rv = *(const float4*)(fir + (size_t)sl * d + c);
-          f[0] = fmaf(rv.x, m * xv[0], f[0]);
-          f[1] = fmaf(rv.y, m * xv[1], f[1]);
-          f[2] = fmaf(rv.z, m * xv[2], f[2]);
-          f[3] = fmaf(rv.w, m * xv[3], f[3]);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) xv[v] *= m;
+          if constexpr (!prime) {
+            const float4 rv = *(const float4*)(fir + (size_t)sl * d + c);
+            f[0] = fmaf(rv.x, xv[0], f[0]);
+            f[1] = fmaf(rv.y, xv[1], f[1]);
+            f[2] = fmaf(rv.z, xv[2], f[2]);
+            f[3] = fmaf(rv.w, xv[3], f[3]);
+          }
+          if (OM != 0 && sl + 1 < R) {
+            const float4 rv2 = *(const float4*)(fir + (size_t)(sl + 1) * d + c);
+            fnx[0] = fmaf(rv2.x, xv[0], fnx[0]);
+            fnx[1] = fmaf(rv2.y, xv[1], fnx[1]);
+            fnx[2] = fmaf(rv2.z, xv[2], fnx[2]);
+            fnx[3] = fmaf(rv2.w, xv[3], fnx[3]);
+          }
         }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           if (jg & 1) acco[v] += f[v]; else acc[v] += f[v];
         }
-        if (jg == 0) Ring4<T>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, x);
       }
+      if (head && jg == 0 && !prime) Ring4<T>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, x);
     }
   }
 #pragma unroll
   for (int v = 0; v < 4; ++v) { sh[jg][q][v] = acc[v]; sho[jg][q][v] = acco[v]; }
+  if (omode && (jg & 1) == 0) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) shf[jg + 1][q][v] = fnx[v];
+  }
   __syncthreads();
   if (jg == 0 && ok) {
+    float onext[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       float e = 0.f, o = 0.f;
 #pragma unroll
-      for (int g = 0; g < LDS_JG; ++g) { e += sh[g][q][v]; o += sho[g][q][v]; }
-      const float out = pair ? DT<T>::rnd(e + o) + DT<T>::rnd(e - o) : scale * (e + o);
-      DT<T>::st(y + (size_t)b * ldy + c + v, res ? rsd[v] + DT<T>::rnd(out) : out);
+      for (int g = 0; g < LDS_JG; ++g) {
+        e += sh[g][q][v];
+        // (omode: what the plain step's odd mode group g holds before the reduction: its bank sum plus its lags)
+        o += (omode && head && (g & 1)) ? sho[g][q][v] + shf[g][q][v] : sho[g][q][v];
+      }
+      onext[v] = o;
+      if (omode) o = ocur[v];
+      if constexpr (!prime) {
+        const float out = pair ? DT<T>::rnd(e + o) + DT<T>::rnd(e - o) : scale * (e + o);
+        DT<T>::st(y + (size_t)b * ldy + c + v, res ? rsd[v] + DT<T>::rnd(out) : out);
+      }
     }
+    if (omode) Ring4<float>::st(ocache + (size_t)b * d + c, onext);
   }
 }
 
@@ -304,7 +395,7 @@ extern "C" int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const f
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
                                void* stream, int pair = 0, void* ring = nullptr, const float* fir = nullptr, int R = 0,
-                               const int* pos_dyn = nullptr, const void* res = nullptr);
+                               const int* pos_dyn = nullptr, const void* res = nullptr, float* ocache = nullptr, int omode = 0);
 
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,
                           int B, int S, int d, int t, const int* dyn, int dtype, void* stream) {
@@ -323,20 +414,45 @@ extern "C" int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, co
                                       const float* co, void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S,
                                       int d, int t, int dtype, void* stream) {
   return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
-                                    stream, nullptr);
+                                    stream, nullptr, nullptr);
 }
 
 // ring / fir / fir_taps: optional exact head of the filter (all three or none).  dyn: device-side {position, step} that
 // supplies the parity; pos_dyn: the same words where only the ring slot is read from them (the parity then comes with t)
 int fstu_stu_step_lds_pair_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co, void* ring,
                                const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t, const int* dyn,
-                               const int* pos_dyn, int dtype, void* stream, const void* res) {
+                               const int* pos_dyn, int dtype, void* stream, const void* res, float* ocache) {
   FSTU_REQUIRE(co, FSTU_ENULL, "fstu_stu_step_lds_pair: null pointer");
   FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_pair: co must be 16-byte aligned");
   FSTU_REQUIRE(fstu_fir_ok(ring, fir, fir_taps), FSTU_EARG,
                "fstu_stu_step_lds_pair: ring, fir and fir_taps (a power of two, 8..1024) go together, 16-byte aligned");
   return stu_step_lds_launch(state, xp, ldxp, a, ce, co, 1.0f, y, ldy, B, S, d, t, dyn, dtype, stream, 1, ring, fir, fir_taps,
-                             dyn ? dyn : pos_dyn, res);
+                             dyn ? dyn : pos_dyn, res, ocache, ocache ? 1 : 0);
+}
+
+// The pair step with the odd-lag sum handed from step to step: ocache (B,d) fp32 holds the O of position t (from the
+// step at t-1 or from fstu_stu_step_lds_prime) and receives the O of position t+1, so the bank of the other parity
+// is not read.  Same values as fstu_stu_step_lds_pair, bit for bit.  res may be NULL; otherwise as in _pair_add.
+extern "C" int fstu_stu_step_lds_pair_cached(float* state, const void* xp, int ldxp, const float* a, const float* ce,
+                                             const float* co, void* ring, const float* fir, int fir_taps, float* ocache,
+                                             const void* res, void* y, int ldy, int B, int S, int d, int t, int dtype,
+                                             void* stream) {
+  FSTU_REQUIRE(ocache, FSTU_ENULL, "fstu_stu_step_lds_pair_cached: ocache is null");
+  return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
+                                    stream, res, ocache);
+}
+
+// ocache = the O of position t+1 as a pair step at position t would leave it, from the state and the ring as they
+// stand after position t (a prompt's last position): nothing else is read or written.
+extern "C" int fstu_stu_step_lds_prime(const float* state, const float* a, const float* co, const void* ring, const float* fir,
+                                       int fir_taps, float* ocache, int B, int S, int d, int t, int dtype, void* stream) {
+  FSTU_REQUIRE(state && a && co && ocache, FSTU_ENULL, "fstu_stu_step_lds_prime: null pointer");
+  FSTU_REQUIRE(fstu_aligned(co, 16), FSTU_EALIGN, "fstu_stu_step_lds_prime: co must be 16-byte aligned");
+  FSTU_REQUIRE(fstu_fir_ok(ring, fir, fir_taps), FSTU_EARG,
+               "fstu_stu_step_lds_prime: ring, fir and fir_taps (a power of two, 8..1024) go together, 16-byte aligned");
+  // (ce, xp and y are not touched in this mode; valid pointers stand in for them)
+  return stu_step_lds_launch(const_cast<float*>(state), ocache, d, a, co, co, 1.0f, ocache, d, B, S, d, t, nullptr, dtype, stream, 1,
+                             const_cast<void*>(ring), fir, fir_taps, nullptr, nullptr, ocache, 2);
 }
 
 // The same step joining the residual stream: y = T(res + T(step output)), rows of stride ldy in both; y may be res
@@ -346,13 +462,16 @@ extern "C" int fstu_stu_step_lds_pair_add(float* state, const void* xp, int ldxp
                                           int ldy, int B, int S, int d, int t, int dtype, void* stream) {
   FSTU_REQUIRE(res, FSTU_ENULL, "fstu_stu_step_lds_pair_add: res is null");
   return fstu_stu_step_lds_pair_dyn(state, xp, ldxp, a, ce, co, ring, fir, fir_taps, y, ldy, B, S, d, t, nullptr, nullptr, dtype,
-                                    stream, res);
+                                    stream, res, nullptr);
 }
 
 static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                                float scale, void* y, int ldy, int B, int S, int d, int t, const int* dyn, int dtype,
-                               void* stream, int pair, void* ring, const float* fir, int R, const int* pos_dyn, const void* res) {
+                               void* stream, int pair, void* ring, const float* fir, int R, const int* pos_dyn, const void* res,
+                               float* ocache, int omode) {
   FSTU_REQUIRE(state && xp && a && ce && y, FSTU_ENULL, "fstu_stu_step_lds: null pointer");
+  FSTU_REQUIRE(omode == 0 || (ocache && co && fstu_aligned(ocache, 16)), FSTU_EARG,
+               "fstu_stu_step_lds: the handed-on odd-lag sum needs co and a 16-byte aligned ocache");
   FSTU_REQUIRE(!res || (fstu_aligned(res, 16) && ldy % 4 == 0), FSTU_EALIGN,
                "fstu_stu_step_lds: the residual rows must be 16-byte aligned with a stride that is a multiple of 4");
   FSTU_REQUIRE(B >= 1 && S >= 1 && d >= 4 && d % 4 == 0, FSTU_ESHAPE, "fstu_stu_step_lds: need d %% 4 == 0 (B=%d S=%d d=%d)", B, S, d);
@@ -360,10 +479,13 @@ static int stu_step_lds_launch(float* state, const void* xp, int ldxp, const flo
   FSTU_REQUIRE(t >= 0, FSTU_EARG, "fstu_stu_step_lds: t<0");
   FSTU_REQUIRE(fstu_aligned(state, 16) && fstu_aligned(ce, 16), FSTU_EALIGN, "fstu_stu_step_lds: state/ce must be 16-byte aligned");
   dim3 grid((d / 4 + 31) / 32, B);
-  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds",
-                      hipLaunchKernelGGL(stu_step_lds_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, state,
-                                         (const T*)xp, ldxp, a, ce, co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair, (T*)ring, fir, R,
-                                         t, pos_dyn, (const T*)res));
+#define STU_STEP_GO(OM)                                                                                               \
+  hipLaunchKernelGGL((stu_step_lds_kernel<T, OM>), grid, dim3(256), 0, (hipStream_t)stream, state, (const T*)xp, ldxp, a, ce, \
+                     co, scale, (T*)y, ldy, S, d, t & 1, dyn, pair, (T*)ring, fir, R, t, pos_dyn, (const T*)res, ocache)
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_step_lds", {
+    if (omode == 1) STU_STEP_GO(1); else if (omode == 2) STU_STEP_GO(2); else STU_STEP_GO(0);
+  });
+#undef STU_STEP_GO
   FSTU_CHECK_LAUNCH("fstu_stu_step_lds");
   return FSTU_OK;
 }

@@ -36,6 +36,8 @@ SIGNATURES = {
     "fstu_stu_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_pair": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_pair_add": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_pair_cached": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_step_lds_prime": [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_step_lds_single": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_bank_step_lds": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_inproj_step": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
@@ -420,12 +422,13 @@ def _fir_args(ring, fir, B, d, dtype):
 def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: torch.Tensor, t: int,
                  out: Optional[torch.Tensor] = None, co: Optional[torch.Tensor] = None, pair: bool = False,
                  ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None,
-                 res: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 res: Optional[torch.Tensor] = None, ocache: Optional[torch.Tensor] = None) -> torch.Tensor:
     """state fp32 (B,2,S,d) advanced in place; xp (B,d) -> y (B,d) = T(2E), E = ce . bank(t).  With co (S,d) and
     O = co . other bank: the single-branch form y = T(E+O) (use_hankel_L), or with pair=True the two sign branches
     rounded separately, y = T(T(E+O) + T(E-O)).  pair=True with ring (B,R,d) and fir (R,d): the exact head of the
     filter on the first R lags (the ring is updated in place).  pair=True with res (B,d): the step joins the residual
-    stream, y = T(res + T(output)); out may be res."""
+    stream, y = T(res + T(output)); out may be res.  pair=True with ocache (B,d) fp32: O comes from ocache (left by the
+    previous step or by stu_step_lds_prime) and the next step's O is left there; the other bank is not read."""
     _dev(state, a, ce, co)
     B, two, S, d = state.shape
     assert two == 2 and state.dtype == torch.float32 and a.dtype == torch.float32 and ce.dtype == torch.float32
@@ -440,6 +443,14 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
         assert co.dtype == torch.float32 and co.shape == (S, d)
         if pair:
             rp, fp, R = _fir_args(ring, fir, B, d, xp.dtype)
+            if ocache is not None:
+                _dev(ocache, res)
+                assert ocache.dtype == torch.float32 and ocache.shape == (B, d) and ocache.is_contiguous()
+                assert res is None or (res.dtype == xp.dtype and res.shape == (B, d) and _rows_view(res)[1] == ldy)
+                _check(load().fstu_stu_step_lds_pair_cached(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(co), rp, fp, R,
+                                                            _p(ocache), _p(res), _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
+                       "fstu_stu_step_lds_pair_cached")
+                return out
             if res is not None:
                 _dev(res)
                 assert res.dtype == xp.dtype and res.shape == (B, d) and _rows_view(res)[1] == ldy
@@ -455,6 +466,24 @@ def stu_step_lds(state: torch.Tensor, xp: torch.Tensor, a: torch.Tensor, ce: tor
         return out
     _check(load().fstu_stu_step_lds(_p(state), _p(xp), ldxp, _p(a), _p(ce), _p(out), ldy, B, S, d, t, _dt(xp), _stream()),
            "fstu_stu_step_lds")
+    return out
+
+
+def stu_step_lds_prime(state: torch.Tensor, a: torch.Tensor, co: torch.Tensor, t: int, dtype: torch.dtype,
+                       ring: Optional[torch.Tensor] = None, fir: Optional[torch.Tensor] = None,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ocache (B,d) fp32 for position t+1 from the state (B,2,S,d) and the ring as they stand after position t: what
+    a pair step with ocache at position t would have left.  dtype: the model dtype (of the ring)."""
+    _dev(state, a, co)
+    B, two, S, d = state.shape
+    assert two == 2 and state.dtype == torch.float32 and a.numel() == S and co.shape == (S, d) and co.dtype == torch.float32
+    rp, fp, R = _fir_args(ring, fir, B, d, dtype)
+    if out is None:
+        out = torch.empty(B, d, dtype=torch.float32, device=state.device)
+    assert out.shape == (B, d) and out.dtype == torch.float32 and out.is_contiguous() and out.is_cuda
+    _check(load().fstu_stu_step_lds_prime(_p(state), _p(a), _p(co), rp, fp, R, _p(out), B, S, d, t,
+                                          FSTU_BF16 if dtype == torch.bfloat16 else FSTU_F32, _stream()),
+           "fstu_stu_step_lds_prime")
     return out
 
 

@@ -27,7 +27,7 @@ _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
 class LayerDesc(ctypes.Structure):
     _fields_ = [("kind", _i), ("norm1_w", _vp), ("mlp_norm_w", _vp), ("w_gate", _vp), ("w_up", _vp), ("w_down", _vp),
-                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_co", _vp), ("lds_state", _vp), ("lds_ring", _vp), ("lds_fir", _vp),
+                ("m_inputs_t", _vp), ("filt", _vp), ("hist", _vp), ("lds_a", _vp), ("lds_ce", _vp), ("lds_co", _vp), ("lds_state", _vp), ("lds_ring", _vp), ("lds_fir", _vp), ("lds_ocache", _vp),
                 ("w_qkv", _vp), ("w_proj", _vp), ("kring", _vp), ("vring", _vp), ("slopes", _vp),
                 ("wp_gate", _vp), ("wp_up", _vp), ("wp_down", _vp), ("wp_m_inputs", _vp), ("wp_qkv", _vp),
                 ("wp_proj", _vp)]
@@ -180,6 +180,13 @@ class DecodeEngine:
                         keep(fir), keep(ring)
                         ld.lds_ring, ld.lds_fir = ring.data_ptr(), fir.data_ptr()
                         fir_taps = fir.shape[0]
+                    if B > _hip.MAX_DECODE_ROWS and dt == torch.bfloat16 and not cfg.use_hankel_L:
+                        # 17..32 rows: the odd-lag sum is handed from step to step, so a step reads one bank only;
+                        # primed here for the first decode position from the state and ring the prompt left
+                        oc = _hip.stu_step_lds_prime(st, a, co, int(pos[0]) - 1, dt,
+                                                     ring=hist[b0:b1] if ld.lds_ring else None, fir=fir if ld.lds_ring else None)
+                        keep(oc)
+                        ld.lds_ocache = oc.data_ptr()
                 else:
                     hs = hist[b0:b1]
                     if hist_cap and hs.shape[1] != hist_cap:

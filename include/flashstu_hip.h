@@ -143,6 +143,19 @@ int fstu_stu_step_lds(float* state, const void* xp, int ldxp, const float* a, co
 int fstu_stu_step_lds_pair(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
                            void* ring, const float* fir, int fir_taps, void* y, int ldy, int B, int S, int d, int t,
                            int dtype, void* stream);
+/* The pair step without the read of the other bank.  The odd-lag sum O of position t weighs the bank that the step at
+ * t-1 advanced and the odd lags of the exact head reach inputs that step already held, so the step at t-1 can form it
+ * while it has that bank in registers: ocache (B,d) fp32 holds the O of position t on entry and the O of position t+1
+ * on return.  Same values as fstu_stu_step_lds_pair, bit for bit (same products in the same order), a third less state
+ * traffic.  res: NULL, or the residual rows as in fstu_stu_step_lds_pair_add.  fstu_stu_step_lds_prime fills ocache for
+ * position t+1 from the state and the ring as they stand after position t (a prompt's last position); it advances and
+ * writes nothing else.  No counterpart in the reference, whose STU layers keep no decode state
+ * (flash_stu/layers/stu_layer.py:99-120). */
+int fstu_stu_step_lds_pair_cached(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
+                                  void* ring, const float* fir, int fir_taps, float* ocache, const void* res, void* y, int ldy,
+                                  int B, int S, int d, int t, int dtype, void* stream);
+int fstu_stu_step_lds_prime(const float* state, const float* a, const float* co, const void* ring, const float* fir,
+                            int fir_taps, float* ocache, int B, int S, int d, int t, int dtype, void* stream);
 /* The same step joining the residual stream (flash_stu/layers/stu_layer.py:93, x = x + stu(stu_norm(x))):
  * y = T(res + T(step output)), rows of stride ldy in both, 16-byte aligned; y may be res. */
 int fstu_stu_step_lds_pair_add(float* state, const void* xp, int ldxp, const float* a, const float* ce, const float* co,
@@ -491,6 +504,8 @@ typedef struct {
   float* lds_state;         /* (B,2,S,d)                          (lds mode) */
   void* lds_ring;           /* (B,lds_fir_taps,d) last projected inputs, model dtype, or NULL (lds mode, with lds_co) */
   const float* lds_fir;     /* (lds_fir_taps,d) phi_proj minus the fitted filter on the first lags, or NULL */
+  float* lds_ocache;        /* (B,d) fp32 or NULL: the odd-lag sum handed from step to step (fstu_stu_step_lds_pair_cached),
+                               primed for the first decode position by fstu_stu_step_lds_prime; used by the 17..32-row step */
   /* attention */
   const void* w_qkv;        /* (3d,d) */
   const void* w_proj;       /* (d,d) */

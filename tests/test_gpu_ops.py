@@ -626,6 +626,39 @@ def test_stu_step_lds_pair_joins_the_residual_stream(hip, dtype):
     assert torch.equal(st1, st2)
 
 
+@pytest.mark.parametrize("dtype,S,R,T0", [(torch.bfloat16, 64, 64, 70), (torch.bfloat16, 64, 64, 1), (torch.bfloat16, 80, 128, 5),
+                                          (torch.float32, 64, 8, 3), (torch.bfloat16, 24, 0, 9), (torch.float32, 72, 256, 300)])
+def test_stu_step_lds_pair_with_the_odd_lag_sum_handed_on(hip, dtype, S, R, T0):
+    """The pair step that takes O from the previous step (or from the priming launch after a prompt of T0 positions)
+    and never reads the other bank equals the plain pair step bit for bit: outputs, both banks and the ring, with and
+    without the exact head (R taps; beyond 64 modes / 64 taps the kernels' loops), with and without a residual row."""
+    B, d = 3, 256
+    g = gen(93)
+    a = dev(torch.rand(S, generator=g) * 0.95)
+    ce, co = dev(torch.randn(S, d, generator=g) / 8), dev(torch.randn(S, d, generator=g) / 8)
+    fir = dev(torch.randn(R, d, generator=g) / 16) if R else None
+    ring_p = torch.zeros(B, R, d, dtype=dtype, device="cuda") if R else None
+    st_p = torch.zeros(B, 2, S, d, device="cuda")
+    xs = torch.randn(T0 + 12, B, d, generator=g).to(dtype)
+    for t in range(T0):                                   # the "prompt", stepped by the plain kernel
+        hip.stu_step_lds(st_p, dev(xs[t]), a, ce, t, co=co, pair=True, ring=ring_p, fir=fir)
+    st_c, ring_c = st_p.clone(), (ring_p.clone() if R else None)
+    oc = hip.stu_step_lds_prime(st_c, a, co, T0 - 1, dtype, ring=ring_c, fir=fir)
+    assert torch.equal(st_c, st_p) and (not R or torch.equal(ring_c, ring_p))      # priming writes nothing else
+    stream = dev(torch.randn(B, d, generator=g).to(dtype))
+    for t in range(T0, T0 + 12):
+        xt = dev(xs[t])
+        want = hip.stu_step_lds(st_p, xt, a, ce, t, co=co, pair=True, ring=ring_p, fir=fir)
+        if t % 3 == 0:                                    # joined with the residual stream now and then
+            got = hip.stu_step_lds(st_c, xt, a, ce, t, co=co, pair=True, ring=ring_c, fir=fir, ocache=oc, res=stream)
+            assert torch.equal(got, stream + want), t
+        else:
+            got = hip.stu_step_lds(st_c, xt, a, ce, t, co=co, pair=True, ring=ring_c, fir=fir, ocache=oc)
+            assert torch.equal(got, want), t
+        assert torch.equal(st_c[:, t & 1], st_p[:, t & 1])
+    assert torch.equal(st_c, st_p) and (not R or torch.equal(ring_c, ring_p))
+
+
 @pytest.mark.parametrize("R", [8, 32, 128, 256])
 def test_stu_step_lds_exact_head(hip, R):
     """The exact head of the distilled filter: fir[s] = phi_proj[s] - fitted filter for the first R lags, applied to a
