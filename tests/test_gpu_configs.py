@@ -255,6 +255,30 @@ def test_c5_shape_bf16_lds_teacher_forced(rows):
     assert float(err.max()) <= 2e-2
 
 
+@pytest.mark.parametrize("P", [1, 20])
+def test_c5_shape_bf16_more_rows_than_one_chunk(P):
+    """40 rows step as a chunk of 32 (packed-weight kernels over two row tiles, the recurrence step handing its
+    odd-lag sum on, primed after a prompt of P positions) and a chunk of 8 (the 16-row kernels): every row's ids are
+    those of its chunk generated alone, its logits agree with that run to rounding, and they meet the teacher-forced
+    oracle."""
+    from test_gpu_model import make_pair, prompt, _teacher_forced
+    ocfg, w, model = make_pair(seed=2, init="healthy", dtype=torch.bfloat16, mlp_scale=2, n_embd=256, n_layers=4,
+                               n_heads=2, window_size=24, num_eigh=24, seq_len=256, vocab_size=2003,
+                               stu_decode_mode="lds")
+    N = 30
+    ids = prompt(40, P, ocfg.vocab_size, 4)
+    got, gl = model.generate(ids.cuda(), max_length=P + N, do_sample=False, return_logits=True)
+    assert torch.equal(model.generate(ids.cuda(), max_length=P + N, do_sample=False), got)        # graph replay
+    for lo, hi in ((0, 32), (32, 40)):
+        part, pl = model.generate(ids[lo:hi].cuda(), max_length=P + N, do_sample=False, return_logits=True)
+        assert torch.equal(part, got[lo:hi])
+        # (the prompt pass picks its GEMM tiles by the number of rows, so the logits agree to rounding, not bit for bit)
+        assert float((pl.float() - gl[lo:hi].float()).abs().max()) <= 2e-2 * float(gl.float().abs().max())
+    ref = _teacher_forced(w, ocfg, got.cpu(), P).float()
+    err = (gl.float().cpu() - ref).abs().amax(-1) / ref.abs().amax(-1)
+    assert float(err.max()) <= 2e-2
+
+
 @pytest.mark.parametrize("d,heads,rows", [(1024, 8, 8), (2048, 16, 8), (2048, 16, 32), (1024, 8, 21)])
 def test_c5_width_bf16_step_kernels(d, heads, rows):
     """Config 5's widths through the whole one-call step (head dim 128, d=2048 takes the 8-k-step variants of the
