@@ -206,10 +206,10 @@ def glu_roofline(eng, cfg, B, K, lib, torch, _hip):
         gbps = glu_bytes / (us * 1e-6) / 1e9
         # HBM bytes per launch from two rocprofv3 --pmc runs (FETCH_SIZE x2.000, WRITE_SIZE x1.000 against the library's
         # plain copy kernel), measured offline for config 5's shape: profiles/decode_c5_hbm_traffic_pmc.txt
-        traffic = 204052787 if packed and (d, I, rows) == (2048, 24576, 32) else None
+        traffic = 204146262 if packed and (d, I, rows) == (2048, 24576, 32) else None
         return {"bound": "hbm", "kernel": name,
                 "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic,
-                "traffic_source": "profiles/decode_c5_hbm_traffic_pmc.txt (counter runs of this launch without its norm, not of this run)" if traffic else None,
+                "traffic_source": "profiles/decode_c5_hbm_traffic_pmc.txt (counter runs of this kernel, not of this run)" if traffic else None,
                 "bytes_per_launch": glu_bytes, "avg_launch_us": us, "launches_timed": n, "rows_per_launch": rows}
     ms_c, n_c = ctypes.c_double(), ctypes.c_int()
     torch.cuda.synchronize()
