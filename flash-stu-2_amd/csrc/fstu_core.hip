@@ -291,6 +291,34 @@ static int launch_add_rmsnorm(void* x, const void* delta, int delta_mode, int ns
   return 0;
 }
 
+// x = T(x + T(sum of nslices fp32 slices)) over rows*d elements, 4 per thread and 64 threads per workgroup, so that the
+// few megabytes of slices are requested by the whole chip at once; the slices are added in the order fstu_add_rmsnorm
+// uses (bit-identical x).  The rows' norm is left to the launch that consumes x.
+__global__ void __launch_bounds__(64)
+add_slices_bf16_kernel(bf16_t* __restrict__ x, const float* __restrict__ slices, int nslices, size_t n) {
+  const size_t i4 = ((size_t)blockIdx.x * 64 + threadIdx.x) * 4;
+  if (i4 >= n) return;
+  const uint2 xr = *(const uint2*)(x + i4);
+  float dv[4];
+  sum_slices4(slices + i4, n, nslices, dv);
+  const float x0 = __uint_as_float(xr.x << 16), x1 = __uint_as_float(xr.x & 0xffff0000u);
+  const float x2 = __uint_as_float(xr.y << 16), x3 = __uint_as_float(xr.y & 0xffff0000u);
+  *(uint2*)(x + i4) = make_uint2(pack2_bf16(x0 + DT<bf16_t>::rnd(dv[0]), x1 + DT<bf16_t>::rnd(dv[1])),
+                                 pack2_bf16(x2 + DT<bf16_t>::rnd(dv[2]), x3 + DT<bf16_t>::rnd(dv[3])));
+}
+
+extern "C" int fstu_add_slices(void* x, const float* slices, int nslices, int rows, int d, int dtype, void* stream) {
+  FSTU_REQUIRE(x && slices, FSTU_ENULL, "fstu_add_slices: null pointer");
+  FSTU_REQUIRE(dtype == FSTU_BF16, FSTU_EDTYPE, "fstu_add_slices: bf16 only");
+  FSTU_REQUIRE(rows >= 1 && d >= 4 && d % 4 == 0 && nslices >= 1, FSTU_ESHAPE, "fstu_add_slices: rows=%d d=%d nslices=%d", rows, d, nslices);
+  FSTU_REQUIRE(fstu_aligned(x, 8) && fstu_aligned(slices, 16), FSTU_EALIGN, "fstu_add_slices: x must be 8-byte, slices 16-byte aligned");
+  const size_t n = (size_t)rows * d;
+  hipLaunchKernelGGL(add_slices_bf16_kernel, dim3((unsigned)((n / 4 + 63) / 64)), dim3(64), 0, (hipStream_t)stream, (bf16_t*)x, slices,
+                     nslices, n);
+  FSTU_CHECK_LAUNCH("fstu_add_slices");
+  return FSTU_OK;
+}
+
 extern "C" int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch,
                                 const void* w, void* y, int rows, int d, float eps, int dtype, void* stream) {
   FSTU_REQUIRE(x, FSTU_ENULL, "fstu_add_rmsnorm: x is null");

@@ -178,19 +178,24 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
     return FSTU_OK;
   };
   TIMED(PC_NORM, fstu_embed_rmsnorm(tok_in, tok_stride, m->emb, m->x, m->layers[0].norm1_w, m->h, B, d, m->V, m->eps, dt, stream, dyn));
+  // raw: the residual stream in m->x has the previous layer's MLP output added but is not normalised yet (m->h is
+  // stale); the layer's first projection, over packed weights, then forms its norm in its own fragments
+  bool raw = false;
   for (int l = 0; l < m->n_layers; ++l) {
     const fstu_layer_desc& L = m->layers[l];
+    const void* xin = raw ? m->x : m->h;
+    const void* nw1 = raw ? L.norm1_w : nullptr;
     // Where the layer's MLP streams packed weights, the sub-layer's last launch adds its output to the residual stream
     // itself (m->x in place) and the gate/up launch normalises the stream in its own fragments: no add+norm launch
     // between them.
     const bool join = packed_mlp && L.wp_gate && L.wp_up && (L.kind == 0 ? L.lds_co != nullptr : L.wp_proj != nullptr);
     if (L.kind == 0) {
       // in-projection on the two halves of the rows (16-row kernel), then one recurrence launch over all rows
-      if (packed_mlp && L.wp_m_inputs) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_m_inputs, m->xp, d, B, d, d, stream));
+      if (packed_mlp && L.wp_m_inputs) TIMED(PC_PROJ, fstu_linear_packed(xin, d, nw1, m->eps, L.wp_m_inputs, m->xp, d, B, d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.m_inputs_t, m->xp, d, d, d));
       TIMED(PC_STU, stu_step(L, m, stu_pos(pos), stu_dyn(dyn), dyn, stream, join ? m->x : nullptr, true));
     } else {
-      if (packed_mlp && L.wp_qkv) TIMED(PC_PROJ, fstu_linear_packed(m->h, d, nullptr, 0.f, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
+      if (packed_mlp && L.wp_qkv) TIMED(PC_PROJ, fstu_linear_packed(xin, d, nw1, m->eps, L.wp_qkv, m->qkv, 3 * d, B, 3 * d, d, stream));
       else TIMED(PC_PROJ, proj(m->h, d, L.w_qkv, m->qkv, 3 * d, 3 * d, d));
       TIMED(PC_SWA, fstu_swa_decode_impl(m->qkv, L.kring, L.vring, m->attn, L.slopes, B, m->n_heads, m->head_dim, m->kv_cap, pos,
                                          m->window, m->softcap, 1, dyn, dt, stream));
@@ -215,7 +220,15 @@ static int decode_step_wide(const fstu_model_desc* m, const int64_t* tok_in, int
     } else {
       TIMED(PC_DOWN, fstu_gemm_bf16_splitk(m->act, I, L.w_down, m->partial, B, d, I, ks, stream));
     }
-    TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
+    // The split-K slices join the stream in a launch that the whole chip shares (one workgroup per row would fetch
+    // 131 KB each); where the next layer's first projection streams packed weights it forms the norm itself
+    raw = false;
+    if (packed_mlp && l + 1 < m->n_layers && d % 4 == 0) {
+      const fstu_layer_desc& Nx = m->layers[l + 1];
+      raw = Nx.kind == 0 ? Nx.wp_m_inputs != nullptr : Nx.wp_qkv != nullptr;
+    }
+    if (raw) TIMED(PC_NORM, fstu_add_slices(m->x, m->partial, nsl, B, d, dt, stream));
+    else TIMED(PC_NORM, fstu_add_rmsnorm(m->x, m->partial, 1, nsl, 0, next_w, m->h, B, d, m->eps, dt, stream));
   }
   if (sample_spread_ok(m, do_sample, top_k)) {
     // the head leaves each row's packed maxima, the sampler spreads every row over the chip and advances {pos, step}

@@ -671,7 +671,7 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
     // two row tiles: the partial sums of both lie in dynamic LDS
     constexpr int DA = KSA <= 3 ? 4 : (KSA == 4 ? 3 : 2);
     const size_t red2 = (size_t)2 * DA * 8 * 512 * sizeof(float);
-    FSTU_REQUIRE(pro == 0 || (pro == 3 && epi == 0), FSTU_ESHAPE, "%s: more than %d rows: no prologue, or the gated pair with the in-register one",
+    FSTU_REQUIRE(pro == 0 || (pro == 3 && epi != 2), FSTU_ESHAPE, "%s: more than %d rows: no prologue, or the in-register one (not on the head)",
                  name, FSTU_MAX_DECODE_ROWS);
 #define GLU_GO2(PRO, EPI)                                                                                                  \
   do {                                                                                                                     \
@@ -682,7 +682,11 @@ static int glu_launch_ksa(GluArgs& a, int pro, int epi, int G, size_t shm, const
                        a.x_in, a.delta, a.x_out, a.norm_w, a.rows, a.d, a.I, a.ldh, a.ldact, a.fpw, a.eps, a.nslices, a.best,  \
                        a.temperature);                                                                                      \
   } while (0)
-    if (pro == 3) GLU_GO2(3, 0); else if (epi == 0) GLU_GO2(0, 0); else if (epi == 2) GLU_GO2(0, 2); else GLU_GO2(0, 1);
+    if (pro == 3 && epi == 0) GLU_GO2(3, 0);
+    else if (pro == 3) GLU_GO2(3, 1);
+    else if (epi == 0) GLU_GO2(0, 0);
+    else if (epi == 2) GLU_GO2(0, 2);
+    else GLU_GO2(0, 1);
 #undef GLU_GO2
     return FSTU_OK;
   }
@@ -773,19 +777,21 @@ extern "C" int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x
 extern "C" int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                                   int rows, int N, int K, void* stream) {
   FSTU_REQUIRE(x && wp && y, FSTU_ENULL, "fstu_linear_packed: null pointer");
+  // 17..32 rows: two row tiles; with norm_w the norm is formed in the matrix-core fragments
+  const bool wide = rows > FSTU_MAX_DECODE_ROWS;
   FSTU_REQUIRE(fstu_glu_packed_supported(rows, K, N) ||
-                   (norm_w == nullptr && rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(FSTU_MAX_DECODE_ROWS, K, N)),
+                   (rows <= 2 * FSTU_MAX_DECODE_ROWS && fstu_glu_packed_supported(FSTU_MAX_DECODE_ROWS, K, N)),
                FSTU_ESHAPE, "fstu_linear_packed: unsupported shape rows=%d K=%d N=%d", rows, K, N);
   FSTU_REQUIRE(ldx >= K && ldx % 8 == 0 && ldy >= N && ldy % 4 == 0, FSTU_ESHAPE, "fstu_linear_packed: ldx=%d ldy=%d", ldx, ldy);
   FSTU_REQUIRE(norm_w == nullptr || ldx == K, FSTU_ESHAPE, "fstu_linear_packed: the norm prologue needs dense rows");
   FSTU_REQUIRE(fstu_aligned(x, 16) && fstu_aligned(norm_w, 16) && fstu_aligned(wp, 16) && fstu_aligned(y, 8), FSTU_EALIGN,
                "fstu_linear_packed: pointers must be 16-byte aligned");
-  FSTU_REQUIRE(norm_w == nullptr || (size_t)rows * (K + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_linear_packed: rows*K too large for LDS");
+  FSTU_REQUIRE(norm_w == nullptr || wide || (size_t)rows * (K + 8) * 2 <= 96 * 1024, FSTU_ESHAPE, "fstu_linear_packed: rows*K too large for LDS");
   GluArgs a = {};
   a.wp_gate = (const uint4*)wp; a.wp_up = (const uint4*)wp; a.act = (bf16_t*)y;
   a.rows = rows; a.d = K; a.I = N; a.ldh = ldx; a.ldact = ldy; a.eps = eps;
   if (norm_w) { a.x_in = (const bf16_t*)x; a.norm_w = (const bf16_t*)norm_w; } else { a.h = (const bf16_t*)x; }
-  return glu_launch(a, norm_w != nullptr ? 1 : 0, 1, "fstu_linear_packed", (hipStream_t)stream);
+  return glu_launch(a, norm_w != nullptr ? (wide ? 3 : 1) : 0, 1, "fstu_linear_packed", (hipStream_t)stream);
 }
 
 // The same projection joining the residual stream: res_out = T(res_in + T(x W^T)), rows of stride N in both (res_out

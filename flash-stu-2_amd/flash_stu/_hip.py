@@ -27,6 +27,7 @@ _vp, _i, _i64, _f, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.
 SIGNATURES = {
     "fstu_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_add_rmsnorm": [_vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _f, _i, _vp],
+    "fstu_add_slices": [_vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_linear_decode": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_glu_decode": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_linear_decode_splitk": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -202,6 +203,15 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], w: Optional[torc
                                    _p(w) if want_norm else None, _p(y) if want_norm else None,
                                    rows, d, float(eps), _dt(x), _stream()), "fstu_add_rmsnorm")
     return y if want_norm else None
+
+
+def add_slices(x: torch.Tensor, slices: torch.Tensor) -> torch.Tensor:
+    """x (rows,d) bf16 += T(sum of the fp32 slices (n,rows,d)) in place, over the whole chip; returns x."""
+    _dev(x, slices)
+    rows, d = x.shape
+    assert x.is_contiguous() and slices.dtype == torch.float32 and slices.is_contiguous() and slices.shape[1:] == (rows, d)
+    _check(load().fstu_add_slices(_p(x), _p(slices), slices.shape[0], rows, d, _dt(x), _stream()), "fstu_add_slices")
+    return x
 
 
 def linear_decode(x: torch.Tensor, W: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -73,6 +73,11 @@ int fstu_embed(const int64_t* ids, const void* table, void* out, int rows, int d
  * layers/attention_layer.py:53-62, model.py:173. */
 int fstu_add_rmsnorm(void* x, const void* delta, int delta_mode, int nslices, int single_branch,
                      const void* w, void* y, int rows, int d, float eps, int dtype, void* stream);
+/* The residual update of delta_mode 1 alone, spread over the whole chip (4 elements per thread): x = T(x + T(sum of
+ * the slices)), the same values as fstu_add_rmsnorm leaves in x; for a consumer that forms the norm itself
+ * (fstu_linear_packed with norm_w at 17..32 rows).  The x.add_() of flash_stu/layers/stu_layer.py:96 and
+ * layers/attention_layer.py:62 behind a split-K down projection.  bf16, d % 4 == 0. */
+int fstu_add_slices(void* x, const float* slices, int nslices, int rows, int d, int dtype, void* stream);
 
 /* ---- skinny linear layers for decode (rows <= 16) -------------------------
  * y[m, n] = T( sum_k x[m,k] * W[n,k] ),  W is (N,K) row-major (nn.Linear layout).
@@ -440,7 +445,7 @@ int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* stream);
  * fstu_glu_packed_supported tells whether a shape is covered (d in {256,512,768,1024,2048}, I % 4 == 0).
  * 17..32 rows (fstu_mlp_packed_rows32_supported: such a d, I % 512 == 0): fstu_glu_packed and fstu_down_packed_splitk
  * take them as two row tiles per weight fragment, so every weight is still read once; of the launches with a norm
- * prologue fstu_glu_packed_norm takes them too (see there), fstu_linear_packed and fstu_linear_packed_res stay at 16 rows. */
+ * prologue fstu_glu_packed_norm and fstu_linear_packed take them too (see there), fstu_linear_packed_res stays at 16 rows. */
 int fstu_glu_packed_supported(int rows, int d, int I);
 int fstu_mlp_packed_rows32_supported(int rows, int d, int I);
 int fstu_glu_packed(const void* h, int ldh, const void* wp_gate, const void* wp_up, void* act, int ldact, int rows,
@@ -456,8 +461,9 @@ int fstu_glu_packed_norm(const void* x_in, const void* delta, void* x_out, const
 
 /* y = T(x W^T) over packed W (N,K) with the same balanced launch; with norm_w != NULL, x is the residual stream
  * (dense rows) and h = rmsnorm(x) * norm_w is formed in the prologue (the sub-layer norm of stu_layer.py:81 /
- * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, bf16, rows <= 16
- * (without norm_w: rows <= 32, the second 16 as another row tile of the same weight fragments). */
+ * attention_layer.py:53 fused into c_attn / M_inputs).  K in {256,512,768,1024,2048}, N % 4 == 0, bf16, rows <= 32
+ * (17..32: the second 16 as another row tile of the same weight fragments, and the norm formed in those fragments
+ * instead of in LDS). */
 int fstu_linear_packed(const void* x, int ldx, const void* norm_w, float eps, const void* wp, void* y, int ldy,
                        int rows, int N, int K, void* stream);
 /* The same projection joining the residual stream (flash_stu/layers/attention_layer.py:57, x = x + attn(attn_norm(x))

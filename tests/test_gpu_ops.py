@@ -1299,6 +1299,37 @@ def test_glu_packed_norm_two_row_tiles(hip, rows, d, I):
     assert float((two != act).float().mean()) <= 0.01
 
 
+@pytest.mark.parametrize("rows,d,ns", [(32, 2048, 16), (17, 768, 4), (5, 260, 3)])
+def test_add_slices_equals_the_residual_update_of_add_rmsnorm(hip, rows, d, ns):
+    g = gen(69)
+    x = dev(torch.randn(rows, d, generator=g).bfloat16())
+    sl = dev(0.3 * torch.randn(ns, rows, d, generator=g))
+    want = x.clone()
+    hip.add_rmsnorm(want, sl, None, 0.0, delta_mode=1, nslices=ns, want_norm=False)
+    got = hip.add_slices(x.clone(), sl)
+    assert torch.equal(got, want)
+    ref = (x.double() + sl.double().sum(0).bfloat16().double()).bfloat16()
+    assert float((got != ref).float().mean()) <= 0.01          # fp32 against float64 summation of the slices
+
+
+@pytest.mark.parametrize("rows,K,N", [(32, 2048, 6144), (20, 1024, 1024), (17, 256, 768)])
+def test_linear_packed_norm_two_row_tiles(hip, rows, K, N):
+    """17..32 rows: y = rmsnorm(x) W^T with the norm formed in the launch's matrix-core fragments: almost everywhere
+    the bits of the norm launch followed by the plain packed projection, and within the bf16 tolerance of float64."""
+    dtype = torch.bfloat16
+    g = gen(70)
+    x = dev(torch.randn(rows, K, generator=g).to(dtype))
+    nw = dev((1 + 0.1 * torch.randn(K, generator=g)).to(dtype))
+    W = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    wp = hip.pack_rows(dev(W))
+    got = hip.linear_packed(x, wp, N, nw, O.RMS_EPS_DEFAULT)
+    h = hip.add_rmsnorm(x.clone(), None, nw, O.RMS_EPS_DEFAULT)
+    two = hip.linear_packed(h, wp, N)
+    assert float((two != got).float().mean()) <= 0.01
+    ref = (O.rms_norm(x.cpu(), nw.cpu(), O.RMS_EPS_DEFAULT).double() @ W.double().t()).to(dtype)
+    check(got, ref, dtype, frac=0.05, atol=2.0 ** -7 * 2e-2 * float(ref.float().abs().max()))   # fp32 against float64 sums of K terms
+
+
 @pytest.mark.parametrize("rows,K,N", [(32, 2048, 2048), (8, 768, 768), (19, 1024, 512), (32, 256, 64)])
 def test_linear_packed_add_joins_the_residual_stream(hip, rows, K, N):
     """res_out = T(res + T(x W^T)) == the plain packed projection followed by a bf16 add, bit for bit; in place too."""
@@ -1401,8 +1432,6 @@ def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
     with pytest.raises(hip.FlashSTUHipError):
         hip.linear_packed(x33, pg, I)
     with pytest.raises(hip.FlashSTUHipError):
-        hip.linear_packed(x20, pg, I, nw, 1e-6)             # the norm prologue stops at 16 rows
-    with pytest.raises(hip.FlashSTUHipError):
         hip.glu_packed_norm(x20, x20, nw, 1e-6, pg, pg, I)  # 17..32 rows take the summed stream only: no delta
     with pytest.raises(hip.FlashSTUHipError):
         hip.glu_packed_norm(x33, None, nw, 1e-6, pg, pg, I)
@@ -1418,6 +1447,7 @@ def test_packed_kernels_refuse_rows_and_shapes_they_do_not_take(hip):
     assert hip.linear_packed(x20, pg, I).shape == (20, I)
     assert hip.glu_packed(x20, pg, pg, I).shape == (20, I)
     assert hip.glu_packed_norm(x20, None, nw, 1e-6, pg, pg, I)[1].shape == (20, I)
+    assert hip.linear_packed(x20, pg, I, nw, 1e-6).shape == (20, I)
 
 
 @pytest.mark.parametrize("rows,d,I,ks", [(8, 768, 9216, 16), (3, 256, 512, 4), (16, 1024, 4096, 8), (8, 2048, 24576, 16), (5, 48, 1024, 4), (8, 768, 9216, 4), (8, 768, 9216, 8),
