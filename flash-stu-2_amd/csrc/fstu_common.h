@@ -32,6 +32,8 @@ void fstu_set_error(const char* fmt, ...);
 // ---- library-internal launchers used by the decode-step driver.  `dyn`, when not null, is a device int[2]
 // {position, sampling step} read by the kernels instead of the host-side values, so that a captured graph of one
 // step can be replayed for every position.
+extern "C" int fstu_stu_lds_state_ring_from_hist(const void* hist, const float* a, float* state, void* ring, int R, int B,
+                                                 int S, int d, int t_last, int cap, int dtype, void* stream);
 int fstu_embed_strided(const int64_t* ids, int64_t id_stride, const void* table, void* out, int rows, int d, int vocab,
                        int dtype, void* stream, const int* dyn);
 int fstu_stu_step_lds_dyn(float* state, const void* xp, int ldxp, const float* a, const float* ce, void* y, int ldy,

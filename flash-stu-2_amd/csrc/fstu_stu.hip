@@ -980,7 +980,7 @@ template <> __device__ __forceinline__ float lsh_load<bf16_t>(__amdgpu_buffer_rs
 template <typename T, int MAXJ, int NG /* waves of a workgroup, each with up to MAXJ modes of the same 64 channels */>
 __global__ void __launch_bounds__(NG * 64)
 lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__ a, float* __restrict__ state, int S,
-                           int d, int t_last, int cap) {
+                           int d, int t_last, int cap, T* __restrict__ ring /*optional (B,R,d): the last R inputs*/, int R) {
   const int b = blockIdx.y, p = blockIdx.z;
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int jg = threadIdx.x >> 6;
@@ -1020,6 +1020,15 @@ lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__
           for (int i = 0; i < MAXJ; ++i) h[i] = fmaf(aj[i], h[i], xs[k]);
         }
       }
+      // the exact head's ring: position t in slot t % R for the last R positions, written by the first wave on the way
+      // (every slot is covered when the sequence has R positions; a shorter one leaves the others as the caller zeroed them)
+      if (ring && jg == 0 && tt0 + 32 * u + 30 > t_last - R) {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const int t = tt0 + 32 * u + 2 * k;
+          if (t <= t_last && t > t_last - R) DT<T>::st(ring + ((size_t)b * R + (t & (R - 1))) * d + c, xs[k]);
+        }
+      }
     }
   }
   float* st = state + (((size_t)b * 2 + p) * S) * d + c;
@@ -1030,7 +1039,14 @@ lds_state_from_hist_kernel(const T* __restrict__ hist, const float* __restrict__
 
 extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, float* state, int B, int S, int d,
                                             int t_last, int cap, int dtype, void* stream) {
+  return fstu_stu_lds_state_ring_from_hist(hist, a, state, nullptr, 0, B, S, d, t_last, cap, dtype, stream);
+}
+
+extern "C" int fstu_stu_lds_state_ring_from_hist(const void* hist, const float* a, float* state, void* ring, int R, int B, int S,
+                                                 int d, int t_last, int cap, int dtype, void* stream) {
   FSTU_REQUIRE(hist && a && state, FSTU_ENULL, "fstu_stu_lds_state_from_hist: null pointer");
+  FSTU_REQUIRE(ring == nullptr || (R >= 8 && R <= 1024 && (R & (R - 1)) == 0), FSTU_EARG,
+               "fstu_stu_lds_state_ring_from_hist: ring length %d is not a power of two in 8..1024", R);
   FSTU_REQUIRE(B >= 1 && d >= 1 && S >= 1 && S <= LSH_JG * LSH_MAXJ, FSTU_ESHAPE,
                "fstu_stu_lds_state_from_hist: S=%d outside 1..%d", S, LSH_JG * LSH_MAXJ);
   FSTU_REQUIRE(t_last >= -1 && t_last < cap, FSTU_EARG, "fstu_stu_lds_state_from_hist: t_last=%d cap=%d", t_last, cap);
@@ -1040,11 +1056,11 @@ extern "C" int fstu_stu_lds_state_from_hist(const void* hist, const float* a, fl
     // 8 waves of 8 modes: two waves per SIMD cover each other's dependent fused multiply-adds
     FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
                         hipLaunchKernelGGL((lds_state_from_hist_kernel<T, 8, 8>), grid, dim3(512), 0, (hipStream_t)stream,
-                                           (const T*)hist, a, state, S, d, t_last, cap));
+                                           (const T*)hist, a, state, S, d, t_last, cap, (T*)ring, R));
   } else {
     FSTU_DISPATCH_DTYPE(dtype, "fstu_stu_lds_state_from_hist",
                         hipLaunchKernelGGL((lds_state_from_hist_kernel<T, LSH_MAXJ, LSH_JG>), grid, dim3(256), 0,
-                                           (hipStream_t)stream, (const T*)hist, a, state, S, d, t_last, cap));
+                                           (hipStream_t)stream, (const T*)hist, a, state, S, d, t_last, cap, (T*)ring, R));
   }
   FSTU_CHECK_LAUNCH("fstu_stu_lds_state_from_hist");
   return FSTU_OK;

@@ -45,6 +45,7 @@ SIGNATURES = {
     "fstu_stu_res_inproj_step": [_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_scan_lds": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_lds_state_from_hist": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_lds_state_ring_from_hist": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_direct": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_fft_length": [_i],
@@ -557,16 +558,23 @@ def stu_res_inproj_step(x: torch.Tensor, partial: torch.Tensor, norm_w: torch.Te
     return x_out, y
 
 
-def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, state: Optional[torch.Tensor] = None) -> torch.Tensor:
-    _dev(hist, a, state)
+def stu_lds_state_from_hist(hist: torch.Tensor, a: torch.Tensor, t_last: int, state: Optional[torch.Tensor] = None,
+                            ring: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """state (B,2,S,d) fp32 of the recurrence after positions 0..t_last of hist (B,cap,d).  ring (B,R,d), optional:
+    also receives hist[:, t] in slot t % R for the last R positions (slots a shorter sequence does not reach stay)."""
+    _dev(hist, a, state, ring)
     B, cap, d = hist.shape
     S = a.numel()
     assert a.dtype == torch.float32
     if state is None:
         state = torch.empty(B, 2, S, d, dtype=torch.float32, device=hist.device)
     assert state.shape == (B, 2, S, d) and state.dtype == torch.float32
-    _check(load().fstu_stu_lds_state_from_hist(_p(hist), _p(a), _p(state), B, S, d, t_last, cap, _dt(hist), _stream()),
-           "fstu_stu_lds_state_from_hist")
+    R = 0
+    if ring is not None:
+        R = ring.shape[1]
+        assert ring.shape == (B, R, d) and ring.dtype == hist.dtype and ring.is_contiguous()
+    _check(load().fstu_stu_lds_state_ring_from_hist(_p(hist), _p(a), _p(state), _p(ring), R, B, S, d, t_last, cap, _dt(hist),
+                                                    _stream()), "fstu_stu_lds_state_ring_from_hist")
     return state
 
 

@@ -344,8 +344,16 @@ class STU(nn.Module):
         if self.decode_mode() == "lds" and (self.use_approx or self._exact_lds_ok()):
             a = (self.lds_single_params()[0] if self._single_lds_ok() else
                  self.lds_params()[0] if self.use_approx else self.bank_lds_params()[0])
-            state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1)
-            return (self._ring_from_sequence(src) if self.use_approx else src.new_empty(B, 0, d), state, pos)
+            # the exact head's ring of the last projected inputs is written by the same launch on its way through them
+            fir = self.lds_fir() if self.use_approx else None
+            if fir is None:
+                ring = None
+            elif T >= fir.shape[0]:
+                ring = src.new_empty(B, fir.shape[0], d)          # every slot is written
+            else:
+                ring = src.new_zeros(B, fir.shape[0], d)          # zeros before the first position
+            state = _hip.stu_lds_state_from_hist(src.contiguous(), a, T - 1, ring=ring)
+            return (ring if ring is not None else src.new_empty(B, 0, d), state, pos)
         cap = max(self.config.seq_len, T)
         hist = src.new_zeros(B, cap, d)
         hist[:, :T] = src

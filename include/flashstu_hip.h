@@ -216,6 +216,11 @@ int fstu_stu_scan_lds(const void* xp, int64_t x_bstride, int64_t x_tstride, cons
  *   of parity p that is <= t_last.  hist is (B,cap,d). */
 int fstu_stu_lds_state_from_hist(const void* hist, const float* a, float* state, int B, int S, int d,
                                  int t_last, int cap, int dtype, void* stream);
+/* The same launch also leaving the exact head's ring (fstu_stu_step_lds_pair): ring (B,R,d) in the model dtype receives
+ * hist[b,t,:] in slot t % R for the last R positions t <= t_last (R a power of two, 8..1024); slots that a sequence
+ * shorter than R does not reach are left as they are (the caller zeroes them).  ring == NULL: as above. */
+int fstu_stu_lds_state_ring_from_hist(const void* hist, const float* a, float* state, void* ring, int R, int B, int S,
+                                      int d, int t_last, int cap, int dtype, void* stream);
 
 /* ---- STU prefill convolution (approx mode), time-domain form ---------------
  * y[b,t,c] = T(E+O) + T(E-O)  (or T(E+O) if single_branch) with E/O the even-/

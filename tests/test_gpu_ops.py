@@ -659,6 +659,25 @@ def test_stu_step_lds_pair_with_the_odd_lag_sum_handed_on(hip, dtype, S, R, T0):
     assert torch.equal(st_c, st_p) and (not R or torch.equal(ring_c, ring_p))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,R", [(600, 64), (64, 64), (65, 64), (40, 64), (1, 8), (300, 256), (1000, 8)])
+def test_state_from_hist_also_leaves_the_ring(hip, dtype, T, R):
+    """The launch that scans a prompt's projected inputs into the recurrence state also writes the exact head's ring:
+    position t in slot t % R for the last R positions, zeros (the caller's) where a short prompt has none; the state
+    is the one the launch without a ring leaves."""
+    B, d, S = 3, 200, 64
+    g = gen(94)
+    xp = dev(torch.randn(B, T, d, generator=g).to(dtype))
+    a = dev(torch.rand(S, generator=g) * 0.95)
+    ring = torch.zeros(B, R, d, dtype=dtype, device="cuda") if T < R else torch.full((B, R, d), float("nan"), dtype=dtype, device="cuda")
+    st = hip.stu_lds_state_from_hist(xp, a, T - 1, ring=ring)
+    assert torch.equal(st, hip.stu_lds_state_from_hist(xp, a, T - 1))
+    want = torch.zeros(B, R, d, dtype=dtype, device="cuda")
+    for t in range(max(0, T - R), T):
+        want[:, t % R] = xp[:, t]
+    assert torch.equal(ring, want)
+
+
 @pytest.mark.parametrize("R", [8, 32, 128, 256])
 def test_stu_step_lds_exact_head(hip, R):
     """The exact head of the distilled filter: fir[s] = phi_proj[s] - fitted filter for the first R lags, applied to a
