@@ -516,8 +516,12 @@ def run_ref(args, torch, _hip):
     ms = (time.perf_counter() - t0) / K * 1e3
     assert bool(torch.isfinite(y.float()).all())
     # the two launches of the operator on their own (HIP events on the launch stream)
-    ms_proj, xp = timed(lambda: stu._project(x), K)
-    ms_conv, _ = timed(lambda: stu._convolve(xp), K)
+    # (x @ M_inputs as time-major slabs, the convolution on them, the transpose of its result)
+    ms_proj, xt = timed(lambda: stu._project_time_major(x), K)
+    yt = torch.empty_like(xt)
+    spec = stu.filter_spectrum(_hip.fft_length(L))
+    ms_conv, _ = timed(lambda: _hip.stu_conv_fft_strided(xt.transpose(1, 2), spec, yt.transpose(1, 2)), K)
+    ms_tr, _ = timed(lambda: _hip.transpose(yt), K)
     conv_bytes = 2 * B * L * d * 2 + L * d * 2          # x_proj in, y out, the filter once
     conv_gbps = conv_bytes / (ms_conv * 1e-3) / 1e9
     flops = 2.0 * B * L * d * d
@@ -530,7 +534,9 @@ def run_ref(args, torch, _hip):
                        "batch": B, "L": L, "d": d, "K": Kf,
                        "published": {"ms_per_call": published_ms, "hardware": "NVIDIA H100 PCIe (another GPU: context, not a like-for-like bar)",
                                      "source": "tests/tilling/standard_memory_profile.txt:48-59"}},
-            "kernels_ms": {"x @ M_inputs (gemm_bf16_kernel)": ms_proj, "spectral convolution (fft_conv_kernel)": ms_conv,
+            "kernels_ms": {"x @ M_inputs (gemm_bf16_kernel, time-major output)": ms_proj,
+                           "spectral convolution (fft_conv_kernel on time-major slabs)": ms_conv,
+                           "result back to (L, d) (transpose_tiles_kernel)": ms_tr,
                            "projection_tflops": flops / (ms_proj * 1e-3) / 1e12},
             "roofline": {"bound": "hbm", "kernel": "fft_conv_kernel (spectral convolution of the projected inputs, both sign branches, one column per workgroup)",
                          "achieved": conv_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": conv_gbps / HBM_PEAK_GBPS,

@@ -705,6 +705,17 @@ extern "C" int fstu_stu_conv_fft(const void* xp, const float* spec, void* y, con
                          T_, d, 1, n, single_branch ? 1 : 0, dtype, stream);
 }
 
+// The same convolution on strided operands: element (b, t, c) of x at x_strides[0]*b + x_strides[1]*t + x_strides[2]*c
+// (elements), y likewise.  Time-major operands (a time stride of 1) make the loads and stores of the one-column
+// kernel coalesce, which is what a few long sequences want (few channels x batch rows, transform length 8192 or more).
+extern "C" int fstu_stu_conv_fft_strided(const void* xp, const int64_t* x_strides, const float* spec, void* y,
+                                         const int64_t* y_strides, const float* tw, int B, int T_, int d, int n,
+                                         int single_branch, int dtype, void* stream) {
+  FSTU_REQUIRE(xp && x_strides && spec && y && y_strides && tw, FSTU_ENULL, "fstu_stu_conv_fft_strided: null pointer");
+  return conv_fft_launch("fstu_stu_conv_fft_strided", xp, x_strides[0], x_strides[1], x_strides[2], spec, y, nullptr, y_strides[0],
+                         y_strides[1], 0, y_strides[2], tw, B, T_, d, 1, n, single_branch ? 1 : 0, dtype, stream);
+}
+
 extern "C" int fstu_stu_conv_bank_fft(const void* x, const int64_t* x_strides, const float* spec, void* u_plus,
                                       void* u_minus, const int64_t* u_strides, const float* tw, int B, int T_, int d,
                                       int K, int n, int dtype, void* stream) {

@@ -39,3 +39,39 @@ extern "C" int fstu_pack_rows(const void* W, void* Wp, int N, int K, void* strea
   FSTU_CHECK_LAUNCH("fstu_pack_rows");
   return FSTU_OK;
 }
+
+// ---------------------------------------------------------------- transpose of the last two dimensions
+// out[b][c][r] = in[b][r][c] through 64 x 64 tiles in LDS (rows padded by one 32-bit word so that the transposed reads
+// fall into different banks): both the loads and the stores walk the contiguous dimension.  Used to hand a few long
+// sequences to the spectral convolution time-major (flash_stu/modules/stu.py:89-98 of the reference convolves
+// (B, L, d) tensors along L).
+template <typename T>
+__global__ void __launch_bounds__(256)
+transpose_tiles_kernel(const T* __restrict__ in, T* __restrict__ out, int R, int C) {
+  __shared__ T tile[64][64 + 4 / sizeof(T) * 1];
+  const int b = blockIdx.z, r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int j = threadIdx.x & 63, i0 = threadIdx.x >> 6;
+  const T* src = in + (size_t)b * R * C;
+  T* dst = out + (size_t)b * R * C;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int i = i0 + 4 * k;
+    if (r0 + i < R && c0 + j < C) tile[i][j] = src[(size_t)(r0 + i) * C + c0 + j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int i = i0 + 4 * k;
+    if (c0 + i < C && r0 + j < R) dst[(size_t)(c0 + i) * R + r0 + j] = tile[j][i];
+  }
+}
+
+extern "C" int fstu_transpose(const void* in, void* out, int B, int R, int C, int dtype, void* stream) {
+  FSTU_REQUIRE(in && out && in != out, FSTU_ENULL, "fstu_transpose: null or aliased pointers");
+  FSTU_REQUIRE(B >= 1 && B <= 65535 && R >= 1 && C >= 1 && (R + 63) / 64 <= 65535, FSTU_ESHAPE, "fstu_transpose: B=%d R=%d C=%d", B, R, C);
+  const dim3 grid((C + 63) / 64, (R + 63) / 64, B);
+  FSTU_DISPATCH_DTYPE(dtype, "fstu_transpose",
+                      hipLaunchKernelGGL(transpose_tiles_kernel<T>, grid, dim3(256), 0, (hipStream_t)stream, (const T*)in, (T*)out, R, C));
+  FSTU_CHECK_LAUNCH("fstu_transpose");
+  return FSTU_OK;
+}

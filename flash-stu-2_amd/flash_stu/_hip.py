@@ -52,6 +52,8 @@ SIGNATURES = {
     "fstu_fft_twiddles": [_vp, _i, _vp],
     "fstu_stu_fft_filter": [_vp, _i64, _i64, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_fft": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_stu_conv_fft_strided": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "fstu_transpose": [_vp, _vp, _i, _i, _i, _i, _vp],
     "fstu_stu_conv_bank_fft": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_append": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "fstu_kv_fill": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -649,6 +651,36 @@ def stu_conv_fft(xp: torch.Tensor, spec: torch.Tensor, single_branch: bool = Fal
         out = torch.empty_like(xp)
     _check(load().fstu_stu_conv_fft(_p(xp), _p(spec), _p(out), _p(fft_twiddles(n, xp.device)), B, T, d, n,
                                     int(single_branch), _dt(xp), _stream()), "fstu_stu_conv_fft")
+    return out
+
+
+def transpose(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(B,R,C) -> (B,C,R), contiguous."""
+    _dev(x, out)
+    B, R, C = x.shape
+    if out is None:
+        out = torch.empty(B, C, R, dtype=x.dtype, device=x.device)
+    assert out.shape == (B, C, R) and out.dtype == x.dtype and out.is_contiguous() and out.data_ptr() != x.data_ptr()
+    _check(load().fstu_transpose(_p(x), _p(out), B, R, C, _dt(x), _stream()), "fstu_transpose")
+    return out
+
+
+def stu_conv_fft_strided(xp: torch.Tensor, spec: torch.Tensor, out: torch.Tensor, single_branch: bool = False) -> torch.Tensor:
+    """xp, out: strided views of logical shape (B,T,d) (e.g. the transposed view of a time-major slab (B,d,T));
+    spec (d,n,2) as for stu_conv_fft.  Written into out."""
+    _dev(spec)
+    if not xp.is_cuda or not out.is_cuda:
+        raise FlashSTUHipError("tensor is not on the GPU: the HIP path has no CPU fallback")
+    B, T, d = xp.shape
+    n = spec.shape[1]
+    if spec.shape != (d, n, 2) or spec.dtype != torch.float32 or not spec.is_contiguous():
+        raise FlashSTUHipError(f"spec must be contiguous ({d}, n, 2) float32")
+    if tuple(out.shape) != (B, T, d) or out.dtype != xp.dtype:
+        raise FlashSTUHipError("out must have the logical shape and dtype of xp")
+    xs = (ctypes.c_int64 * 3)(*xp.stride())
+    ys = (ctypes.c_int64 * 3)(*out.stride())
+    _check(load().fstu_stu_conv_fft_strided(_p(xp), xs, _p(spec), _p(out), ys, _p(fft_twiddles(n, xp.device)), B, T, d, n,
+                                            int(single_branch), _dt(xp), _stream()), "fstu_stu_conv_fft_strided")
     return out
 
 

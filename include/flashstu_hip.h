@@ -269,6 +269,15 @@ int fstu_stu_fft_filter(const void* filt, int64_t f_ls, int64_t f_cs, float* spe
                         int ncols, int n, int single_branch, int dtype, void* stream);
 int fstu_stu_conv_fft(const void* xp, const float* spec, void* y, const float* tw, int B, int T, int d, int n,
                       int single_branch, int dtype, void* stream);
+/* The same on strided operands: element (b,t,c) of xp at x_strides[0]*b + x_strides[1]*t + x_strides[2]*c (elements), y
+ * likewise.  With a time stride of 1 (time-major slabs (B,d,T)) every load and store of the one-column kernel is
+ * coalesced: the form for a few long sequences (transform length 8192 or 16384 and fewer than 512 groups of 8
+ * channels x batch rows), where the channel-contiguous kernel leaves compute units idle. */
+int fstu_stu_conv_fft_strided(const void* xp, const int64_t* x_strides, const float* spec, void* y, const int64_t* y_strides,
+                              const float* tw, int B, int T, int d, int n, int single_branch, int dtype, void* stream);
+/* out[b][c][r] = in[b][r][c] for (B,R,C) tensors in either dtype (out must not be in): the copy that hands (B,L,d)
+ * activations to fstu_stu_conv_fft_strided as time-major slabs and takes the result back. */
+int fstu_transpose(const void* in, void* out, int B, int R, int C, int dtype, void* stream);
 int fstu_stu_conv_bank_fft(const void* x, const int64_t* x_strides, const float* spec, void* u_plus, void* u_minus,
                            const int64_t* u_strides, const float* tw, int B, int T, int d, int K, int n, int dtype,
                            void* stream);

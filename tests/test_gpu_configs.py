@@ -40,6 +40,39 @@ def _exact_stu(dtype, d, L, K, seed):
     return stu.cuda(), phi, p
 
 
+@pytest.mark.parametrize("dtype,B,T,d", [(torch.bfloat16, 1, 4096, 256), (torch.bfloat16, 2, 2300, 128), (torch.float32, 1, 2304, 64)])
+def test_stu_forward_of_a_few_long_sequences_goes_time_major(dtype, B, T, d):
+    """Approx-mode STU.forward on a few long sequences (the shape class of the reference's own benchmark,
+    tests/benchmark_tilling.py:157-165): without a cache the projected inputs are formed as time-major slabs by the
+    prompt GEMM with swapped operands and convolved as such; with a cache they are transposed in front of the same
+    convolution.  Both give the oracle's values, and the same bits as each other where the GEMM is the same."""
+    from flash_stu import STU, FlashSTUConfig
+    L, K = 4096, 8
+    cfg = FlashSTUConfig(n_embd=d, n_heads=1, n_layers=1, seq_len=L, num_eigh=K, use_approx=True, torch_dtype=dtype,
+                         vocab_size=3, stu_decode_mode="lds")
+    phi = _filters(L, K, dtype)
+    g = torch.Generator().manual_seed(11)
+    stu = STU(cfg, phi, O.nearest_power_of_two(2 * L - 1, True))
+    with torch.no_grad():
+        stu.M_inputs.copy_((torch.randn(d, d, generator=g) / math.sqrt(d)).to(dtype))
+        stu.M_filters.copy_((torch.randn(K, d, generator=g) / math.sqrt(K)).to(dtype))
+    p = {"M_inputs": stu.M_inputs.detach().clone(), "M_filters": stu.M_filters.detach().clone()}
+    stu = stu.cuda()
+    x = torch.randn(B, T, d, generator=g).to(dtype)
+    assert stu._few_long_sequences(B, T, d, x.element_size())
+    y = stu(x.cuda())
+    y2, _ = stu(x.cuda(), use_cache=True)
+    ref = O.stu_forward(x, phi, p, 8192, use_approx=True).float()
+    scale = float(ref.abs().max())
+    for out in (y, y2):
+        err = (out.float().cpu() - ref).abs()
+        if dtype == torch.float32:
+            assert float(err.max()) <= 2e-4 * scale
+        else:
+            assert float(err.max()) <= 3e-2 * scale and float(err.mean()) <= 3e-3 * scale
+    assert float((y != y2).float().mean()) <= (0.0 if dtype == torch.float32 else 0.02)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("T", [200, 384, 20])
 def test_c3_exact_mode_ragged_lengths_and_both_dtypes(dtype, T):

@@ -660,6 +660,30 @@ def test_stu_step_lds_pair_with_the_odd_lag_sum_handed_on(hip, dtype, S, R, T0):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,R,C", [(1, 4096, 2048), (3, 100, 70), (2, 64, 64), (1, 1, 5), (2, 129, 1)])
+def test_transpose(hip, dtype, B, R, C):
+    x = dev(torch.randn(B, R, C, generator=gen(95)).to(dtype))
+    assert torch.equal(hip.transpose(x), x.transpose(1, 2).contiguous())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,T,d", [(1, 4096, 256), (2, 2100, 64), (1, 600, 40)])
+def test_stu_conv_fft_on_time_major_slabs(hip, dtype, B, T, d):
+    """The strided entry on time-major slabs gives the bits of the channel-contiguous call (every transform length,
+    both kernels behind them)."""
+    g = gen(96)
+    xp = dev(torch.randn(B, T, d, generator=g).to(dtype))
+    filt = dev((torch.randn(T, d, generator=g) / 30).to(dtype))
+    n = hip.fft_length(T)
+    spec = hip.stu_fft_filter(filt, n)
+    want = hip.stu_conv_fft(xp, spec)
+    xt = hip.transpose(xp)
+    yt = torch.empty_like(xt)
+    hip.stu_conv_fft_strided(xt.transpose(1, 2), spec, yt.transpose(1, 2))
+    assert torch.equal(hip.transpose(yt), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,R", [(600, 64), (64, 64), (65, 64), (40, 64), (1, 8), (300, 256), (1000, 8)])
 def test_state_from_hist_also_leaves_the_ring(hip, dtype, T, R):
     """The launch that scans a prompt's projected inputs into the recurrence state also writes the exact head's ring:
